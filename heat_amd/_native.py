@@ -1,0 +1,176 @@
+"""
+ctypes binding of libhkm, the C-ABI library holding the gfx950 kernels (see include/hkm.h).
+
+The library is built in-tree (``heat_amd/csrc/libhkm.so``) by ``heat_amd/csrc/Makefile``.  There
+is no fallback: if the library is missing, every compute entry point raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int32, c_int64, c_size_t, c_void_p
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
+_lib: Optional[ctypes.CDLL] = None
+
+HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
+WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE = 1, 2, 3, 4
+
+# name -> (restype, argtypes); must list every symbol declared in include/hkm.h
+SIGNATURES = {
+    "hkm_version": (ctypes.c_int, []),
+    "hkm_last_error": (c_char_p, []),
+    "hkm_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int32]),
+    "hkm_assign_kernel_name": (c_char_p, [c_int64, c_int32, c_int32]),
+    "hkm_assign_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                      c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_update_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
+                                      c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_shift_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
+    "hkm_functional_value_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_cdist_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
+                                     c_void_p, c_int64, c_int32, c_void_p]),
+    "hkm_widen_labels_i64": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
+}
+
+
+class HkmError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libhkm error {code}: {message}")
+        self.code = code
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load libhkm once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(
+                f"{_LIB_PATH} is missing: build it with `make -C heat_amd/csrc` "
+                "(or __graft_entry__.build()). heat_amd has no CPU fallback."
+            )
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().hkm_last_error().decode()
+
+
+def check(rc: int) -> None:
+    if rc != HKM_OK:
+        raise HkmError(rc, last_error())
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "heat_amd computes on the GPU only: got a tensor on "
+                f"'{t.device}'. Create the DNDarray with device='gpu'."
+            )
+
+
+class Workspace:
+    """A reusable device scratch buffer, grown on demand."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self.buf: Optional[torch.Tensor] = None
+
+    def get(self, nbytes: int) -> torch.Tensor:
+        if self.buf is None or self.buf.numel() < nbytes:
+            self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+        return self.buf
+
+
+def workspace_bytes(n: int, d: int, k: int, flags: int) -> int:
+    return int(load().hkm_workspace_bytes(n, d, k, flags))
+
+
+def assign_kernel_name(n: int, d: int, k: int) -> str:
+    return load().hkm_assign_kernel_name(n, d, k).decode()
+
+
+def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optional[torch.Tensor],
+           ws: Workspace) -> None:
+    _require_gpu(x, c, labels, min_d2)
+    n, d = x.shape
+    k = c.shape[0]
+    need = workspace_bytes(n, d, k, WS_ASSIGN)
+    buf = ws.get(need)
+    check(load().hkm_assign_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k, c.stride(0) if k > 1 else d,
+                                _ptr(labels), _ptr(min_d2), _ptr(buf), buf.numel(), _stream()))
+
+
+def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: Optional[torch.Tensor],
+           ws: Workspace) -> None:
+    _require_gpu(x, labels, c_new, counts)
+    n, d = x.shape
+    k = c_new.shape[0]
+    need = workspace_bytes(n, d, k, WS_UPDATE)
+    buf = ws.get(need)
+    check(load().hkm_update_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k, _ptr(c_new),
+                                c_new.stride(0) if k > 1 else d, _ptr(counts), _ptr(buf), buf.numel(), _stream()))
+
+
+def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: torch.Tensor,
+               shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace) -> None:
+    _require_gpu(x, c, c_new, labels, shift, sse)
+    n, d = x.shape
+    k = c.shape[0]
+    flags = WS_LLOYD | (WS_SSE if sse is not None else 0)
+    need = workspace_bytes(n, d, k, flags)
+    buf = ws.get(need)
+    check(load().hkm_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
+                                    _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
+
+
+def shift(c_old: torch.Tensor, c_new: torch.Tensor, out: torch.Tensor) -> None:
+    _require_gpu(c_old, c_new, out)
+    k, d = c_old.shape
+    check(load().hkm_shift_f32(_ptr(c_old), _ptr(c_new), k, d, _ptr(out), _stream()))
+
+
+def functional_value(min_d2: torch.Tensor, out: torch.Tensor, ws: Workspace) -> None:
+    _require_gpu(min_d2, out)
+    n = min_d2.numel()
+    need = workspace_bytes(n, 1, 1, WS_ASSIGN)
+    buf = ws.get(need)
+    check(load().hkm_functional_value_f32(_ptr(min_d2), n, _ptr(out), _ptr(buf), buf.numel(), _stream()))
+
+
+def cdist(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, sqrt: bool = True) -> None:
+    _require_gpu(x, y, out)
+    m, d = x.shape
+    nn = y.shape[0]
+    check(load().hkm_cdist_f32(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn, y.stride(0) if nn > 1 else d,
+                               d, _ptr(out), out.stride(0) if m > 1 else nn, 1 if sqrt else 0, _stream()))
+
+
+def widen_labels(labels32: torch.Tensor, out64: torch.Tensor) -> None:
+    _require_gpu(labels32, out64)
+    check(load().hkm_widen_labels_i64(_ptr(labels32), labels32.numel(), _ptr(out64), _stream()))

@@ -1,0 +1,3 @@
+"""Clustering estimators (subset of heat/cluster)."""
+from .kmeans import KMeans  # noqa: F401
+from ._kcluster import _KCluster  # noqa: F401

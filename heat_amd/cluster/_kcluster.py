@@ -1,0 +1,173 @@
+"""
+Base of the k-clustering estimators, with the interface of heat/cluster/_kcluster.py:13-415.
+
+The reference composes assignment from generic array ops (cdist -> argmin); here
+``_assign_to_cluster`` is one call into the fused distance+argmin kernel, so the N x K matrix is
+never built.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from .. import _native
+from ..core import types
+from ..core.base import BaseEstimator, ClusteringMixin
+from ..core.dndarray import DNDarray
+
+
+class _KCluster(ClusteringMixin, BaseEstimator):
+    def __init__(self, metric, n_clusters: int, init: Union[str, DNDarray], max_iter: int, tol: float,
+                 random_state: Optional[int]):  # noqa: D107
+        self.n_clusters = n_clusters
+        self.init = init
+        self.max_iter = max_iter
+        self.tol = tol
+        self.random_state = random_state
+
+        self._metric = metric
+        self._cluster_centers = None
+        self._functional_value = None
+        self._labels = None
+        self._inertia = None
+        self._n_iter = None
+        self._p = None
+        self._ws = None
+
+    # ---- read-only results (heat/cluster/_kcluster.py:63-98) -----------------------------------
+    @property
+    def cluster_centers_(self) -> DNDarray:
+        return self._cluster_centers
+
+    @property
+    def labels_(self) -> DNDarray:
+        return self._labels
+
+    @property
+    def inertia_(self):
+        """Squared centroid movement of the last iteration (what the reference stores, kmeans.py:141)."""
+        return self._inertia
+
+    @property
+    def n_iter_(self) -> int:
+        return self._n_iter
+
+    @property
+    def functional_value_(self) -> DNDarray:
+        return self._functional_value
+
+    # ---- helpers ---------------------------------------------------------------------------
+    def _workspace(self, device: torch.device) -> _native.Workspace:
+        if self._ws is None or self._ws.device != device:
+            self._ws = _native.Workspace(device)
+        return self._ws
+
+    @staticmethod
+    def _local_f32(x: DNDarray) -> torch.Tensor:
+        """The local tensor as a row-major float32 matrix (ints are widened as the reference's
+        promote(X, C, float32) does; float64 is outside the float32 kernels)."""
+        t = x.larray
+        if t.dim() != 2:
+            raise NotImplementedError("Only 2D data matrices are currently supported")
+        if t.dtype == torch.float64 or types.promote_types(x.dtype, types.float32) is not types.float32:
+            raise NotImplementedError(
+                f"the gfx950 kernels compute in float32; input dtype {x.dtype.__name__} promotes to float64"
+            )
+        if t.dtype != torch.float32:
+            t = t.to(torch.float32)
+        if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+            t = t.contiguous()
+        return t
+
+    @staticmethod
+    def _check_split(x: DNDarray) -> None:
+        # the reference raises this from cdist (heat/spatial/distance.py:386-390)
+        if x.split is not None and x.split != 0:
+            raise NotImplementedError(
+                f"Input splits were X.split = {x.split}, Y.split = None. Splittings other than 0 or None currently not supported."
+            )
+
+    def _initialize_cluster_centers(self, x: DNDarray, oversampling: float, iter_multiplier: float):
+        """
+        Initial centroids; checks in the order of heat/cluster/_kcluster.py:116-143,276-281.
+        Built: ``"random"`` (K rows drawn with a generator seeded by ``random_state``) and an explicit
+        (K, D) DNDarray, which is copied so later changes by the caller do not leak in.
+        """
+        if not isinstance(x, DNDarray):
+            raise ValueError(f"Input x needs to be a ht.DNDarray, but was {type(x)}")
+        if oversampling < 2:
+            raise ValueError(f"Oversampling factor should be at least 2, but was {oversampling}")
+        if iter_multiplier < 1:
+            raise ValueError(f"Iteration multiplier should be at least 1, but was {iter_multiplier}")
+
+        if isinstance(self.init, str) and self.init == "random":
+            gen = torch.Generator(device="cpu")
+            if self.random_state is not None:
+                gen.manual_seed(int(self.random_state))
+            else:
+                gen.seed()
+            # same index range as the reference: randint(0, n - 1) excludes the last row
+            hi = max(x.shape[0] - 1, 1)
+            idx = torch.randint(0, hi, (self.n_clusters,), generator=gen).to(x.larray.device)
+            cent = x.larray[idx, :].clone()
+            self._cluster_centers = DNDarray(cent, tuple(cent.shape), x.dtype, None, x.device, x.comm, True)
+        elif isinstance(self.init, DNDarray):
+            if len(self.init.shape) != 2:
+                raise ValueError(f"passed centroids need to be two-dimensional, but are {len(self.init)}")
+            if self.init.shape[0] != self.n_clusters or self.init.shape[1] != x.shape[1]:
+                raise ValueError("passed centroids do not match cluster count or data shape")
+            self._cluster_centers = self.init.resplit(None)
+        elif isinstance(self.init, str) and self.init == "probability_based":
+            if x.split is None or x.split == 0:
+                raise NotImplementedError('init="probability_based" (k-means||) is not built in heat_amd')
+            raise NotImplementedError("Not implemented for other splitting-axes")
+        elif isinstance(self.init, str) and self.init == "batchparallel":
+            if x.split == 0:
+                raise NotImplementedError('init="batchparallel" is not built in heat_amd')
+            raise NotImplementedError(
+                f"Batch parallel initalization only implemented for split = 0, but split was {x.split}"
+            )
+        else:
+            raise ValueError(
+                'init needs to be one of "random", ht.DNDarray, "kmeans++", or "batchparallel", but was {}'.format(
+                    self.init
+                )
+            )
+
+    def _assign_to_cluster(self, x: DNDarray, eval_functional_value: bool = False) -> DNDarray:
+        """
+        (N, 1) int64 labels of the closest centroid, ``split = x.split``; optionally sets
+        ``functional_value_`` = ||min_k dist||_2 ** 2 (heat/cluster/_kcluster.py:352-370).
+        """
+        self._check_split(x)
+        xt = self._local_f32(x)
+        ct = self._local_f32(self._cluster_centers)
+        if xt.shape[1] != ct.shape[1]:
+            raise ValueError("Inputs must have same shape[1]")
+        dev = xt.device
+        n = xt.shape[0]
+        ws = self._workspace(dev)
+        lab32 = torch.empty((n,), dtype=torch.int32, device=dev)
+        min_d2 = torch.empty((n,), dtype=torch.float32, device=dev) if eval_functional_value else None
+        _native.assign(xt, ct, lab32, min_d2, ws)
+        lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
+        _native.widen_labels(lab32, lab64)
+        if eval_functional_value:
+            fv = torch.empty((), dtype=torch.float32, device=dev)
+            _native.functional_value(min_d2, fv, ws)
+            self._functional_value = DNDarray(fv, (), types.float32, None, x.device, x.comm, True)
+        return DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
+
+    def _update_centroids(self, x: DNDarray, matching_centroids: DNDarray):
+        raise NotImplementedError()
+
+    def fit(self, x: DNDarray):
+        raise NotImplementedError()
+
+    def predict(self, x: DNDarray) -> DNDarray:
+        """Index of the closest centroid for every row of ``x`` (heat/cluster/_kcluster.py:398-415)."""
+        if not isinstance(x, DNDarray):
+            raise ValueError(f"input needs to be a ht.DNDarray, but was  {type(x)}")
+        return self._assign_to_cluster(x, eval_functional_value=True)

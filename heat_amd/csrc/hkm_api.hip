@@ -1,0 +1,231 @@
+// C ABI of libhkm: host-side validation, workspace carving and kernel dispatch.
+// Nothing here allocates device memory or synchronises; every entry point only enqueues kernels.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "hkm_common.h"
+
+namespace hkm {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HKM_EHIP, "%s: %s", what, hipGetErrorString(e));
+    return HKM_OK;
+}
+
+int num_cus() {
+    static thread_local int cached_dev = -1;
+    static thread_local int cached_cus = 256;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev != cached_dev) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cached_cus = n;
+        cached_dev = dev;
+    }
+    return cached_cus;
+}
+
+AssignKind assign_kind(int32_t D, int32_t K) {
+    if (D <= 16) return ASSIGN_VALU;
+    if (D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024) return ASSIGN_MFMA_RESIDENT;
+    return ASSIGN_MFMA_STREAM;
+}
+
+static size_t cn_pad(int32_t K) { return (size_t(K) + 127) / 128 * 128; }
+
+Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
+    Workspace w;
+    memset(&w, 0, sizeof(w));
+    char* p = static_cast<char*>(base);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* r = p ? p + off : nullptr;
+        off += align_up(bytes, 256);
+        return r;
+    };
+    w.red = reinterpret_cast<double*>(take(size_t(RED_SLOTS) * sizeof(double)));
+    if (flags & HKM_WS_ASSIGN) w.cn = reinterpret_cast<float*>(take(cn_pad(K) * sizeof(float)));
+    if (flags & HKM_WS_UPDATE) {
+        const UpdateGeom g = update_geom(N, D, K);
+        w.part_sum = reinterpret_cast<float*>(take(size_t(g.S) * K * g.J * 32 * sizeof(float)));
+        w.part_cnt = reinterpret_cast<int32_t*>(take(size_t(g.S) * K * sizeof(int32_t)));
+        w.counts = reinterpret_cast<int64_t*>(take(size_t(K) * sizeof(int64_t)));
+    }
+    if (flags & HKM_WS_SSE) w.min_d2 = reinterpret_cast<float*>(take(size_t(N < 1 ? 1 : N) * sizeof(float)));
+    w.total = off;
+    return w;
+}
+
+static int check_matrix(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
+    if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);
+    if (reinterpret_cast<uintptr_t>(p) & 3u) return fail(HKM_EINVAL, "%s is not 4-byte aligned", name);
+    if (ld < cols) return fail(HKM_EINVAL, "leading dimension of %s (%lld) < columns (%d)", name, (long long)ld, cols);
+    return HKM_OK;
+}
+
+static int check_shape(int64_t N, int32_t D, int32_t K) {
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
+    return HKM_OK;
+}
+
+static int check_ws(void* ws, size_t ws_bytes, size_t need) {
+    if (!ws) return fail(HKM_EWORKSPACE, "workspace is NULL (%zu bytes needed)", need);
+    if (reinterpret_cast<uintptr_t>(ws) & 255u) return fail(HKM_EWORKSPACE, "workspace is not 256-byte aligned");
+    if (ws_bytes < need) return fail(HKM_EWORKSPACE, "workspace too small: %zu bytes given, %zu needed", ws_bytes, need);
+    return HKM_OK;
+}
+
+static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                     int64_t ldc, int32_t* labels, float* min_d2, const Workspace& w,
+                     hipStream_t st) {
+    if (N == 0) return HKM_OK;
+    switch (assign_kind(D, K)) {
+        case ASSIGN_VALU:
+            return launch_assign_valu(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
+        case ASSIGN_MFMA_RESIDENT:
+            return launch_assign_mfma_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
+        default: {
+            int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
+            if (rc) return rc;
+            return launch_assign_mfma_stream(X, N, D, ldx, C, K, ldc, w.cn, labels, min_d2, st);
+        }
+    }
+}
+
+}  // namespace hkm
+
+using namespace hkm;
+
+extern "C" {
+
+int hkm_version(void) { return 100; }
+
+const char* hkm_last_error(void) { return g_err; }
+
+size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags) {
+    if (N < 0 || D < 1 || K < 1) return 0;
+    return carve(nullptr, N, D, K, flags).total;
+}
+
+const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K) {
+    (void)N;
+    if (D < 1 || K < 1) return "invalid";
+    switch (assign_kind(D, K)) {
+        case ASSIGN_VALU: return "valu";
+        case ASSIGN_MFMA_RESIDENT: return "mfma_resident";
+        default: return "mfma_stream";
+    }
+}
+
+int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                   int64_t ldc, int32_t* labels, float* min_d2, void* ws, size_t ws_bytes,
+                   void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C", C, K, D, ldc))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    const size_t need = carve(nullptr, N, D, K, HKM_WS_ASSIGN).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const Workspace w = carve(ws, N, D, K, HKM_WS_ASSIGN);
+    return do_assign(X, N, D, ldx, C, K, ldc, labels, min_d2, w, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, void* ws,
+                   size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C_new", C_new, K, D, ldcn))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    const size_t need = carve(nullptr, N, D, K, HKM_WS_UPDATE).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const Workspace w = carve(ws, N, D, K, HKM_WS_UPDATE);
+    return launch_update(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                       float* C_new, int32_t K, int32_t* labels, float* shift, float* sse, void* ws,
+                       size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C", C, K, D, D))) return rc;
+    if ((rc = check_matrix("C_new", C_new, K, D, D))) return rc;
+    if (C == C_new) return fail(HKM_EINVAL, "C and C_new must not alias");
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (!shift) return fail(HKM_EINVAL, "shift is NULL");
+    const int32_t flags = HKM_WS_LLOYD | (sse ? HKM_WS_SSE : 0);
+    const size_t need = carve(nullptr, N, D, K, flags).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const Workspace w = carve(ws, N, D, K, flags);
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;
+    if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, st))) return rc;
+    if ((rc = launch_shift(C, C_new, K, D, shift, st))) return rc;
+    if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
+    return rc;
+}
+
+int hkm_shift_f32(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
+                  void* hip_stream) {
+    g_err[0] = 0;
+    if (K < 1 || D < 1) return fail(HKM_EINVAL, "K = %d and D = %d must be >= 1", K, D);
+    if (!C_old || !C_new || !shift) return fail(HKM_EINVAL, "NULL pointer argument");
+    return launch_shift(C_old, C_new, K, D, shift, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_functional_value_f32(const float* min_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
+                             void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (!min_d2 || !out) return fail(HKM_EINVAL, "NULL pointer argument");
+    const size_t need = carve(nullptr, N, 1, 1, HKM_WS_ASSIGN).total;
+    int rc = check_ws(ws, ws_bytes, need);
+    if (rc) return rc;
+    const Workspace w = carve(ws, N, 1, 1, HKM_WS_ASSIGN);
+    return launch_sum_min_d2(min_d2, N, out, w.red, 2, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                  int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 0 || Nn < 0) return fail(HKM_EINVAL, "negative row count (M = %lld, Nn = %lld)", (long long)M, (long long)Nn);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    int rc;
+    if ((rc = check_matrix("X", X, M, D, ldx))) return rc;
+    if ((rc = check_matrix("Y", Y, Nn, D, ldy))) return rc;
+    if (!out) return fail(HKM_EINVAL, "out is NULL");
+    if (ldo < Nn) return fail(HKM_EINVAL, "leading dimension of out (%lld) < columns (%lld)", (long long)ldo, (long long)Nn);
+    if (M == 0 || Nn == 0) return HKM_OK;
+    return launch_cdist(X, M, ldx, Y, Nn, ldy, D, out, ldo, sqrt_flag, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (!in || !out) return fail(HKM_EINVAL, "NULL pointer argument");
+    if (N == 0) return HKM_OK;
+    return launch_widen(in, N, out, static_cast<hipStream_t>(hip_stream));
+}
+
+}  // extern "C"

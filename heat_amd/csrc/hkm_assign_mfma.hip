@@ -1,0 +1,349 @@
+// Fused distance + argmin on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), for D > 16.
+//
+// Operand roles: the A operand (M = 32 rows) carries CENTROIDS, the B operand (N = 32 columns)
+// carries POINTS.  In the 32x32 accumulator a lane then owns one point (column lane%32) and 16
+// centroid rows (8*(v/4) + 4*(lane/32) + v%4 for register v), so the min/argmin over centroids is a
+// scan over the lane's own registers, followed by ONE exchange between lane and lane^32.
+//
+// The contraction index is permuted: lane-half h feeds k = h*DP/2 + 4j + t at step (j, t), which
+// lets both operands be fetched as 16-byte vectors.  A and B use the same permutation, so every k
+// is consumed exactly once.
+//
+// Arithmetic mirrors heat/spatial/distance.py:59-64: d2 = (|x|^2 + |c|^2) - 2*(x.c), clamped at 0;
+// first index wins ties (torch.min, heat/core/statistics.py:177).
+#include "hkm_common.h"
+
+namespace hkm {
+
+#define MFMA32(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
+
+__device__ __forceinline__ floatx4 ld4(const float* p) {
+    return *reinterpret_cast<const floatx4*>(p);
+}
+
+// 16 bytes of row `p` starting at column c; columns >= D read as zero.  VEC: p + c is 16-B aligned
+// and D % 4 == 0, so a group is either fully inside or fully outside the row.
+template <bool VEC>
+__device__ __forceinline__ floatx4 load_row4(const float* row, int c, int D) {
+    floatx4 v = {0.f, 0.f, 0.f, 0.f};
+    if (VEC) {
+        if (c < D) v = ld4(row + c);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (c + t < D) v[t] = row[c + t];
+    }
+    return v;
+}
+
+__device__ __forceinline__ void scan16(const floatx16& acc, float xn, const float* cn_lds_or_glb,
+                                       int kbase, int h, float& m, int& mi) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const floatx4 cn4 = ld4(cn_lds_or_glb + 8 * g + 4 * h);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            float d = fmaf(-2.0f, acc[4 * g + t], xn + cn4[t]);
+            d = fmaxf(d, 0.0f);
+            if (d < m) {
+                m = d;
+                mi = kbase + 8 * g + 4 * h + t;
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void merge_halves(float& m, int& mi) {
+    const float om = __shfl_xor(m, 32);
+    const int oi = __shfl_xor(mi, 32);
+    if (om < m || (om == m && oi < mi)) {
+        m = om;
+        mi = oi;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Resident variant: the whole centroid matrix (zero-padded to KP x DP) and its squared norms live
+// in LDS for the lifetime of a persistent workgroup; each wave streams its own 32*PB points from
+// global memory straight into B-operand registers.  No barrier inside the tile loop.
+// ------------------------------------------------------------------------------------------------
+template <int DP, int PB, bool VEC>
+__global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
+    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles) {
+    extern __shared__ __align__(16) float lds[];
+    constexpr int LDC = DP + 4;  // row stride: +4 floats keeps 16-B vector reads conflict-free
+    constexpr int NJ = DP / 8;   // 16-byte groups per lane-half
+    const int KP = (K + 31) & ~31;
+    float* sC = lds;
+    float* sCn = lds + KP * LDC;
+    const int tid = threadIdx.x;
+
+    for (int i = tid; i < KP * DP; i += 256) {
+        const int r = i / DP, c = i - r * DP;
+        sC[r * LDC + c] = (r < K && c < D) ? C[int64_t(r) * ldc + c] : 0.f;
+    }
+    __syncthreads();
+    for (int r = tid; r < KP; r += 256) {
+        float s = HKM_INF;
+        if (r < K) {
+            s = 0.f;
+            for (int c = 0; c < D; ++c) s = fmaf(sC[r * LDC + c], sC[r * LDC + c], s);
+        }
+        sCn[r] = s;
+    }
+    __syncthreads();
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int p = lane & 31, h = lane >> 5;
+    const int ncb = KP >> 5;
+
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
+        floatx4 b[PB][NJ];
+        float xn[PB], m[PB];
+        int mi[PB];
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            int64_t r = row0 + pb * 32 + p;
+            r = r < N ? r : N - 1;
+            const float* xr = X + r * ldx;
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                b[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
+            }
+            xn[pb] = s + __shfl_xor(s, 32);
+            m[pb] = HKM_INF;
+            mi[pb] = 0;
+        }
+
+        for (int cb = 0; cb < ncb; ++cb) {
+            floatx16 acc[PB];
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[pb][v] = 0.f;
+            const float* arow = sC + (cb * 32 + p) * LDC + h * (DP / 2);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const floatx4 a = ld4(arow + 4 * j);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int pb = 0; pb < PB; ++pb) acc[pb] = MFMA32(a[t], b[pb][j][t], acc[pb]);
+            }
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb)
+                scan16(acc[pb], xn[pb], sCn + cb * 32, cb * 32, h, m[pb], mi[pb]);
+        }
+
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            merge_halves(m[pb], mi[pb]);
+            const int64_t r = row0 + pb * 32 + p;
+            if (h == 0 && r < N) {
+                labels[r] = mi[pb];
+                if (min_d2) min_d2[r] = m[pb];
+            }
+        }
+    }
+}
+
+template <int DP, bool VEC>
+static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                             int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
+                             hipStream_t st) {
+    constexpr int PB = 2;
+    const int64_t ntiles = (N + 4 * PB * 32 - 1) / (4 * PB * 32);
+    const size_t lds = resident_lds_bytes(D, K);
+    auto kern = assign_mfma_resident_kernel<DP, PB, VEC>;
+    int64_t grid = int64_t(num_cus()) * 3;
+    if (grid > ntiles) grid = ntiles;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc,
+                       labels, min_d2, ntiles);
+    return check_launch("assign_mfma_resident_kernel");
+}
+
+int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                                int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
+                                hipStream_t st) {
+    const bool vec = aligned16(X) && (ldx % 4 == 0) && (D % 4 == 0);
+    const int dp = resident_dp(D);
+#define HKM_CASE(d)                                                                         \
+    case d:                                                                                 \
+        return vec ? launch_resident_t<d, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, st) \
+                   : launch_resident_t<d, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
+    switch (dp) {
+        HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
+        default:
+            return fail(HKM_EUNSUPPORTED, "assign_mfma_resident: D=%d", D);
+    }
+#undef HKM_CASE
+}
+
+// ------------------------------------------------------------------------------------------------
+// Streaming variant for any K and D: a workgroup owns 256 points (4 waves x 64) and walks over
+// centroid tiles of 64 and feature chunks of 32.  The centroid panel of a (tile, chunk) step is
+// staged through a double-buffered LDS tile by all 256 threads; the point operand of the step is
+// loaded by each lane straight into registers.  Global loads of step i+1 are issued before the
+// MFMAs of step i.  Squared centroid norms come from global memory (padded with +inf).
+// ------------------------------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
+    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, const float* __restrict__ cn, int32_t* __restrict__ labels,
+    float* __restrict__ min_d2, int64_t ntiles) {
+    constexpr int PB = 2, CB = 2, CT = CB * 32, DC = 32, LDA = DC + 4;
+    __shared__ __align__(16) float sA[2][CT * LDA];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int p = lane & 31, h = lane >> 5;
+    const int nct = (K + CT - 1) / CT;
+    const int ndc = (D + DC - 1) / DC;
+    const int64_t my_tiles = (ntiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const int64_t nsteps = my_tiles * nct * ndc;
+
+    // staging role of this thread: 2 x 16-byte groups of the 64 x 32 panel
+    const int sr = tid >> 3;        // panel rows sr and sr + 32
+    const int sc = (tid & 7) * 4;   // column group
+
+    floatx4 pa[2];
+    floatx4 bn[PB][4];
+    auto issue = [&](int64_t tile, int ct, int dc) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int r = ct * CT + sr + 32 * q;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (r < K) v = load_row4<VEC>(C + int64_t(r) * ldc, dc * DC + sc, D);
+            pa[q] = v;
+        }
+        const int64_t row0 = tile * 256 + wave * 64;
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            int64_t r = row0 + pb * 32 + p;
+            r = r < N ? r : N - 1;
+            const float* xr = X + r * ldx;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bn[pb][j] = load_row4<VEC>(xr, dc * DC + h * 16 + 4 * j, D);
+        }
+    };
+
+    int64_t tile = blockIdx.x;
+    int ct = 0, dc = 0;
+    if (nsteps > 0) issue(tile, ct, dc);
+
+    floatx16 acc[PB][CB];
+    float xn[PB] = {0.f, 0.f}, xs[PB] = {0.f, 0.f}, m[PB];
+    int mi[PB];
+
+    for (int64_t it = 0; it < nsteps; ++it) {
+        const int buf = int(it & 1);
+        // publish the prefetched panel, take the prefetched point operand
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+            *reinterpret_cast<floatx4*>(&sA[buf][(sr + 32 * q) * LDA + sc]) = pa[q];
+        floatx4 b[PB][4];
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[pb][j] = bn[pb][j];
+        __syncthreads();
+
+        const int64_t cur_tile = tile;
+        const int cur_ct = ct, cur_dc = dc;
+        // advance the (tile, ct, dc) odometer and issue the next step's loads
+        if (++dc == ndc) {
+            dc = 0;
+            if (++ct == nct) {
+                ct = 0;
+                tile += gridDim.x;
+            }
+        }
+        if (it + 1 < nsteps) issue(tile, ct, dc);
+
+        if (cur_dc == 0) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[pb][cb][v] = 0.f;
+            if (cur_ct == 0) {
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) {
+                    xs[pb] = 0.f;
+                    m[pb] = HKM_INF;
+                    mi[pb] = 0;
+                }
+            }
+        }
+        if (cur_ct == 0) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) xs[pb] = fmaf(b[pb][j][t], b[pb][j][t], xs[pb]);
+        }
+
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const float* arow = &sA[buf][(cb * 32 + p) * LDA + h * 16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const floatx4 a = ld4(arow + 4 * j);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int pb = 0; pb < PB; ++pb)
+                        acc[pb][cb] = MFMA32(a[t], b[pb][j][t], acc[pb][cb]);
+            }
+        }
+
+        if (cur_dc == ndc - 1) {
+            if (cur_ct == 0) {
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) xn[pb] = xs[pb] + __shfl_xor(xs[pb], 32);
+            }
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb)
+                    scan16(acc[pb][cb], xn[pb], cn + cur_ct * CT + cb * 32, cur_ct * CT + cb * 32,
+                           h, m[pb], mi[pb]);
+            if (cur_ct == nct - 1) {
+                const int64_t row0 = cur_tile * 256 + wave * 64;
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) {
+                    merge_halves(m[pb], mi[pb]);
+                    const int64_t r = row0 + pb * 32 + p;
+                    if (h == 0 && r < N) {
+                        labels[r] = mi[pb];
+                        if (min_d2) min_d2[r] = m[pb];
+                    }
+                }
+            }
+        }
+    }
+}
+
+int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
+                              float* min_d2, hipStream_t st) {
+    const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
+    const int64_t ntiles = (N + 255) / 256;
+    int64_t grid = int64_t(num_cus()) * 2;
+    if (grid > ntiles) grid = ntiles;
+    if (vec)
+        hipLaunchKernelGGL(assign_mfma_stream_kernel<true>, dim3((unsigned)grid), dim3(256), 0, st, X,
+                           N, D, ldx, C, K, ldc, cn, labels, min_d2, ntiles);
+    else
+        hipLaunchKernelGGL(assign_mfma_stream_kernel<false>, dim3((unsigned)grid), dim3(256), 0, st,
+                           X, N, D, ldx, C, K, ldc, cn, labels, min_d2, ntiles);
+    return check_launch("assign_mfma_stream_kernel");
+}
+
+}  // namespace hkm

@@ -1,0 +1,101 @@
+// Full pairwise distance matrix (quadratic expansion) for the public cdist API.
+// out[i, j] = max(0, (|x_i|^2 + |y_j|^2) - 2 x_i.y_j), optionally square-rooted
+// (heat/spatial/distance.py:32-64).  The output is M x Nn floats, so for the feature counts cdist is
+// used with the kernel is bound by writing the matrix; a 64 x 64 output tile per workgroup with a
+// 4 x 4 register block per lane keeps the X / Y re-reads in L2 and the stores 16 bytes wide.
+#include "hkm_common.h"
+
+namespace hkm {
+
+static constexpr int CD_T = 64;   // tile edge
+static constexpr int CD_KC = 16;  // feature chunk
+
+__global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X, int64_t M,
+                                                    int64_t ldx, const float* __restrict__ Y,
+                                                    int64_t Nn, int64_t ldy, int D,
+                                                    float* __restrict__ out, int64_t ldo,
+                                                    int sqrt_flag, int64_t tiles_n) {
+    __shared__ float sX[CD_KC][CD_T + 4];
+    __shared__ float sY[CD_KC][CD_T + 4];
+    __shared__ float sXn[CD_T], sYn[CD_T];
+    const int tid = threadIdx.x;
+    const int64_t tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int64_t i0 = tm * CD_T, j0 = tn * CD_T;
+
+    // squared norms of the tile's rows / columns, each summed in feature order
+    if (tid < 2 * CD_T) {
+        const bool is_x = tid < CD_T;
+        const int r = is_x ? tid : tid - CD_T;
+        const int64_t g = (is_x ? i0 : j0) + r;
+        const int64_t lim = is_x ? M : Nn;
+        float s = 0.f;
+        if (g < lim) {
+            const float* row = is_x ? X + g * ldx : Y + g * ldy;
+            for (int d = 0; d < D; ++d) s = fmaf(row[d], row[d], s);
+        }
+        (is_x ? sXn : sYn)[r] = s;
+    }
+
+    const int tx = tid & 15, ty = tid >> 4;
+    float acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
+
+    // staging role: element (row lr, feature lk) of both tiles, 4 passes of 16 rows
+    const int lk = tid & 15, lr = tid >> 4;
+    for (int d0 = 0; d0 < D; d0 += CD_KC) {
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int r = lr + 16 * q;
+            const int d = d0 + lk;
+            const int64_t gi = i0 + r, gj = j0 + r;
+            sX[lk][r] = (gi < M && d < D) ? X[gi * ldx + d] : 0.f;
+            sY[lk][r] = (gj < Nn && d < D) ? Y[gj * ldy + d] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < CD_KC; ++k) {
+            float xa[4], yb[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) xa[a] = sX[k][ty * 4 + a];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) yb[b] = sY[k][tx * 4 + b];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 4; ++b) acc[a][b] = fmaf(xa[a], yb[b], acc[a][b]);
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int64_t gi = i0 + ty * 4 + a;
+        if (gi >= M) continue;
+        const float xn = sXn[ty * 4 + a];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int64_t gj = j0 + tx * 4 + b;
+            if (gj >= Nn) continue;
+            float d = fmaf(-2.0f, acc[a][b], xn + sYn[tx * 4 + b]);
+            d = fmaxf(d, 0.0f);
+            if (sqrt_flag) d = sqrtf(d);
+            out[gi * ldo + gj] = d;
+        }
+    }
+}
+
+int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                 int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, hipStream_t st) {
+    const int64_t tiles_m = (M + CD_T - 1) / CD_T, tiles_n = (Nn + CD_T - 1) / CD_T;
+    const int64_t total = tiles_m * tiles_n;
+    if (total > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "cdist: %lld tiles exceed the grid limit", (long long)total);
+    hipLaunchKernelGGL(cdist_kernel, dim3((unsigned)total), dim3(256), 0, st, X, M, ldx, Y, Nn, ldy,
+                       D, out, ldo, sqrt_flag, tiles_n);
+    return check_launch("cdist_kernel");
+}
+
+}  // namespace hkm

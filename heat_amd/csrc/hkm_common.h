@@ -1,0 +1,83 @@
+// Internal declarations shared by the translation units of libhkm (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "hkm.h"
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define HKM_WAVE 64
+#define HKM_INF __builtin_inff()
+
+namespace hkm {
+
+// ---- error plumbing (hkm_api.hip) -----------------------------------------------------------
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- kernel family selection ------------------------------------------------------------------
+enum AssignKind { ASSIGN_VALU = 0, ASSIGN_MFMA_RESIDENT = 1, ASSIGN_MFMA_STREAM = 2 };
+AssignKind assign_kind(int32_t D, int32_t K);
+
+// padded feature count used by the resident MFMA kernel (24, 32, 48 or 64)
+static inline int resident_dp(int32_t D) { return D <= 24 ? 24 : D <= 32 ? 32 : D <= 48 ? 48 : 64; }
+static inline size_t resident_lds_bytes(int32_t D, int32_t K) {
+    size_t kp = (size_t(K) + 31) / 32 * 32;
+    return kp * (resident_dp(D) + 4) * sizeof(float) + kp * sizeof(float);
+}
+
+// ---- geometry of the deterministic update ----------------------------------------------------
+struct UpdateGeom {
+    int64_t rows_per_chunk;  // rows summed in fp32 inside one workgroup before the fp64 reduction
+    int32_t S;               // number of row chunks
+    int32_t J;               // number of 32-column slices of D
+    int32_t Z;               // number of cluster ranges
+    int32_t KR;              // clusters per range (LDS accumulator rows)
+};
+UpdateGeom update_geom(int64_t N, int32_t D, int32_t K);
+
+// ---- workspace layout --------------------------------------------------------------------------
+struct Workspace {
+    float* cn;          // squared centroid norms, padded to a multiple of 128 with +inf
+    float* part_sum;    // [S][K][J*32] fp32 partial sums
+    int32_t* part_cnt;  // [S][K]
+    int64_t* counts;    // [K]
+    double* red;        // [RED_SLOTS] scratch for scalar reductions
+    float* min_d2;      // [N] (only with the SSE flag)
+    size_t total;
+};
+static const int RED_SLOTS = 2048;
+Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags);
+
+// ---- launchers (one per .hip file) ------------------------------------------------------------
+int launch_norms(const float* C, int32_t K, int32_t D, int64_t ldc, float* cn, int32_t kpad,
+                 hipStream_t st);
+int launch_assign_valu(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                       int64_t ldc, int32_t* labels, float* min_d2, hipStream_t st);
+int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                                int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
+                                hipStream_t st);
+int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
+                              float* min_d2, hipStream_t st);
+int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                  int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                  hipStream_t st);
+int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
+                 hipStream_t st);
+int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, int mode,
+                      hipStream_t st);
+int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                 int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, hipStream_t st);
+int launch_widen(const int32_t* in, int64_t N, int64_t* out, hipStream_t st);
+
+int num_cus();
+
+}  // namespace hkm

@@ -1,0 +1,118 @@
+/*
+ * hkm.h -- C ABI of libhkm: the k-means Lloyd step (distance -> argmin -> per-cluster mean) as
+ * hand-written gfx950 kernels.
+ *
+ * The reference (helmholtz-analytics/heat) has no FFI for this path: it is a chain of PyTorch calls
+ * behind plain Python functions.  Each entry point below therefore cites the Python function whose
+ * arithmetic it replaces; the Python host package binds them with ctypes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer (except where noted), row-major, fp32 unless the name says
+ *     otherwise; `ld*` are leading dimensions in ELEMENTS (ld >= number of columns);
+ *   - X, C, Y and out base pointers must be 4-byte aligned; 16-byte alignment together with
+ *     ld % 4 == 0 enables the vector-load fast paths;
+ *   - return value: HKM_OK or a negative HKM_E* code; a human-readable message for the last error
+ *     of the calling thread is available from hkm_last_error();
+ *   - argument validation runs on the host before anything is launched, so it is testable without
+ *     a GPU;
+ *   - every call only ENQUEUES work on `hip_stream` (a hipStream_t, NULL = default stream); nothing
+ *     synchronises; the library allocates nothing: the caller passes a workspace of at least
+ *     hkm_workspace_bytes(N, D, K, flags) bytes (256-byte aligned) that must stay alive until the
+ *     enqueued work has finished.  Concurrent calls must use different workspaces;
+ *   - all reductions use a fixed order: the same inputs give bit-identical outputs on every run.
+ */
+#ifndef HKM_H
+#define HKM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HKM_OK 0
+#define HKM_EINVAL (-1)       /* bad argument (null pointer, negative size, ld < D, misalignment) */
+#define HKM_EWORKSPACE (-2)   /* workspace missing or too small */
+#define HKM_EHIP (-3)         /* a HIP runtime call failed; message holds hipGetErrorString */
+#define HKM_EUNSUPPORTED (-4) /* shape outside what the kernels cover */
+
+/* flags for hkm_workspace_bytes */
+#define HKM_WS_ASSIGN 1
+#define HKM_WS_UPDATE 2
+#define HKM_WS_LLOYD 3 /* assign + update */
+#define HKM_WS_SSE 4   /* add when hkm_lloyd_step_f32 is called with sse != NULL (N floats of scratch) */
+
+/* Library version: major*10000 + minor*100 + patch. */
+int hkm_version(void);
+
+/* Message of the last error raised on the calling thread ("" if none). Host pointer, static storage. */
+const char* hkm_last_error(void);
+
+/* Bytes of device workspace needed by the entry points below for this problem size. */
+size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags);
+
+/*
+ * Fused distance + argmin; the N x K matrix is never materialised.
+ *   labels[i] = argmin_k max(0, (|x_i|^2 + |c_k|^2) - 2 x_i.c_k), first index on ties
+ *   min_d2[i] = that minimum (clamped, NOT square-rooted); may be NULL.
+ * Replaces heat/spatial/distance.py:47-64 (_quadratic_expand), :32-44 (_euclidian_fast; the
+ * monotone sqrt is dropped under the argmin) and the argmin of heat/cluster/_kcluster.py:352-370
+ * (heat/core/statistics.py:129-200).
+ */
+int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                   int64_t ldc, int32_t* labels, float* min_d2, void* ws, size_t ws_bytes,
+                   void* hip_stream);
+
+/*
+ * Deterministic per-cluster mean: C_new[k] = (sum over {i: labels[i]==k} of x_i) / count_k, sums
+ * in fp64, count rounded through fp32 like the reference does; an empty cluster gives a zero row.
+ * counts (int64[K]) may be NULL.  labels outside [0, K) are ignored.
+ * Replaces heat/cluster/kmeans.py:76-103 (KMeans._update_centroids).
+ */
+int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, void* ws,
+                   size_t ws_bytes, void* hip_stream);
+
+/*
+ * One Lloyd iteration: labels against C, C_new = per-cluster means, *shift = sum((C - C_new)^2)
+ * (fp32 value, device scalar), optional *sse = sum_i min_d2[i] (device scalar; NULL to skip).
+ * C and C_new are K x D with leading dimension D.
+ * Replaces the loop body of heat/cluster/kmeans.py:131-143 (KMeans.fit).
+ */
+int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                       float* C_new, int32_t K, int32_t* labels, float* shift, float* sse, void* ws,
+                       size_t ws_bytes, void* hip_stream);
+
+/* *shift = sum((C_old - C_new)^2), fixed order.  Replaces heat/cluster/kmeans.py:141. */
+int hkm_shift_f32(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
+                  void* hip_stream);
+
+/*
+ * Clustering functional of predict(): *out = (sqrt(sum_i sqrt(min_d2[i])^2))^2 in fp32, the sum
+ * taken in fp64 in a fixed order.  ws needs hkm_workspace_bytes(N, 1, 1, HKM_WS_ASSIGN) bytes.
+ * Replaces heat/cluster/_kcluster.py:367-368 (norm(distances.min(axis=1), 2) ** 2).
+ */
+int hkm_functional_value_f32(const float* min_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
+                             void* hip_stream);
+
+/*
+ * Full distance matrix for the public cdist API:
+ *   out[i, j] = max(0, (|x_i|^2 + |y_j|^2) - 2 x_i.y_j), square-rooted when sqrt_flag != 0.
+ * X is M x D, Y is Nn x D, out is M x Nn with leading dimension ldo.
+ * Replaces heat/spatial/distance.py:136-156 (cdist, quadratic_expansion=True) on local tensors.
+ */
+int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                  int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, void* hip_stream);
+
+/* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
+int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
+
+/* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "mfma_resident",
+ * "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
+const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HKM_H */

@@ -1,0 +1,217 @@
+"""
+GPU parity of the C-ABI entry points against the CPU oracle, kernel by kernel.
+Every call goes through libhkm via ctypes (heat_amd._native).
+
+Tolerances (fp32 path): labels must agree except where the fp64 best/second-best squared distances
+are within 1e-5 relative; min_d2 within 2e-5 * (|x|^2 + |c|^2) absolute (cancellation in the quadratic
+expansion); centroids within 1e-5 relative to max|C|; counts exact; two runs bit-identical.
+"""
+import numpy as np
+import pytest
+import torch
+
+from heat_amd import _native
+from oracle import heat_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+# (N, D, K): covers the VALU kernel (D <= 16), the LDS-resident MFMA kernel and the streaming MFMA
+# kernel, with ragged sizes, K not a multiple of 32, D not a multiple of 4 (scalar-load path)
+ASSIGN_SHAPES = [
+    (1, 3, 8), (1000, 3, 8), (5000, 8, 16), (777, 16, 40), (300, 1, 5), (2000, 5, 700),
+    (4096, 32, 256), (1000, 20, 33), (999, 17, 1), (3000, 64, 100), (1300, 50, 37), (257, 24, 64),
+    (2048, 64, 1024), (1500, 100, 70), (900, 512, 130), (700, 33, 500), (513, 130, 1030),
+]
+
+
+def _data(n, d, k, seed, spread=3.0):
+    g = torch.Generator().manual_seed(seed)
+    c = torch.randn((k, d), generator=g) * spread
+    lab = torch.randint(0, k, (n,), generator=g)
+    x = c[lab] + torch.randn((n, d), generator=g)
+    return x.contiguous(), c.contiguous()
+
+
+def _assign_gpu(x, c, dev, want_min=True):
+    xs, cs = x.to(dev), c.to(dev)
+    lab = torch.full((x.shape[0],), -7, dtype=torch.int32, device=dev)
+    md = torch.full((x.shape[0],), -1.0, dtype=torch.float32, device=dev) if want_min else None
+    _native.assign(xs, cs, lab, md, _native.Workspace(dev))
+    torch.cuda.synchronize()
+    return lab.cpu(), (md.cpu() if want_min else None)
+
+
+@pytest.mark.parametrize("n,d,k", ASSIGN_SHAPES)
+def test_assign_matches_oracle(cuda, n, d, k):
+    print(f"assign n={n} d={d} k={k} kernel={_native.assign_kernel_name(n, d, k)}", flush=True)
+    x, c = _data(n, d, k, seed=n + d + k)
+    lab, md = _assign_gpu(x, c, cuda)
+    ref_lab, _ = orc.assign_to_cluster_literal(x, c)
+    assert lab.min() >= 0 and lab.max() < k
+    rep = orc.label_agreement(x, c, lab, ref_lab)
+    assert rep["n_unexcused"] == 0, rep
+    assert rep["agreement"] >= 0.999, rep
+    ref_q = orc.quadratic_expand(x, c).gather(1, lab.view(-1, 1).long()).view(-1)
+    scale = (x.double() ** 2).sum(1) + (c.double() ** 2).sum(1).max()
+    assert torch.all((md.double() - ref_q.double()).abs() <= 2e-5 * scale + 1e-6)
+    # against the mathematical definition too
+    d2 = orc.brute_force_d2(x, c).min(dim=1).values
+    assert torch.all((md.double() - d2).abs() <= 2e-5 * scale + 1e-6)
+
+
+def test_assign_ties_take_first_index(cuda):
+    # Duplicated centroids give bit-identical distances in the kernels (same instruction sequence for
+    # every centroid), i.e. exact ties; torch.min's rule -- the first index wins -- must then hold.
+    # The CPU sgemm does NOT always produce exact ties for duplicated columns (it blocks columns), so
+    # the oracle is compared modulo the duplication.
+    g = torch.Generator().manual_seed(5)
+    for d in (3, 32, 80):
+        base = torch.randn((6, d), generator=g)
+        c = torch.cat([base, base, base])  # k = 18, centroid j == j+6 == j+12
+        x = base[torch.randint(0, 6, (500,), generator=g)] + 0.01 * torch.randn((500, d), generator=g)
+        lab, _ = _assign_gpu(x, c, cuda)
+        ref, _ = orc.assign_to_cluster_literal(x, c)
+        assert int(lab.max()) < 6, d
+        assert bool((lab.long() == ref.view(-1) % 6).all()), d
+
+
+def test_assign_point_equals_centroid_clamps_at_zero(cuda):
+    # x_i == c_k: the expansion may go slightly negative and must be clamped to exactly 0
+    g = torch.Generator().manual_seed(6)
+    for d in (8, 32, 128):
+        c = torch.randn((40, d), generator=g) * 50
+        x = c[torch.arange(40).repeat(10)].contiguous()
+        lab, md = _assign_gpu(x, c, cuda)
+        assert torch.equal(lab.long(), torch.arange(40).repeat(10))
+        assert md.min() >= 0.0
+        assert md.max() <= 2e-6 * float((c.double() ** 2).sum(1).max())
+
+
+def test_assign_strided_rows(cuda):
+    # X and C as column slices of wider buffers: ld > D, base pointers not 16-byte aligned
+    g = torch.Generator().manual_seed(7)
+    for d, k in ((3, 8), (32, 64), (96, 200)):
+        xw = torch.randn((1200, d + 5), generator=g)
+        cw = torch.randn((k, d + 3), generator=g)
+        xs, cs = xw.to(cuda)[:, 1 : 1 + d], cw.to(cuda)[:, 2 : 2 + d]
+        lab = torch.empty((1200,), dtype=torch.int32, device=cuda)
+        _native.assign(xs, cs, lab, None, _native.Workspace(cuda))
+        ref, _ = orc.assign_to_cluster_literal(xw[:, 1 : 1 + d].contiguous(), cw[:, 2 : 2 + d].contiguous())
+        rep = orc.label_agreement(xw[:, 1 : 1 + d], cw[:, 2 : 2 + d], lab.cpu(), ref)
+        assert rep["n_unexcused"] == 0, (d, k, rep)
+
+
+UPDATE_SHAPES = [(1000, 3, 8), (5000, 8, 16), (4096, 32, 256), (3000, 64, 100), (70000, 20, 33),
+                 (900, 512, 130), (2500, 130, 1030), (100000, 32, 7)]
+
+
+@pytest.mark.parametrize("n,d,k", UPDATE_SHAPES)
+def test_update_matches_oracle(cuda, n, d, k):
+    print(f"update n={n} d={d} k={k}", flush=True)
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.randn((n, d), generator=g) * 4 + 1
+    lab = torch.randint(0, k, (n,), generator=g)
+    lab[lab == k // 2] = 0  # force an empty cluster (k >= 2)
+    c_new = torch.full((k, d), 123.0, device=cuda)
+    cnt = torch.full((k,), -1, dtype=torch.int64, device=cuda)
+    _native.update(x.to(cuda), lab.to(torch.int32).to(cuda), c_new, cnt, _native.Workspace(cuda))
+    torch.cuda.synchronize()
+    ref, ref_cnt = orc.update_centroids_fast(x, lab.view(-1, 1), k)
+    assert torch.equal(cnt.cpu(), ref_cnt)
+    assert int(cnt.sum()) == n
+    assert orc.rel_err_centers(c_new.cpu(), ref) <= 1e-5
+    if k >= 2:
+        assert torch.all(c_new[k // 2] == 0)
+    if n * k <= 2_000_000:
+        lit = orc.update_centroids_literal(x, lab.view(-1, 1), torch.zeros((k, d)))
+        assert orc.rel_err_centers(c_new.cpu(), lit) <= 1e-5
+
+
+def test_update_ignores_out_of_range_labels(cuda):
+    x = torch.arange(40, dtype=torch.float32).view(10, 4)
+    lab = torch.tensor([0, 1, -1, 5, 1, 0, 99, 1, 0, 1], dtype=torch.int32)
+    c_new = torch.empty((2, 4), device=cuda)
+    cnt = torch.empty((2,), dtype=torch.int64, device=cuda)
+    _native.update(x.to(cuda), lab.to(cuda), c_new, cnt, _native.Workspace(cuda))
+    assert cnt.tolist() == [3, 4]
+    assert torch.allclose(c_new.cpu()[0], x[[0, 5, 8]].mean(0))
+    assert torch.allclose(c_new.cpu()[1], x[[1, 4, 7, 9]].mean(0))
+
+
+@pytest.mark.parametrize("n,d,k", [(20000, 3, 8), (20000, 8, 16), (30000, 32, 256), (5000, 64, 1024), (4000, 512, 96)])
+def test_lloyd_step_matches_oracle_and_is_deterministic(cuda, n, d, k):
+    print(f"lloyd n={n} d={d} k={k}", flush=True)
+    x, _ = _data(n, d, k, seed=11 * n + k)
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(3))[:k]].contiguous()
+    xs, cs = x.to(cuda), c0.to(cuda)
+    outs = []
+    for _ in range(2):
+        c_new = torch.empty_like(cs)
+        lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+        shift = torch.empty((), device=cuda)
+        sse = torch.empty((), device=cuda)
+        _native.lloyd_step(xs, cs, c_new, lab, shift, sse, _native.Workspace(cuda))
+        torch.cuda.synchronize()
+        outs.append((c_new.cpu(), lab.cpu(), shift.cpu(), sse.cpu()))
+    for a, b in zip(outs[0], outs[1]):
+        assert torch.equal(a, b), "two runs must be bit-identical"
+    c_new, lab, shift, sse = outs[0]
+    ref_lab, _ = orc.assign_to_cluster_literal(x, c0)
+    rep = orc.label_agreement(x, c0, lab, ref_lab)
+    assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, rep
+    ref_c, _ = orc.update_centroids_fast(x, lab.view(-1, 1).long(), k)  # same labels -> isolates the update
+    assert orc.rel_err_centers(c_new, ref_c) <= 1e-5
+    ref_shift = orc.centroid_shift(c0, c_new)
+    assert orc.rel_err_scalar(float(shift), float(ref_shift), floor=1e-12) <= 1e-5
+    ref_sse = orc.sse(x, c0, lab.long())
+    assert orc.rel_err_scalar(float(sse), ref_sse) <= 1e-4
+
+
+def test_shift_and_functional_value(cuda):
+    g = torch.Generator().manual_seed(9)
+    a, b = torch.randn((37, 19), generator=g), torch.randn((37, 19), generator=g)
+    out = torch.empty((), device=cuda)
+    _native.shift(a.to(cuda), b.to(cuda), out)
+    assert orc.rel_err_scalar(float(out), float(orc.centroid_shift(a, b))) <= 1e-6
+    _native.shift(a.to(cuda), a.to(cuda), out)
+    assert float(out) == 0.0
+    md = torch.rand((100003,), generator=g) * 7
+    _native.functional_value(md.to(cuda), out, _native.Workspace(cuda))
+    m = torch.sqrt(md)
+    ref = torch.sqrt(torch.dot(m, m)) ** 2
+    assert orc.rel_err_scalar(float(out), float(ref)) <= 1e-5
+
+
+def test_cdist_known_answers_and_oracle(cuda):
+    # known answers of the reference's tests/spatial/test_distances.py:16-58
+    X, Y = torch.ones((4, 4)), torch.zeros((4, 4))
+    out = torch.empty((4, 4), device=cuda)
+    _native.cdist(X.to(cuda), Y.to(cuda), out, sqrt=True)
+    assert torch.equal(out.cpu(), torch.full((4, 4), 2.0))
+    _native.cdist(X.to(cuda), X.to(cuda), out, sqrt=True)
+    assert torch.equal(out.cpu(), torch.zeros((4, 4)))
+    g = torch.Generator().manual_seed(10)
+    for m, n, d in ((100, 70, 3), (130, 257, 64), (65, 64, 200), (1, 1, 1)):
+        a, b = torch.randn((m, d), generator=g) * 3, torch.randn((n, d), generator=g) * 3
+        out = torch.empty((m, n), device=cuda)
+        _native.cdist(a.to(cuda), b.to(cuda), out, sqrt=False)
+        ref = orc.quadratic_expand(a, b)
+        scale = float((a.double() ** 2).sum(1).max() + (b.double() ** 2).sum(1).max())
+        assert float((out.cpu() - ref).abs().max()) <= 2e-6 * scale
+        _native.cdist(a.to(cuda), b.to(cuda), out, sqrt=True)
+        bf = orc.brute_force_d2(a, b).sqrt()
+        assert float((out.cpu().double() - bf).abs().max()) <= 1e-3
+
+
+def test_widen_and_empty_inputs(cuda):
+    lab = torch.tensor([3, 0, 2147483647, 5], dtype=torch.int32, device=cuda)
+    out = torch.empty((4,), dtype=torch.int64, device=cuda)
+    _native.widen_labels(lab, out)
+    assert out.tolist() == [3, 0, 2147483647, 5]
+    # N = 0: nothing to do, no launch, no error
+    x = torch.empty((0, 8), device=cuda)
+    c = torch.randn((4, 8), device=cuda)
+    _native.assign(x, c, torch.empty((0,), dtype=torch.int32, device=cuda), None, _native.Workspace(cuda))
+    c_new = torch.full((4, 8), 9.0, device=cuda)
+    _native.update(x, torch.empty((0,), dtype=torch.int32, device=cuda), c_new, None, _native.Workspace(cuda))
+    assert torch.all(c_new == 0)
