@@ -40,8 +40,13 @@ def array(obj, dtype=None, copy=None, ndmin: int = 0, order: str = "C", split: O
         t = obj.larray
         sp = obj.split if split is None and is_split is None else (split if split is not None else is_split)
     else:
-        dev = devices.sanitize_device(device)
         sp = split if split is not None else is_split
+        if isinstance(obj, torch.Tensor) and device is None:
+            # a tensor keeps its own device (the reference would move it to the default device;
+            # here that would silently pull GPU data back to the host)
+            dev = devices.sanitize_device(obj.device.type)
+        else:
+            dev = devices.sanitize_device(device)
         if isinstance(obj, torch.Tensor):
             t = obj
         else:
