@@ -4,7 +4,10 @@
 //
 // Arithmetic mirrors heat/spatial/distance.py:59-64: d2 = (|x|^2 + |c|^2) - 2*(x.c), clamped at 0,
 // scanned over k ascending with a strict '<' so the first index wins ties
-// (torch.min semantics, heat/core/statistics.py:177).
+// (torch.min semantics, heat/core/statistics.py:177).  The squared norms are sums of ROUNDED squares
+// in feature order and the dot product is an FMA chain in feature order: for D <= 8 that is the
+// order torch's CPU reduction and sgemm use, so the fp32 distances agree bit for bit with the
+// reference's there.
 #include "hkm_common.h"
 
 namespace hkm {
@@ -18,7 +21,7 @@ __global__ void norms_kernel(const float* __restrict__ C, int K, int D, int64_t 
     if (k < K) {
         s = 0.f;
         const float* c = C + int64_t(k) * ldc;
-        for (int d = 0; d < D; ++d) s = fmaf(c[d], c[d], s);
+        for (int d = 0; d < D; ++d) s = __fadd_rn(s, __fmul_rn(c[d], c[d]));
     }
     cn[k] = s;
 }
@@ -54,7 +57,7 @@ __global__ __launch_bounds__(VALU_THREADS) void assign_valu_kernel(
         for (int r = tid; r < kn; r += VALU_THREADS) {
             float s = 0.f;
 #pragma unroll
-            for (int d = 0; d < D; ++d) s = fmaf(sC[r * S + d], sC[r * S + d], s);
+            for (int d = 0; d < D; ++d) s = __fadd_rn(s, __fmul_rn(sC[r * S + d], sC[r * S + d]));
             sC[r * S + D] = s;
         }
         __syncthreads();
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(VALU_THREADS) void assign_valu_kernel(
         for (int d = 0; d < D; ++d) x[d] = xp[d];
         float xn = 0.f;
 #pragma unroll
-        for (int d = 0; d < D; ++d) xn = fmaf(x[d], x[d], xn);
+        for (int d = 0; d < D; ++d) xn = __fadd_rn(xn, __fmul_rn(x[d], x[d]));
 
         float m = HKM_INF;
         int mi = 0;

@@ -279,9 +279,15 @@ def label_agreement(
 ):
     """
     Compare two labelings of ``x`` against ``centers``.  For every row where they differ, the fp64
-    best / second-best squared distances (direct ``sum((x-c)**2)``) are evaluated; a disagreement is
-    *excused* when ``(d2_second - d2_best) <= rel_gap * d2_best`` (a numerical tie at fp32 accuracy)
-    AND both labels are among the (near-)tied candidates.
+    squared distances (direct ``sum((x-c)**2)``) of both chosen centroids are compared with the best
+    one; a disagreement is *excused* (a numerical tie) when both lie within
+
+        rel_gap * d2_best  +  max(2, sqrt(D)/4) * eps32 * (|x|^2 + |c|^2)
+
+    of the best.  The first term is the stated gap rule.  The second is the resolution of the
+    reference's own arithmetic: in fp32, ``(|x|^2 + |c|^2) - 2 x.c`` is a difference of two numbers of
+    that magnitude, so its value is a multiple of their ulp and carries the rounding of a D-term dot
+    product; squared distances closer than that are not ordered reliably by the reference either.
 
     Returns dict(n, n_diff, n_unexcused, agreement).
     """
@@ -291,6 +297,8 @@ def label_agreement(
     diff = torch.nonzero(a != b).view(-1)
     n_unexcused = 0
     c64 = centers.to(torch.float64).cpu()
+    cn = (c64**2).sum(1)
+    dfac = max(2.0, math.sqrt(x.shape[1]) / 4.0) * float(torch.finfo(torch.float32).eps)
     for s in range(0, diff.numel(), chunk):
         rows = diff[s : s + chunk]
         xr = x[rows].to(torch.float64).cpu()
@@ -298,7 +306,8 @@ def label_agreement(
         best = d2.min(dim=1).values
         da = d2.gather(1, a[rows].view(-1, 1)).view(-1)
         db = d2.gather(1, b[rows].view(-1, 1)).view(-1)
-        lim = best * (1.0 + rel_gap) + 1e-300
+        mag = (xr**2).sum(1) + torch.maximum(cn[a[rows]], cn[b[rows]])
+        lim = best * (1.0 + rel_gap) + dfac * mag + 1e-300
         ok = (da <= lim) & (db <= lim)
         n_unexcused += int((~ok).sum())
     return {

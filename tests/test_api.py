@@ -1,0 +1,224 @@
+"""
+Host-side tests that need no GPU: the estimator protocol and exception matrix of the reference's
+tests/cluster/test_kmeans.py:18-34,68-100 and tests/spatial/test_distances.py:190-205 restated for
+heat_amd, the DNDarray/array surface callers use, and the C ABI (every symbol of include/hkm.h is
+exported; argument validation returns the documented codes before anything is launched).
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import heat_amd as ht
+from heat_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+IRIS = np.loadtxt(os.path.join(ROOT, "tests", "golden", "iris.csv"), delimiter=";", dtype=np.float32)
+
+
+# ---- estimator protocol -----------------------------------------------------------------------
+def test_clusterer_protocol():
+    km = ht.cluster.KMeans()
+    assert ht.is_estimator(km) and ht.is_clusterer(km)
+    assert isinstance(km, ht.BaseEstimator) and isinstance(km, ht.ClusteringMixin)
+
+
+def test_get_and_set_params():
+    km = ht.cluster.KMeans()
+    params = km.get_params()
+    assert params == {"n_clusters": 8, "init": "random", "max_iter": 300, "tol": 1e-4, "random_state": None}
+    params["n_clusters"] = 10
+    km.set_params(**params)
+    assert km.n_clusters == 10
+    with pytest.raises(ValueError):
+        km.set_params(foo="bar")
+    assert "KMeans(" in repr(km)
+    assert ht.cluster.KMeans(init="kmeans++").init == "probability_based"
+    for attr in ("cluster_centers_", "labels_", "inertia_", "n_iter_", "functional_value_"):
+        assert getattr(km, attr) is None
+
+
+def test_exception_matrix():
+    iris_split1 = ht.array(torch.from_numpy(IRIS), split=1)
+    iris = ht.array(torch.from_numpy(IRIS), split=0)
+    k = 3
+    with pytest.raises(NotImplementedError):  # split = 1 is refused by the distance
+        ht.cluster.KMeans(n_clusters=k).fit(iris_split1)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=k, init="random_number").fit(iris_split1)
+    with pytest.raises(NotImplementedError):
+        ht.cluster.KMeans(n_clusters=k, init="batchparallel").fit(iris_split1)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=k, init=np.array([1, 2, 3])).fit(iris_split1)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=k).fit(iris_split1, oversampling=-1)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=k).fit(iris_split1, iter_multiplier=-1)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=k, init=ht.array([1, 2])).fit(iris_split1)
+    with pytest.raises(NotImplementedError):
+        ht.cluster.KMeans(n_clusters=k, init="probability_based").fit(iris_split1)
+    with pytest.raises(ValueError):  # (K, D) mismatch
+        ht.cluster.KMeans(n_clusters=k, init=ht.array(torch.zeros((2, 4)))).fit(iris)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=k, init=ht.array(torch.zeros((3, 5)))).fit(iris)
+    with pytest.raises(TypeError):  # fit wants a DNDarray
+        ht.cluster.KMeans(n_clusters=k).fit(IRIS)
+    with pytest.raises(ValueError):  # predict wants a DNDarray
+        ht.cluster.KMeans(n_clusters=k).predict(IRIS)
+
+
+def test_no_cpu_fallback():
+    # data on the host: the product must refuse, not compute on the CPU
+    iris = ht.array(torch.from_numpy(IRIS), split=0)
+    init = ht.array(torch.from_numpy(IRIS[:3].copy()))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ht.cluster.KMeans(n_clusters=3, init=init, max_iter=2).fit(iris)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ht.spatial.cdist(iris, init, quadratic_expansion=True)
+
+
+def test_cdist_exceptions():
+    X = ht.ones((4, 4), split=1)
+    Y = ht.zeros((4, 4))
+    with pytest.raises(NotImplementedError):
+        ht.spatial.cdist(X, quadratic_expansion=True)
+    with pytest.raises(NotImplementedError):
+        ht.spatial.cdist(X, Y, quadratic_expansion=True)
+    with pytest.raises(NotImplementedError):
+        ht.spatial.cdist(ht.ones((4, 4)), ht.zeros((4, 4), split=1), quadratic_expansion=True)
+    Z = ht.ones((4, 6, 3))
+    with pytest.raises(NotImplementedError):
+        ht.spatial.cdist(Z, quadratic_expansion=True)
+    with pytest.raises(NotImplementedError):
+        ht.spatial.cdist(ht.ones((4, 4)), Z, quadratic_expansion=True)
+    with pytest.raises(ValueError):
+        ht.spatial.cdist(ht.ones((4, 4)), ht.ones((4, 5)), quadratic_expansion=True)
+    with pytest.raises(NotImplementedError):  # float64 is outside the float32 kernels
+        ht.spatial.cdist(ht.ones((4, 4), dtype=ht.float64), quadratic_expansion=True)
+
+
+# ---- array surface ----------------------------------------------------------------------------
+def test_array_and_dndarray_surface():
+    t = torch.arange(12, dtype=torch.float32).view(4, 3)
+    a = ht.array(t, split=0)
+    assert a.larray.data_ptr() == t.data_ptr()  # shared, not copied
+    assert a.shape == (4, 3) == a.gshape == a.lshape and a.split == 0 and a.dtype is ht.float32
+    assert a.device == ht.cpu and a.comm.size == 1 and a.comm.rank == 0 and a.balanced
+    assert not a.is_distributed() and a.ndim == 2 and a.size == 12 and len(a) == 4
+    b = a.resplit(None)
+    assert b.split is None and b.larray.data_ptr() != t.data_ptr()  # resplit copies
+    c = a.astype(ht.int64)
+    assert c.dtype is ht.int64 and c.larray.dtype == torch.int64
+    assert a.copy().larray.data_ptr() != t.data_ptr()
+    # DNDarray == "string" is False instead of raising (the reference relies on this)
+    assert (a == "kmeans++") is False
+    assert bool(ht.array(3.0) <= 4.0) and not bool(ht.array(5.0) <= 4.0)
+    with pytest.raises(TypeError):
+        bool(a)
+    assert ht.array([1, 2]).shape == (2,)
+    assert ht.zeros((2, 2)).larray.sum() == 0 and ht.ones((2, 2), dtype=ht.int32).dtype is ht.int32
+    with pytest.raises(ValueError):
+        ht.array(t, split=0, is_split=0)
+    assert a[1:3].shape == (2, 3) and a[1:3].split == 0
+
+
+def test_type_promotion():
+    assert ht.promote_types(ht.int32, ht.float32) is ht.float32
+    assert ht.promote_types(ht.int64, ht.float32) is ht.float64
+    assert ht.promote_types(ht.int8, ht.uint8) is ht.int16
+    assert ht.promote_types(ht.uint8, ht.uint8) is ht.uint8
+    assert ht.promote_types("i8", "f4") is ht.float64
+    assert ht.float32.torch_type() == torch.float32
+    assert ht.iinfo(ht.int64).max == 9223372036854775807
+    assert ht.heat_type_of(torch.zeros(1, dtype=torch.int16)) is ht.int16
+
+
+def test_devices():
+    assert str(ht.cpu) == "cpu:0" and ht.cpu.torch_device == "cpu"
+    assert ht.get_device() == ht.cpu
+    assert ht.sanitize_device("cpu") is ht.cpu
+    with pytest.raises(ValueError):
+        ht.sanitize_device("tpu")
+
+
+# ---- C ABI -----------------------------------------------------------------------------------
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hkm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hkm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _native.load()
+    names = _declared_symbols()
+    assert len(names) >= 11
+    for name in names:
+        assert hasattr(lib, name), name
+        assert name in _native.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(_native.SIGNATURES) == names
+    assert lib.hkm_version() >= 100
+
+
+def test_workspace_and_kernel_selection():
+    assert _native.workspace_bytes(-1, 3, 8, 3) == 0
+    assert _native.workspace_bytes(10, 0, 8, 3) == 0
+    a = _native.workspace_bytes(10_000_000, 32, 256, _native.WS_LLOYD)
+    b = _native.workspace_bytes(10_000_000, 32, 256, _native.WS_LLOYD | _native.WS_SSE)
+    assert 0 < a < b and b - a >= 40_000_000 and a % 256 == 0
+    assert _native.assign_kernel_name(200_000_000, 3, 8).startswith("valu")
+    assert _native.assign_kernel_name(100_000, 8, 16).startswith("valu")
+    assert _native.assign_kernel_name(10_000_000, 32, 256) == "mfma_resident"
+    assert _native.assign_kernel_name(1 << 20, 64, 1024) == "mfma_stream"
+    assert _native.assign_kernel_name(2_000_000, 512, 1024) == "mfma_stream"
+
+
+def test_argument_validation_happens_on_the_host():
+    lib = _native.load()
+    P = ctypes.c_void_p
+    good, ws = P(4096), P(1 << 20)  # never dereferenced: every call below fails validation first
+    big = 1 << 30
+
+    def err():
+        return lib.hkm_last_error().decode()
+
+    assert lib.hkm_assign_f32(None, 10, 3, 3, good, 8, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert "X is NULL" in err()
+    assert lib.hkm_assign_f32(good, -1, 3, 3, good, 8, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_f32(good, 10, 0, 3, good, 8, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_f32(good, 10, 3, 3, good, 0, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_f32(good, 10, 3, 2, good, 8, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert "leading dimension" in err()
+    assert lib.hkm_assign_f32(P(4098), 10, 3, 3, good, 8, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert "aligned" in err()
+    assert lib.hkm_assign_f32(good, 10, 3, 3, good, 8, 3, None, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_f32(good, 10, 3, 3, good, 8, 3, good, None, None, 0, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_assign_f32(good, 10, 3, 3, good, 8, 3, good, None, ws, 16, None) == _native.HKM_EWORKSPACE
+    assert "too small" in err()
+    assert lib.hkm_assign_f32(good, 10, 3, 3, good, 8, 3, good, None, P((1 << 20) + 8), big, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_update_f32(good, 10, 3, 3, None, 8, good, 3, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_update_f32(good, 10, 3, 3, good, 8, good, 2, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_update_f32(good, 10, 3, 3, good, 8, good, 3, None, ws, 8, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_lloyd_step_f32(good, 10, 3, 3, good, good, 8, good, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert "alias" in err()
+    assert lib.hkm_lloyd_step_f32(good, 10, 3, 3, good, P(8192), 8, good, None, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_shift_f32(None, good, 8, 3, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_shift_f32(good, good, 0, 3, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_cdist_f32(good, 4, 3, good, 4, 3, 3, good, 3, 1, None) == _native.HKM_EINVAL  # ldo < Nn
+    assert lib.hkm_cdist_f32(good, -4, 3, good, 4, 3, 3, good, 4, 1, None) == _native.HKM_EINVAL
+    assert lib.hkm_widen_labels_i64(None, 4, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_functional_value_f32(good, -1, good, ws, big, None) == _native.HKM_EINVAL
+    # zero-sized problems succeed without touching the device
+    assert lib.hkm_widen_labels_i64(good, 0, good, None) == _native.HKM_OK
+    assert lib.hkm_cdist_f32(None, 0, 3, good, 4, 3, 3, good, 4, 1, None) == _native.HKM_OK
+    assert err() == ""
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "_LIB_PATH", "/nonexistent/libhkm.so")
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        _native.load()

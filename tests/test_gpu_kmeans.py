@@ -1,0 +1,243 @@
+"""
+GPU parity of the public surface -- ht.cluster.KMeans(...).fit/predict and ht.spatial.cdist -- against
+the CPU oracle and the committed golden vectors, on the five benchmark workloads (scaled where the
+oracle would not finish in seconds) and, at full size, through size-independent properties.
+
+Bar (fp32): labels equal wherever the fp64 best/second-best squared distances differ by more than
+1e-5 relative and >= 99.99 % overall; centroids, inertia_ (the last centroid shift) and
+functional_value_ within 1e-4 relative (shift with an absolute floor of 1e-6 * mean|c|^2);
+n_iter_ equal; repeated runs bit-identical.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import heat_amd as ht
+from heat_amd.utils import synthetic
+from oracle import heat_oracle as orc
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _fit(x_cpu, init_cpu, k, iters, tol, dev):
+    x = ht.array(x_cpu.to(dev), split=0)
+    init = ht.array(init_cpu.to(dev))
+    km = ht.cluster.KMeans(n_clusters=k, init=init, max_iter=iters, tol=tol).fit(x)
+    torch.cuda.synchronize()
+    return km, x
+
+
+def _check_fit(km, x_cpu, ref_centers, ref_labels, ref_inertia, ref_n_iter, tie_flips=0):
+    """End-to-end comparison of a whole fit.  ``tie_flips`` = number of numerically tied points that the
+    two implementations resolved differently somewhere along the trajectory (found by
+    _stepwise_parity).  One such point moves a centroid by |x - c| / n_k and Lloyd's iteration
+    amplifies that before convergence, so the 1e-4 bar on centroids and shift applies to trajectories
+    without flips; with flips the run must still reach the same objective (SSE within 1e-4) in the
+    same number of iterations (labels are compared step by step in _stepwise_parity; here >= 99 %)."""
+    c = km.cluster_centers_.larray.cpu()
+    lab = km.labels_.larray.cpu()
+    assert km.cluster_centers_.shape == tuple(ref_centers.shape) and km.cluster_centers_.split is None
+    assert km.labels_.shape == (x_cpu.shape[0], 1) and km.labels_.dtype is ht.int64 and km.labels_.split == 0
+    assert km.n_iter_ == ref_n_iter, (km.n_iter_, ref_n_iter)
+    agree = float((lab == ref_labels).float().mean())
+    if tie_flips == 0:
+        assert orc.rel_err_centers(c, ref_centers) <= 1e-4, orc.rel_err_centers(c, ref_centers)
+        floor = 1e-6 * float((ref_centers.double() ** 2).sum(1).mean())
+        assert orc.rel_err_scalar(float(km.inertia_), float(ref_inertia), floor=floor) <= 1e-4
+        assert agree >= 0.9999, agree
+    else:
+        a = orc.sse(x_cpu, c, orc.assign_to_cluster_fast(x_cpu, c)[0])
+        b = orc.sse(x_cpu, ref_centers, orc.assign_to_cluster_fast(x_cpu, ref_centers)[0])
+        assert orc.rel_err_scalar(a, b) <= 1e-4, (a, b, tie_flips)
+        assert agree >= 0.99, agree
+
+
+def _stepwise_parity(w, dev, iters, literal):
+    """Walk the ORACLE's trajectory; at every iteration run one GPU Lloyd step from the oracle's current
+    centroids and compare: labels (gap rule, no unexcused difference), centroids against the oracle's
+    update of the GPU's own labels (1e-5) and against the oracle's new centroids when the labels are
+    identical (1e-5), shift (1e-4).  Returns the number of excused tie flips and the oracle's result."""
+    from heat_amd import _native
+
+    x = w.x.to(dev)
+    n = w.x.shape[0]
+    ws = _native.Workspace(dev)
+    lab = torch.empty((n,), dtype=torch.int32, device=dev)
+    shift = torch.empty((), device=dev)
+    c_ref = w.init.clone()
+    flips = 0
+    n_iter = 0
+    for _ in range(iters):
+        n_iter += 1
+        c_in = c_ref.to(dev)
+        c_out = torch.empty_like(c_in)
+        _native.lloyd_step(x, c_in, c_out, lab, shift, None, ws)
+        if literal:
+            ref_lab, _ = orc.assign_to_cluster_literal(w.x, c_ref)
+            ref_new = orc.update_centroids_literal(w.x, ref_lab, c_ref)
+        else:
+            ref_lab, _ = orc.assign_to_cluster_fast(w.x, c_ref)
+            ref_new, _ = orc.update_centroids_fast(w.x, ref_lab, w.k)
+        rep = orc.label_agreement(w.x, c_ref, lab.cpu(), ref_lab)
+        assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, (n_iter, rep)
+        flips += rep["n_diff"]
+        own, _ = orc.update_centroids_fast(w.x, lab.cpu().long().view(-1, 1), w.k)
+        assert orc.rel_err_centers(c_out.cpu(), own) <= 1e-5, n_iter
+        if rep["n_diff"] == 0:
+            assert orc.rel_err_centers(c_out.cpu(), ref_new) <= 1e-5, n_iter
+        ref_shift = orc.centroid_shift(c_ref, c_out.cpu())
+        floor = 1e-6 * float((c_ref.double() ** 2).sum(1).mean())
+        assert orc.rel_err_scalar(float(shift), float(ref_shift), floor=floor) <= 1e-4, n_iter
+        inertia = orc.centroid_shift(c_ref, ref_new)
+        c_ref = ref_new.clone()
+        if bool(inertia <= 0.0):
+            break
+    return flips, dict(cluster_centers=c_ref, labels=ref_lab, inertia=inertia, n_iter=n_iter)
+
+
+@pytest.mark.parametrize("name", ["iris_k3", "edge_k4", "translated_k2"])
+def test_golden_fixtures(cuda, name):
+    z = np.load(os.path.join(GOLD, name + ".npz"))
+    x, c0 = torch.from_numpy(z["x"]), torch.from_numpy(z["init"])
+    km, xd = _fit(x, c0, c0.shape[0], int(z["max_iter"]), 0.0, cuda)
+    _check_fit(km, x, torch.from_numpy(z["centers"]), torch.from_numpy(z["labels"]), z["inertia"], int(z["n_iter"]))
+    pred = km.predict(xd)
+    assert pred.shape == (x.shape[0], 1) and pred.dtype is ht.int64
+    assert float((pred.larray.cpu() == torch.from_numpy(z["predict_labels"])).float().mean()) >= 0.99
+    assert orc.rel_err_scalar(float(km.functional_value_), float(z["functional_value"])) <= 1e-4
+    # first-iteration distances through the public cdist (square-rooted)
+    d = ht.spatial.cdist(xd, ht.array(c0.to(cuda)), quadratic_expansion=True)
+    assert d.shape == (x.shape[0], c0.shape[0]) and d.split == 0 and d.dtype is ht.float32
+    ref = np.sqrt(z["d2_first"])
+    assert np.allclose(d.larray.cpu().numpy(), ref, rtol=1e-4, atol=2e-3)
+
+
+def test_fit_restarts_from_cluster_centers(cuda):
+    # KMeans has no resume; passing cluster_centers_ as init continues the iteration
+    z = np.load(os.path.join(GOLD, "iris_k3.npz"))
+    x, c0 = torch.from_numpy(z["x"]), torch.from_numpy(z["init"])
+    a, _ = _fit(x, c0, 3, 2, None, cuda)
+    b, _ = _fit(x, a.cluster_centers_.larray.cpu(), 3, 3, None, cuda)
+    full, _ = _fit(x, c0, 3, 5, None, cuda)
+    assert torch.equal(b.cluster_centers_.larray, full.cluster_centers_.larray)
+    assert np.allclose(full.cluster_centers_.numpy(), z["centers"], rtol=1e-5)
+
+
+def test_config1_full_size_against_literal_oracle(cuda):
+    w = synthetic.config1()
+    flips, ref = _stepwise_parity(w, cuda, w.max_iter, literal=True)
+    print(f"config1: {flips} excused tie flips over {ref['n_iter']} iterations", flush=True)
+    km, xd = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
+    _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
+    lab, fv = orc.predict(w.x, ref["cluster_centers"])
+    ref_km, _ = _fit(w.x, ref["cluster_centers"], w.k, 1, None, cuda)
+    pred = ref_km.predict(ht.array(w.x.to(cuda), split=0))  # predicts against centroids after 1 more step
+    pred0 = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(ref["cluster_centers"].to(cuda)), max_iter=1)
+    pred0._cluster_centers = ht.array(ref["cluster_centers"].to(cuda))
+    p = pred0.predict(xd)
+    assert float((p.larray.cpu() == lab).float().mean()) >= 0.9999
+    assert orc.rel_err_scalar(float(pred0.functional_value_), float(fv)) <= 1e-4
+    assert pred.shape == (w.x.shape[0], 1)
+    km2, _ = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
+    assert torch.equal(km.cluster_centers_.larray, km2.cluster_centers_.larray)
+    assert torch.equal(km.labels_.larray, km2.labels_.larray)
+    assert float(km.inertia_) == float(km2.inertia_)
+
+
+@pytest.mark.parametrize("cfg,scale", [("c3", 0.01), ("c4", 0.004), ("c5", 0.005)])
+def test_scaled_configs_against_oracle(cuda, cfg, scale):
+    w = synthetic.CONFIGS[cfg](scale)
+    print(f"{w.name} scaled to {tuple(w.x.shape)}", flush=True)
+    flips, ref = _stepwise_parity(w, cuda, w.max_iter, literal=False)
+    print(f"{w.name}: {flips} excused tie flips over {ref['n_iter']} iterations", flush=True)
+    km, _ = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
+    _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
+
+
+@pytest.mark.parametrize("scale", [1.0 / 16, 1.0])
+def test_config2_cdist_argmin(cuda, scale):
+    from heat_amd import _native
+
+    w = synthetic.config2(scale)
+    n = w.x.shape[0]
+    lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+    md = torch.empty((n,), dtype=torch.float32, device=cuda)
+    _native.assign(w.x.to(cuda), w.y.to(cuda), lab, md, _native.Workspace(cuda))
+    ref_lab, ref_md = orc.assign_to_cluster_fast(w.x, w.y, want_min=True)
+    rep = orc.label_agreement(w.x, w.y, lab.cpu(), ref_lab)
+    assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, rep
+    same = lab.cpu().long() == ref_lab.view(-1)
+    assert torch.allclose(md.cpu()[same], ref_md[same], rtol=1e-4, atol=1e-3)
+
+
+def _full_size_properties(w, dev, iters):
+    """Properties that hold at any size: counts sum to N, sum_k n_k C_k = sum_i x_i, the shift
+    sequence is what the centroids say, SSE does not increase, predict == re-assignment, a random row
+    sample agrees with the oracle, and two runs are bit-identical."""
+    from heat_amd import _native
+
+    n, d = w.x.shape
+    x = w.x.to(dev)
+    xd = ht.array(x, split=0)
+    ws = _native.Workspace(dev)
+    c_cur = w.init.to(dev).clone()
+    c_nxt = torch.empty_like(c_cur)
+    lab = torch.empty((n,), dtype=torch.int32, device=dev)
+    shift = torch.empty((), device=dev)
+    sse = torch.empty((), device=dev)
+    xsum = x.sum(0, dtype=torch.float64)
+    sse_hist = []
+    for it in range(iters):
+        _native.lloyd_step(x, c_cur, c_nxt, lab, shift, sse, ws)
+        cnt = torch.bincount(lab.long(), minlength=w.k)
+        assert int(cnt.sum()) == n
+        recon = (c_nxt.double() * cnt.view(-1, 1)).sum(0)
+        assert float((recon - xsum).abs().max()) <= 1e-5 * float(xsum.abs().max() + n * 1e-3)
+        ref_shift = ((c_cur.double() - c_nxt.double()) ** 2).sum()
+        assert orc.rel_err_scalar(float(shift), float(ref_shift), floor=1e-12) <= 1e-4
+        sse_hist.append(float(sse))
+        if it == 0:
+            # a seeded row sample against the oracle, same centroids
+            idx = torch.randperm(n, generator=torch.Generator().manual_seed(1))[:200_000]
+            ref_lab, _ = orc.assign_to_cluster_fast(w.x[idx], w.init)
+            rep = orc.label_agreement(w.x[idx], w.init, lab[idx.to(dev)].cpu(), ref_lab)
+            assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, rep
+        c_cur, c_nxt = c_nxt, c_cur
+    assert all(b <= a * (1 + 1e-5) for a, b in zip(sse_hist, sse_hist[1:])), sse_hist
+    km = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(dev)), max_iter=iters, tol=0.0).fit(xd)
+    assert torch.equal(km.cluster_centers_.larray, c_cur), "fit() and the step loop must agree bit for bit"
+    assert torch.equal(km.labels_.larray.view(-1), lab.long())
+    pred = km.predict(xd)
+    lab2 = torch.empty_like(lab)
+    _native.assign(x, c_cur, lab2, None, ws)
+    assert torch.equal(pred.larray.view(-1), lab2.long())
+
+
+def test_config3_full_size_properties(cuda):
+    _full_size_properties(synthetic.config3(), cuda, iters=3)
+
+
+def test_config5_full_size_properties(cuda):
+    _full_size_properties(synthetic.config5(), cuda, iters=2)
+
+
+def test_config4_full_size_properties(cuda):
+    _full_size_properties(synthetic.config4(), cuda, iters=2)
+
+
+def test_random_init_and_fit_predict(cuda):
+    w = synthetic.config1(0.2)
+    x = ht.array(w.x.to(cuda), split=0)
+    a = ht.cluster.KMeans(n_clusters=5, init="random", max_iter=5, random_state=3).fit(x)
+    b = ht.cluster.KMeans(n_clusters=5, init="random", max_iter=5, random_state=3).fit(x)
+    assert a.cluster_centers_.shape == (5, 8)
+    assert torch.equal(a.cluster_centers_.larray, b.cluster_centers_.larray)
+    lab = ht.cluster.KMeans(n_clusters=5, init="random", max_iter=5, random_state=3).fit_predict(x)
+    assert lab.shape == (w.x.shape[0], 1) and int(lab.larray.max()) < 5
+    # int32 data is promoted to float32, unsplit data is accepted
+    xi = ht.array((w.x * 10).to(torch.int32).to(cuda))
+    c = ht.cluster.KMeans(n_clusters=4, init="random", max_iter=3, random_state=1).fit(xi)
+    assert c.cluster_centers_.shape == (4, 8) and c.cluster_centers_.dtype is ht.float32

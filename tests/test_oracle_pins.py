@@ -1,0 +1,232 @@
+"""
+Pins of the CPU oracle (oracle/heat_oracle.py): every function is checked against something it was
+NOT written from -- the known-answer vectors of the reference's own tests, closed forms, brute
+force in fp64, library routines (torch.cdist, torch.argmin, scikit-learn's Lloyd) -- chosen so
+that a dropped term, a wrong sign or a transposed operand fails.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import heat_oracle as orc
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+# ---- distances --------------------------------------------------------------------------------
+def test_cdist_known_answers_of_reference_tests():
+    # tests/spatial/test_distances.py:16-58 of the reference: ones vs zeros with D = 4 -> 2.0,
+    # X vs X -> 0.0, for both metrics
+    X, Y = torch.ones((4, 4)), torch.zeros((4, 4))
+    for qe in (True, False):
+        assert torch.equal(orc.cdist(X, Y, quadratic_expansion=qe), torch.full((4, 4), 2.0))
+        assert torch.allclose(orc.cdist(X, quadratic_expansion=qe), torch.zeros((4, 4)))
+        assert torch.allclose(orc.cdist(X, X, quadratic_expansion=qe), torch.zeros((4, 4)))
+
+
+def test_cdist_row_scaled_ones_vs_torch_cdist():
+    # tests/spatial/test_distances.py:207-222: rows i * ones(6); compared with torch.cdist, atol 1e-5
+    A = torch.ones((8, 6)) * torch.arange(8, dtype=torch.float32).view(-1, 1)
+    ref = torch.cdist(A, A)
+    assert torch.allclose(orc.cdist(A, A, quadratic_expansion=True), ref, atol=1e-5)
+    assert torch.allclose(orc.cdist(A, A.to(torch.int32), quadratic_expansion=True), ref, atol=1e-5)
+    assert orc.cdist(A, A.to(torch.int32)).dtype == torch.float32  # int32 + float32 -> float32
+    assert orc.cdist(A, A.to(torch.int64)).dtype == torch.float64  # int64 + float32 -> float64
+    assert orc.cdist(A.double(), A).dtype == torch.float64
+    # analytic: |i - j| * sqrt(6)
+    i = torch.arange(8, dtype=torch.float64)
+    assert torch.allclose(orc.cdist(A, A).double(), (i.view(-1, 1) - i.view(1, -1)).abs() * 6**0.5, atol=1e-5)
+
+
+def test_quadratic_expand_vs_bruteforce_and_invariants():
+    g = torch.Generator().manual_seed(1)
+    x, y = torch.randn((50, 7), generator=g) * 3, torch.randn((30, 7), generator=g) * 3
+    q = orc.quadratic_expand(x, y)
+    bf = orc.brute_force_d2(x, y)
+    assert q.shape == (50, 30)  # a transposed operand would give (30, 50) or fail
+    assert torch.allclose(q.double(), bf, rtol=1e-4, atol=1e-4)
+    assert float(q.min()) >= 0.0
+    qq = orc.quadratic_expand(x, x)
+    assert torch.allclose(qq, qq.T, atol=1e-4)
+    assert float(qq.diag().abs().max()) <= 1e-3
+    # sign of the cross term: moving y towards x must decrease the distance
+    assert float(orc.quadratic_expand(x[:1], x[:1] * 0.9)[0, 0]) < float(orc.quadratic_expand(x[:1], -x[:1])[0, 0])
+    assert torch.equal(orc.euclidian_fast(x, y), torch.sqrt(q))
+
+
+def test_cdist_rejects_3d():
+    with pytest.raises(NotImplementedError):
+        orc.cdist(torch.ones((2, 3, 4)))
+
+
+# ---- assignment -------------------------------------------------------------------------------
+def test_assign_is_torch_argmin_keepdim_with_first_index_ties():
+    # tests/core/test_statistics.py:136-143 pins ht.argmin(keepdims=True) == torch.argmin(keepdim=True)
+    g = torch.Generator().manual_seed(2)
+    x, c = torch.randn((200, 5), generator=g), torch.randn((9, 5), generator=g)
+    lab, _ = orc.assign_to_cluster_literal(x, c)
+    assert lab.shape == (200, 1) and lab.dtype == torch.int64
+    assert torch.equal(lab, torch.argmin(orc.cdist(x, c), dim=1, keepdim=True))
+    bf = orc.brute_force_d2(x, c).argmin(dim=1)
+    assert float((lab.view(-1) == bf).float().mean()) == 1.0
+    # exact tie -> first index (torch.min semantics)
+    m, i = torch.min(torch.tensor([[1.0, 0.0, 0.0, 2.0], [3.0, 3.0, 3.0, 3.0]]), dim=1)
+    assert i.tolist() == [1, 0]
+    # the point IS centroid 1 and centroid 2: distance clamps to 0 for both, label 1
+    c2 = torch.stack([x[0] + 5, x[0], x[0]])
+    lab2, _ = orc.assign_to_cluster_literal(x[:1], c2)
+    assert int(lab2) == 1
+
+
+def test_fast_assign_matches_literal():
+    g = torch.Generator().manual_seed(3)
+    x, c = torch.randn((5000, 16), generator=g), torch.randn((33, 16), generator=g)
+    a, _ = orc.assign_to_cluster_literal(x, c)
+    b, md = orc.assign_to_cluster_fast(x, c, chunk=777, want_min=True)
+    rep = orc.label_agreement(x, c, a, b)
+    assert rep["n_unexcused"] == 0 and rep["agreement"] > 0.999
+    assert torch.allclose(md.double(), orc.brute_force_d2(x, c).min(1).values, rtol=1e-4, atol=1e-4)
+
+
+def test_functional_value_is_sse():
+    g = torch.Generator().manual_seed(4)
+    x, c = torch.randn((300, 6), generator=g), torch.randn((5, 6), generator=g)
+    lab, fv = orc.predict(x, c)
+    assert abs(float(fv) - orc.sse(x, c, lab)) <= 1e-4 * orc.sse(x, c, lab)
+    _, fv2 = orc.predict(x, c, literal=False)
+    assert abs(float(fv) - float(fv2)) <= 1e-5 * float(fv)
+
+
+# ---- update -----------------------------------------------------------------------------------
+def _mean_bruteforce(x, lab, k):
+    out = np.zeros((k, x.shape[1]), dtype=np.float64)
+    cnt = np.zeros(k, dtype=np.int64)
+    for row, l in zip(x.numpy().astype(np.float64), lab.view(-1).tolist()):
+        out[l] += row
+        cnt[l] += 1
+    return out / np.maximum(cnt, 1)[:, None], cnt
+
+
+def test_update_literal_vs_python_loop_and_invariants():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((400, 5), generator=g) * 2 + 1
+    lab = torch.randint(0, 7, (400, 1), generator=g)
+    lab[lab == 3] = 2  # cluster 3 empty
+    lit = orc.update_centroids_literal(x, lab, torch.full((7, 5), 9.0))
+    bf, cnt = _mean_bruteforce(x, lab, 7)
+    assert lit.dtype == torch.float32
+    assert np.allclose(lit.numpy(), bf, rtol=1e-6, atol=1e-7)
+    assert torch.all(lit[3] == 0)  # empty cluster -> zero row, not the old centroid (9.0)
+    fast, fcnt = orc.update_centroids_fast(x, lab, 7)
+    assert np.array_equal(fcnt.numpy(), cnt) and int(fcnt.sum()) == 400
+    assert torch.allclose(fast, lit, rtol=1e-6, atol=1e-7)
+    # sum_k cnt_k * C_k == sum_i x_i
+    assert np.allclose((fast.double() * fcnt.view(-1, 1)).sum(0).numpy(), x.double().sum(0).numpy(), rtol=1e-5)
+    # the sum-then-divide formulation of the reference's own torch baseline
+    # (benchmarks/2020/kmeans/torch-cpu.py:36-50) gives the same means
+    for i in range(7):
+        sel = (lab == i).float()
+        alt = (x * sel).sum(0) / sel.sum().clamp(1.0)
+        assert torch.allclose(alt, lit[i], rtol=1e-5, atol=1e-6)
+
+
+def test_count_passes_through_fp32():
+    # clamp(1.0, int64max) of an int64 tensor yields float32 under torch: 25 000 001 -> 25 000 000
+    c = torch.tensor([[25000001]], dtype=torch.int64).clamp(1.0, orc.INT64_MAX)
+    assert c.dtype == torch.float32 and float(c) == 25000000.0
+
+
+# ---- the loop ---------------------------------------------------------------------------------
+def test_fit_closed_forms():
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((500, 4), generator=g)
+    # K = 1: the centroid is the global mean after one iteration, shift 0 in the second
+    r = orc.kmeans_fit(x, x[:1].clone(), 5, 0.0)
+    assert torch.allclose(r["cluster_centers"][0], x.double().mean(0).float(), atol=1e-6)
+    assert r["n_iter"] == 2 and float(r["inertia"]) == 0.0
+    # K = N distinct points: fixed point, stops after the first iteration with shift exactly 0
+    xs = x[:20]
+    r = orc.kmeans_fit(xs, xs.clone(), 7, 0.0)
+    assert r["n_iter"] == 1 and float(r["inertia"]) == 0.0
+    assert torch.equal(r["labels"].view(-1), torch.arange(20))
+    # tol=None never stops early
+    r = orc.kmeans_fit(xs, xs.clone(), 7, None)
+    assert r["n_iter"] == 7
+    # init at the optimum of two far-apart blobs: converged in <= 2 iterations, labels are the blobs
+    blobs = torch.cat([x[:250] * 0.1 + 10, x[250:] * 0.1 - 10])
+    c0 = torch.stack([blobs[:250].mean(0), blobs[250:].mean(0)])
+    r = orc.kmeans_fit(blobs, c0, 10, 0.0)
+    assert r["n_iter"] <= 2
+    assert torch.equal(r["labels"].view(-1), torch.cat([torch.zeros(250), torch.ones(250)]).long())
+    # labels_ belong to the centroids BEFORE the last update (kmeans.py:146)
+    r = orc.kmeans_fit(x, x[:3].clone(), 1, None)
+    lab0, _ = orc.assign_to_cluster_literal(x, x[:3])
+    assert torch.equal(r["labels"], lab0)
+    # wrong init shapes
+    with pytest.raises(ValueError):
+        orc.kmeans_fit(x, torch.ones(4), 1, 0.0)
+    with pytest.raises(ValueError):
+        orc.kmeans_fit(x, torch.ones((3, 5)), 1, 0.0)
+
+
+def test_fit_matches_sklearn_lloyd():
+    sk = pytest.importorskip("sklearn.cluster")
+    g = torch.Generator().manual_seed(7)
+    cent = torch.randn((5, 6), generator=g) * 6
+    x = (cent[torch.randint(0, 5, (3000,), generator=g)] + torch.randn((3000, 6), generator=g)).contiguous()
+    c0 = x[:5].clone()
+    r = orc.kmeans_fit(x, c0, 8, None)
+    km = sk.KMeans(n_clusters=5, init=c0.numpy(), n_init=1, max_iter=8, tol=0.0, algorithm="lloyd").fit(x.numpy())
+    # no empty clusters here, so both implement the same iteration
+    assert np.allclose(r["cluster_centers"].numpy(), km.cluster_centers_, rtol=1e-4, atol=1e-4)
+    lab_final, _ = orc.assign_to_cluster_literal(x, r["cluster_centers"])
+    assert float((lab_final.view(-1).numpy() == km.labels_).mean()) > 0.999
+
+
+def test_fast_fit_matches_literal_fit():
+    g = torch.Generator().manual_seed(8)
+    cent = torch.randn((12, 8), generator=g) * 4
+    x = (cent[torch.randint(0, 12, (6000,), generator=g)] + torch.randn((6000, 8), generator=g)).contiguous()
+    a = orc.kmeans_fit(x, x[:12].clone(), 6, 0.0, literal=True)
+    b = orc.kmeans_fit(x, x[:12].clone(), 6, 0.0, literal=False, chunk=1000)
+    assert a["n_iter"] == b["n_iter"]
+    assert orc.rel_err_centers(a["cluster_centers"], b["cluster_centers"]) <= 1e-6
+    assert float((a["labels"] == b["labels"]).float().mean()) >= 0.9995
+
+
+# ---- golden fixtures --------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["iris_k3", "edge_k4", "translated_k2"])
+def test_oracle_reproduces_golden(name):
+    z = np.load(os.path.join(GOLD, name + ".npz"))
+    x, c0 = torch.from_numpy(z["x"]), torch.from_numpy(z["init"])
+    r = orc.kmeans_fit(x, c0, int(z["max_iter"]), 0.0)
+    assert r["n_iter"] == int(z["n_iter"])
+    assert np.allclose(r["cluster_centers"].numpy(), z["centers"], rtol=1e-6, atol=1e-7)
+    assert np.array_equal(r["labels"].numpy(), z["labels"])
+    assert np.allclose(np.asarray(r["shifts"]), z["shifts"], rtol=1e-5, atol=1e-12)
+
+
+def test_golden_translated_copies_invariant():
+    # doc/source/tutorials/tutorial_clustering.rst:22-80 of the reference: two translated copies of
+    # one cloud split 100/100 and the centroids differ by exactly the translation (4.0 per axis)
+    z = np.load(os.path.join(GOLD, "translated_k2.npz"))
+    assert np.bincount(z["labels"].ravel()).tolist() == [100, 100]
+    assert np.allclose(z["centers"][0] - z["centers"][1], 4.0, atol=1e-5)
+
+
+def test_golden_iris_file_is_the_reference_dataset():
+    iris = np.loadtxt(os.path.join(GOLD, "iris.csv"), delimiter=";", dtype=np.float32)
+    assert iris.shape == (150, 4)
+    assert iris[0].tolist() == pytest.approx([5.1, 3.5, 1.4, 0.2])
+    # textbook means of the iris columns
+    assert iris.mean(0).tolist() == pytest.approx([5.8433, 3.054, 3.7587, 1.1987], abs=2e-3)
+
+
+def test_label_agreement_excuses_only_numerical_ties():
+    x = torch.tensor([[0.0, 0.0], [1.0, 0.0]])
+    c = torch.tensor([[-1.0, 0.0], [1.0 + 1e-7, 0.0], [5.0, 5.0]])
+    a = torch.tensor([0, 1])
+    assert orc.label_agreement(x, c, a, torch.tensor([1, 1]))["n_unexcused"] == 0  # row 0: near tie
+    assert orc.label_agreement(x, c, a, torch.tensor([2, 1]))["n_unexcused"] == 1  # row 0: wrong
