@@ -58,6 +58,8 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
     };
     w.red = reinterpret_cast<double*>(take(size_t(RED_SLOTS) * sizeof(double)));
     if (flags & HKM_WS_ASSIGN) w.cn = reinterpret_cast<float*>(take(cn_pad(K) * sizeof(float)));
+    if ((flags & HKM_WS_UPDATE) && small_eligible(D, K))
+        w.small_part = reinterpret_cast<double*>(take(size_t(SMALL_MAX_GRID) * (size_t(K) * (D + 1) + 1) * sizeof(double)));
     if (flags & HKM_WS_UPDATE) {
         const UpdateGeom g = update_geom(N, D, K);
         w.part_sum = reinterpret_cast<float*>(take(size_t(g.S) * K * g.J * 32 * sizeof(float)));
@@ -96,6 +98,8 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
     if (N == 0) return HKM_OK;
     switch (assign_kind(D, K)) {
         case ASSIGN_VALU:
+            if (small_eligible(D, K))
+                return launch_small(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, 0, st);
             return launch_assign_valu(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_RESIDENT:
             return launch_assign_mfma_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
@@ -126,7 +130,7 @@ const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K) {
     (void)N;
     if (D < 1 || K < 1) return "invalid";
     switch (assign_kind(D, K)) {
-        case ASSIGN_VALU: return "valu";
+        case ASSIGN_VALU: return small_eligible(D, K) ? "valu_fused" : "valu";
         case ASSIGN_MFMA_RESIDENT: return "mfma_resident";
         default: return "mfma_stream";
     }
@@ -179,6 +183,11 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const Workspace w = carve(ws, N, D, K, flags);
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    if (small_eligible(D, K) && N > 0) {
+        // one sweep over X: labels + private per-lane sums, then a single-workgroup finish
+        if ((rc = launch_small(X, N, D, ldx, C, K, D, labels, nullptr, w.small_part, sse ? 3 : 1, st))) return rc;
+        return launch_small_finalize(w.small_part, small_grid(N, D, K), K, D, C, C_new, D, nullptr, shift, sse, st);
+    }
     if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;
     if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, st))) return rc;
     if ((rc = launch_shift(C, C_new, K, D, shift, st))) return rc;

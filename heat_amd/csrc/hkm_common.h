@@ -51,9 +51,11 @@ struct Workspace {
     int64_t* counts;    // [K]
     double* red;        // [RED_SLOTS] scratch for scalar reductions
     float* min_d2;      // [N] (only with the SSE flag)
+    double* small_part; // [SMALL_MAX_GRID][K*(D+1)+1] partial rows of the one-sweep small-D step
     size_t total;
 };
 static const int RED_SLOTS = 2048;
+static const int SMALL_MAX_GRID = 2048;
 Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags);
 
 // ---- launchers (one per .hip file) ------------------------------------------------------------
@@ -67,6 +69,14 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                               int32_t K, int64_t ldc, const float* cn, int32_t* labels,
                               float* min_d2, hipStream_t st);
+bool small_eligible(int32_t D, int32_t K);
+int small_grid(int64_t N, int32_t D, int32_t K);
+int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                 int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
+                 hipStream_t st);
+int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, const float* C_old,
+                          float* C_new, int64_t ldcn, int64_t* counts, float* shift, float* sse,
+                          hipStream_t st);
 int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                   hipStream_t st);

@@ -1,0 +1,488 @@
+// One-sweep Lloyd step for small feature counts (D <= 8) and small K*(D+1): X is read from HBM
+// exactly once per iteration (4D bytes per point) and only the labels are written (4 bytes).
+//
+// Assignment: a lane owns PPT consecutive points in registers; centroids and their squared norms
+// sit in LDS and are read as wave-wide broadcasts; d2 = (|x|^2 + |c|^2) - 2 x.c exactly in the
+// reference's evaluation order (heat/spatial/distance.py:59-64), first index wins ties
+// (torch.min, heat/core/statistics.py:177).  The clamp at 0 is applied lazily: a negative minimum
+// (a point that coincides with a centroid up to rounding) triggers a rescan with the clamp applied
+// to every candidate, so the result equals clamping first.
+//
+// Update (heat/cluster/kmeans.py:76-103) without atomics, two strategies with a fixed summation order:
+//   K*(D+1) <= 48: every lane owns a private fp32 column per (cluster, coordinate) in LDS and adds
+//     its own points in program order; the read-add-write round trips of a round are deferred to the
+//     next round and interleaved with its arithmetic.  At the end lanes' columns are added in a fixed
+//     fp64 tree.
+//   otherwise: for every cluster k and coordinate d the wavefront forms
+//     sum over lanes of [label == k] * x_d with a fixed DPP tree (row shifts, then row broadcasts;
+//     the total lands in lane 63) and lane 63 adds it to the wave's private fp64 row in LDS.
+// Either way the workgroup writes one fp64 partial row; a single-workgroup kernel adds the rows in a
+// fixed order, divides by the count (rounded through fp32 like the reference,
+// heat/core/rounding.py:156-164) and computes the centroid shift (kmeans.py:141).
+#include <type_traits>
+
+#include "hkm_common.h"
+
+namespace hkm {
+
+__device__ __forceinline__ floatx4 ldg4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
+
+template <int D>
+struct SmallCfg {
+    // points per lane so that a lane's chunk is a whole number of 16-byte vectors
+    static constexpr int PPT = (D % 4 == 0) ? 2 : (D % 2 == 0) ? 2 : 4;
+    static constexpr int SC = (D + 1 + 3) / 4 * 4;  // LDS centroid row: D coords, |c|^2, pad
+};
+
+bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
+static constexpr int SMALL_T = 256;
+int small_grid(int64_t N, int32_t D, int32_t K) {
+    (void)K;
+    const int ppt = (D % 2 == 0) ? 2 : 4;
+    const int64_t groups = (N + ppt - 1) / ppt;
+    // at least 8 groups per lane where the input allows it, at most 4 workgroups per CU
+    int64_t want = (groups + SMALL_T * 8 - 1) / (SMALL_T * 8);
+    int64_t cap = int64_t(num_cus()) * 4;
+    if (cap > SMALL_MAX_GRID) cap = SMALL_MAX_GRID;
+    if (want > cap) want = cap;
+    if (want < 1) want = 1;
+    return int(want);
+}
+
+// sum over the 64 lanes with a fixed tree; the total is valid in lane 63
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+#define HKM_DPP_ADD(ctrl, rmask, bmask)                                                              \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, \
+                                                               rmask, bmask, true))
+    HKM_DPP_ADD(0x111, 0xf, 0xf);  // row_shr:1
+    HKM_DPP_ADD(0x112, 0xf, 0xf);  // row_shr:2
+    HKM_DPP_ADD(0x114, 0xf, 0xf);  // row_shr:4
+    HKM_DPP_ADD(0x118, 0xf, 0xf);  // row_shr:8  -> lane 15 of each row holds the row sum
+    HKM_DPP_ADD(0x142, 0xa, 0xf);  // row_bcast:15 into rows 1 and 3
+    HKM_DPP_ADD(0x143, 0xc, 0xf);  // row_bcast:31 into rows 2 and 3
+#undef HKM_DPP_ADD
+    return v;
+}
+
+template <int D, int PPT, bool CLAMP>
+__device__ __forceinline__ void scan_centroids(const float* sC, int k0, int k1,
+                                               const float (&x)[PPT][D], const float (&xn)[PPT],
+                                               float (&m)[PPT], int (&mi)[PPT]) {
+    constexpr int SC = SmallCfg<D>::SC;
+#pragma unroll 2
+    for (int k = k0; k < k1; ++k) {
+        float c[SC];
+#pragma unroll
+        for (int q = 0; q < SC / 4; ++q) {
+            const floatx4 v = *reinterpret_cast<const floatx4*>(sC + k * SC + 4 * q);
+            c[4 * q] = v[0];
+            c[4 * q + 1] = v[1];
+            c[4 * q + 2] = v[2];
+            c[4 * q + 3] = v[3];
+        }
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            float dot = x[p][0] * c[0];
+#pragma unroll
+            for (int d = 1; d < D; ++d) dot = fmaf(x[p][d], c[d], dot);
+            float dist = fmaf(-2.0f, dot, xn[p] + c[D]);
+            if (CLAMP) dist = fmaxf(dist, 0.0f);
+            mi[p] = dist < m[p] ? k : mi[p];
+            m[p] = fminf(m[p], dist);
+        }
+    }
+}
+
+// ACC: 0 = labels only, 1 = per-lane private LDS columns, 2 = DPP wave tree + per-wave fp64 rows
+template <int D, int ACC, bool WANT_MIN, bool WANT_SSE>
+__global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
+    const float* __restrict__ X, int64_t N, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2,
+    double* __restrict__ part, int vec) {
+    constexpr int T = SMALL_T;
+    constexpr int PPT = SmallCfg<D>::PPT;
+    constexpr int SC = SmallCfg<D>::SC;
+    constexpr int NV = PPT * D / 4;  // 16-byte vectors per lane
+    constexpr int NW = T / 64;
+    extern __shared__ __align__(16) float lds[];
+    float* sC = lds;  // [K][SC]
+    const int slots = K * (D + 1);
+    constexpr bool ACCUM = ACC != 0;
+    float* stage = lds + ((K * SC + 3) & ~3);                        // [NW][NV*64*4] transpose buffer
+    float* after = stage + NW * NV * 256;
+    double* wacc_all = reinterpret_cast<double*>(after);             // ACC==2: [NW][slots]
+    float* cols = after;                                             // ACC==1: [slots][T]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    double* wacc = wacc_all + wave * slots;
+    float* wstage = stage + wave * NV * 256;
+
+    for (int i = tid; i < K * SC; i += T) {
+        const int r = i / SC, c = i - r * SC;
+        sC[i] = c < D ? C[int64_t(r) * ldc + c] : 0.f;
+    }
+    if (ACC == 2)
+        for (int i = tid; i < NW * slots; i += T) wacc_all[i] = 0.0;
+    if (ACC == 1)
+        for (int i = tid; i < (slots + D + 1) * T; i += T) cols[i] = 0.f;
+    __syncthreads();
+    for (int r = tid; r < K; r += T) {
+        float s = 0.f;
+#pragma unroll
+        for (int d = 0; d < D; ++d) s = __fadd_rn(s, __fmul_rn(sC[r * SC + d], sC[r * SC + d]));
+        sC[r * SC + D] = s;
+    }
+    __syncthreads();
+
+    double sse = 0.0;
+    const int64_t groups = (N + PPT - 1) / PPT;
+    const int64_t full = vec ? N / PPT : 0;  // groups served by the 16-byte vector path
+    const int64_t stride = int64_t(gridDim.x) * T;
+
+    // ACC == 1: the additions of a round are deferred to the NEXT round and interleaved with its
+    // arithmetic, so that the LDS read -> add -> write round trips of the PPT points (which must stay
+    // sequential: two points of a lane may share a cluster) hide behind independent work.  A lane's
+    // pending points live in pcol (column offset of their cluster, or of a dummy cluster that
+    // collects nothing useful) and px.
+    const int dummy_col = slots * T + tid;
+    int pcol[PPT];
+    float px[PPT][D + 1];
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) {
+        pcol[p] = dummy_col;
+#pragma unroll
+        for (int d = 0; d <= D; ++d) px[p][d] = 0.f;
+    }
+    auto rmw_read = [&](int p, float (&r)[D + 1]) {
+#pragma unroll
+        for (int d = 0; d <= D; ++d) r[d] = cols[pcol[p] + d * T];
+    };
+    auto rmw_write = [&](int p, const float (&r)[D + 1]) {
+#pragma unroll
+        for (int d = 0; d <= D; ++d) cols[pcol[p] + d * T] = r[d] + px[p][d];
+    };
+
+    // label + accumulate one group of PPT points held in registers.  Executed by ALL lanes of the
+    // wave (the DPP tree needs them); GUARD: rows >= N contribute nothing and store nothing.
+    auto process = [&](int64_t i0, const float (&x)[PPT][D], auto guard_tag) {
+        constexpr bool GUARD = decltype(guard_tag)::value;
+        float xn[PPT], m[PPT];
+        int mi[PPT];
+        float r[D + 1];
+        if (ACC == 1) rmw_read(0, r);
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            float s = 0.f;
+#pragma unroll
+            for (int d = 0; d < D; ++d) s = __fadd_rn(s, __fmul_rn(x[p][d], x[p][d]));
+            xn[p] = s;
+            m[p] = HKM_INF;
+            mi[p] = 0;
+        }
+        const int kh = K >> 1;
+        if (ACC == 1 && PPT == 4) {
+            rmw_write(0, r);
+            rmw_read(1, r);
+        }
+        scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
+        if (ACC == 1) {
+            rmw_write(PPT == 4 ? 1 : 0, r);
+            rmw_read(PPT == 4 ? 2 : 1, r);
+        }
+        scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
+        if (ACC == 1 && PPT == 4) {
+            rmw_write(2, r);
+            rmw_read(3, r);
+        }
+        bool neg = false;
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) neg |= (m[p] < 0.f);
+        if (__any(neg)) {
+#pragma unroll
+            for (int p = 0; p < PPT; ++p) {
+                m[p] = HKM_INF;
+                mi[p] = 0;
+            }
+            scan_centroids<D, PPT, true>(sC, 0, K, x, xn, m, mi);
+        }
+
+        if constexpr (!GUARD) {
+            if constexpr (PPT == 4) {
+                *reinterpret_cast<int4*>(labels + i0) = make_int4(mi[0], mi[1], mi[2], mi[3]);
+            } else {
+                *reinterpret_cast<int2*>(labels + i0) = make_int2(mi[0], mi[1]);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            const bool ok = !GUARD || i0 + p < N;
+            if (ok) {
+                if (GUARD) labels[i0 + p] = mi[p];
+                if (WANT_MIN) min_d2[i0 + p] = m[p];
+                if (WANT_SSE) sse += double(m[p]);
+            } else {
+                mi[p] = -1;  // matches no cluster below
+            }
+        }
+        if (ACC == 1) {
+            rmw_write(PPT - 1, r);
+            // this round's points become the pending ones
+#pragma unroll
+            for (int p = 0; p < PPT; ++p) {
+                pcol[p] = (GUARD && mi[p] < 0) ? dummy_col : (mi[p] * (D + 1)) * T + tid;
+#pragma unroll
+                for (int d = 0; d < D; ++d) px[p][d] = x[p][d];
+                px[p][D] = 1.0f;
+            }
+        }
+        if (ACC == 2) {
+            for (int k = 0; k < K; ++k) {
+                float f[PPT], v[D + 1];
+#pragma unroll
+                for (int p = 0; p < PPT; ++p) f[p] = (mi[p] == k) ? 1.0f : 0.0f;
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    v[d] = f[0] * x[0][d];
+#pragma unroll
+                    for (int p = 1; p < PPT; ++p) v[d] = fmaf(f[p], x[p][d], v[d]);
+                }
+                v[D] = f[0];
+#pragma unroll
+                for (int p = 1; p < PPT; ++p) v[D] += f[p];
+#pragma unroll
+                for (int d = 0; d <= D; ++d) v[d] = wave_sum_to_lane63(v[d]);
+                if (lane == 63) {
+#pragma unroll
+                    for (int d = 0; d <= D; ++d) wacc[k * (D + 1) + d] += double(v[d]);
+                }
+            }
+        }
+    };
+
+    // Main loop, identical trip count for every lane of the workgroup.  Rounds in which the whole
+    // workgroup lies inside the vector-loadable range take the fast path; the next round's rows are
+    // requested before the current round is processed.
+    const int64_t wg0 = int64_t(blockIdx.x) * T;
+    int64_t base = wg0;
+    {
+        // A wave's 64 groups are NV*1024 contiguous bytes: fetched as NV fully coalesced 16-byte
+        // loads per lane, then redistributed through a wave-private LDS buffer so that every lane
+        // ends up with its own PPT consecutive points.
+        constexpr int PF = 3;  // rounds in flight: enough bytes per CU to cover the HBM latency
+        floatx4 nxt[PF][NV];
+        const float* wsrc = X + (base + wave * 64) * (PPT * D) + lane * 4;
+        const int64_t rstride = stride * (PPT * D);
+#pragma unroll
+        for (int f = 0; f < PF; ++f) {
+            if (base + f * stride + T <= full) {
+#pragma unroll
+                for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + f * rstride + v * 256);
+            }
+        }
+        // The loop is unrolled PF times so that each round's buffer is a fixed set of registers: a
+        // register rotation would make every round wait for ALL outstanding loads.
+        bool more = base + T <= full;
+        while (more) {
+#pragma unroll
+            for (int f = 0; f < PF; ++f) {
+                if (more) {
+                    float x[PPT][D];
+#pragma unroll
+                    for (int v = 0; v < NV; ++v)
+                        *reinterpret_cast<floatx4*>(wstage + v * 256 + lane * 4) = nxt[f][v];
+                    if (base + PF * stride + T <= full) {
+#pragma unroll
+                        for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + PF * rstride + v * 256);
+                    }
+                    wsrc += rstride;
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        const floatx4 q =
+                            *reinterpret_cast<const floatx4*>(wstage + lane * (PPT * D) + 4 * v);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) x[(4 * v + t) / D][(4 * v + t) % D] = q[t];
+                    }
+                    process((base + tid) * PPT, x, std::false_type{});
+                    base += stride;
+                    more = base + T <= full;
+                }
+            }
+        }
+    }
+    // remaining rounds: unaligned / strided inputs and the ragged end, rows clamped and guarded
+    for (; base < groups; base += stride) {
+        const int64_t i0 = (base + tid) * PPT;
+        float x[PPT][D];
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            const int64_t r = (i0 + p < N) ? i0 + p : N - 1;
+#pragma unroll
+            for (int d = 0; d < D; ++d) x[p][d] = X[r * ldx + d];
+        }
+        process(i0, x, std::true_type{});
+    }
+
+    if (ACC == 1) {
+        // the last round's points are still pending
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            float r[D + 1];
+            rmw_read(p, r);
+            rmw_write(p, r);
+        }
+    }
+    if (ACCUM || WANT_SSE) {
+        __syncthreads();
+        double* prow = part + int64_t(blockIdx.x) * (slots + 1);
+        if (ACC == 2) {
+            for (int s = tid; s < slots; s += T) {
+                double v = 0.0;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) v += wacc_all[w * slots + s];
+                prow[s] = v;
+            }
+        }
+        if (ACC == 1) {
+            // lanes add their T/64 columns in ascending order, then a butterfly over the 64 lanes
+            for (int s = wave; s < slots; s += NW) {
+                double v = 0.0;
+                for (int t = lane; t < T; t += 64) v += double(cols[s * T + t]);
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+                if (lane == 0) prow[s] = v;
+            }
+        }
+        if (WANT_SSE) {
+            __shared__ double ssh[NW];
+            double v = sse;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+            if (lane == 0) ssh[wave] = v;
+            __syncthreads();
+            if (tid == 0) {
+                double t = 0.0;
+                for (int w = 0; w < NW; ++w) t += ssh[w];
+                prow[slots] = t;
+            }
+        }
+    }
+}
+
+// One workgroup of 1024 threads finishes the step.  Thread (j, s) adds the partial rows g = j, j+J,
+// ... of slot s in ascending order (8 independent loads in flight, additions still in row order);
+// thread (0, s) then adds the J strided sums in ascending j.  The order depends only on (G, slots).
+__global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
+    const double* __restrict__ part, int G, int K, int D, const float* __restrict__ C_old,
+    float* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts,
+    float* __restrict__ shift, float* __restrict__ sse_out, int have_sse, int spad) {
+    __shared__ double strided[1024];
+    __shared__ double tot[256];
+    __shared__ double red[1024];
+    const int tid = threadIdx.x;
+    const int slots = K * (D + 1);
+    const int nslot = slots + 1;  // last = sum of min d2
+    const int J = 1024 / spad;
+    const int s = tid % spad, j = tid / spad;
+    double v = 0.0;
+    if (s < nslot && (s < slots || have_sse)) {
+        int g = j;
+        for (; g + 7 * J < G; g += 8 * J) {
+            double t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = part[int64_t(g + u * J) * nslot + s];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v += t[u];
+        }
+        for (; g < G; g += J) v += part[int64_t(g) * nslot + s];
+    }
+    strided[tid] = v;
+    __syncthreads();
+    if (j == 0 && s < nslot) {
+        double t = 0.0;
+        for (int q = 0; q < J; ++q) t += strided[q * spad + s];
+        tot[s] = t;
+    }
+    __syncthreads();
+    double sq = 0.0;
+    for (int i = tid; i < K * D; i += 1024) {
+        const int k = i / D, d = i - k * D;
+        const int64_t n = (int64_t)tot[k * (D + 1) + D];
+        const double cnt = double(float(n < 1 ? 1 : n));
+        const float c = float(tot[k * (D + 1) + d] / cnt);
+        C_new[int64_t(k) * ldcn + d] = c;
+        if (C_old) {
+            const float df = C_old[int64_t(k) * D + d] - c;
+            sq += double(df * df);
+        }
+        if (d == 0 && counts) counts[k] = n;
+    }
+    red[tid] = sq;
+    __syncthreads();
+    for (int w = 512; w > 0; w >>= 1) {
+        if (tid < w) red[tid] += red[tid + w];
+        __syncthreads();
+    }
+    if (tid == 0) {
+        if (shift) *shift = float(red[0]);
+        if (sse_out && have_sse) *sse_out = float(tot[slots]);
+    }
+}
+
+template <int D>
+static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C, int32_t K,
+                          int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
+                          int grid, hipStream_t st) {
+    constexpr int SC = SmallCfg<D>::SC;
+    const bool accum = mode & 1, want_sse = mode & 2, want_min = min_d2 != nullptr;
+    constexpr int NV = SmallCfg<D>::PPT * D / 4;
+    const int slots = K * (D + 1);
+    // per-lane LDS columns while they fit (slots * 1 KB), the DPP tree otherwise
+    const int acc_mode = !accum ? 0 : (slots <= 48 ? 1 : 2);
+    const size_t lds = size_t((K * SC + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * NV * 256 * sizeof(float) +
+                       (acc_mode == 2 ? size_t(SMALL_T / 64) * slots * sizeof(double)
+                        : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float) : 0);
+    const int vec = (ldx == D) && aligned16(X) && aligned16(labels);
+#define HKM_GO(A, M, S)                                                                             \
+    hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S>), dim3(grid), dim3(SMALL_T), lds, st, X, N, ldx, \
+                       C, K, ldc, labels, min_d2, part, vec)
+    if (acc_mode == 1) {
+        if (want_sse) HKM_GO(1, false, true);
+        else HKM_GO(1, false, false);
+    } else if (acc_mode == 2) {
+        if (want_sse) HKM_GO(2, false, true);
+        else HKM_GO(2, false, false);
+    } else {
+        if (want_min) HKM_GO(0, true, false);
+        else HKM_GO(0, false, false);
+    }
+#undef HKM_GO
+    return check_launch("lloyd_small_kernel");
+}
+
+// mode bit 0: accumulate per-cluster sums into `part`; bit 1: also the sum of min d2
+int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                 int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
+                 hipStream_t st) {
+    const int grid = small_grid(N, D, K);
+#define HKM_T(d) \
+    case d:      \
+        return launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, mode, grid, st);
+    switch (D) {
+        HKM_T(1) HKM_T(2) HKM_T(3) HKM_T(4) HKM_T(5) HKM_T(6) HKM_T(7) HKM_T(8)
+        default:
+            return fail(HKM_EUNSUPPORTED, "lloyd_small: D=%d outside 1..8", D);
+    }
+#undef HKM_T
+}
+
+int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, const float* C_old,
+                          float* C_new, int64_t ldcn, int64_t* counts, float* shift, float* sse,
+                          hipStream_t st) {
+    int spad = 1;
+    while (spad < K * (D + 1) + 1) spad <<= 1;  // <= 256 because K*(D+1) <= 240
+    hipLaunchKernelGGL(lloyd_small_finalize_kernel, dim3(1), dim3(1024), 0, st, part, grid, K, D,
+                       C_old, C_new, ldcn, counts, shift, sse, sse ? 1 : 0, spad);
+    return check_launch("lloyd_small_finalize_kernel");
+}
+
+}  // namespace hkm
