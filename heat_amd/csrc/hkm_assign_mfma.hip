@@ -63,34 +63,106 @@ __device__ __forceinline__ void merge_halves(float& m, int& mi) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Resident variant: the whole centroid matrix (zero-padded to KP x DP) and its squared norms live
-// in LDS for the lifetime of a persistent workgroup; each wave streams its own 32*PB points from
-// global memory straight into B-operand registers.  No barrier inside the tile loop.
+// Resident variant: the whole centroid matrix and its squared norms live in LDS for the lifetime of
+// a persistent workgroup; each wave streams its own 32*PB points from global memory straight into
+// B-operand registers.  No barrier inside the tile loop.
+//
+// On this hardware every VALU instruction takes issue time away from the fp32 MFMA pipe (there is no
+// co-execution), so the epilogue is kept to three VALU instructions per distance:
+//   * the norms ride along in the contraction: LDS row k holds [-2*c_k (zero-padded to DP), |c_k|^2,
+//     1] and the point operand is extended by [1, |x|^2], so the accumulator IS
+//     (|x|^2 + |c|^2) - 2 x.c.  The extra step goes first, i.e. the accumulator starts at the rounded
+//     sum of the two norms like the reference's x_norm + y_norm, and scaling by -2 is exact;
+//   * the clamp at 0 is applied lazily: only if some running minimum went negative (a point that
+//     coincides with a centroid up to rounding) the tile is rescanned with the clamp on every value;
+//   * per value: compare, select index, select value (see resident_scan).  The lane-half term of the
+//     index is added once per tile.
 // ------------------------------------------------------------------------------------------------
+// One centroid block (32 rows) against the wave's PB point blocks: 1 + DP/2 MFMAs per point block.
+template <int DP, int PB>
+__device__ __forceinline__ void resident_block(const float* arow, int h, const floatx4 (&b)[PB][DP / 8],
+                                               const float (&baug)[PB], floatx16 (&acc)[PB]) {
+    constexpr int NJ = DP / 8;
+    const float aaug = arow[DP + h];
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb) {
+        floatx16 z;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) z[v] = 0.f;
+        acc[pb] = MFMA32(aaug, baug[pb], z);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const floatx4 a = ld4(arow + h * (DP / 2) + 4 * j);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) acc[pb] = MFMA32(a[t], b[pb][j][t], acc[pb]);
+    }
+}
+
+// Scan of all centroid blocks: per distance compare, select index, select value; the block-local
+// first minimum (candidate indices are small literals) is merged into the running minimum once per
+// block.  Strict '<' everywhere keeps the first index on ties.  CLAMP applies max(., 0) to every
+// value (the rescan of a tile whose lazy minimum came out negative).
+template <int DP, int PB, bool CLAMP>
+__device__ __forceinline__ void resident_scan(const float* sC, int ncb, int p, int h,
+                                              const floatx4 (&b)[PB][DP / 8],
+                                              const float (&baug)[PB], float (&m)[PB],
+                                              int (&mi)[PB]) {
+    constexpr int LDC = DP + 4;
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb) {
+        m[pb] = HKM_INF;
+        mi[pb] = 0;
+    }
+    for (int cb = 0; cb < ncb; ++cb) {
+        floatx16 acc[PB];
+        resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, h, b, baug, acc);
+        const int kb = cb * 32;
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            float bm = CLAMP ? fmaxf(acc[pb][0], 0.0f) : acc[pb][0];
+            int bi = 0;
+#pragma unroll
+            for (int v = 1; v < 16; ++v) {
+                float d = acc[pb][v];
+                if (CLAMP) d = fmaxf(d, 0.0f);
+                const bool lt = d < bm;
+                bi = lt ? 8 * (v >> 2) + (v & 3) : bi;
+                bm = lt ? d : bm;
+            }
+            const bool lt = bm < m[pb];
+            mi[pb] = lt ? kb + bi : mi[pb];
+            m[pb] = lt ? bm : m[pb];
+        }
+    }
+}
+
 template <int DP, int PB, bool VEC>
 __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles) {
     extern __shared__ __align__(16) float lds[];
-    constexpr int LDC = DP + 4;  // row stride: +4 floats keeps 16-B vector reads conflict-free
+    constexpr int LDC = DP + 4;  // row: DP scaled coordinates, |c|^2, 1, 2 pad; also keeps 16-B reads conflict-free
     constexpr int NJ = DP / 8;   // 16-byte groups per lane-half
     const int KP = (K + 31) & ~31;
-    float* sC = lds;
-    float* sCn = lds + KP * LDC;
+    float* sC = lds;  // [KP][LDC]
     const int tid = threadIdx.x;
 
     for (int i = tid; i < KP * DP; i += 256) {
         const int r = i / DP, c = i - r * DP;
-        sC[r * LDC + c] = (r < K && c < D) ? C[int64_t(r) * ldc + c] : 0.f;
+        sC[r * LDC + c] = (r < K && c < D) ? -2.0f * C[int64_t(r) * ldc + c] : 0.f;
     }
-    __syncthreads();
     for (int r = tid; r < KP; r += 256) {
-        float s = HKM_INF;
+        float s = HKM_INF;  // padding rows can never win
         if (r < K) {
             s = 0.f;
-            for (int c = 0; c < D; ++c) s = fmaf(sC[r * LDC + c], sC[r * LDC + c], s);
+            const float* c = C + int64_t(r) * ldc;
+            for (int d = 0; d < D; ++d) s = fmaf(c[d], c[d], s);
         }
-        sCn[r] = s;
+        sC[r * LDC + DP] = s;
+        sC[r * LDC + DP + 1] = 1.0f;
     }
     __syncthreads();
 
@@ -101,7 +173,7 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
         floatx4 b[PB][NJ];
-        float xn[PB], m[PB];
+        float baug[PB], m[PB];
         int mi[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
@@ -115,33 +187,19 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 #pragma unroll
                 for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
             }
-            xn[pb] = s + __shfl_xor(s, 32);
-            m[pb] = HKM_INF;
-            mi[pb] = 0;
+            const float xn = s + __shfl_xor(s, 32);
+            baug[pb] = h ? xn : 1.0f;  // pairs with [|c|^2, 1] of the centroid row
         }
 
-        for (int cb = 0; cb < ncb; ++cb) {
-            floatx16 acc[PB];
+        resident_scan<DP, PB, false>(sC, ncb, p, h, b, baug, m, mi);
+        bool neg = false;
 #pragma unroll
-            for (int pb = 0; pb < PB; ++pb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[pb][v] = 0.f;
-            const float* arow = sC + (cb * 32 + p) * LDC + h * (DP / 2);
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const floatx4 a = ld4(arow + 4 * j);
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int pb = 0; pb < PB; ++pb) acc[pb] = MFMA32(a[t], b[pb][j][t], acc[pb]);
-            }
-#pragma unroll
-            for (int pb = 0; pb < PB; ++pb)
-                scan16(acc[pb], xn[pb], sCn + cb * 32, cb * 32, h, m[pb], mi[pb]);
-        }
+        for (int pb = 0; pb < PB; ++pb) neg |= m[pb] < 0.f;
+        if (__any(neg)) resident_scan<DP, PB, true>(sC, ncb, p, h, b, baug, m, mi);
 
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
+            mi[pb] += 4 * h;
             merge_halves(m[pb], mi[pb]);
             const int64_t r = row0 + pb * 32 + p;
             if (h == 0 && r < N) {

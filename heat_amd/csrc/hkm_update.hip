@@ -6,8 +6,8 @@
 // half-waves OWNS the clusters k with k % 8 == q and is the only one that ever touches their
 // accumulator rows; it visits the rows of the chunk in ascending order.  Every accumulator element
 // therefore has exactly one writer with a fixed order of additions.
-// Pass 2 (update_finalize_kernel): one thread per (k, d) adds the chunk partials in ascending chunk
-// order in fp64, divides by the count and rounds to fp32.
+// Pass 2 (update_finalize_kernel): four threads per (k, d) add the chunk partials in a fixed strided
+// order in fp64; the result is divided by the count and rounded to fp32.
 //
 // Arithmetic follows heat/cluster/kmeans.py:88-101: mean in float64 (types.py:945-959 promotes
 // x * selection), count clipped to >= 1 and rounded through fp32 (rounding.py:156-164), result
@@ -25,11 +25,11 @@ UpdateGeom update_geom(int64_t N, int32_t D, int32_t K) {
     g.J = (D + 31) / 32;
     g.Z = (K + UPD_KR_MAX - 1) / UPD_KR_MAX;
     g.KR = (K + g.Z - 1) / g.Z;
-    // aim at ~2048 workgroups overall; keep fp32 runs <= 32768 rows, chunks >= 2048 rows
-    int64_t want_s = 2048 / (int64_t(g.J) * g.Z);
+    // aim at ~1024 workgroups overall; keep fp32 runs <= 32768 rows and chunks >= 1024 rows
+    int64_t want_s = 1024 / (int64_t(g.J) * g.Z);
     if (want_s < 1) want_s = 1;
     int64_t rpc = (N + want_s - 1) / want_s;
-    if (rpc < 2048) rpc = 2048;
+    if (rpc < 1024) rpc = 1024;
     if (rpc > 32768) rpc = 32768;
     rpc = (rpc + 63) / 64 * 64;
     g.rows_per_chunk = rpc;
@@ -62,19 +62,23 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
     const int64_t r_begin = int64_t(s) * rows_per_chunk;
     const int64_t r_end = min(N, r_begin + rows_per_chunk);
 
+    int lab_next = -1;
+    if (r_begin + lane < r_end) lab_next = labels[r_begin + lane];
     for (int64_t base = r_begin; base < r_end; base += 64) {
-        const int64_t ri = base + lane;
-        int lab = -1;
-        if (ri < r_end) lab = labels[ri];
+        const int lab = lab_next;
+        // the next batch's labels are requested before this batch's rows: one round trip per batch
+        lab_next = -1;
+        if (base + 64 + lane < r_end) lab_next = labels[base + 64 + lane];
         const bool in_rng = lab >= kbase && lab < kend;
         unsigned long long own0 = __ballot(in_rng && (lab & (UPD_HALVES - 1)) == q0);
         unsigned long long own1 = __ballot(in_rng && (lab & (UPD_HALVES - 1)) == q1);
         while (own0 | own1) {
-            // up to 4 rows per half-wave in flight
-            int rr[4], ll[4];
-            float xv[4];
+            // up to 8 rows per half-wave in flight
+            constexpr int U = 8;
+            int rr[U], ll[U];
+            float xv[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 int r0 = -1, r1 = -1;
                 if (own0) {
                     r0 = __builtin_ctzll(own0);
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
                 if (rr[u] >= 0 && col_ok) xv[u] = X[(base + rr[u]) * ldx + col];
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 if (rr[u] >= 0) {
                     const int k = ll[u] - kbase;
                     acc[k * 32 + c] += xv[u];
@@ -112,23 +116,55 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
             part_cnt[int64_t(s) * K + kbase + i] = cnt[i];
 }
 
-__global__ void update_finalize_kernel(const float* __restrict__ part_sum,
-                                       const int32_t* __restrict__ part_cnt, int S, int K, int D,
-                                       int DPAD, float* __restrict__ C_new, int64_t ldcn,
-                                       int64_t* __restrict__ counts) {
-    const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= int64_t(K) * D) return;
-    const int k = int(i / D), d = int(i - int64_t(k) * D);
+// 256 threads = 64 (k, d) pairs x 4 strided lanes over the chunks.  Lane q adds chunks q, q+4, ...
+// in ascending order (8 loads in flight, additions in order); lane 0 then adds the four lane sums in
+// lane order.  The order depends only on S.
+__global__ __launch_bounds__(256) void update_finalize_kernel(
+    const float* __restrict__ part_sum, const int32_t* __restrict__ part_cnt, int S, int K, int D,
+    int DPAD, float* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts) {
+    __shared__ double ssum[4][64];
+    __shared__ int64_t scnt[4][64];
+    const int e = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const int64_t i = int64_t(blockIdx.x) * 64 + e;
+    const bool ok = i < int64_t(K) * D;
+    const int k = ok ? int(i / D) : 0, d = ok ? int(i - int64_t(k) * D) : 0;
     double sum = 0.0;
     int64_t n = 0;
-    for (int s = 0; s < S; ++s) {
-        sum += double(part_sum[(int64_t(s) * K + k) * DPAD + d]);
-        n += part_cnt[int64_t(s) * K + k];
+    if (ok) {
+        const float* ps = part_sum + int64_t(k) * DPAD + d;
+        const int32_t* pc = part_cnt + k;
+        const int64_t sstride = int64_t(K) * DPAD;
+        int s = q;
+        for (; s + 28 < S; s += 32) {
+            float t[8];
+            int32_t c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                t[u] = ps[(s + 4 * u) * sstride];
+                c[u] = pc[int64_t(s + 4 * u) * K];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                sum += double(t[u]);
+                n += c[u];
+            }
+        }
+        for (; s < S; s += 4) {
+            sum += double(ps[s * sstride]);
+            n += pc[int64_t(s) * K];
+        }
     }
-    // the reference's count passes through fp32 (clamp of an int64 tensor with a float bound)
-    const double cnt = double(float(n < 1 ? 1 : n));
-    C_new[int64_t(k) * ldcn + d] = float(sum / cnt);
-    if (d == 0 && counts) counts[k] = n;
+    ssum[q][e] = sum;
+    scnt[q][e] = n;
+    __syncthreads();
+    if (q == 0 && ok) {
+        sum = ((ssum[0][e] + ssum[1][e]) + ssum[2][e]) + ssum[3][e];
+        n = scnt[0][e] + scnt[1][e] + scnt[2][e] + scnt[3][e];
+        // the reference's count passes through fp32 (clamp of an int64 tensor with a float bound)
+        const double cnt = double(float(n < 1 ? 1 : n));
+        C_new[int64_t(k) * ldcn + d] = float(sum / cnt);
+        if (d == 0 && counts) counts[k] = n;
+    }
 }
 
 int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
@@ -142,7 +178,7 @@ int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32
     int rc = check_launch("update_partial_kernel");
     if (rc) return rc;
     const int64_t tot = int64_t(K) * D;
-    hipLaunchKernelGGL(update_finalize_kernel, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL(update_finalize_kernel, dim3((unsigned)((tot + 63) / 64)), dim3(256), 0, st,
                        w.part_sum, w.part_cnt, g.S, K, D, dpad, C_new, ldcn, counts);
     return check_launch("update_finalize_kernel");
 }
