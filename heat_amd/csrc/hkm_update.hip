@@ -18,7 +18,7 @@ namespace hkm {
 
 static constexpr int UPD_THREADS = 256;
 static constexpr int UPD_HALVES = 8;
-static constexpr int UPD_KR_MAX = 480;  // 480 x (32 x 4 + 4) B = 61.9 KB of LDS, under the 64 KB dynamic limit
+static constexpr int UPD_KR_MAX = 448;  // (448 + 1) x (32 x 4 + 4) B + 4.6 KB of row lists = 63.9 KB of LDS (64 KB dynamic limit)
 
 UpdateGeom update_geom(int64_t N, int32_t D, int32_t K) {
     UpdateGeom g;
@@ -42,16 +42,19 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const int32_t* __restrict__ labels,
     int K, int KR, int64_t rows_per_chunk, float* __restrict__ part_sum,
     int32_t* __restrict__ part_cnt, int DPAD) {
+    constexpr int U = 4;          // rows per half-wave and pass
+    constexpr int LIST = 64 + U;  // a batch has 64 rows; room for the padding to a multiple of U
     extern __shared__ __align__(16) float lds[];
-    float* acc = lds;                                       // [KR][32]
-    int32_t* cnt = reinterpret_cast<int32_t*>(lds + KR * 32);  // [KR]
+    float* acc = lds;                                                 // [KR + 1][32], last row = sink
+    int32_t* cnt = reinterpret_cast<int32_t*>(lds + (KR + 1) * 32);   // [KR + 1]
+    int2* lists = reinterpret_cast<int2*>(cnt + ((KR + 1 + 1) & ~1)); // [8 half-waves][LIST]
     const int tid = threadIdx.x;
     const int s = blockIdx.x, j = blockIdx.y, z = blockIdx.z;
     const int kbase = z * KR;
     const int kend = min(K, kbase + KR);
 
-    for (int i = tid; i < KR * 32; i += UPD_THREADS) acc[i] = 0.f;
-    for (int i = tid; i < KR; i += UPD_THREADS) cnt[i] = 0;
+    for (int i = tid; i < (KR + 1) * 32; i += UPD_THREADS) acc[i] = 0.f;
+    for (int i = tid; i < KR + 1; i += UPD_THREADS) cnt[i] = 0;
     __syncthreads();
 
     const int lane = tid & 63, wave = tid >> 6;
@@ -59,48 +62,50 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
     const int col = j * 32 + c;
     const bool col_ok = col < D;
     const int q0 = wave * 2, q1 = wave * 2 + 1;
+    int2* my_list = lists + (wave * 2 + h) * LIST;  // list of the half-wave this lane belongs to
+    int2* list0 = lists + q0 * LIST;
+    int2* list1 = lists + q1 * LIST;
+    const bool count_here = (c == 0) && (j == 0);
     const int64_t r_begin = int64_t(s) * rows_per_chunk;
     const int64_t r_end = min(N, r_begin + rows_per_chunk);
+    const float* xcol = X + (col_ok ? col : 0);
 
     int lab_next = -1;
     if (r_begin + lane < r_end) lab_next = labels[r_begin + lane];
     for (int64_t base = r_begin; base < r_end; base += 64) {
         const int lab = lab_next;
-        // the next batch's labels are requested before this batch's rows: one round trip per batch
+        // the next batch's labels are requested before this batch's rows
         lab_next = -1;
         if (base + 64 + lane < r_end) lab_next = labels[base + 64 + lane];
+
+        // Each half-wave collects the rows of the batch whose cluster it owns, in ascending row order,
+        // as (row, local cluster) pairs in its LDS list; the list is padded to a multiple of U with
+        // entries that add row 0 of the batch to the sink row.
         const bool in_rng = lab >= kbase && lab < kend;
-        unsigned long long own0 = __ballot(in_rng && (lab & (UPD_HALVES - 1)) == q0);
-        unsigned long long own1 = __ballot(in_rng && (lab & (UPD_HALVES - 1)) == q1);
-        while (own0 | own1) {
-            // up to 8 rows per half-wave in flight
-            constexpr int U = 8;
-            int rr[U], ll[U];
+        const bool p0 = in_rng && (lab & (UPD_HALVES - 1)) == q0;
+        const bool p1 = in_rng && (lab & (UPD_HALVES - 1)) == q1;
+        const unsigned long long m0 = __ballot(p0), m1 = __ballot(p1);
+        const int n0 = __popcll(m0), n1 = __popcll(m1);
+        const int rank0 = __builtin_amdgcn_mbcnt_hi(unsigned(m0 >> 32), __builtin_amdgcn_mbcnt_lo(unsigned(m0), 0));
+        const int rank1 = __builtin_amdgcn_mbcnt_hi(unsigned(m1 >> 32), __builtin_amdgcn_mbcnt_lo(unsigned(m1), 0));
+        if (p0) list0[rank0] = make_int2(lane, lab - kbase);
+        if (p1) list1[rank1] = make_int2(lane, lab - kbase);
+        const int nmax = max(n0, n1);
+        const int npad = (nmax + U - 1) / U * U;
+        if (lane < npad - n0) list0[n0 + lane] = make_int2(0, KR);
+        if (lane < npad - n1) list1[n1 + lane] = make_int2(0, KR);
+
+        for (int t = 0; t < npad; t += U) {
+            int2 e[U];
             float xv[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                int r0 = -1, r1 = -1;
-                if (own0) {
-                    r0 = __builtin_ctzll(own0);
-                    own0 &= own0 - 1;
-                }
-                if (own1) {
-                    r1 = __builtin_ctzll(own1);
-                    own1 &= own1 - 1;
-                }
-                rr[u] = h ? r1 : r0;
-                const int src = rr[u] < 0 ? 0 : rr[u];
-                ll[u] = __shfl(lab, src);
-                xv[u] = 0.f;
-                if (rr[u] >= 0 && col_ok) xv[u] = X[(base + rr[u]) * ldx + col];
-            }
+            for (int u = 0; u < U; ++u) e[u] = my_list[t + u];
+#pragma unroll
+            for (int u = 0; u < U; ++u) xv[u] = xcol[(base + e[u].x) * ldx];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (rr[u] >= 0) {
-                    const int k = ll[u] - kbase;
-                    acc[k * 32 + c] += xv[u];
-                    if (c == 0 && j == 0) cnt[k] += 1;
-                }
+                acc[e[u].y * 32 + c] += col_ok ? xv[u] : 0.f;
+                if (count_here) cnt[e[u].y] += 1;
             }
         }
     }
@@ -172,7 +177,8 @@ int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32
                   hipStream_t st) {
     const UpdateGeom g = update_geom(N, D, K);
     const int dpad = g.J * 32;
-    const size_t lds = size_t(g.KR) * 32 * sizeof(float) + size_t(g.KR) * sizeof(int32_t);
+    const size_t lds = size_t(g.KR + 1) * 32 * sizeof(float) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
+                       size_t(UPD_HALVES) * (64 + 8) * sizeof(int2);
     hipLaunchKernelGGL(update_partial_kernel, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
                        D, ldx, labels, K, g.KR, g.rows_per_chunk, w.part_sum, w.part_cnt, dpad);
     int rc = check_launch("update_partial_kernel");
