@@ -41,6 +41,7 @@ int num_cus() {
 AssignKind assign_kind(int32_t D, int32_t K) {
     if (D <= 16) return ASSIGN_VALU;
     if (D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024) return ASSIGN_MFMA_RESIDENT;
+    if (D <= 64) return ASSIGN_MFMA_TILED;
     return ASSIGN_MFMA_STREAM;
 }
 
@@ -103,6 +104,11 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
             return launch_assign_valu(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_RESIDENT:
             return launch_assign_mfma_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
+        case ASSIGN_MFMA_TILED: {
+            int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
+            if (rc) return rc;
+            return launch_assign_mfma_tiled(X, N, D, ldx, C, K, ldc, w.cn, labels, min_d2, st);
+        }
         default: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
             if (rc) return rc;
@@ -132,6 +138,7 @@ const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K) {
     switch (assign_kind(D, K)) {
         case ASSIGN_VALU: return small_eligible(D, K) ? "valu_fused" : "valu";
         case ASSIGN_MFMA_RESIDENT: return "mfma_resident";
+        case ASSIGN_MFMA_TILED: return "mfma_tiled";
         default: return "mfma_stream";
     }
 }

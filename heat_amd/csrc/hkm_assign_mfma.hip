@@ -36,23 +36,6 @@ __device__ __forceinline__ floatx4 load_row4(const float* row, int c, int D) {
     return v;
 }
 
-__device__ __forceinline__ void scan16(const floatx16& acc, float xn, const float* cn_lds_or_glb,
-                                       int kbase, int h, float& m, int& mi) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const floatx4 cn4 = ld4(cn_lds_or_glb + 8 * g + 4 * h);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            float d = fmaf(-2.0f, acc[4 * g + t], xn + cn4[t]);
-            d = fmaxf(d, 0.0f);
-            if (d < m) {
-                m = d;
-                mi = kbase + 8 * g + 4 * h + t;
-            }
-        }
-    }
-}
-
 __device__ __forceinline__ void merge_halves(float& m, int& mi) {
     const float om = __shfl_xor(m, 32);
     const int oi = __shfl_xor(mi, 32);
@@ -210,6 +193,171 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Tiled variant for 16 < D <= 64 when the centroids do not fit in LDS: same wave-level scheme as the
+// resident kernel (a wave keeps its 32*PB points in B-operand registers for the whole feature range
+// and scans centroid blocks), but the centroids pass through LDS in tiles of 128 rows, double
+// buffered; all 256 threads fetch the next tile while the current one is scanned, one barrier per
+// tile (every 4*(1+DP/2)*PB MFMAs per wave).  The running (min, argmin) is carried across tiles, so
+// the clamp is applied eagerly here.  Squared centroid norms come from global memory.
+// ------------------------------------------------------------------------------------------------
+template <int DP, int PB, bool VEC>
+__global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
+    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, const float* __restrict__ cn, int32_t* __restrict__ labels,
+    float* __restrict__ min_d2, int64_t ntiles) {
+    extern __shared__ __align__(16) float lds[];
+    constexpr int LDC = DP + 4;
+    constexpr int NJ = DP / 8;
+    constexpr int TC = 128;                 // centroid rows per LDS tile
+    constexpr int GPR = DP / 4;             // 16-byte groups per row
+    constexpr int NQ = TC * GPR / 256;      // groups per thread and tile
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int p = lane & 31, h = lane >> 5;
+    const int nct = (K + TC - 1) / TC;
+    const int64_t my_tiles = (ntiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const int64_t nsteps = my_tiles * nct;
+
+    floatx4 pc[NQ];
+    float pcn = 0.f;  // squared norm of row `tid` of the tile (threads 0..127)
+    auto issue = [&](int ct) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int g = tid + 256 * q;
+            const int r = ct * TC + g / GPR, c = (g % GPR) * 4;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (r < K) v = load_row4<VEC>(C + int64_t(r) * ldc, c, D);
+            pc[q] = v;
+        }
+        if (tid < TC) pcn = cn[ct * TC + tid];  // padded with +inf beyond K
+    };
+
+    int64_t tile = blockIdx.x;
+    int ct = 0;
+    if (nsteps > 0) issue(0);
+
+    floatx4 b[PB][NJ];
+    float baug[PB], m[PB];
+    int mi[PB];
+
+    for (int64_t it = 0; it < nsteps; ++it) {
+        float* sC = lds + (it & 1) * (TC * LDC);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int g = tid + 256 * q;
+            *reinterpret_cast<floatx4*>(sC + (g / GPR) * LDC + (g % GPR) * 4) = -2.0f * pc[q];
+        }
+        if (tid < TC) {
+            sC[tid * LDC + DP] = pcn;
+            sC[tid * LDC + DP + 1] = 1.0f;
+        }
+        __syncthreads();
+
+        const int64_t cur_tile = tile;
+        const int cur_ct = ct;
+        if (++ct == nct) {
+            ct = 0;
+            tile += gridDim.x;
+        }
+        if (it + 1 < nsteps) issue(ct);
+
+        const int64_t row0 = cur_tile * (4 * PB * 32) + wave * (PB * 32);
+        if (cur_ct == 0) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                int64_t r = row0 + pb * 32 + p;
+                r = r < N ? r : N - 1;
+                const float* xr = X + r * ldx;
+                float s = 0.f;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    b[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
+                }
+                const float xn = s + __shfl_xor(s, 32);
+                baug[pb] = h ? xn : 1.0f;
+                m[pb] = HKM_INF;
+                mi[pb] = 0;
+            }
+        }
+
+#pragma unroll 1
+        for (int cb = 0; cb < TC / 32; ++cb) {
+            floatx16 acc[PB];
+            resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, h, b, baug, acc);
+            const int kb = cur_ct * TC + cb * 32;
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                float bm = fmaxf(acc[pb][0], 0.0f);
+                int bi = 0;
+#pragma unroll
+                for (int v = 1; v < 16; ++v) {
+                    const float d = fmaxf(acc[pb][v], 0.0f);
+                    const bool lt = d < bm;
+                    bi = lt ? 8 * (v >> 2) + (v & 3) : bi;
+                    bm = lt ? d : bm;
+                }
+                const bool lt = bm < m[pb];
+                mi[pb] = lt ? kb + bi : mi[pb];
+                m[pb] = lt ? bm : m[pb];
+            }
+        }
+
+        if (cur_ct == nct - 1) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                float mm = m[pb];
+                int ii = mi[pb] + 4 * h;
+                merge_halves(mm, ii);
+                const int64_t r = row0 + pb * 32 + p;
+                if (h == 0 && r < N) {
+                    labels[r] = ii;
+                    if (min_d2) min_d2[r] = mm;
+                }
+            }
+        }
+    }
+}
+
+template <int DP, bool VEC>
+static int launch_tiled_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                          int32_t K, int64_t ldc, const float* cn, int32_t* labels, float* min_d2,
+                          hipStream_t st) {
+    constexpr int PB = 2;
+    const int64_t ntiles = (N + 4 * PB * 32 - 1) / (4 * PB * 32);
+    const size_t lds = size_t(2) * 128 * (DP + 4) * sizeof(float);
+    auto kern = assign_mfma_tiled_kernel<DP, PB, VEC>;
+    int64_t grid = int64_t(num_cus()) * 2;
+    if (grid > ntiles) grid = ntiles;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+        if (e != hipSuccess) return fail(HKM_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc, cn,
+                       labels, min_d2, ntiles);
+    return check_launch("assign_mfma_tiled_kernel");
+}
+
+int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                             int32_t K, int64_t ldc, const float* cn, int32_t* labels,
+                             float* min_d2, hipStream_t st) {
+    const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
+    const int dp = resident_dp(D);
+#define HKM_CASE(d)                                                                              \
+    case d:                                                                                      \
+        return vec ? launch_tiled_t<d, true>(X, N, D, ldx, C, K, ldc, cn, labels, min_d2, st)    \
+                   : launch_tiled_t<d, false>(X, N, D, ldx, C, K, ldc, cn, labels, min_d2, st);
+    switch (dp) {
+        HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
+        default:
+            return fail(HKM_EUNSUPPORTED, "assign_mfma_tiled: D=%d", D);
+    }
+#undef HKM_CASE
+}
+
 template <int DP, bool VEC>
 static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                              int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
@@ -243,49 +391,50 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
 }
 
 // ------------------------------------------------------------------------------------------------
-// Streaming variant for any K and D: a workgroup owns 256 points (4 waves x 64) and walks over
-// centroid tiles of 64 and feature chunks of 32.  The centroid panel of a (tile, chunk) step is
-// staged through a double-buffered LDS tile by all 256 threads; the point operand of the step is
-// loaded by each lane straight into registers.  Global loads of step i+1 are issued before the
-// MFMAs of step i.  Squared centroid norms come from global memory (padded with +inf).
+// Streaming variant for any K and D.  A workgroup owns 128 points and walks over centroid tiles of
+// 128 and feature chunks of 32; its four waves form a 2 x 2 grid, each computing 64 points x 64
+// centroids per step (2 x 2 MFMA blocks, 64 MFMAs).  Both operand panels of a step (128 x 32 floats
+// each) are fetched with fully coalesced 16-byte loads by all 256 threads one step ahead and staged
+// through double-buffered LDS (row stride 36 floats keeps the 16-byte operand reads conflict-free).
+// After the last chunk of a centroid tile one more MFMA adds (-|c|^2/2) * 1 + 1 * (-|x|^2/2), so the
+// accumulator is minus half the squared distance (squared centroid norms come from global memory, padded with
+// +inf; |x|^2 is accumulated from the point operand while the first centroid tile is processed).
+// The (min, argmin) of the two waves that share a point are merged through LDS at the end of a tile.
 // ------------------------------------------------------------------------------------------------
 template <bool VEC>
 __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, const float* __restrict__ cn, int32_t* __restrict__ labels,
     float* __restrict__ min_d2, int64_t ntiles) {
-    constexpr int PB = 2, CB = 2, CT = CB * 32, DC = 32, LDA = DC + 4;
-    __shared__ __align__(16) float sA[2][CT * LDA];
+    constexpr int PB = 2, CB = 2, TP = 128, TC = 128, DC = 32, LDS_LD = DC + 4;
+    __shared__ __align__(16) float sA[2][TC * LDS_LD];
+    __shared__ __align__(16) float sB[2][TP * LDS_LD];
+    __shared__ float sM[2][TP];
+    __shared__ int sI[2][TP];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
+    const int wp = wave & 1, wc = wave >> 1;  // this wave: points [64 wp, +64), centroids [64 wc, +64)
     const int p = lane & 31, h = lane >> 5;
-    const int nct = (K + CT - 1) / CT;
+    const int nct = (K + TC - 1) / TC;
     const int ndc = (D + DC - 1) / DC;
     const int64_t my_tiles = (ntiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
     const int64_t nsteps = my_tiles * nct * ndc;
 
-    // staging role of this thread: 2 x 16-byte groups of the 64 x 32 panel
-    const int sr = tid >> 3;        // panel rows sr and sr + 32
-    const int sc = (tid & 7) * 4;   // column group
+    // staging role of this thread: rows sr + 32 q (q = 0..3) of both panels, column group sc
+    const int sr = tid >> 3;
+    const int sc = (tid & 7) * 4;
 
-    floatx4 pa[2];
-    floatx4 bn[PB][4];
+    floatx4 pa[4], pb_[4];
     auto issue = [&](int64_t tile, int ct, int dc) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const int r = ct * CT + sr + 32 * q;
+        for (int q = 0; q < 4; ++q) {
+            const int rc = ct * TC + sr + 32 * q;
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if (r < K) v = load_row4<VEC>(C + int64_t(r) * ldc, dc * DC + sc, D);
+            if (rc < K) v = load_row4<VEC>(C + int64_t(rc) * ldc, dc * DC + sc, D);
             pa[q] = v;
-        }
-        const int64_t row0 = tile * 256 + wave * 64;
-#pragma unroll
-        for (int pb = 0; pb < PB; ++pb) {
-            int64_t r = row0 + pb * 32 + p;
-            r = r < N ? r : N - 1;
-            const float* xr = X + r * ldx;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) bn[pb][j] = load_row4<VEC>(xr, dc * DC + h * 16 + 4 * j, D);
+            int64_t rp = tile * TP + sr + 32 * q;
+            rp = rp < N ? rp : N - 1;
+            pb_[q] = load_row4<VEC>(X + rp * ldx, dc * DC + sc, D);
         }
     };
 
@@ -294,25 +443,20 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     if (nsteps > 0) issue(tile, ct, dc);
 
     floatx16 acc[PB][CB];
-    float xn[PB] = {0.f, 0.f}, xs[PB] = {0.f, 0.f}, m[PB];
+    float xs[PB] = {0.f, 0.f}, baug[PB] = {0.f, 0.f}, m[PB];
     int mi[PB];
 
     for (int64_t it = 0; it < nsteps; ++it) {
         const int buf = int(it & 1);
-        // publish the prefetched panel, take the prefetched point operand
 #pragma unroll
-        for (int q = 0; q < 2; ++q)
-            *reinterpret_cast<floatx4*>(&sA[buf][(sr + 32 * q) * LDA + sc]) = pa[q];
-        floatx4 b[PB][4];
-#pragma unroll
-        for (int pb = 0; pb < PB; ++pb)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) b[pb][j] = bn[pb][j];
+        for (int q = 0; q < 4; ++q) {
+            *reinterpret_cast<floatx4*>(&sA[buf][(sr + 32 * q) * LDS_LD + sc]) = pa[q];
+            *reinterpret_cast<floatx4*>(&sB[buf][(sr + 32 * q) * LDS_LD + sc]) = pb_[q];
+        }
         __syncthreads();
 
         const int64_t cur_tile = tile;
         const int cur_ct = ct, cur_dc = dc;
-        // advance the (tile, ct, dc) odometer and issue the next step's loads
         if (++dc == ndc) {
             dc = 0;
             if (++ct == nct) {
@@ -333,10 +477,19 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
 #pragma unroll
                 for (int pb = 0; pb < PB; ++pb) {
                     xs[pb] = 0.f;
-                    m[pb] = HKM_INF;
+                    m[pb] = -HKM_INF;
                     mi[pb] = 0;
                 }
             }
+        }
+
+        // this lane-half's 16 features of the chunk, for both operands
+        floatx4 b[PB][4];
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            const float* brow = &sB[buf][(wp * 64 + pb * 32 + p) * LDS_LD + h * 16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[pb][j] = ld4(brow + 4 * j);
         }
         if (cur_ct == 0) {
 #pragma unroll
@@ -346,10 +499,9 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
 #pragma unroll
                     for (int t = 0; t < 4; ++t) xs[pb] = fmaf(b[pb][j][t], b[pb][j][t], xs[pb]);
         }
-
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
-            const float* arow = &sA[buf][(cb * 32 + p) * LDA + h * 16];
+            const float* arow = &sA[buf][(wc * 64 + cb * 32 + p) * LDS_LD + h * 16];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const floatx4 a = ld4(arow + 4 * j);
@@ -364,23 +516,60 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         if (cur_dc == ndc - 1) {
             if (cur_ct == 0) {
 #pragma unroll
-                for (int pb = 0; pb < PB; ++pb) xn[pb] = xs[pb] + __shfl_xor(xs[pb], 32);
+                for (int pb = 0; pb < PB; ++pb) {
+                    const float xn = xs[pb] + __shfl_xor(xs[pb], 32);
+                    baug[pb] = h ? -0.5f * xn : 1.0f;
+                }
             }
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-                for (int pb = 0; pb < PB; ++pb)
-                    scan16(acc[pb][cb], xn[pb], cn + cur_ct * CT + cb * 32, cur_ct * CT + cb * 32,
-                           h, m[pb], mi[pb]);
-            if (cur_ct == nct - 1) {
-                const int64_t row0 = cur_tile * 256 + wave * 64;
+            for (int cb = 0; cb < CB; ++cb) {
+                const int kb = cur_ct * TC + wc * 64 + cb * 32;
+                const float aaug = h ? 1.0f : -0.5f * cn[kb + p];
 #pragma unroll
                 for (int pb = 0; pb < PB; ++pb) {
+                    // g = x.c - |c|^2/2 - |x|^2/2 = -d2/2 (halving is exact): the nearest centroid has
+                    // the LARGEST g; the clamp of d2 at 0 is a clamp of g at 0 from above
+                    const floatx16 g16 = MFMA32(aaug, baug[pb], acc[pb][cb]);
+                    float bm = fminf(g16[0], 0.0f);
+                    int bi = 0;
+#pragma unroll
+                    for (int v = 1; v < 16; ++v) {
+                        const float g = fminf(g16[v], 0.0f);
+                        const bool gt = g > bm;
+                        bi = gt ? 8 * (v >> 2) + (v & 3) : bi;
+                        bm = gt ? g : bm;
+                    }
+                    const bool gt = bm > m[pb];
+                    mi[pb] = gt ? kb + bi : mi[pb];
+                    m[pb] = gt ? bm : m[pb];
+                }
+            }
+            if (cur_ct == nct - 1) {
+                // merge lane halves, then the two waves that cover the same points
+#pragma unroll
+                for (int pb = 0; pb < PB; ++pb) {
+                    mi[pb] += 4 * h;
+                    m[pb] = -2.0f * m[pb];  // back to the squared distance
                     merge_halves(m[pb], mi[pb]);
-                    const int64_t r = row0 + pb * 32 + p;
-                    if (h == 0 && r < N) {
-                        labels[r] = mi[pb];
-                        if (min_d2) min_d2[r] = m[pb];
+                    if (h == 0) {
+                        sM[wc][wp * 64 + pb * 32 + p] = m[pb];
+                        sI[wc][wp * 64 + pb * 32 + p] = mi[pb];
+                    }
+                }
+                __syncthreads();
+                if (tid < TP) {
+                    float m0 = sM[0][tid];
+                    int i0 = sI[0][tid];
+                    const float m1 = sM[1][tid];
+                    const int i1 = sI[1][tid];
+                    if (m1 < m0 || (m1 == m0 && i1 < i0)) {
+                        m0 = m1;
+                        i0 = i1;
+                    }
+                    const int64_t r = cur_tile * TP + tid;
+                    if (r < N) {
+                        labels[r] = i0;
+                        if (min_d2) min_d2[r] = m0;
                     }
                 }
             }
@@ -392,7 +581,7 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
                               int32_t K, int64_t ldc, const float* cn, int32_t* labels,
                               float* min_d2, hipStream_t st) {
     const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
-    const int64_t ntiles = (N + 255) / 256;
+    const int64_t ntiles = (N + 127) / 128;
     int64_t grid = int64_t(num_cus()) * 2;
     if (grid > ntiles) grid = ntiles;
     if (vec)

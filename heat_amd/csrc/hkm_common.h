@@ -23,7 +23,7 @@ static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- kernel family selection ------------------------------------------------------------------
-enum AssignKind { ASSIGN_VALU = 0, ASSIGN_MFMA_RESIDENT = 1, ASSIGN_MFMA_STREAM = 2 };
+enum AssignKind { ASSIGN_VALU = 0, ASSIGN_MFMA_RESIDENT = 1, ASSIGN_MFMA_STREAM = 2, ASSIGN_MFMA_TILED = 3 };
 AssignKind assign_kind(int32_t D, int32_t K);
 
 // padded feature count used by the resident MFMA kernel (24, 32, 48 or 64)
@@ -66,6 +66,9 @@ int launch_assign_valu(const float* X, int64_t N, int32_t D, int64_t ldx, const 
 int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                                 int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
                                 hipStream_t st);
+int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                             int32_t K, int64_t ldc, const float* cn, int32_t* labels,
+                             float* min_d2, hipStream_t st);
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                               int32_t K, int64_t ldc, const float* cn, int32_t* labels,
                               float* min_d2, hipStream_t st);

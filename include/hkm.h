@@ -108,8 +108,8 @@ int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 
-/* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "mfma_resident",
- * "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
+/* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "mfma_resident",
+ * "mfma_tiled", "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
 const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K);
 
 #ifdef __cplusplus

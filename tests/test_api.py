@@ -172,7 +172,7 @@ def test_workspace_and_kernel_selection():
     assert _native.assign_kernel_name(200_000_000, 3, 8).startswith("valu")
     assert _native.assign_kernel_name(100_000, 8, 16).startswith("valu")
     assert _native.assign_kernel_name(10_000_000, 32, 256) == "mfma_resident"
-    assert _native.assign_kernel_name(1 << 20, 64, 1024) == "mfma_stream"
+    assert _native.assign_kernel_name(1 << 20, 64, 1024) == "mfma_tiled"
     assert _native.assign_kernel_name(2_000_000, 512, 1024) == "mfma_stream"
 
 
