@@ -66,6 +66,7 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         w.part_sum = reinterpret_cast<float*>(take(size_t(g.S) * K * g.J * 32 * sizeof(float)));
         w.part_cnt = reinterpret_cast<int32_t*>(take(size_t(g.S) * K * sizeof(int32_t)));
         w.counts = reinterpret_cast<int64_t*>(take(size_t(K) * sizeof(int64_t)));
+        w.shift_part = reinterpret_cast<double*>(take((size_t(K) * D / 64 + 1) * sizeof(double)));
     }
     if (flags & HKM_WS_SSE) w.min_d2 = reinterpret_cast<float*>(take(size_t(N < 1 ? 1 : N) * sizeof(float)));
     w.total = off;
@@ -170,7 +171,8 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
     const size_t need = carve(nullptr, N, D, K, HKM_WS_UPDATE).total;
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const Workspace w = carve(ws, N, D, K, HKM_WS_UPDATE);
-    return launch_update(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, static_cast<hipStream_t>(hip_stream));
+    return launch_update(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, nullptr, nullptr,
+                         static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
@@ -196,8 +198,7 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
         return launch_small_finalize(w.small_part, small_grid(N, D, K), K, D, C, C_new, D, nullptr, shift, sse, st);
     }
     if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;
-    if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, st))) return rc;
-    if ((rc = launch_shift(C, C_new, K, D, shift, st))) return rc;
+    if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
     if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
     return rc;
 }

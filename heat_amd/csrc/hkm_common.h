@@ -51,6 +51,7 @@ struct Workspace {
     int64_t* counts;    // [K]
     double* red;        // [RED_SLOTS] scratch for scalar reductions
     float* min_d2;      // [N] (only with the SSE flag)
+    double* shift_part; // [ceil(K*D/64)] per-block shares of the squared centroid shift
     double* small_part; // [SMALL_MAX_GRID][K*(D+1)+1] partial rows of the one-sweep small-D step
     size_t total;
 };
@@ -82,7 +83,7 @@ int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, co
                           hipStream_t st);
 int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
-                  hipStream_t st);
+                  const float* C_old, float* shift, hipStream_t st);
 int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
                  hipStream_t st);
 int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, int mode,

@@ -40,8 +40,8 @@ int small_grid(int64_t N, int32_t D, int32_t K) {
     (void)K;
     const int ppt = (D % 2 == 0) ? 2 : 4;
     const int64_t groups = (N + ppt - 1) / ppt;
-    // at least 8 groups per lane where the input allows it, at most 4 workgroups per CU
-    int64_t want = (groups + SMALL_T * 8 - 1) / (SMALL_T * 8);
+    // one group per lane until 4 workgroups per CU are reached, then grid-stride
+    int64_t want = (groups + SMALL_T - 1) / SMALL_T;
     int64_t cap = int64_t(num_cus()) * 4;
     if (cap > SMALL_MAX_GRID) cap = SMALL_MAX_GRID;
     if (want > cap) want = cap;

@@ -126,8 +126,10 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
 // lane order.  The order depends only on S.
 __global__ __launch_bounds__(256) void update_finalize_kernel(
     const float* __restrict__ part_sum, const int32_t* __restrict__ part_cnt, int S, int K, int D,
-    int DPAD, float* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts) {
+    int DPAD, float* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts,
+    const float* __restrict__ C_old, double* __restrict__ shift_part) {
     __shared__ double ssum[4][64];
+    __shared__ double ssq[64];
     __shared__ int64_t scnt[4][64];
     const int e = threadIdx.x & 63, q = threadIdx.x >> 6;
     const int64_t i = int64_t(blockIdx.x) * 64 + e;
@@ -167,14 +169,46 @@ __global__ __launch_bounds__(256) void update_finalize_kernel(
         n = scnt[0][e] + scnt[1][e] + scnt[2][e] + scnt[3][e];
         // the reference's count passes through fp32 (clamp of an int64 tensor with a float bound)
         const double cnt = double(float(n < 1 ? 1 : n));
-        C_new[int64_t(k) * ldcn + d] = float(sum / cnt);
+        const float cnew = float(sum / cnt);
+        C_new[int64_t(k) * ldcn + d] = cnew;
         if (d == 0 && counts) counts[k] = n;
+        if (C_old) {
+            const float df = C_old[int64_t(k) * D + d] - cnew;  // square taken in fp32 (kmeans.py:141)
+            ssq[e] = double(df * df);
+        }
+    }
+    if (C_old) {
+        // this block's share of sum((C - C_new)^2), added in element order
+        if (q == 0 && !ok) ssq[e] = 0.0;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double t = 0.0;
+            for (int i = 0; i < 64; ++i) t += ssq[i];
+            shift_part[blockIdx.x] = t;
+        }
+    }
+}
+
+// one workgroup adds the per-block shares in block order
+__global__ __launch_bounds__(256) void shift_final_kernel(const double* __restrict__ part, int nb,
+                                                          float* __restrict__ out) {
+    __shared__ double sh[256];
+    const int per = (nb + 255) / 256;
+    double acc = 0.0;
+    const int b0 = threadIdx.x * per, b1 = min(nb, b0 + per);
+    for (int i = b0; i < b1; ++i) acc += part[i];
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int i = 0; i < 256; ++i) t += sh[i];
+        *out = float(t);
     }
 }
 
 int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
-                  hipStream_t st) {
+                  const float* C_old, float* shift, hipStream_t st) {
     const UpdateGeom g = update_geom(N, D, K);
     const int dpad = g.J * 32;
     const size_t lds = size_t(g.KR + 1) * 32 * sizeof(float) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
@@ -184,9 +218,13 @@ int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32
     int rc = check_launch("update_partial_kernel");
     if (rc) return rc;
     const int64_t tot = int64_t(K) * D;
-    hipLaunchKernelGGL(update_finalize_kernel, dim3((unsigned)((tot + 63) / 64)), dim3(256), 0, st,
-                       w.part_sum, w.part_cnt, g.S, K, D, dpad, C_new, ldcn, counts);
-    return check_launch("update_finalize_kernel");
+    const int nb = int((tot + 63) / 64);
+    hipLaunchKernelGGL(update_finalize_kernel, dim3(nb), dim3(256), 0, st, w.part_sum, w.part_cnt,
+                       g.S, K, D, dpad, C_new, ldcn, counts, C_old, w.shift_part);
+    rc = check_launch("update_finalize_kernel");
+    if (rc || !C_old) return rc;
+    hipLaunchKernelGGL(shift_final_kernel, dim3(1), dim3(256), 0, st, w.shift_part, nb, shift);
+    return check_launch("shift_final_kernel");
 }
 
 // ---- scalar reductions: one workgroup, fixed order ------------------------------------------
