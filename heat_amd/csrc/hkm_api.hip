@@ -58,7 +58,11 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         return r;
     };
     w.red = reinterpret_cast<double*>(take(size_t(RED_SLOTS) * sizeof(double)));
-    if (flags & HKM_WS_ASSIGN) w.cn = reinterpret_cast<float*>(take(cn_pad(K) * sizeof(float)));
+    if (flags & HKM_WS_ASSIGN) {
+        w.cn = reinterpret_cast<float*>(take(cn_pad(K) * sizeof(float)));
+        if (assign_kind(D, K) == ASSIGN_MFMA_STREAM)
+            w.keys = reinterpret_cast<unsigned long long*>(take(size_t(N < 1 ? 1 : N) * sizeof(unsigned long long)));
+    }
     if ((flags & HKM_WS_UPDATE) && small_eligible(D, K))
         w.small_part = reinterpret_cast<double*>(take(size_t(SMALL_MAX_GRID) * (size_t(K) * (D + 1) + 1) * sizeof(double)));
     if (flags & HKM_WS_UPDATE) {
@@ -113,7 +117,7 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
         default: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
             if (rc) return rc;
-            return launch_assign_mfma_stream(X, N, D, ldx, C, K, ldc, w.cn, labels, min_d2, st);
+            return launch_assign_mfma_stream(X, N, D, ldx, C, K, ldc, w.cn, w.keys, labels, min_d2, st);
         }
     }
 }

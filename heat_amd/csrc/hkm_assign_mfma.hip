@@ -391,21 +391,70 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
 }
 
 // ------------------------------------------------------------------------------------------------
-// Streaming variant for any K and D.  A workgroup owns 128 points and walks over centroid tiles of
-// 128 and feature chunks of 32; its four waves form a 2 x 2 grid, each computing 64 points x 64
-// centroids per step (2 x 2 MFMA blocks, 64 MFMAs).  Both operand panels of a step (128 x 32 floats
-// each) are fetched with fully coalesced 16-byte loads by all 256 threads one step ahead and staged
-// through double-buffered LDS (row stride 36 floats keeps the 16-byte operand reads conflict-free).
-// After the last chunk of a centroid tile one more MFMA adds (-|c|^2/2) * 1 + 1 * (-|x|^2/2), so the
-// accumulator is minus half the squared distance (squared centroid norms come from global memory, padded with
-// +inf; |x|^2 is accumulated from the point operand while the first centroid tile is processed).
-// The (min, argmin) of the two waves that share a point are merged through LDS at the end of a tile.
+// Streaming variant for any K and D, 2-D decomposition.  A work item is (tile of 128 points) x (tile
+// of 128 centroids) over all features in chunks of 32; the four waves of a workgroup form a 2 x 2 grid,
+// each computing 64 points x 64 centroids per chunk (2 x 2 MFMA blocks, 64 MFMAs).  Both operand
+// panels of a chunk (128 x 32 floats each) are fetched with fully coalesced 16-byte loads by all 256
+// threads one chunk ahead and staged through double-buffered LDS (row stride 36 floats keeps the
+// 16-byte operand reads conflict-free).  After the last chunk one more MFMA adds
+// (-|c|^2/2) * 1 + 1 * (-|x|^2/2), so the accumulator is minus half the squared distance (squared
+// centroid norms come from global memory, padded with +inf; |x|^2 is accumulated from the point
+// operand on the way).
+//
+// Work items are laid out so that the workgroups of one XCD (workgroup b runs on XCD b % 8) work on
+// the SAME few point tiles at the same time, one centroid tile each: a point tile is then read from
+// HBM once and served to the other workgroups from that XCD's L2, instead of once per centroid tile.
+// The per-item (min, argmin) of a point are merged across centroid tiles with a 64-bit unsigned
+// atomic min on the key (bits of the clamped d2) << 32 | index: for non-negative floats the bit
+// pattern orders like the value, so the smallest distance wins and, among equal distances, the
+// smallest index -- an order-independent, hence deterministic, merge.
 // ------------------------------------------------------------------------------------------------
+struct StreamPlan {
+    int nct, ndc, W, PG;  // centroid tiles, feature chunks, workgroups per XCD, point tiles in flight per XCD
+    int grid;
+};
+static StreamPlan stream_plan(int64_t N, int32_t D, int32_t K) {
+    StreamPlan pl;
+    pl.nct = (K + 127) / 128;
+    pl.ndc = (D + 31) / 32;
+    const int w_max = num_cus() * 2 / 8;  // two workgroups per CU
+    if (pl.nct <= w_max) {
+        pl.PG = w_max / pl.nct;
+        const int64_t per_xcd = ((N + 127) / 128 + 7) / 8;  // point tiles per XCD
+        if (pl.PG > per_xcd) pl.PG = int(per_xcd < 1 ? 1 : per_xcd);
+        pl.W = pl.PG * pl.nct;
+    } else {
+        pl.PG = 1;
+        pl.W = w_max;
+    }
+    pl.grid = pl.W * 8;
+    return pl;
+}
+
+__global__ void fill_keys_kernel(unsigned long long* __restrict__ keys, int64_t n) {
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += int64_t(gridDim.x) * blockDim.x)
+        keys[i] = ~0ull;
+}
+
+__global__ void unpack_keys_kernel(const unsigned long long* __restrict__ keys, int64_t n,
+                                   int32_t* __restrict__ labels, float* __restrict__ min_d2) {
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += int64_t(gridDim.x) * blockDim.x) {
+        const unsigned long long k = keys[i];
+        const unsigned hi = unsigned(k >> 32);
+        // a row whose distances were all NaN never lowered its key: label 0 like the reference's
+        // torch.min on an all-NaN row
+        labels[i] = hi == 0xffffffffu ? 0 : int32_t(unsigned(k));
+        if (min_d2) min_d2[i] = __uint_as_float(hi);
+    }
+}
+
 template <bool VEC>
 __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
-    int64_t ldc, const float* __restrict__ cn, int32_t* __restrict__ labels,
-    float* __restrict__ min_d2, int64_t ntiles) {
+    int64_t ldc, const float* __restrict__ cn, unsigned long long* __restrict__ keys, int64_t ntiles,
+    int nct, int ndc, int W, int PG) {
     constexpr int PB = 2, CB = 2, TP = 128, TC = 128, DC = 32, LDS_LD = DC + 4;
     __shared__ __align__(16) float sA[2][TC * LDS_LD];
     __shared__ __align__(16) float sB[2][TP * LDS_LD];
@@ -415,36 +464,40 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     const int lane = tid & 63, wave = tid >> 6;
     const int wp = wave & 1, wc = wave >> 1;  // this wave: points [64 wp, +64), centroids [64 wc, +64)
     const int p = lane & 31, h = lane >> 5;
-    const int nct = (K + TC - 1) / TC;
-    const int ndc = (D + DC - 1) / DC;
-    const int64_t my_tiles = (ntiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
-    const int64_t nsteps = my_tiles * nct * ndc;
 
-    // staging role of this thread: rows sr + 32 q (q = 0..3) of both panels, column group sc
-    const int sr = tid >> 3;
-    const int sc = (tid & 7) * 4;
+    // items of this workgroup: item q = (point tile xt0 + 8 PG (q / cpw), centroid tile ct0 + W (q % cpw))
+    const int xcd = blockIdx.x & 7, l = blockIdx.x >> 3;
+    const bool spread = nct <= W;  // one centroid tile per workgroup, PG point tiles in flight
+    const int ct0 = spread ? l % nct : l;
+    const int64_t xt0 = xcd + 8 * int64_t(spread ? l / nct : 0);
+    const int cpw = spread ? 1 : (nct - l + W - 1) / W;
+    const int64_t xstep = 8 * int64_t(PG);
+    const int64_t nx = xt0 < ntiles ? (ntiles - xt0 + xstep - 1) / xstep : 0;
+    const int64_t nsteps = nx * cpw * ndc;
+
+    const int sr = tid >> 3;         // staging: rows sr + 32 q (q = 0..3) of both panels
+    const int sc = (tid & 7) * 4;    // column group
 
     floatx4 pa[4], pb_[4];
-    auto issue = [&](int64_t tile, int ct, int dc) {
+    auto issue = [&](int64_t xt, int ct, int dc) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int rc = ct * TC + sr + 32 * q;
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
             if (rc < K) v = load_row4<VEC>(C + int64_t(rc) * ldc, dc * DC + sc, D);
             pa[q] = v;
-            int64_t rp = tile * TP + sr + 32 * q;
+            int64_t rp = xt * TP + sr + 32 * q;
             rp = rp < N ? rp : N - 1;
             pb_[q] = load_row4<VEC>(X + rp * ldx, dc * DC + sc, D);
         }
     };
 
-    int64_t tile = blockIdx.x;
-    int ct = 0, dc = 0;
-    if (nsteps > 0) issue(tile, ct, dc);
+    int64_t xi = 0;  // index of the point tile within this workgroup's sequence
+    int ci = 0, dc = 0;
+    if (nsteps > 0) issue(xt0, ct0, 0);
 
     floatx16 acc[PB][CB];
-    float xs[PB] = {0.f, 0.f}, baug[PB] = {0.f, 0.f}, m[PB];
-    int mi[PB];
+    float xs[PB] = {0.f, 0.f};
 
     for (int64_t it = 0; it < nsteps; ++it) {
         const int buf = int(it & 1);
@@ -455,31 +508,25 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         }
         __syncthreads();
 
-        const int64_t cur_tile = tile;
-        const int cur_ct = ct, cur_dc = dc;
+        const int64_t cur_xt = xt0 + xi * xstep;
+        const int cur_ct = ct0 + ci * W, cur_dc = dc;
         if (++dc == ndc) {
             dc = 0;
-            if (++ct == nct) {
-                ct = 0;
-                tile += gridDim.x;
+            if (++ci == cpw) {
+                ci = 0;
+                ++xi;
             }
         }
-        if (it + 1 < nsteps) issue(tile, ct, dc);
+        if (it + 1 < nsteps) issue(xt0 + xi * xstep, ct0 + ci * W, dc);
 
         if (cur_dc == 0) {
 #pragma unroll
-            for (int pb = 0; pb < PB; ++pb)
+            for (int pb = 0; pb < PB; ++pb) {
+                xs[pb] = 0.f;
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) acc[pb][cb][v] = 0.f;
-            if (cur_ct == 0) {
-#pragma unroll
-                for (int pb = 0; pb < PB; ++pb) {
-                    xs[pb] = 0.f;
-                    m[pb] = -HKM_INF;
-                    mi[pb] = 0;
-                }
             }
         }
 
@@ -489,15 +536,11 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         for (int pb = 0; pb < PB; ++pb) {
             const float* brow = &sB[buf][(wp * 64 + pb * 32 + p) * LDS_LD + h * 16];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[pb][j] = ld4(brow + 4 * j);
-        }
-        if (cur_ct == 0) {
+            for (int j = 0; j < 4; ++j) {
+                b[pb][j] = ld4(brow + 4 * j);
 #pragma unroll
-            for (int pb = 0; pb < PB; ++pb)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) xs[pb] = fmaf(b[pb][j][t], b[pb][j][t], xs[pb]);
+                for (int t = 0; t < 4; ++t) xs[pb] = fmaf(b[pb][j][t], b[pb][j][t], xs[pb]);
+            }
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
@@ -514,22 +557,21 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         }
 
         if (cur_dc == ndc - 1) {
-            if (cur_ct == 0) {
+            float m[PB];
+            int mi[PB];
 #pragma unroll
-                for (int pb = 0; pb < PB; ++pb) {
-                    const float xn = xs[pb] + __shfl_xor(xs[pb], 32);
-                    baug[pb] = h ? -0.5f * xn : 1.0f;
-                }
-            }
+            for (int pb = 0; pb < PB; ++pb) {
+                const float xn = xs[pb] + __shfl_xor(xs[pb], 32);
+                const float baug = h ? -0.5f * xn : 1.0f;
+                m[pb] = -HKM_INF;
+                mi[pb] = 0;
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                const int kb = cur_ct * TC + wc * 64 + cb * 32;
-                const float aaug = h ? 1.0f : -0.5f * cn[kb + p];
-#pragma unroll
-                for (int pb = 0; pb < PB; ++pb) {
+                for (int cb = 0; cb < CB; ++cb) {
+                    const int kb = cur_ct * TC + wc * 64 + cb * 32;
+                    const float aaug = h ? 1.0f : -0.5f * cn[kb + p];
                     // g = x.c - |c|^2/2 - |x|^2/2 = -d2/2 (halving is exact): the nearest centroid has
                     // the LARGEST g; the clamp of d2 at 0 is a clamp of g at 0 from above
-                    const floatx16 g16 = MFMA32(aaug, baug[pb], acc[pb][cb]);
+                    const floatx16 g16 = MFMA32(aaug, baug, acc[pb][cb]);
                     float bm = fminf(g16[0], 0.0f);
                     int bi = 0;
 #pragma unroll
@@ -543,34 +585,32 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
                     mi[pb] = gt ? kb + bi : mi[pb];
                     m[pb] = gt ? bm : m[pb];
                 }
-            }
-            if (cur_ct == nct - 1) {
                 // merge lane halves, then the two waves that cover the same points
-#pragma unroll
-                for (int pb = 0; pb < PB; ++pb) {
-                    mi[pb] += 4 * h;
-                    m[pb] = -2.0f * m[pb];  // back to the squared distance
-                    merge_halves(m[pb], mi[pb]);
-                    if (h == 0) {
-                        sM[wc][wp * 64 + pb * 32 + p] = m[pb];
-                        sI[wc][wp * 64 + pb * 32 + p] = mi[pb];
-                    }
+                mi[pb] += 4 * h;
+                // back to the squared distance (+inf if every g was NaN or -inf); the "+ 0" turns a
+                // -0.0 into +0.0, whose bit pattern is the smallest key
+                m[pb] = -2.0f * m[pb] + 0.0f;
+                merge_halves(m[pb], mi[pb]);
+                if (h == 0) {
+                    sM[wc][wp * 64 + pb * 32 + p] = m[pb];
+                    sI[wc][wp * 64 + pb * 32 + p] = mi[pb];
                 }
-                __syncthreads();
-                if (tid < TP) {
-                    float m0 = sM[0][tid];
-                    int i0 = sI[0][tid];
-                    const float m1 = sM[1][tid];
-                    const int i1 = sI[1][tid];
-                    if (m1 < m0 || (m1 == m0 && i1 < i0)) {
-                        m0 = m1;
-                        i0 = i1;
-                    }
-                    const int64_t r = cur_tile * TP + tid;
-                    if (r < N) {
-                        labels[r] = i0;
-                        if (min_d2) min_d2[r] = m0;
-                    }
+            }
+            __syncthreads();
+            if (tid < TP) {
+                float m0 = sM[0][tid];
+                int i0 = sI[0][tid];
+                const float m1 = sM[1][tid];
+                const int i1 = sI[1][tid];
+                if (m1 < m0 || (m1 == m0 && i1 < i0)) {
+                    m0 = m1;
+                    i0 = i1;
+                }
+                const int64_t r = cur_xt * TP + tid;
+                if (r < N && m0 < HKM_INF) {
+                    const unsigned long long key =
+                        (static_cast<unsigned long long>(__float_as_uint(m0)) << 32) | unsigned(i0);
+                    atomicMin(keys + r, key);
                 }
             }
         }
@@ -578,19 +618,26 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
 }
 
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
-                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
-                              float* min_d2, hipStream_t st) {
+                              int32_t K, int64_t ldc, const float* cn, unsigned long long* keys,
+                              int32_t* labels, float* min_d2, hipStream_t st) {
     const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
     const int64_t ntiles = (N + 127) / 128;
-    int64_t grid = int64_t(num_cus()) * 2;
-    if (grid > ntiles) grid = ntiles;
+    const StreamPlan pl = stream_plan(N, D, K);
+    int64_t fgrid = (N + 255) / 256;
+    const int64_t fcap = int64_t(num_cus()) * 8;
+    if (fgrid > fcap) fgrid = fcap;
+    hipLaunchKernelGGL(fill_keys_kernel, dim3((unsigned)fgrid), dim3(256), 0, st, keys, N);
+    int rc = check_launch("fill_keys_kernel");
+    if (rc) return rc;
     if (vec)
-        hipLaunchKernelGGL(assign_mfma_stream_kernel<true>, dim3((unsigned)grid), dim3(256), 0, st, X,
-                           N, D, ldx, C, K, ldc, cn, labels, min_d2, ntiles);
+        hipLaunchKernelGGL(assign_mfma_stream_kernel<true>, dim3(pl.grid), dim3(256), 0, st, X, N, D, ldx,
+                           C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
     else
-        hipLaunchKernelGGL(assign_mfma_stream_kernel<false>, dim3((unsigned)grid), dim3(256), 0, st,
-                           X, N, D, ldx, C, K, ldc, cn, labels, min_d2, ntiles);
-    return check_launch("assign_mfma_stream_kernel");
+        hipLaunchKernelGGL(assign_mfma_stream_kernel<false>, dim3(pl.grid), dim3(256), 0, st, X, N, D,
+                           ldx, C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
+    if ((rc = check_launch("assign_mfma_stream_kernel"))) return rc;
+    hipLaunchKernelGGL(unpack_keys_kernel, dim3((unsigned)fgrid), dim3(256), 0, st, keys, N, labels, min_d2);
+    return check_launch("unpack_keys_kernel");
 }
 
 }  // namespace hkm

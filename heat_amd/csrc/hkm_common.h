@@ -46,6 +46,7 @@ UpdateGeom update_geom(int64_t N, int32_t D, int32_t K);
 // ---- workspace layout --------------------------------------------------------------------------
 struct Workspace {
     float* cn;          // squared centroid norms, padded to a multiple of 128 with +inf
+    unsigned long long* keys;  // [N] packed (d2 bits, index) merge keys of the streaming kernel
     float* part_sum;    // [S][K][J*32] fp32 partial sums
     int32_t* part_cnt;  // [S][K]
     int64_t* counts;    // [K]
@@ -71,8 +72,8 @@ int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, 
                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
                              float* min_d2, hipStream_t st);
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
-                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
-                              float* min_d2, hipStream_t st);
+                              int32_t K, int64_t ldc, const float* cn, unsigned long long* keys,
+                              int32_t* labels, float* min_d2, hipStream_t st);
 bool small_eligible(int32_t D, int32_t K);
 int small_grid(int64_t N, int32_t D, int32_t K);
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
