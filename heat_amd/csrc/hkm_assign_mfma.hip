@@ -153,6 +153,21 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     const int p = lane & 31, h = lane >> 5;
     const int ncb = KP >> 5;
 
+    // the rows of the next tile are requested before the current tile is scanned
+    floatx4 bn[PB][NJ];
+    auto fetch = [&](int64_t tile) {
+        const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            int64_t r = row0 + pb * 32 + p;
+            r = r < N ? r : N - 1;
+            const float* xr = X + r * ldx;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bn[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+        }
+    };
+    if (int64_t(blockIdx.x) < ntiles) fetch(blockIdx.x);
+
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
         floatx4 b[PB][NJ];
@@ -160,19 +175,17 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
         int mi[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
-            int64_t r = row0 + pb * 32 + p;
-            r = r < N ? r : N - 1;
-            const float* xr = X + r * ldx;
             float s = 0.f;
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                b[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+                b[pb][j] = bn[pb][j];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
             }
             const float xn = s + __shfl_xor(s, 32);
             baug[pb] = h ? xn : 1.0f;  // pairs with [|c|^2, 1] of the centroid row
         }
+        if (tile + gridDim.x < ntiles) fetch(tile + gridDim.x);
 
         resident_scan<DP, PB, false>(sC, ncb, p, h, b, baug, m, mi);
         bool neg = false;
