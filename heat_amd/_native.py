@@ -36,6 +36,8 @@ SIGNATURES = {
     "hkm_functional_value_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_cdist_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
                                      c_void_p, c_int64, c_int32, c_void_p]),
+    "hkm_pairwise_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
+                                        c_void_p, c_int64, c_int32, ctypes.c_float, c_void_p]),
     "hkm_widen_labels_i64": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
 }
 
@@ -169,6 +171,18 @@ def cdist(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, sqrt: bool = True
     nn = y.shape[0]
     check(load().hkm_cdist_f32(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn, y.stride(0) if nn > 1 else d,
                                d, _ptr(out), out.stride(0) if m > 1 else nn, 1 if sqrt else 0, _stream()))
+
+
+METRIC_EUCLID_QE, METRIC_EUCLID, METRIC_GAUSS_QE, METRIC_GAUSS, METRIC_MANHATTAN = 0, 1, 2, 3, 4
+
+
+def pairwise(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, metric: int, sigma: float = 1.0) -> None:
+    _require_gpu(x, y, out)
+    m, d = x.shape
+    nn = y.shape[0]
+    check(load().hkm_pairwise_f32(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn,
+                                  y.stride(0) if nn > 1 else d, d, _ptr(out), out.stride(0) if m > 1 else nn,
+                                  metric, float(sigma), _stream()))
 
 
 def widen_labels(labels32: torch.Tensor, out64: torch.Tensor) -> None:

@@ -238,7 +238,28 @@ int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_
     if (!out) return fail(HKM_EINVAL, "out is NULL");
     if (ldo < Nn) return fail(HKM_EINVAL, "leading dimension of out (%lld) < columns (%lld)", (long long)ldo, (long long)Nn);
     if (M == 0 || Nn == 0) return HKM_OK;
-    return launch_cdist(X, M, ldx, Y, Nn, ldy, D, out, ldo, sqrt_flag, static_cast<hipStream_t>(hip_stream));
+    return launch_cdist(X, M, ldx, Y, Nn, ldy, D, out, ldo, 0, sqrt_flag, 0.f, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                     int32_t D, float* out, int64_t ldo, int32_t metric, float sigma, void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 0 || Nn < 0) return fail(HKM_EINVAL, "negative row count (M = %lld, Nn = %lld)", (long long)M, (long long)Nn);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    if (metric < HKM_METRIC_EUCLID_QE || metric > HKM_METRIC_MANHATTAN) return fail(HKM_EINVAL, "unknown metric %d", metric);
+    const bool gaussian = metric == HKM_METRIC_GAUSS_QE || metric == HKM_METRIC_GAUSS;
+    if (gaussian && !(sigma > 0.f)) return fail(HKM_EINVAL, "sigma = %g must be > 0", double(sigma));
+    int rc;
+    if ((rc = check_matrix("X", X, M, D, ldx))) return rc;
+    if ((rc = check_matrix("Y", Y, Nn, D, ldy))) return rc;
+    if (!out) return fail(HKM_EINVAL, "out is NULL");
+    if (ldo < Nn) return fail(HKM_EINVAL, "leading dimension of out (%lld) < columns (%lld)", (long long)ldo, (long long)Nn);
+    if (M == 0 || Nn == 0) return HKM_OK;
+    const int form = (metric == HKM_METRIC_EUCLID_QE || metric == HKM_METRIC_GAUSS_QE) ? 0
+                     : metric == HKM_METRIC_MANHATTAN                                   ? 2
+                                                                                        : 1;
+    const float gauss = gaussian ? 1.0f / (2.0f * sigma * sigma) : 0.f;
+    return launch_cdist(X, M, ldx, Y, Nn, ldy, D, out, ldo, form, 1, gauss, static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream) {

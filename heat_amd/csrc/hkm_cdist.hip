@@ -1,8 +1,9 @@
-// Full pairwise distance matrix (quadratic expansion) for the public cdist API.
-// out[i, j] = max(0, (|x_i|^2 + |y_j|^2) - 2 x_i.y_j), optionally square-rooted
-// (heat/spatial/distance.py:32-64).  The output is M x Nn floats, so for the feature counts cdist is
-// used with the kernel is bound by writing the matrix; a 64 x 64 output tile per workgroup with a
-// 4 x 4 register block per lane keeps the X / Y re-reads in L2 and the stores 16 bytes wide.
+// Full pairwise distance matrices for the public cdist / rbf / manhattan API
+// (heat/spatial/distance.py:17-133): quadratic expansion max(0, (|x|^2 + |y|^2) - 2 x.y), the direct
+// form sum((x-y)^2) and sum|x-y|, followed by sqrt or exp(-d2 / (2 sigma^2)).  The output is M x Nn
+// floats, so for the feature counts these functions are used with the kernel is bound by writing the
+// matrix; a 64 x 64 output tile per workgroup with a 4 x 4 register block per lane keeps the X / Y
+// re-reads in L2 and the stores 16 bytes wide.
 #include "hkm_common.h"
 
 namespace hkm {
@@ -10,11 +11,14 @@ namespace hkm {
 static constexpr int CD_T = 64;   // tile edge
 static constexpr int CD_KC = 16;  // feature chunk
 
+// METRIC: 0 = quadratic expansion (squared, optional sqrt), 1 = direct sum((x-y)^2) (optional sqrt),
+//         2 = sum |x-y|;  gauss != 0 applies exp(-d2 * gauss) to the squared distance instead of sqrt
+template <int METRIC>
 __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X, int64_t M,
                                                     int64_t ldx, const float* __restrict__ Y,
                                                     int64_t Nn, int64_t ldy, int D,
                                                     float* __restrict__ out, int64_t ldo,
-                                                    int sqrt_flag, int64_t tiles_n) {
+                                                    int sqrt_flag, float gauss, int64_t tiles_n) {
     __shared__ float sX[CD_KC][CD_T + 4];
     __shared__ float sY[CD_KC][CD_T + 4];
     __shared__ float sXn[CD_T], sYn[CD_T];
@@ -66,7 +70,16 @@ __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X,
 #pragma unroll
             for (int a = 0; a < 4; ++a)
 #pragma unroll
-                for (int b = 0; b < 4; ++b) acc[a][b] = fmaf(xa[a], yb[b], acc[a][b]);
+                for (int b = 0; b < 4; ++b) {
+                    if (METRIC == 0) {
+                        acc[a][b] = fmaf(xa[a], yb[b], acc[a][b]);
+                    } else if (METRIC == 1) {
+                        const float df = xa[a] - yb[b];
+                        acc[a][b] = fmaf(df, df, acc[a][b]);
+                    } else {
+                        acc[a][b] += fabsf(xa[a] - yb[b]);
+                    }
+                }
         }
     }
     __syncthreads();
@@ -80,21 +93,33 @@ __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X,
         for (int b = 0; b < 4; ++b) {
             const int64_t gj = j0 + tx * 4 + b;
             if (gj >= Nn) continue;
-            float d = fmaf(-2.0f, acc[a][b], xn + sYn[tx * 4 + b]);
-            d = fmaxf(d, 0.0f);
-            if (sqrt_flag) d = sqrtf(d);
+            float d = acc[a][b];
+            if (METRIC == 0) {
+                d = fmaf(-2.0f, d, xn + sYn[tx * 4 + b]);
+                d = fmaxf(d, 0.0f);
+            }
+            if (METRIC != 2) {
+                if (gauss != 0.f) d = expf(-d * gauss);
+                else if (sqrt_flag) d = sqrtf(d);
+            }
             out[gi * ldo + gj] = d;
         }
     }
 }
 
 int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
-                 int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, hipStream_t st) {
+                 int32_t D, float* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, float gauss,
+                 hipStream_t st) {
     const int64_t tiles_m = (M + CD_T - 1) / CD_T, tiles_n = (Nn + CD_T - 1) / CD_T;
     const int64_t total = tiles_m * tiles_n;
     if (total > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "cdist: %lld tiles exceed the grid limit", (long long)total);
-    hipLaunchKernelGGL(cdist_kernel, dim3((unsigned)total), dim3(256), 0, st, X, M, ldx, Y, Nn, ldy,
-                       D, out, ldo, sqrt_flag, tiles_n);
+#define HKM_GO(MET)                                                                              \
+    hipLaunchKernelGGL(cdist_kernel<MET>, dim3((unsigned)total), dim3(256), 0, st, X, M, ldx, Y, Nn, \
+                       ldy, D, out, ldo, sqrt_flag, gauss, tiles_n)
+    if (metric == 0) HKM_GO(0);
+    else if (metric == 1) HKM_GO(1);
+    else HKM_GO(2);
+#undef HKM_GO
     return check_launch("cdist_kernel");
 }
 

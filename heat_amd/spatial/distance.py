@@ -1,7 +1,6 @@
 """
-Pairwise distances with the interface of heat/spatial/distance.py:136-156 (``cdist``), backed by
-the hkm_cdist_f32 kernel.  Only the quadratic-expansion metric on float32 is computed here; that
-is the branch KMeans uses (heat/cluster/kmeans.py:67).
+Pairwise distances with the interface of heat/spatial/distance.py:136-206 (``cdist``, ``rbf``,
+``manhattan``), backed by the hkm_pairwise_f32 kernel, computed in float32 on one rank.
 """
 
 from __future__ import annotations
@@ -14,7 +13,7 @@ from .. import _native
 from ..core import types
 from ..core.dndarray import DNDarray
 
-__all__ = ["cdist"]
+__all__ = ["cdist", "manhattan", "rbf"]
 
 
 def _check_inputs(X: DNDarray, Y: Optional[DNDarray]):
@@ -65,20 +64,10 @@ def _as_f32_matrix(a: DNDarray, promoted) -> torch.Tensor:
     return t
 
 
-def cdist(X: DNDarray, Y: Optional[DNDarray] = None, quadratic_expansion: bool = False) -> DNDarray:
-    """
-    Euclidean distance between all rows of ``X`` (m x f) and ``Y`` (n x f): an (m, n) DNDarray of
-    square-rooted distances in promote(X, Y, float32), ``split = X.split`` (1 when only ``Y`` is
-    split).  ``Y=None`` means ``Y = X``.
-
-    Only ``quadratic_expansion=True`` is built: |x-y|^2 = |x|^2 + |y|^2 - 2xy clamped at 0, in
-    float32.  The other metric of the reference (``torch.cdist``) is not part of this package.
-    """
+def _pairwise(X: DNDarray, Y: Optional[DNDarray], metric: int, sigma: float = 1.0) -> DNDarray:
+    """Shared driver of cdist / rbf / manhattan: the checks and promotion of ``_dist``
+    (heat/spatial/distance.py:209-414) at one rank, then one kernel launch."""
     split = _check_inputs(X, Y)
-    if not quadratic_expansion:
-        raise NotImplementedError(
-            "cdist(quadratic_expansion=False) is not built in heat_amd; use quadratic_expansion=True"
-        )
     promoted = types.promote_types(X.dtype, types.float32)
     if Y is not None:
         promoted = types.promote_types(types.promote_types(X.dtype, Y.dtype), types.float32)
@@ -87,5 +76,29 @@ def cdist(X: DNDarray, Y: Optional[DNDarray] = None, quadratic_expansion: bool =
     if x.shape[1] != y.shape[1]:
         raise ValueError("Inputs must have same shape[1]")
     out = torch.empty((x.shape[0], y.shape[0]), dtype=torch.float32, device=x.device)
-    _native.cdist(x, y, out, sqrt=True)
+    _native.pairwise(x, y, out, metric, sigma)
     return DNDarray(out, tuple(out.shape), types.float32, split, X.device, X.comm, True)
+
+
+def cdist(X: DNDarray, Y: Optional[DNDarray] = None, quadratic_expansion: bool = False) -> DNDarray:
+    """
+    Euclidean distance between all rows of ``X`` (m x f) and ``Y`` (n x f): an (m, n) DNDarray of
+    square-rooted distances in promote(X, Y, float32), ``split = X.split`` (1 when only ``Y`` is
+    split).  ``Y=None`` means ``Y = X``.  Computed in float32.
+
+    ``quadratic_expansion=True``: |x-y|^2 = |x|^2 + |y|^2 - 2xy clamped at 0 (the metric KMeans
+    uses); ``False``: sum((x-y)^2) directly (heat/spatial/distance.py:136-156).
+    """
+    return _pairwise(X, Y, _native.METRIC_EUCLID_QE if quadratic_expansion else _native.METRIC_EUCLID)
+
+
+def rbf(X: DNDarray, Y: Optional[DNDarray] = None, sigma: float = 1.0,
+        quadratic_expansion: bool = False) -> DNDarray:
+    """Gaussian kernel exp(-|x-y|^2 / (2 sigma^2)) between all rows (heat/spatial/distance.py:159-183)."""
+    return _pairwise(X, Y, _native.METRIC_GAUSS_QE if quadratic_expansion else _native.METRIC_GAUSS, sigma)
+
+
+def manhattan(X: DNDarray, Y: Optional[DNDarray] = None, expand: bool = False) -> DNDarray:
+    """Manhattan distance sum|x_i - y_i| between all rows; ``expand`` selects between two evaluation
+    strategies in the reference and has no effect here (heat/spatial/distance.py:186-206)."""
+    return _pairwise(X, Y, _native.METRIC_MANHATTAN)

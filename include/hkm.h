@@ -105,6 +105,23 @@ int hkm_functional_value_f32(const float* min_d2, int64_t N, float* out, void* w
 int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                   int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, void* hip_stream);
 
+/*
+ * The other pairwise functions of heat/spatial/distance.py on local tensors, out is M x Nn:
+ *   HKM_METRIC_EUCLID_QE  sqrt(max(0, |x|^2+|y|^2-2x.y))        cdist(quadratic_expansion=True),  :32-64
+ *   HKM_METRIC_EUCLID     sqrt(sum((x-y)^2))                     cdist(quadratic_expansion=False), :17-29
+ *   HKM_METRIC_GAUSS_QE   exp(-max(0, expansion) / (2 sigma^2))  rbf(quadratic_expansion=True),    :87-103
+ *   HKM_METRIC_GAUSS      exp(-sum((x-y)^2) / (2 sigma^2))       rbf(quadratic_expansion=False),   :67-84
+ *   HKM_METRIC_MANHATTAN  sum(|x-y|)                             manhattan(expand=True/False),     :106-133
+ * sigma is read for the two Gaussian metrics only.
+ */
+#define HKM_METRIC_EUCLID_QE 0
+#define HKM_METRIC_EUCLID 1
+#define HKM_METRIC_GAUSS_QE 2
+#define HKM_METRIC_GAUSS 3
+#define HKM_METRIC_MANHATTAN 4
+int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                     int32_t D, float* out, int64_t ldo, int32_t metric, float sigma, void* hip_stream);
+
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 

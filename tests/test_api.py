@@ -99,6 +99,10 @@ def test_cdist_exceptions():
         ht.spatial.cdist(ht.ones((4, 4)), ht.ones((4, 5)), quadratic_expansion=True)
     with pytest.raises(NotImplementedError):  # float64 is outside the float32 kernels
         ht.spatial.cdist(ht.ones((4, 4), dtype=ht.float64), quadratic_expansion=True)
+    with pytest.raises(NotImplementedError):
+        ht.spatial.rbf(X)
+    with pytest.raises(NotImplementedError):
+        ht.spatial.manhattan(ht.ones((4, 4)), Z)
 
 
 # ---- array surface ----------------------------------------------------------------------------
@@ -155,7 +159,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) >= 11
+    assert len(names) >= 12
     for name in names:
         assert hasattr(lib, name), name
         assert name in _native.SIGNATURES, f"{name} has no ctypes signature"
@@ -209,6 +213,9 @@ def test_argument_validation_happens_on_the_host():
     assert lib.hkm_shift_f32(good, good, 0, 3, good, None) == _native.HKM_EINVAL
     assert lib.hkm_cdist_f32(good, 4, 3, good, 4, 3, 3, good, 3, 1, None) == _native.HKM_EINVAL  # ldo < Nn
     assert lib.hkm_cdist_f32(good, -4, 3, good, 4, 3, 3, good, 4, 1, None) == _native.HKM_EINVAL
+    assert lib.hkm_pairwise_f32(good, 4, 3, good, 4, 3, 3, good, 4, 9, 1.0, None) == _native.HKM_EINVAL  # metric
+    assert lib.hkm_pairwise_f32(good, 4, 3, good, 4, 3, 3, good, 4, _native.METRIC_GAUSS, 0.0, None) == _native.HKM_EINVAL
+    assert "sigma" in err()
     assert lib.hkm_widen_labels_i64(None, 4, good, None) == _native.HKM_EINVAL
     assert lib.hkm_functional_value_f32(good, -1, good, ws, big, None) == _native.HKM_EINVAL
     # zero-sized problems succeed without touching the device

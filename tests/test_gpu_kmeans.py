@@ -241,3 +241,53 @@ def test_random_init_and_fit_predict(cuda):
     xi = ht.array((w.x * 10).to(torch.int32).to(cuda))
     c = ht.cluster.KMeans(n_clusters=4, init="random", max_iter=3, random_state=1).fit(xi)
     assert c.cluster_centers_.shape == (4, 8) and c.cluster_centers_.dtype is ht.float32
+
+
+def test_spatial_known_answers_all_metrics(cuda):
+    # tests/spatial/test_distances.py:16-58 of the reference: ones vs zeros with 4 features
+    import math
+
+    X = ht.array(torch.ones((4, 4), device=cuda))
+    Y = ht.array(torch.zeros((4, 4), device=cuda))
+    Xs = ht.array(torch.ones((4, 4), device=cuda), split=0)
+    for qe in (False, True):
+        d = ht.spatial.cdist(X, quadratic_expansion=qe)
+        assert torch.allclose(d.larray.cpu(), torch.zeros((4, 4))) and d.split is None
+        d = ht.spatial.cdist(X, Y, quadratic_expansion=qe)
+        assert torch.allclose(d.larray.cpu(), torch.full((4, 4), 2.0))
+        d = ht.spatial.rbf(X, quadratic_expansion=qe)
+        assert torch.allclose(d.larray.cpu(), torch.ones((4, 4)))
+        d = ht.spatial.rbf(X, Y, sigma=math.sqrt(2.0), quadratic_expansion=qe)
+        assert torch.allclose(d.larray.cpu(), torch.full((4, 4), math.exp(-1.0)))
+        d = ht.spatial.cdist(Xs, Y, quadratic_expansion=qe)
+        assert d.split == 0
+    for ex in (False, True):
+        d = ht.spatial.manhattan(X, expand=ex)
+        assert torch.allclose(d.larray.cpu(), torch.zeros((4, 4)))
+        d = ht.spatial.manhattan(Xs, Y, expand=ex)
+        assert torch.allclose(d.larray.cpu(), torch.full((4, 4), 4.0)) and d.split == 0
+    with pytest.raises(NotImplementedError):
+        ht.spatial.rbf(ht.array(torch.ones((4, 4), device=cuda), split=1))
+    with pytest.raises(NotImplementedError):
+        ht.spatial.manhattan(ht.array(torch.ones((4, 4, 2), device=cuda)))
+
+
+def test_spatial_metrics_against_torch(cuda):
+    # the reference's own cross-check (tests/spatial/test_distances.py:207-265): row-scaled ones
+    # against torch.cdist, plus random inputs against torch.cdist (p = 2, p = 1) in float64
+    A = torch.ones((8, 6)) * torch.arange(8, dtype=torch.float32).view(-1, 1)
+    Ad = ht.array(A.to(cuda), split=0)
+    ref = torch.cdist(A, A)
+    assert torch.allclose(ht.spatial.cdist(Ad, quadratic_expansion=False).larray.cpu(), ref, atol=1e-5)
+    assert torch.allclose(ht.spatial.cdist(Ad, ht.array(A.to(torch.int32).to(cuda), split=0)).larray.cpu(), ref, atol=1e-5)
+    g = torch.Generator().manual_seed(12)
+    for m, n, d in ((100, 70, 3), (130, 257, 64), (65, 64, 200)):
+        a, b = torch.randn((m, d), generator=g) * 2, torch.randn((n, d), generator=g) * 2
+        ad, bd = ht.array(a.to(cuda), split=0), ht.array(b.to(cuda))
+        e = torch.cdist(a.double(), b.double())
+        assert torch.allclose(ht.spatial.cdist(ad, bd).larray.cpu().double(), e, rtol=1e-5, atol=1e-5)
+        assert torch.allclose(ht.spatial.cdist(ad, bd, quadratic_expansion=True).larray.cpu().double(), e, rtol=1e-4, atol=2e-3)
+        assert torch.allclose(ht.spatial.manhattan(ad, bd).larray.cpu().double(), torch.cdist(a.double(), b.double(), p=1), rtol=1e-5, atol=1e-4)
+        for qe in (False, True):
+            r = ht.spatial.rbf(ad, bd, sigma=3.0, quadratic_expansion=qe).larray.cpu().double()
+            assert torch.allclose(r, torch.exp(-e * e / 18.0), rtol=1e-4, atol=1e-5)
