@@ -38,6 +38,10 @@ SIGNATURES = {
                                      c_void_p, c_int64, c_int32, c_void_p]),
     "hkm_pairwise_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
                                         c_void_p, c_int64, c_int32, ctypes.c_float, c_void_p]),
+    "hkm_min_dist_sum_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_sample_select_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_void_p, ctypes.c_float, c_void_p,
+                                             c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_label_counts_i64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
     "hkm_widen_labels_i64": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
 }
 
@@ -183,6 +187,33 @@ def pairwise(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, metric: int, s
     check(load().hkm_pairwise_f32(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn,
                                   y.stride(0) if nn > 1 else d, d, _ptr(out), out.stride(0) if m > 1 else nn,
                                   metric, float(sigma), _stream()))
+
+
+def min_dist_sum(min_d2: torch.Tensor, out: torch.Tensor, ws: Workspace) -> None:
+    """out = sum_i sqrt(min_d2[i]) (device scalar)."""
+    _require_gpu(min_d2, out)
+    n = min_d2.numel()
+    buf = ws.get(workspace_bytes(n, 1, 1, WS_ASSIGN))
+    check(load().hkm_min_dist_sum_f32(_ptr(min_d2), n, _ptr(out), _ptr(buf), buf.numel(), _stream()))
+
+
+def sample_select(min_d2: torch.Tensor, u: torch.Tensor, cost: torch.Tensor, oversampling: float,
+                  idx: torch.Tensor, count: torch.Tensor, ws: Workspace) -> None:
+    """idx[:count] = ascending rows i with u[i] <= oversampling * sqrt(min_d2[i]) / max(cost, 1e-12)."""
+    _require_gpu(min_d2, u, cost, idx, count)
+    n = min_d2.numel()
+    if u.numel() != n:
+        raise ValueError(f"u has {u.numel()} elements, expected {n}")
+    buf = ws.get(workspace_bytes(n, 1, 1, WS_ASSIGN))
+    check(load().hkm_sample_select_f32(_ptr(min_d2), _ptr(u), n, _ptr(cost), float(oversampling), _ptr(idx),
+                                       idx.numel(), _ptr(count), _ptr(buf), buf.numel(), _stream()))
+
+
+def label_counts(labels32: torch.Tensor, k: int, counts: torch.Tensor) -> None:
+    _require_gpu(labels32, counts)
+    if counts.numel() != k:
+        raise ValueError(f"counts has {counts.numel()} elements, expected {k}")
+    check(load().hkm_label_counts_i64(_ptr(labels32), labels32.numel(), k, _ptr(counts), _stream()))
 
 
 def widen_labels(labels32: torch.Tensor, out64: torch.Tensor) -> None:

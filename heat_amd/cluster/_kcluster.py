@@ -8,6 +8,8 @@ never built.
 
 from __future__ import annotations
 
+import math
+import warnings
 from typing import Optional, Union
 
 import torch
@@ -16,6 +18,7 @@ from .. import _native
 from ..core import types
 from ..core.base import BaseEstimator, ClusteringMixin
 from ..core.dndarray import DNDarray
+from ._sampling import DeviceSampler
 
 
 class _KCluster(ClusteringMixin, BaseEstimator):
@@ -92,8 +95,9 @@ class _KCluster(ClusteringMixin, BaseEstimator):
     def _initialize_cluster_centers(self, x: DNDarray, oversampling: float, iter_multiplier: float):
         """
         Initial centroids; checks in the order of heat/cluster/_kcluster.py:116-143,276-281.
-        Built: ``"random"`` (K rows drawn with a generator seeded by ``random_state``) and an explicit
-        (K, D) DNDarray, which is copied so later changes by the caller do not leak in.
+        ``"random"`` (K rows drawn with a generator seeded by ``random_state``), an explicit (K, D)
+        DNDarray, which is copied so later changes by the caller do not leak in,
+        ``"probability_based"`` (k-means||) and ``"batchparallel"``.
         """
         if not isinstance(x, DNDarray):
             raise ValueError(f"Input x needs to be a ht.DNDarray, but was {type(x)}")
@@ -121,20 +125,109 @@ class _KCluster(ClusteringMixin, BaseEstimator):
             self._cluster_centers = self.init.resplit(None)
         elif isinstance(self.init, str) and self.init == "probability_based":
             if x.split is None or x.split == 0:
-                raise NotImplementedError('init="probability_based" (k-means||) is not built in heat_amd')
-            raise NotImplementedError("Not implemented for other splitting-axes")
+                cent = self._kmeans_parallel(x, oversampling, iter_multiplier)
+                self._cluster_centers = DNDarray(cent, tuple(cent.shape), types.float32, None, x.device, x.comm, True)
+            else:
+                raise NotImplementedError("Not implemented for other splitting-axes")
         elif isinstance(self.init, str) and self.init == "batchparallel":
             if x.split == 0:
-                raise NotImplementedError('init="batchparallel" is not built in heat_amd')
-            raise NotImplementedError(
-                f"Batch parallel initalization only implemented for split = 0, but split was {x.split}"
-            )
+                if self._p == 2:
+                    from .batchparallelclustering import BatchParallelKMeans
+
+                    clusterer = BatchParallelKMeans(n_clusters=self.n_clusters, init="k-means++", max_iter=100,
+                                                    random_state=self.random_state)
+                elif self._p == 1:
+                    raise NotImplementedError("BatchParallelKMedians is not built in heat_amd")
+                else:
+                    raise ValueError("Batch parallel initialization only implemented for KMeans and KMedians")
+                clusterer.fit(x)
+                self._cluster_centers = clusterer.cluster_centers_
+            else:
+                raise NotImplementedError(
+                    f"Batch parallel initalization only implemented for split = 0, but split was {x.split}"
+                )
         else:
             raise ValueError(
                 'init needs to be one of "random", ht.DNDarray, "kmeans++", or "batchparallel", but was {}'.format(
                     self.init
                 )
             )
+
+    # ---- k-means|| (heat/cluster/_kcluster.py:146-247, 283-350) --------------------------------
+    def _make_sampler(self, device: torch.device):
+        """Source of the initialiser's random draws; replaced in tests to feed fixed numbers."""
+        return DeviceSampler(device, self.random_state)
+
+    def _centroid_sampling_helper(self, xt: torch.Tensor, centroids: torch.Tensor, oversampling: float,
+                                  num_iters: int, sampler, ws) -> torch.Tensor:
+        """
+        ``num_iters`` rounds of: distance of every row to its closest current candidate, then every
+        row joins the candidates with probability ``oversampling * distance / sum(distance)``
+        (heat/cluster/_kcluster.py:283-350).  One fused distance+argmin launch, one reduction and one
+        ordered selection per round; only the number of new candidates comes back to the host.
+        """
+        n = xt.shape[0]
+        dev = xt.device
+        lab = torch.empty((n,), dtype=torch.int32, device=dev)
+        d2 = torch.empty((n,), dtype=torch.float32, device=dev)
+        cost = torch.empty((), dtype=torch.float32, device=dev)
+        count = torch.zeros((), dtype=torch.int64, device=dev)
+        idx = torch.empty((max(1024, int(16 * oversampling)),), dtype=torch.int64, device=dev)
+        for _ in range(num_iters):
+            _native.assign(xt, centroids, lab, d2, ws)
+            _native.min_dist_sum(d2, cost, ws)
+            u = sampler.uniform(n)
+            _native.sample_select(d2, u, cost, oversampling, idx, count, ws)
+            c = int(count.item())
+            if c > idx.numel():
+                idx = torch.empty((c,), dtype=torch.int64, device=dev)
+                _native.sample_select(d2, u, cost, oversampling, idx, count, ws)
+            centroids = torch.cat((centroids, xt[idx[:c]]), dim=0)
+        return centroids
+
+    def _kmeans_parallel(self, x: DNDarray, oversampling: float, iter_multiplier: float) -> torch.Tensor:
+        """(K, D) initial centroids by k-means|| and a weighted k-means++ reclustering of the candidates."""
+        from .batchparallelclustering import _kmex
+
+        xt = self._local_f32(x)
+        n = xt.shape[0]
+        dev = xt.device
+        ws = self._workspace(dev)
+        sampler = self._make_sampler(dev)
+        # randint(0, n - 1) of the reference excludes the last row
+        first = sampler.randint(max(n - 1, 1))
+        init_centroids = xt[first : first + 1].clone()
+        lab = torch.empty((n,), dtype=torch.int32, device=dev)
+        d2 = torch.empty((n,), dtype=torch.float32, device=dev)
+        cost = torch.empty((), dtype=torch.float32, device=dev)
+        _native.assign(xt, init_centroids, lab, d2, ws)
+        _native.min_dist_sum(d2, cost, ws)
+        init_cost = float(cost.item())
+        # the order of magnitude of the initial cost sets the number of rounds (_kcluster.py:172-175);
+        # all rows equal gives cost 0, where the reference fails in int(-inf): one round instead
+        num_iters = max(1, int(iter_multiplier * math.log(init_cost))) if init_cost > 0.0 else 1
+        centroids = self._centroid_sampling_helper(xt, init_centroids, oversampling, num_iters, sampler, ws)
+        if centroids.shape[0] <= self.n_clusters:
+            warnings.warn(
+                f"Oversampling={oversampling} is too low for data set."
+                "Increasing it by factor 10 automatically. And restarting centroid initialization.",
+                UserWarning,
+            )
+            oversampling = 10 * oversampling
+            centroids = self._centroid_sampling_helper(xt, init_centroids, oversampling, num_iters, sampler, ws)
+        if centroids.shape[0] <= self.n_clusters:
+            raise ValueError(
+                f"The parameter oversampling={oversampling} and/or iter_multiplier={iter_multiplier} "
+                "are chosen too small for the initialization of cluster centers."
+            )
+        # weight of a candidate = number of rows closest to it (_kcluster.py:198-208)
+        m = centroids.shape[0]
+        _native.assign(xt, centroids, lab, None, ws)
+        counts = torch.empty((m,), dtype=torch.int64, device=dev)
+        _native.label_counts(lab, m, counts)
+        weights = counts.to(torch.float32)
+        centers, _ = _kmex(centroids, 2, self.n_clusters, "++", self.max_iter, self.tol, sampler, weights, ws)
+        return centers
 
     def _assign_to_cluster(self, x: DNDarray, eval_functional_value: bool = False) -> DNDarray:
         """

@@ -1,0 +1,226 @@
+"""
+Single-device k-means++ seeding and Lloyd iteration on a local matrix, and the batch-parallel
+estimator built from them; interface of heat/cluster/batchparallelclustering.py.
+
+The reference runs these helpers with ``torch.cdist`` / ``torch.argmin`` / ``torch.mean``; here every
+distance + argmin is one call of the fused kernel (``hkm_assign_f32``) and every mean one call of the
+deterministic update (``hkm_update_f32``), torch only supplies memory, the random draws and a few
+elementwise operations on K x D or N-element vectors.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple, Union
+from warnings import warn
+
+import torch
+
+from .. import _native
+from ..core import types
+from ..core.base import BaseEstimator, ClusteringMixin
+from ..core.dndarray import DNDarray
+from ._sampling import DeviceSampler
+
+
+def _dist_to_row(x: torch.Tensor, row: torch.Tensor) -> torch.Tensor:
+    """Euclidean distance sqrt(sum((x_i - row)^2)) of every row of x to one row (direct form: exactly
+    zero for the row itself, which a quadratic expansion does not guarantee)."""
+    out = torch.empty((x.shape[0], 1), dtype=torch.float32, device=x.device)
+    _native.pairwise(x, row.reshape(1, -1).contiguous(), out, _native.METRIC_EUCLID)
+    return out.view(-1)
+
+
+def _initialize_plus_plus(x: torch.Tensor, n_clusters: int, p: int, sampler, weights=1.0,
+                          max_samples: int = 2**24 - 1, ws: Optional[_native.Workspace] = None) -> torch.Tensor:
+    """
+    k-means++ seeding as heat/cluster/batchparallelclustering.py:22-46 does it: the first centre
+    uniformly, every further one with probability proportional to ``weights * distance`` (the plain
+    distance to the closest centre chosen so far, not its square).  More than ``max_samples`` rows
+    are subsampled first because a categorical draw is limited to 2**24 categories.  The reference
+    recomputes the distances to all chosen centres in every step; the running minimum kept here is
+    the same number and needs one N x 1 distance column per step.
+    """
+    if p != 2:
+        raise NotImplementedError("only the Euclidean (p=2) seeding is built")
+    if x.shape[0] > max_samples:
+        sub = torch.tensor([sampler.randint(x.shape[0]) for _ in range(max_samples)], device=x.device)
+        x = x[sub].contiguous()
+    idxs = [sampler.randint(x.shape[0])]
+    dist = _dist_to_row(x, x[idxs[0]])
+    for i in range(1, n_clusters):
+        idxs.append(sampler.multinomial(weights * dist))
+        if i + 1 < n_clusters:
+            dist = torch.minimum(dist, _dist_to_row(x, x[idxs[-1]]))
+    return x[torch.tensor(idxs, device=x.device)]
+
+
+def _kmex(x: torch.Tensor, p: int, n_clusters: int, init: Union[str, torch.Tensor], max_iter: int, tol: float,
+          sampler=None, weights=1.0, ws: Optional[_native.Workspace] = None) -> Tuple[torch.Tensor, int]:
+    """
+    Lloyd iteration on a local matrix (heat/cluster/batchparallelclustering.py:49-88): an empty
+    cluster KEEPS its centre (unlike KMeans._update_centroids), the loop stops when
+    ``allclose(centers, previous, atol=tol)`` (rtol 1e-5).  Returns (centers, iterations run).
+    """
+    if p != 2:
+        raise NotImplementedError("only p=2 (k-means) is built")
+    _native._require_gpu(x)
+    ws = ws or _native.Workspace(x.device)
+    sampler = sampler or DeviceSampler(x.device)
+    if isinstance(init, torch.Tensor):
+        if init.shape != (n_clusters, x.shape[1]):
+            raise ValueError("if a torch tensor, init must have shape (n_clusters, n_features).")
+        centers = init.to(torch.float32).contiguous()
+    elif init == "++":
+        centers = _initialize_plus_plus(x, n_clusters, p, sampler, weights, ws=ws)
+    elif init == "random":
+        centers = x[torch.tensor([sampler.randint(x.shape[0]) for _ in range(n_clusters)], device=x.device)]
+    else:
+        raise ValueError("init must be a torch tensor with initial centers, string '++', or 'random'.")
+    n = x.shape[0]
+    lab = torch.empty((n,), dtype=torch.int32, device=x.device)
+    counts = torch.empty((n_clusters,), dtype=torch.int64, device=x.device)
+    means = torch.empty_like(centers)
+    it = 0
+    for it in range(max_iter):
+        _native.assign(x, centers, lab, None, ws)
+        _native.update(x, lab, means, counts, ws)
+        new = torch.where(counts.unsqueeze(1) > 0, means, centers)
+        done = bool(torch.allclose(new, centers, atol=tol))
+        centers = new
+        if done:
+            break
+    return centers, it + 1
+
+
+class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
+    """Checks and result attributes of heat/cluster/batchparallelclustering.py:99-331 at one rank."""
+
+    def __init__(self, p: int, n_clusters: int, init: str, max_iter: int, tol: float,
+                 random_state: Optional[int], n_procs_to_merge: Optional[int]):  # noqa: D107
+        if not isinstance(n_clusters, int):
+            raise TypeError(f"n_clusters must be int, but was {type(n_clusters)}")
+        if n_clusters <= 0:
+            raise ValueError(f"n_clusters must be positive, but was {n_clusters}")
+        if not isinstance(max_iter, int):
+            raise TypeError(f"max_iter must be int, but was {type(max_iter)}")
+        if max_iter <= 0:
+            raise ValueError(f"max_iter must be positive, but was {max_iter}")
+        if not isinstance(tol, float):
+            raise TypeError(f"tol must be float, but was {type(tol)}")
+        if tol <= 0:
+            raise ValueError(f"tol must be positive, but was {tol}")
+        if not isinstance(random_state, int) and random_state is not None:
+            raise TypeError(f"random_state must be int or None, but was {type(random_state)}")
+        if not isinstance(n_procs_to_merge, int) and n_procs_to_merge is not None:
+            raise TypeError(f"procs_to_merge must be int or None, but was {type(n_procs_to_merge)}")
+        if n_procs_to_merge is not None and n_procs_to_merge <= 1:
+            raise ValueError(f"If an integer, procs_to_merge must be > 1, but was {n_procs_to_merge}.")
+
+        self.n_clusters = n_clusters
+        self._init = init
+        self.max_iter = max_iter
+        self.tol = tol
+        self.random_state = random_state
+        self.n_procs_to_merge = n_procs_to_merge
+        if not (p == 1 or p == 2):
+            warn(
+                "p should be 1 (k-Medians) or 2 (k-Means). For other choice of p, we proceed as for p=2 and hope for the best.",
+                UserWarning,
+            )
+        self._p = p
+        self._cluster_centers = None
+        self._n_iter = None
+        self._functional_value = None
+        self._ws = None
+
+    @property
+    def cluster_centers_(self) -> DNDarray:
+        return self._cluster_centers
+
+    @property
+    def n_iter_(self):
+        return self._n_iter
+
+    @property
+    def functional_value_(self):
+        return self._functional_value
+
+    def _make_sampler(self, device: torch.device, rank: int = 0):
+        seed = None if self.random_state is None else self.random_state + rank
+        return DeviceSampler(device, seed)
+
+    @staticmethod
+    def _local_f32(x: DNDarray) -> torch.Tensor:
+        t = x.larray
+        if t.dtype == torch.float64:
+            raise NotImplementedError("the gfx950 kernels compute in float32; float64 input is not supported")
+        if t.dtype != torch.float32:
+            t = t.to(torch.float32)
+        return t.contiguous()
+
+    def fit(self, x: DNDarray):
+        """One rank: the local clustering is the global one (batchparallelclustering.py:177-269)."""
+        if not isinstance(x, DNDarray):
+            raise TypeError(f"input needs to be a ht.DNDarray, but was {type(x)}")
+        if not x.ndim == 2:
+            raise ValueError(f"input needs to be 2D, but was {x.ndim}D")
+        if x.split != 0:
+            raise ValueError(f"input needs to be split along the sample axis, but was split along {x.split}")
+        xt = self._local_f32(x)
+        if self._ws is None or self._ws.device != xt.device:
+            self._ws = _native.Workspace(xt.device)
+        centers, n_iter = _kmex(xt, self._p, self.n_clusters, self._init, self.max_iter, self.tol,
+                                self._make_sampler(xt.device, x.comm.rank), ws=self._ws)
+        self._cluster_centers = DNDarray(centers, (self.n_clusters, x.shape[1]), types.float32, None, x.device,
+                                         x.comm, True)
+        self._n_iter = n_iter
+        return self
+
+    def predict(self, x: DNDarray) -> DNDarray:
+        """(N, 1) int32 labels; sets ``functional_value_`` (batchparallelclustering.py:271-331)."""
+        if not isinstance(x, DNDarray):
+            raise TypeError(f"input needs to be a ht.DNDarray, but was {type(x)}")
+        if not x.ndim == 2:
+            raise ValueError(f"input needs to be 2D, but was {x.ndim}D")
+        if x.split != 0:
+            raise ValueError(f"input needs to be split along the sample axis, but was split along {x.split}")
+        if self._cluster_centers is None:
+            raise RuntimeError("fit needs to be called before predict")
+        if x.shape[1] != self._cluster_centers.shape[1]:
+            raise ValueError(
+                f"input needs to have {self._cluster_centers.shape[1]} features, but has {x.shape[1]}"
+            )
+        if self._p != 2:
+            raise NotImplementedError("only p=2 (k-means) is built")
+        xt = self._local_f32(x)
+        if self._ws is None or self._ws.device != xt.device:
+            self._ws = _native.Workspace(xt.device)
+        n = xt.shape[0]
+        lab = torch.empty((n, 1), dtype=torch.int32, device=xt.device)
+        d2 = torch.empty((n,), dtype=torch.float32, device=xt.device)
+        _native.assign(xt, self._cluster_centers.larray, lab.view(-1), d2, self._ws)
+        fv = torch.empty((), dtype=torch.float32, device=xt.device)
+        # ||x - C[labels]||_F ** 2 = sum of the squared distances to the closest centre
+        _native.functional_value(d2, fv, self._ws)
+        self._functional_value = fv.item()
+        return DNDarray(lab, (n, 1), types.int32, x.split, x.device, x.comm, x.balanced)
+
+
+class BatchParallelKMeans(_BatchParallelKCluster):
+    """Batch-parallel k-means (heat/cluster/batchparallelclustering.py:339-397)."""
+
+    def __init__(self, n_clusters: int = 8, init: str = "k-means++", max_iter: int = 300, tol: float = 1e-4,
+                 random_state: Optional[int] = None, n_procs_to_merge: Optional[int] = None):  # noqa: D107
+        if not isinstance(init, str):
+            raise TypeError(f"init must be str, but was {type(init)}")
+        if init == "k-means++":
+            _init = "++"
+        elif init == "random":
+            raise NotImplementedError(
+                "random initialization for batch parallel k-means is currently not supported due to instable behaviour of the algorithm. Use init='k-means++' instead."
+            )
+        else:
+            raise ValueError(f"init must be 'k-means++' or 'random', but was {init}")
+        super().__init__(p=2, n_clusters=n_clusters, init=_init, max_iter=max_iter, tol=tol,
+                         random_state=random_state, n_procs_to_merge=n_procs_to_merge)
+        self.init = init

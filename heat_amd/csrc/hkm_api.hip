@@ -227,6 +227,44 @@ int hkm_functional_value_f32(const float* min_d2, int64_t N, float* out, void* w
     return launch_sum_min_d2(min_d2, N, out, w.red, 2, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_min_dist_sum_f32(const float* min_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
+                         void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if ((!min_d2 && N > 0) || !out) return fail(HKM_EINVAL, "NULL pointer argument");
+    const size_t need = carve(nullptr, N, 1, 1, HKM_WS_ASSIGN).total;
+    int rc = check_ws(ws, ws_bytes, need);
+    if (rc) return rc;
+    const Workspace w = carve(ws, N, 1, 1, HKM_WS_ASSIGN);
+    return launch_sum_min_d2(min_d2, N, out, w.red, 3, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_sample_select_f32(const float* min_d2, const float* u, int64_t N, const float* cost,
+                          float oversampling, int64_t* idx, int64_t cap, int64_t* count, void* ws,
+                          size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (cap < 0) return fail(HKM_EINVAL, "cap = %lld is negative", (long long)cap);
+    if (!(oversampling > 0.f)) return fail(HKM_EINVAL, "oversampling = %g must be > 0", double(oversampling));
+    if (N > 0 && (!min_d2 || !u)) return fail(HKM_EINVAL, "NULL pointer argument");
+    if (!cost || !count || (cap > 0 && !idx)) return fail(HKM_EINVAL, "NULL pointer argument");
+    const size_t need = carve(nullptr, N, 1, 1, HKM_WS_ASSIGN).total;
+    int rc = check_ws(ws, ws_bytes, need);
+    if (rc) return rc;
+    const Workspace w = carve(ws, N, 1, 1, HKM_WS_ASSIGN);
+    return launch_select(min_d2, u, N, cost, oversampling, idx, cap, count, w.red,
+                         static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* counts,
+                         void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
+    if ((N > 0 && !labels) || !counts) return fail(HKM_EINVAL, "NULL pointer argument");
+    return launch_label_counts(labels, N, K, counts, static_cast<hipStream_t>(hip_stream));
+}
+
 int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                   int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, void* hip_stream) {
     g_err[0] = 0;

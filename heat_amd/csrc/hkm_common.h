@@ -92,6 +92,10 @@ int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, i
 int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                  int32_t D, float* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, float gauss,
                  hipStream_t st);
+int launch_select(const float* d2, const float* u, int64_t N, const float* cost, float os,
+                  int64_t* idx, int64_t cap, int64_t* count, double* red, hipStream_t st);
+int launch_label_counts(const int32_t* labels, int64_t N, int32_t K, int64_t* counts,
+                        hipStream_t st);
 int launch_widen(const int32_t* in, int64_t N, int64_t* out, hipStream_t st);
 
 int num_cus();

@@ -231,6 +231,7 @@ int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32
 // mode 0: sum of (a[i]-b[i])^2 with the square taken in fp32 (heat/cluster/kmeans.py:141)
 // mode 1: sum of v[i]                      (sum of clamped squared distances)
 // mode 2: sum of sqrtf(v[i])^2, then (sqrtf(total))^2   (heat/cluster/_kcluster.py:367-368)
+// mode 3: sum of sqrtf(v[i])               (clustering cost of k-means||, _kcluster.py:163-170,312-316)
 __device__ __forceinline__ double block_sum_fixed(double v, double* sh) {
     const int tid = threadIdx.x;
     sh[tid] = v;
@@ -275,6 +276,8 @@ __global__ __launch_bounds__(256) void sum_partial_kernel(const float* __restric
         if (mode == 2) {
             const float r = sqrtf(x);
             x = r * r;
+        } else if (mode == 3) {
+            x = sqrtf(x);
         }
         acc += double(x);
     }

@@ -134,3 +134,20 @@ def config5(scale: float = 1.0) -> Workload:
 
 
 CONFIGS = {"c1": config1, "c2": config2, "c3": config3, "c4": config4, "c5": config5}
+
+
+def spherical_dataset(num_samples_cluster: int, radius: float = 1.0, offset: float = 4.0,
+                      dtype: torch.dtype = torch.float32, seed: int = 1) -> torch.Tensor:
+    """
+    Four balls of ``num_samples_cluster`` points each, centred on the space diagonal of R^3 at
+    (+-offset) and (+-2 offset) in every coordinate: the shape of the data set the reference's
+    clustering tests use (heat/utils/data/spherical.py:7-55).  The same points (polar coordinates
+    with uniform radius and angles) are shifted to all four centres.
+    """
+    gen = torch.Generator().manual_seed(int(seed))
+    r = torch.rand(num_samples_cluster, generator=gen) * radius
+    theta = torch.rand(num_samples_cluster, generator=gen) * 3.1415
+    phi = torch.rand(num_samples_cluster, generator=gen) * 2 * 3.1415
+    pts = torch.stack((r * theta.sin() * phi.cos(), r * theta.sin() * phi.sin(), r * theta.cos()), dim=1)
+    data = torch.cat([pts + s * offset for s in (1.0, 2.0, -1.0, -2.0)], dim=0)
+    return data.to(dtype)

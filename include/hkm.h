@@ -122,6 +122,29 @@ int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_
 int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                      int32_t D, float* out, int64_t ldo, int32_t metric, float sigma, void* hip_stream);
 
+/*
+ * Pieces of the k-means|| initialisation (heat/cluster/_kcluster.py:146-247, 283-350); the distance
+ * work itself is hkm_assign_f32 with its min_d2 output.
+ *
+ * hkm_min_dist_sum_f32: *out = sum_i sqrt(min_d2[i]) (fp64 accumulation, fixed order): the
+ *   clustering cost `distance.min(axis=1).sum()` of _kcluster.py:163-170 and :312-316.
+ *   ws as for hkm_functional_value_f32.
+ * hkm_sample_select_f32: row i is a candidate iff u[i] <= (oversampling * sqrt(min_d2[i])) /
+ *   max(*cost, 1e-12) in fp32 (_kcluster.py:314-322: `where(sample <= prob)`); the selected row
+ *   indices are written to idx in ascending order (at most cap of them) and their number, which may
+ *   exceed cap, to *count.  cost and count are device pointers, no host synchronisation.
+ *   ws needs hkm_workspace_bytes(N, 1, 1, HKM_WS_ASSIGN) bytes.
+ * hkm_label_counts_i64: counts[k] = #{i : labels[i] == k}, the candidate weights of
+ *   _kcluster.py:206-208; labels outside [0, K) are ignored.
+ */
+int hkm_min_dist_sum_f32(const float* min_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
+                         void* hip_stream);
+int hkm_sample_select_f32(const float* min_d2, const float* u, int64_t N, const float* cost,
+                          float oversampling, int64_t* idx, int64_t cap, int64_t* count, void* ws,
+                          size_t ws_bytes, void* hip_stream);
+int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* counts,
+                         void* hip_stream);
+
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 

@@ -37,6 +37,14 @@ Pins (what each function is checked against, see tests/test_oracle_pins.py):
   End-to-end KMeans numerics are not pinned by any value stored in the reference
   (``tests/cluster/test_kmeans.py`` asserts types and shapes only): for the composed loop the parity
   statement rests on the per-function pins above plus these closed forms.
+* centroid_sampling_helper / kmeans_parallel_init / initialize_plus_plus / kmex (k-means||
+  initialisation and its k-means++ reclustering): closed forms (probabilities sum to the
+  oversampling factor, so the expected number of new candidates per round equals it; a row at
+  distance 0 is never drawn; with a huge oversampling factor every row at non-zero distance is
+  drawn), the D-sampling law of k-means++ on a hand-made case, the empty-cluster-keeps-its-centre
+  rule and the allclose stop of ``_kmex``, and recovery of well-separated blobs.  **Parity unpinned**
+  for the random draws themselves: the reference takes them from Heat's counter-based generator and
+  from torch's unseeded global generator, and stores no seeded result anywhere.
 """
 
 from __future__ import annotations
@@ -48,6 +56,105 @@ import numpy as np
 import torch
 
 INT64_MAX = 9223372036854775807
+
+
+class CpuSampler:
+    """
+    Random draws for the initialisers from one seeded torch CPU generator, with the interface the
+    product's sampler has (randint / uniform / multinomial).  ``device`` only says where ``uniform``
+    puts its result, the numbers are always generated on the CPU, so two implementations constructed
+    with the same seed see the same draws.  The categorical draw is an inverse-CDF lookup in fp64 so
+    that it depends on the weights only through their cumulative sums.
+    """
+
+    def __init__(self, seed: int, device="cpu"):
+        self._gen = torch.Generator(device="cpu")
+        self._gen.manual_seed(int(seed))
+        self.device = torch.device(device)
+
+    def randint(self, high: int) -> int:
+        return int(torch.randint(0, int(high), (1,), generator=self._gen).item())
+
+    def uniform(self, n: int) -> torch.Tensor:
+        return torch.rand((int(n),), generator=self._gen, dtype=torch.float32).to(self.device)
+
+    def multinomial(self, weights: torch.Tensor) -> int:
+        w = weights.detach().to("cpu", torch.float64)
+        cdf = torch.cumsum(w, 0)
+        r = torch.rand((1,), generator=self._gen, dtype=torch.float64) * cdf[-1]
+        i = int(torch.searchsorted(cdf, r, right=True).item())
+        return min(i, w.numel() - 1)
+
+
+class RecordingSampler(CpuSampler):
+    """A CpuSampler that keeps every draw (and the weights of every categorical draw) in ``tape``."""
+
+    def __init__(self, seed: int):
+        super().__init__(seed, "cpu")
+        self.tape = []
+
+    def randint(self, high: int) -> int:
+        r = super().randint(high)
+        self.tape.append(("randint", int(high), r))
+        return r
+
+    def uniform(self, n: int) -> torch.Tensor:
+        u = super().uniform(n)
+        self.tape.append(("uniform", int(n), u))
+        return u
+
+    def multinomial(self, weights: torch.Tensor) -> int:
+        i = super().multinomial(weights)
+        self.tape.append(("multinomial", weights.detach().clone(), i))
+        return i
+
+
+class ReplaySampler:
+    """
+    Replays the tape of a RecordingSampler to a second implementation, so both walk the same random
+    path even where a draw sits close to a decision boundary.  Each call must be the same kind of draw
+    with the same argument; for a categorical draw the weights must agree with the recorded ones to
+    ``rtol`` relative plus ``atol_frac`` of the largest weight.  The absolute part is there for the
+    rows already chosen as centres: their distance is exactly 0 in a direct evaluation, while
+    ``torch.cdist`` switches to a quadratic expansion above 25 rows and returns about
+    sqrt(eps) * |x| instead, which is then multiplied by a weight of up to thousands.
+    """
+
+    def __init__(self, tape, device="cpu", rtol: float = 1e-3, atol_frac: float = 1e-2):
+        self.tape = list(tape)
+        self.pos = 0
+        self.device = torch.device(device)
+        self.rtol, self.atol_frac = rtol, atol_frac
+
+    def _next(self, kind: str):
+        assert self.pos < len(self.tape), f"more draws than recorded (next would be {kind})"
+        rec = self.tape[self.pos]
+        self.pos += 1
+        assert rec[0] == kind, f"draw {self.pos - 1}: recorded {rec[0]}, asked for {kind}"
+        return rec
+
+    def randint(self, high: int) -> int:
+        rec = self._next("randint")
+        assert rec[1] == int(high), (rec[1], high)
+        return rec[2]
+
+    def uniform(self, n: int) -> torch.Tensor:
+        rec = self._next("uniform")
+        assert rec[1] == int(n), (rec[1], n)
+        return rec[2].to(self.device)
+
+    def multinomial(self, weights: torch.Tensor) -> int:
+        rec = self._next("multinomial")
+        w = weights.detach().to("cpu", torch.float32)
+        ref = rec[1].to(torch.float32)
+        assert w.shape == ref.shape, (w.shape, ref.shape)
+        tol = self.rtol * ref.abs() + self.atol_frac * float(ref.abs().max())
+        bad = (w - ref).abs() > tol
+        assert not bool(bad.any()), f"categorical weights differ at {int(bad.sum())} of {w.numel()} entries"
+        return rec[2]
+
+    def exhausted(self) -> bool:
+        return self.pos == len(self.tape)
 
 
 # --------------------------------------------------------------------------------------------------
@@ -366,3 +473,98 @@ __all__ = [
     "brute_force_d2",
     "sse",
 ]
+
+
+# --------------------------------------------------------------------------------------------------
+# k-means|| initialisation and its k-means++ reclustering
+# --------------------------------------------------------------------------------------------------
+def _min_distance(x: torch.Tensor, centroids: torch.Tensor, chunk: int = 1 << 15) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``cdist(x, centroids, quadratic_expansion=True)`` then min / argmin over axis 1, in row chunks."""
+    vals, idxs = [], []
+    for i0 in range(0, x.shape[0], chunk):
+        v, i = torch.min(euclidian_fast(x[i0 : i0 + chunk], centroids), dim=1)
+        vals.append(v)
+        idxs.append(i)
+    return torch.cat(vals), torch.cat(idxs)
+
+
+def centroid_sampling_helper(x: torch.Tensor, centroids: torch.Tensor, oversampling: float, num_iters: int,
+                             sampler) -> torch.Tensor:
+    """Follows heat/cluster/_kcluster.py:283-350 at one rank."""
+    for _ in range(num_iters):
+        min_distance, _i = _min_distance(x, centroids)
+        min_dist_sum = torch.maximum(min_distance.sum(), torch.tensor(1e-12))
+        prob = oversampling * min_distance / min_dist_sum
+        sample = sampler.uniform(x.shape[0])
+        idx = torch.where(sample <= prob)[0]
+        centroids = torch.cat((centroids, x[idx].reshape(-1, x.shape[1])), dim=0)
+    return centroids
+
+
+def initialize_plus_plus(x: torch.Tensor, n_clusters: int, sampler, weights=1.0) -> torch.Tensor:
+    """Follows heat/cluster/batchparallelclustering.py:22-46 (p = 2, no subsampling)."""
+    idxs = torch.zeros(n_clusters, dtype=torch.long)
+    idxs[0] = sampler.randint(x.shape[0])
+    for i in range(1, n_clusters):
+        dist = torch.cdist(x, x[idxs[:i]], p=2)
+        dist = torch.min(dist, dim=1)[0]
+        idxs[i] = sampler.multinomial(weights * dist)
+    return x[idxs]
+
+
+def kmex(x: torch.Tensor, n_clusters: int, init, max_iter: int, tol: float, sampler=None,
+         weights=1.0) -> Tuple[torch.Tensor, int]:
+    """Follows heat/cluster/batchparallelclustering.py:49-88 (p = 2)."""
+    if isinstance(init, torch.Tensor):
+        if init.shape != (n_clusters, x.shape[1]):
+            raise ValueError("if a torch tensor, init must have shape (n_clusters, n_features).")
+        centers = init.clone()
+    elif init == "++":
+        centers = initialize_plus_plus(x, n_clusters, sampler, weights)
+    elif init == "random":
+        centers = x[torch.tensor([sampler.randint(x.shape[0]) for _ in range(n_clusters)])]
+    else:
+        raise ValueError("init must be a torch tensor with initial centers, string '++', or 'random'.")
+    it = 0
+    for it in range(max_iter):
+        dist = torch.cdist(x, centers, p=2)
+        labels = torch.argmin(dist, dim=1)
+        centers_old = centers.clone()
+        for i in range(n_clusters):
+            if (labels == i).any():
+                centers[i] = torch.mean(x[labels == i], dim=0)
+        if torch.allclose(centers, centers_old, atol=tol):
+            break
+    return centers, it + 1
+
+
+def kmeans_parallel_init(x: torch.Tensor, n_clusters: int, oversampling: float, iter_multiplier: float,
+                         max_iter: int, tol: float, sampler) -> Tuple[torch.Tensor, dict]:
+    """
+    ``init="probability_based"`` of heat/cluster/_kcluster.py:146-247 at one rank.  Returns the
+    (K, D) centres and a dict with the intermediate quantities (number of rounds, candidates,
+    weights) for step-wise comparisons.
+    """
+    n = x.shape[0]
+    init_idx = sampler.randint(max(n - 1, 1))
+    init_centroids = x[init_idx : init_idx + 1].clone()
+    init_min_distance, _i = _min_distance(x, init_centroids)
+    init_cost = init_min_distance.sum()
+    num_iters = max(1, int(iter_multiplier * torch.log(init_cost))) if float(init_cost) > 0 else 1
+    centroids = centroid_sampling_helper(x, init_centroids, oversampling, num_iters, sampler)
+    if centroids.shape[0] <= n_clusters:
+        oversampling = 10 * oversampling
+        centroids = centroid_sampling_helper(x, init_centroids, oversampling, num_iters, sampler)
+    if centroids.shape[0] <= n_clusters:
+        raise ValueError(
+            f"The parameter oversampling={oversampling} and/or iter_multiplier={iter_multiplier} "
+            "are chosen too small for the initialization of cluster centers."
+        )
+    _d, final_idx = _min_distance(x, centroids)
+    weights = torch.zeros(centroids.shape[0])
+    for i in range(centroids.shape[0]):
+        weights[i] = torch.sum(final_idx == i)
+    centers, n_it = kmex(centroids, n_clusters, "++", max_iter, tol, sampler, weights)
+    info = {"init_idx": init_idx, "init_cost": float(init_cost), "num_iters": num_iters,
+            "candidates": centroids, "weights": weights, "kmex_iters": n_it, "oversampling": oversampling}
+    return centers, info

@@ -159,7 +159,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) >= 12
+    assert len(names) >= 15
     for name in names:
         assert hasattr(lib, name), name
         assert name in _native.SIGNATURES, f"{name} has no ctypes signature"
@@ -217,6 +217,15 @@ def test_argument_validation_happens_on_the_host():
     assert lib.hkm_pairwise_f32(good, 4, 3, good, 4, 3, 3, good, 4, _native.METRIC_GAUSS, 0.0, None) == _native.HKM_EINVAL
     assert "sigma" in err()
     assert lib.hkm_widen_labels_i64(None, 4, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_min_dist_sum_f32(good, -1, good, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_min_dist_sum_f32(good, 8, good, None, 0, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_sample_select_f32(good, good, 8, good, 0.0, good, 4, good, ws, big, None) == _native.HKM_EINVAL
+    assert "oversampling" in err()
+    assert lib.hkm_sample_select_f32(good, None, 8, good, 2.0, good, 4, good, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_sample_select_f32(good, good, 8, good, 2.0, good, -4, good, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_sample_select_f32(good, good, 8, good, 2.0, good, 4, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_label_counts_i64(good, 8, 0, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_label_counts_i64(None, 8, 4, good, None) == _native.HKM_EINVAL
     assert lib.hkm_functional_value_f32(good, -1, good, ws, big, None) == _native.HKM_EINVAL
     # zero-sized problems succeed without touching the device
     assert lib.hkm_widen_labels_i64(good, 0, good, None) == _native.HKM_OK
@@ -229,3 +238,38 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_native, "_LIB_PATH", "/nonexistent/libhkm.so")
     with pytest.raises(ImportError, match="no CPU fallback"):
         _native.load()
+
+
+def test_batchparallel_kmeans_surface():
+    # tests/cluster/test_batchparallelclustering.py:46-84,135-190 of the reference (constructor part)
+    from heat_amd.cluster.batchparallelclustering import _BatchParallelKCluster
+
+    bp = ht.cluster.BatchParallelKMeans()
+    assert ht.is_estimator(bp) and ht.is_clusterer(bp)
+    params = bp.get_params()
+    assert params == {"n_clusters": 8, "init": "k-means++", "max_iter": 300, "tol": 1e-4, "random_state": None,
+                      "n_procs_to_merge": None}
+    params["n_clusters"] = 10
+    params["n_procs_to_merge"] = 4
+    bp.set_params(**params)
+    assert bp.n_clusters == 10
+    with pytest.raises(TypeError):
+        _BatchParallelKCluster(2, 10, "++", 100, 1e-2, random_state=3.14, n_procs_to_merge=None)
+    with pytest.warns(UserWarning):
+        _BatchParallelKCluster(3, 10, "++", 100, 1e-2, random_state=None, n_procs_to_merge=None)
+    with pytest.raises(TypeError):
+        _BatchParallelKCluster(2, 10, "++", 100, 1e-2, random_state=None, n_procs_to_merge=2.7183)
+    with pytest.raises(ValueError):
+        _BatchParallelKCluster(2, 10, "++", 100, 1e-2, random_state=None, n_procs_to_merge=1)
+    for kwargs, exc in (({"n_clusters": -1}, ValueError), ({"n_clusters": "abc"}, TypeError),
+                        ({"max_iter": -10}, ValueError), ({"max_iter": 0.1}, TypeError),
+                        ({"tol": -0.5}, ValueError), ({"tol": "abc"}, TypeError), ({"init": "abc"}, ValueError),
+                        ({"init": 3.14}, TypeError), ({"init": "random"}, NotImplementedError)):
+        with pytest.raises(exc):
+            ht.cluster.BatchParallelKMeans(**kwargs)
+    with pytest.raises(TypeError):
+        bp.fit("abc")
+    with pytest.raises(RuntimeError):  # host data: refused, not computed on the CPU
+        ht.cluster.BatchParallelKMeans(n_clusters=2).fit(ht.array(torch.rand(16, 2), split=0))
+    with pytest.raises(RuntimeError):
+        ht.cluster.KMeans(n_clusters=2, init="probability_based").fit(ht.array(torch.rand(16, 2), split=0))

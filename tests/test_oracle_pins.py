@@ -230,3 +230,107 @@ def test_label_agreement_excuses_only_numerical_ties():
     a = torch.tensor([0, 1])
     assert orc.label_agreement(x, c, a, torch.tensor([1, 1]))["n_unexcused"] == 0  # row 0: near tie
     assert orc.label_agreement(x, c, a, torch.tensor([2, 1]))["n_unexcused"] == 1  # row 0: wrong
+
+
+# ---- k-means|| initialisation -------------------------------------------------------------------
+class _RecordingSampler(orc.CpuSampler):
+    """Keeps what the initialisers hand to the categorical draw."""
+
+    def __init__(self, seed, first=None):
+        super().__init__(seed)
+        self.first = first
+        self.seen = []
+
+    def randint(self, high):
+        r = super().randint(high)
+        return r if self.first is None else self.first
+
+    def multinomial(self, weights):
+        self.seen.append(weights.clone())
+        return super().multinomial(weights)
+
+
+def test_sampling_round_closed_forms():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((20000, 3), generator=g)
+    x[7] = x[0]  # a duplicate of the first centroid: distance 0, probability 0
+    c0 = x[0:1].clone()
+    # probabilities sum to the oversampling factor => the expected number of rows drawn per round is
+    # the factor itself (variance below it): 40 independent single rounds
+    counts = [orc.centroid_sampling_helper(x, c0, 8.0, 1, orc.CpuSampler(s)).shape[0] - 1 for s in range(40)]
+    assert abs(np.mean(counts) - 8.0) < 4 * np.sqrt(8.0 / 40)
+    # new candidates are rows of x, appended in ascending row order after the old ones
+    cand = orc.centroid_sampling_helper(x, c0, 50.0, 1, orc.CpuSampler(1))
+    rows = [int(torch.where((x == r).all(1))[0][0]) for r in cand[1:]]
+    assert rows == sorted(rows) and len(set(rows)) == len(rows) and torch.equal(cand[0], x[0])
+    # with a factor beyond sum/min every row at non-zero distance is drawn, the two rows at distance
+    # zero are not
+    cand = orc.centroid_sampling_helper(x, c0, 1e12, 1, orc.CpuSampler(2))
+    assert cand.shape[0] - 1 == x.shape[0] - 2
+    # all rows equal: cost 0 is clamped to 1e-12, nothing is drawn, nothing divides by zero
+    same = torch.ones((100, 3))
+    assert orc.centroid_sampling_helper(same, same[:1].clone(), 4.0, 3, orc.CpuSampler(3)).shape[0] == 1
+
+
+def test_plus_plus_draws_proportional_to_weight_times_distance():
+    # points on a line at 0, 1, 3, 7; first centre forced to row 0: the categorical draw must see
+    # weights * DISTANCE (not its square) = w * [0, 1, 3, 7]; after row 3 joins: w * [0, 1, 3, 0]
+    x = torch.tensor([[0.0], [1.0], [3.0], [7.0]])
+    w = torch.tensor([1.0, 2.0, 1.0, 0.5])
+
+    class Forced(_RecordingSampler):
+        def multinomial(self, weights):
+            self.seen.append(weights.clone())
+            return 3 if len(self.seen) == 1 else 2
+
+    smp = Forced(0, first=0)
+    c = orc.initialize_plus_plus(x, 3, smp, w)
+    assert torch.allclose(smp.seen[0], w * torch.tensor([0.0, 1.0, 3.0, 7.0]))
+    assert torch.allclose(smp.seen[1], w * torch.tensor([0.0, 1.0, 3.0, 0.0]))
+    assert torch.equal(c, x[[0, 3, 2]])
+    # the inverse-CDF draw follows the weights: frequencies over many draws
+    smp = orc.CpuSampler(11)
+    wts = torch.tensor([0.0, 1.0, 3.0, 0.0, 4.0])
+    freq = np.bincount([smp.multinomial(wts) for _ in range(8000)], minlength=5) / 8000.0
+    assert freq[0] == 0 and freq[3] == 0 and np.allclose(freq, [0, 0.125, 0.375, 0, 0.5], atol=0.02)
+
+
+def test_kmex_lloyd_rules():
+    g = torch.Generator().manual_seed(9)
+    x = torch.cat([torch.randn((300, 2), generator=g) + 6.0, torch.randn((300, 2), generator=g) - 6.0])
+    # an empty cluster keeps its centre (KMeans._update_centroids would zero it)
+    far = torch.tensor([[6.0, 6.0], [-6.0, -6.0], [500.0, 500.0]])
+    c, n_it = orc.kmex(x, 3, far.clone(), 50, 1e-4)
+    assert torch.equal(c[2], far[2])
+    assert torch.allclose(c[0], x[:300].mean(0), atol=1e-5) and torch.allclose(c[1], x[300:].mean(0), atol=1e-5)
+    assert n_it == 2  # one step moves the centres, the second finds them unchanged and stops
+    # without empty clusters it is Lloyd's iteration: same centres as the KMeans restatement
+    c0 = x[[0, 1, 300, 301]].clone()
+    c_kmex, n_kmex = orc.kmex(x, 4, c0.clone(), 100, 1e-7)
+    ref = orc.kmeans_fit(x, c0.clone(), max_iter=n_kmex, tol=None)
+    assert torch.allclose(c_kmex, ref["cluster_centers"], atol=1e-5)
+    with pytest.raises(ValueError):
+        orc.kmex(x, 3, torch.zeros((2, 2)), 5, 1e-4)
+    with pytest.raises(ValueError):
+        orc.kmex(x, 3, "farthest", 5, 1e-4)
+
+
+def test_kmeans_parallel_init_composition():
+    g = torch.Generator().manual_seed(21)
+    cent = (torch.rand((6, 5), generator=g) - 0.5) * 40
+    x = cent[torch.randint(0, 6, (6000,), generator=g)] + torch.randn((6000, 5), generator=g)
+    centers, info = orc.kmeans_parallel_init(x, 6, 12.0, 1.0, 100, 1e-4, orc.CpuSampler(4))
+    cost = float(torch.cdist(x, x[info["init_idx"]][None]).sum())
+    assert abs(info["init_cost"] - cost) <= 1e-4 * cost
+    assert info["num_iters"] == max(1, int(np.log(info["init_cost"])))
+    cand, w = info["candidates"], info["weights"]
+    assert cand.shape[0] > 6 and float(w.sum()) == 6000.0
+    # every candidate is a row of x; the weights are the sizes of the candidates' Voronoi cells
+    assert all(bool((x == r).all(1).any()) for r in cand)
+    lab = torch.cdist(x, cand).argmin(1)
+    assert (torch.bincount(lab, minlength=cand.shape[0]).float() - w).abs().sum() <= 4  # ties only
+    assert centers.shape == (6, 5) and torch.isfinite(centers).all()
+    # too few candidates even after the automatic x10: the reference's ValueError
+    tiny = torch.ones((50, 2))
+    with pytest.raises(ValueError):
+        orc.kmeans_parallel_init(tiny, 3, 2.0, 1.0, 10, 1e-4, orc.CpuSampler(0))
