@@ -5,11 +5,15 @@ Benchmark of the k-means Lloyd step on one MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3] [--no-cpu-baseline]
 
 A step is one Lloyd iteration (labels, per-cluster means, centroid shift) over the whole synthetic
-data set, issued exactly as KMeans.fit issues it: one hkm_lloyd_step_f32 call, then the host reads
-the 4-byte shift.  Inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+data set, issued exactly as KMeans.fit issues it (heat_amd.cluster._lloyd.LloydLoop): one
+hkm_lloyd_step_f32 call per iteration, the host reads every 4-byte shift, and the next step is
+already enqueued while it does.  Inputs are resident in HBM before the timed region.  Prints ONE
+JSON line.  The default warm-up is 30 steps because a kernel launched on an idle device runs up to
+30 % longer during the first ~25 ms of load than afterwards (measured per launch with rocprofv3).
 
 value      points*iterations / s over the timed region (wall clock, synchronised both sides)
-roofline   the dominant kernel (fused distance+argmin) timed with events on the launch stream:
+roofline   the dominant kernel (fused distance+argmin; for the one-sweep shapes the whole step, whose
+           other launches take some 15 us) timed with events on the launch stream:
            algorithmic flops 2*N*K*D (MFMA-bound shapes) or bytes N*(4D+4) (HBM-bound shapes) per
            launch divided by its mean duration
 cpu_baseline  the CPU restatement of the reference's op sequence (oracle/, torch CPU, all host
@@ -34,8 +38,8 @@ CPU_SAMPLE_DIV = {"c1": 1, "c2": 16, "c3": 32, "c4": 256, "c5": 128}
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink N (testing only; invalidates the figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -62,7 +66,8 @@ def main() -> int:
     n, d = w.x.shape
     k = w.k
     x = w.x.to(dev)
-    kernel = _native.assign_kernel_name(n, d, k)
+    kernel = _native.assign_kernel_name(n, d, k) if args.config == "c2" else _native.lloyd_kernel_name(n, d, k)
+    kernel = kernel.replace("+update", "")
     ws = _native.Workspace(dev)
     lab = torch.empty((n,), dtype=torch.int32, device=dev)
 
@@ -72,40 +77,44 @@ def main() -> int:
         y = w.y.to(dev)
         md = torch.empty((n,), dtype=torch.float32, device=dev)
 
-        def step():
-            _native.assign(x, y, lab, md, ws)
+        def steps(count):
+            for _ in range(count):
+                _native.assign(x, y, lab, md, ws)
 
         def kernel_only():
             _native.assign(x, y, lab, md, ws)
     else:
-        c_cur = w.init.to(dev).clone()
-        c_nxt = torch.empty_like(c_cur)
-        shift = torch.zeros((), dtype=torch.float32, device=dev)
-        state = {"cur": c_cur, "nxt": c_nxt}
+        # the loop of KMeans.fit: per iteration one hkm_lloyd_step_f32 and a 4-byte read of the shift
+        # (tol = -1: the host looks at every shift, as with tol = 0, but never stops early)
+        from heat_amd.cluster._lloyd import LloydLoop
 
-        def step():
-            _native.lloyd_step(x, state["cur"], state["nxt"], lab, shift, None, ws)
-            state["cur"], state["nxt"] = state["nxt"], state["cur"]
-            shift.item()  # the convergence test of KMeans.fit: a 4-byte read per iteration
+        loop = LloydLoop(x, w.init.to(dev), ws)
+        shift = torch.zeros((), dtype=torch.float32, device=dev)
+        c_tmp = torch.empty_like(loop.centers)
+
+        def steps(count):
+            assert loop.run(count, -1.0) == count
 
         def kernel_only():
-            _native.assign(x, state["cur"], lab, None, ws)
+            if kernel.startswith("lloyd_"):
+                # one-sweep shapes: the step IS the dominant kernel plus a few finishing launches of
+                # some 10 us; timed as a whole, without the host read
+                _native.lloyd_step(x, loop.centers, c_tmp, lab, shift, None, ws)
+            else:
+                _native.assign(x, loop.centers, lab, None, ws)
 
-    for _ in range(args.warmup):
-        step()
+    steps(args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    steps(args.steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
     # dominant kernel alone, event-timed on the stream it is launched on (torch's current stream)
-    fused_small_d = kernel == "valu_fused"
     for _ in range(args.steps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        step() if fused_small_d else kernel_only()
+        kernel_only()
         e1.record()
         torch.cuda.synchronize()
         ev_ms.append(e0.elapsed_time(e1))

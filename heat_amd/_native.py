@@ -26,6 +26,7 @@ SIGNATURES = {
     "hkm_last_error": (c_char_p, []),
     "hkm_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int32]),
     "hkm_assign_kernel_name": (c_char_p, [c_int64, c_int32, c_int32]),
+    "hkm_lloyd_kernel_name": (c_char_p, [c_int64, c_int32, c_int32]),
     "hkm_assign_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_update_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
@@ -121,6 +122,10 @@ def assign_kernel_name(n: int, d: int, k: int) -> str:
     return load().hkm_assign_kernel_name(n, d, k).decode()
 
 
+def lloyd_kernel_name(n: int, d: int, k: int) -> str:
+    return load().hkm_lloyd_kernel_name(n, d, k).decode()
+
+
 def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optional[torch.Tensor],
            ws: Workspace) -> None:
     _require_gpu(x, c, labels, min_d2)
@@ -145,7 +150,11 @@ def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: O
 
 def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: torch.Tensor,
                shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace) -> None:
-    _require_gpu(x, c, c_new, labels, shift, sse)
+    _require_gpu(x, c, c_new, labels, sse)
+    if not (shift.is_cuda or shift.is_pinned()):
+        # a pinned host scalar is written by the kernel itself over the bus: no copy engine, no
+        # extra stream operation between two steps
+        raise RuntimeError("shift must live on the GPU or in pinned host memory")
     n, d = x.shape
     k = c.shape[0]
     flags = WS_LLOYD | (WS_SSE if sse is not None else 0)

@@ -11,6 +11,7 @@ from typing import Optional, Union
 import torch
 
 from .. import _native
+from ._lloyd import LloydLoop
 from ..core import types
 from ..core.dndarray import DNDarray
 from ..spatial import distance
@@ -76,19 +77,13 @@ class KMeans(_KCluster):
         dev = xt.device
         n, d = xt.shape
         k = self.n_clusters
-        c_cur = self._local_f32(self._cluster_centers).clone()
-        c_nxt = torch.empty_like(c_cur)
-        lab32 = torch.empty((n,), dtype=torch.int32, device=dev)
-        shift = torch.zeros((), dtype=torch.float32, device=dev)
-        ws = self._workspace(dev)
-
-        for _ in range(self.max_iter):
-            self._n_iter += 1
-            _native.lloyd_step(xt, c_cur, c_nxt, lab32, shift, None, ws)
-            c_cur, c_nxt = c_nxt, c_cur
-            # the reference evaluates ``inertia <= tol`` on the host every iteration (kmeans.py:143)
-            if self.tol is not None and shift.item() <= self.tol:
-                break
+        # the reference evaluates ``inertia <= tol`` on the host every iteration (kmeans.py:143); the
+        # loop keeps the next step enqueued while the host looks at the shift of the current one
+        loop = LloydLoop(xt, self._local_f32(self._cluster_centers), self._workspace(dev))
+        self._n_iter = loop.run(self.max_iter, self.tol)
+        if self._n_iter == 0:
+            raise ValueError(f"max_iter must be positive, but was {self.max_iter}")
+        c_cur, lab32, shift = loop.centers, loop.labels, loop.last_shift
 
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         _native.widen_labels(lab32, lab64)

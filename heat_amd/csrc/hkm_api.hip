@@ -45,6 +45,11 @@ AssignKind assign_kind(int32_t D, int32_t K) {
     return ASSIGN_MFMA_STREAM;
 }
 
+// the one-sweep MFMA step needs the centroids, fp64 accumulators and counts of a workgroup in LDS
+bool fused_eligible(int32_t D, int32_t K) {
+    return assign_kind(D, K) == ASSIGN_MFMA_RESIDENT && fused_lds_bytes(D, K) <= 160 * 1024;
+}
+
 static size_t cn_pad(int32_t K) { return (size_t(K) + 127) / 128 * 128; }
 
 Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
@@ -71,6 +76,11 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         w.part_cnt = reinterpret_cast<int32_t*>(take(size_t(g.S) * K * sizeof(int32_t)));
         w.counts = reinterpret_cast<int64_t*>(take(size_t(K) * sizeof(int64_t)));
         w.shift_part = reinterpret_cast<double*>(take((size_t(K) * D / 64 + 1) * sizeof(double)));
+    }
+    if ((flags & HKM_WS_LLOYD) == HKM_WS_LLOYD && fused_eligible(D, K)) {
+        w.fsum = reinterpret_cast<double*>(take(size_t(FUSED_MAX_GRID) * K * D * sizeof(double)));
+        w.fcnt = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * K * sizeof(int32_t)));
+        w.fflags = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * sizeof(int32_t)));
     }
     if (flags & HKM_WS_SSE) w.min_d2 = reinterpret_cast<float*>(take(size_t(N < 1 ? 1 : N) * sizeof(float)));
     w.total = off;
@@ -148,6 +158,19 @@ const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K) {
     }
 }
 
+const char* hkm_lloyd_kernel_name(int64_t N, int32_t D, int32_t K) {
+    (void)N;
+    if (D < 1 || K < 1) return "invalid";
+    if (small_eligible(D, K)) return "lloyd_small";
+    if (fused_eligible(D, K)) return "lloyd_mfma_resident";
+    switch (assign_kind(D, K)) {
+        case ASSIGN_VALU: return "valu+update";
+        case ASSIGN_MFMA_RESIDENT: return "mfma_resident+update";
+        case ASSIGN_MFMA_TILED: return "mfma_tiled+update";
+        default: return "mfma_stream+update";
+    }
+}
+
 int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                    int64_t ldc, int32_t* labels, float* min_d2, void* ws, size_t ws_bytes,
                    void* hip_stream) {
@@ -201,8 +224,17 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
         if ((rc = launch_small(X, N, D, ldx, C, K, D, labels, nullptr, w.small_part, sse ? 3 : 1, st))) return rc;
         return launch_small_finalize(w.small_part, small_grid(N, D, K), K, D, C, C_new, D, nullptr, shift, sse, st);
     }
-    if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;
-    if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
+    if (fused_eligible(D, K) && N > 0) {
+        // one sweep over X on the matrix cores: labels + fp64 per-cluster sums in LDS
+        if ((rc = launch_lloyd_mfma_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum,
+                                             w.fcnt, w.fflags, st)))
+            return rc;
+        if ((rc = launch_update_fused(X, N, D, ldx, labels, K, C_new, D, nullptr, w, fused_grid(N), C, shift, st)))
+            return rc;
+    } else {
+        if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;
+        if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
+    }
     if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
     return rc;
 }

@@ -207,6 +207,153 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// One-sweep Lloyd step for the resident shapes: the same persistent kernel, and once the labels of a
+// wave's points are final the point rows -- still in the B-operand registers -- are added to
+// per-workgroup fp64 accumulators in LDS with ds_add_f64.  X is read from HBM once per iteration.
+//
+// Atomic additions arrive in any order, so the sums are made ORDER-INDEPENDENT instead: every row is
+// first rounded to a multiple of q_i = 2^(E_i - 28), where 2^E_i bounds the row's largest
+// coordinate (taken from |x_i|^2, which the distance needs anyway), by (v + B_i) - B_i with
+// B_i = 1.5 * 2^52 * q_i.  All addends of a workgroup are then multiples of 2^(Emin - 28) and every
+// partial sum is below n_wg * 2^Emax, so as long as Emax - Emin <= 53 - 28 - ceil(log2 n_wg) every
+// addition is exact in fp64 and the result does not depend on the order.  The rounding keeps 28 bits
+// below the row's largest coordinate (error <= 2^-29 of it per addend).  A workgroup whose rows
+// violate the range condition (or hold inf / NaN) raises its flag; the step then falls back to the
+// two-pass update, whose kernels start by looking at the flags.
+// ------------------------------------------------------------------------------------------------
+static constexpr int FUSED_QBITS = 28;
+static constexpr int FUSED_THREADS = 768;
+
+template <int DP, int PB, bool VEC>
+__global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
+    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles,
+    double* __restrict__ fsum, int32_t* __restrict__ fcnt, int32_t* __restrict__ flags,
+    int range_bits) {
+    extern __shared__ __align__(16) float lds[];
+    constexpr int LDC = DP + 4;
+    constexpr int LDA = DP + 1;  // odd row stride (in doubles): rows of different clusters spread over the banks
+    constexpr int NJ = DP / 8;
+    const int KP = (K + 31) & ~31;
+    float* sC = lds;                                              // [KP][LDC]
+    double* sA = reinterpret_cast<double*>(lds + KP * LDC);       // [K][LDA]
+    int* sN = reinterpret_cast<int*>(sA + size_t(K) * LDA);       // [K] counts, then Emin, Emax
+    const int tid = threadIdx.x, nthr = blockDim.x;
+
+    for (int i = tid; i < KP * DP; i += nthr) {
+        const int r = i / DP, c = i - r * DP;
+        sC[r * LDC + c] = (r < K && c < D) ? -2.0f * C[int64_t(r) * ldc + c] : 0.f;
+    }
+    for (int r = tid; r < KP; r += nthr) {
+        float s = HKM_INF;
+        if (r < K) {
+            s = 0.f;
+            const float* c = C + int64_t(r) * ldc;
+            for (int d = 0; d < D; ++d) s = fmaf(c[d], c[d], s);
+        }
+        sC[r * LDC + DP] = s;
+        sC[r * LDC + DP + 1] = 1.0f;
+    }
+    for (int i = tid; i < K * LDA; i += nthr) sA[i] = 0.0;
+    for (int i = tid; i < K; i += nthr) sN[i] = 0;
+    if (tid == 0) {
+        sN[K] = 0x7fffffff;
+        sN[K + 1] = -0x7fffffff;
+    }
+    __syncthreads();
+
+    const int lane = tid & 63, wave = tid >> 6, nw = nthr >> 6;
+    const int p = lane & 31, h = lane >> 5;
+    const int ncb = KP >> 5;
+    const int64_t tile_rows = int64_t(nw) * PB * 32;
+    int emin = 0x7fffffff, emax = -0x7fffffff;
+
+    floatx4 bn[PB][NJ];
+    auto fetch = [&](int64_t tile) {
+        const int64_t row0 = tile * tile_rows + wave * (PB * 32);
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            int64_t r = row0 + pb * 32 + p;
+            r = r < N ? r : N - 1;
+            const float* xr = X + r * ldx;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bn[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+        }
+    };
+    if (int64_t(blockIdx.x) < ntiles) fetch(blockIdx.x);
+
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t row0 = tile * tile_rows + wave * (PB * 32);
+        floatx4 b[PB][NJ];
+        float baug[PB], xnr[PB], m[PB];
+        int mi[PB];
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                b[pb][j] = bn[pb][j];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
+            }
+            xnr[pb] = s + __shfl_xor(s, 32);
+            baug[pb] = h ? xnr[pb] : 1.0f;
+        }
+        if (tile + gridDim.x < ntiles) fetch(tile + gridDim.x);
+
+        resident_scan<DP, PB, false>(sC, ncb, p, h, b, baug, m, mi);
+        bool neg = false;
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) neg |= m[pb] < 0.f;
+        if (__any(neg)) resident_scan<DP, PB, true>(sC, ncb, p, h, b, baug, m, mi);
+
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            mi[pb] += 4 * h;
+            merge_halves(m[pb], mi[pb]);
+            const int64_t r = row0 + pb * 32 + p;
+            const bool valid = r < N;
+            if (h == 0 && valid) {
+                labels[r] = mi[pb];
+                if (min_d2) min_d2[r] = m[pb];
+                atomicAdd(&sN[mi[pb]], 1);
+            }
+            if (valid && xnr[pb] != 0.f) {  // an all-zero row adds nothing
+                // |x_d| < 2^E: |x|^2 < 2^(e2+1) up to rounding, one more bit of slack
+                const int e2 = (__float_as_int(xnr[pb]) >> 23) - 127;
+                const int E = (e2 >> 1) + 2;
+                emin = min(emin, E);
+                emax = max(emax, E);
+                const double B = __hiloint2double(((1023 + 52 - FUSED_QBITS + E) << 20) | 0x80000, 0);
+                double* row = sA + size_t(mi[pb]) * LDA + h * (DP / 2);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const double v = (double(b[pb][j][t]) + B) - B;
+                        __hip_atomic_fetch_add(row + 4 * j + t, v, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+            }
+        }
+    }
+
+    atomicMin(&sN[K], emin);
+    atomicMax(&sN[K + 1], emax);
+    __syncthreads();
+    double* gs = fsum + size_t(blockIdx.x) * K * D;
+    for (int i = tid; i < K * D; i += nthr) {
+        const int k = i / D, d = i - k * D;
+        gs[i] = sA[size_t(k) * LDA + d];
+    }
+    for (int i = tid; i < K; i += nthr) fcnt[size_t(blockIdx.x) * K + i] = sN[i];
+    if (tid == 0) {
+        const int lo = sN[K], hi = sN[K + 1];
+        flags[blockIdx.x] = (hi >= lo && hi - lo > range_bits) ? 1 : 0;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Tiled variant for 16 < D <= 64 when the centroids do not fit in LDS: same wave-level scheme as the
 // resident kernel (a wave keeps its 32*PB points in B-operand registers for the whole feature range
 // and scans centroid blocks), but the centroids pass through LDS in tiles of 128 rows, double
@@ -384,6 +531,64 @@ static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, 
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc,
                        labels, min_d2, ntiles);
     return check_launch("assign_mfma_resident_kernel");
+}
+
+size_t fused_lds_bytes(int32_t D, int32_t K) {
+    const size_t kp = (size_t(K) + 31) / 32 * 32;
+    const int dp = resident_dp(D);
+    return kp * (dp + 4) * sizeof(float) + size_t(K) * (dp + 1) * sizeof(double) + (size_t(K) + 4) * sizeof(int);
+}
+
+int fused_grid(int64_t N) {
+    constexpr int PB = 2;
+    const int64_t tile_rows = int64_t(FUSED_THREADS / 64) * PB * 32;
+    const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
+    int64_t grid = num_cus();
+    if (grid > FUSED_MAX_GRID) grid = FUSED_MAX_GRID;
+    if (grid > ntiles) grid = ntiles;
+    return int(grid < 1 ? 1 : grid);
+}
+
+template <int DP, bool VEC>
+static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                          int64_t ldc, int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt,
+                          int32_t* flags, hipStream_t st) {
+    constexpr int PB = 2;
+    const int64_t tile_rows = int64_t(FUSED_THREADS / 64) * PB * 32;
+    const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
+    const int grid = fused_grid(N);
+    const size_t lds = fused_lds_bytes(D, K);
+    auto kern = lloyd_mfma_resident_kernel<DP, PB, VEC>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+        if (e != hipSuccess) return fail(HKM_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    // rows one workgroup adds up, as a power of two
+    const int64_t per_wg = (ntiles + grid - 1) / grid * tile_rows;
+    int lg = 0;
+    while ((int64_t(1) << lg) < per_wg) ++lg;
+    const int range_bits = 53 - FUSED_QBITS - lg;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(FUSED_THREADS), lds, st, X, N, D, ldx, C, K, ldc,
+                       labels, min_d2, ntiles, fsum, fcnt, flags, range_bits);
+    return check_launch("lloyd_mfma_resident_kernel");
+}
+
+int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                               int32_t K, int64_t ldc, int32_t* labels, float* min_d2, double* fsum,
+                               int32_t* fcnt, int32_t* flags, hipStream_t st) {
+    const bool vec = aligned16(X) && (ldx % 4 == 0) && (D % 4 == 0);
+    const int dp = resident_dp(D);
+#define HKM_CASE(d)                                                                                         \
+    case d:                                                                                                 \
+        return vec ? launch_fused_t<d, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st) \
+                   : launch_fused_t<d, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);
+    switch (dp) {
+        HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
+        default:
+            return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
+    }
+#undef HKM_CASE
 }
 
 int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,

@@ -54,10 +54,14 @@ struct Workspace {
     float* min_d2;      // [N] (only with the SSE flag)
     double* shift_part; // [ceil(K*D/64)] per-block shares of the squared centroid shift
     double* small_part; // [SMALL_MAX_GRID][K*(D+1)+1] partial rows of the one-sweep small-D step
+    double* fsum;       // [FUSED_MAX_GRID][K][D] fp64 partial sums of the one-sweep MFMA step
+    int32_t* fcnt;      // [FUSED_MAX_GRID][K]
+    int32_t* fflags;    // [FUSED_MAX_GRID] 1 = this workgroup's sums may depend on the addition order
     size_t total;
 };
 static const int RED_SLOTS = 2048;
 static const int SMALL_MAX_GRID = 2048;
+static const int FUSED_MAX_GRID = 512;
 Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags);
 
 // ---- launchers (one per .hip file) ------------------------------------------------------------
@@ -74,6 +78,15 @@ int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, 
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                               int32_t K, int64_t ldc, const float* cn, unsigned long long* keys,
                               int32_t* labels, float* min_d2, hipStream_t st);
+bool fused_eligible(int32_t D, int32_t K);
+size_t fused_lds_bytes(int32_t D, int32_t K);
+int fused_grid(int64_t N);
+int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                               int32_t K, int64_t ldc, int32_t* labels, float* min_d2, double* fsum,
+                               int32_t* fcnt, int32_t* flags, hipStream_t st);
+int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                        int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                        int fgrid, const float* C_old, float* shift, hipStream_t st);
 bool small_eligible(int32_t D, int32_t K);
 int small_grid(int64_t N, int32_t D, int32_t K);
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,

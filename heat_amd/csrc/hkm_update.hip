@@ -41,7 +41,13 @@ UpdateGeom update_geom(int64_t N, int32_t D, int32_t K) {
 __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const int32_t* __restrict__ labels,
     int K, int KR, int64_t rows_per_chunk, float* __restrict__ part_sum,
-    int32_t* __restrict__ part_cnt, int DPAD) {
+    int32_t* __restrict__ part_cnt, int DPAD, const int32_t* __restrict__ gate, int ngate) {
+    // behind the one-sweep MFMA step this pass only runs if some workgroup there raised its flag
+    if (gate) {
+        int any = 0;
+        for (int i = threadIdx.x; i < ngate; i += UPD_THREADS) any |= gate[i];
+        if (!__syncthreads_or(any)) return;
+    }
     constexpr int U = 4;          // rows per half-wave and pass
     constexpr int LIST = 64 + U;  // a batch has 64 rows; room for the padding to a multiple of U
     extern __shared__ __align__(16) float lds[];
@@ -124,10 +130,14 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
 // 256 threads = 64 (k, d) pairs x 4 strided lanes over the chunks.  Lane q adds chunks q, q+4, ...
 // in ascending order (8 loads in flight, additions in order); lane 0 then adds the four lane sums in
 // lane order.  The order depends only on S.
+// With fsum != NULL the partials of the one-sweep MFMA step ([G][K][D] fp64, [G][K] counts) are used
+// unless one of its workgroups raised its flag; then the fp32 partials of pass 1 are.
 __global__ __launch_bounds__(256) void update_finalize_kernel(
     const float* __restrict__ part_sum, const int32_t* __restrict__ part_cnt, int S, int K, int D,
     int DPAD, float* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts,
-    const float* __restrict__ C_old, double* __restrict__ shift_part) {
+    const float* __restrict__ C_old, double* __restrict__ shift_part,
+    const double* __restrict__ fsum, const int32_t* __restrict__ fcnt,
+    const int32_t* __restrict__ fflags, int G) {
     __shared__ double ssum[4][64];
     __shared__ double ssq[64];
     __shared__ int64_t scnt[4][64];
@@ -137,7 +147,36 @@ __global__ __launch_bounds__(256) void update_finalize_kernel(
     const int k = ok ? int(i / D) : 0, d = ok ? int(i - int64_t(k) * D) : 0;
     double sum = 0.0;
     int64_t n = 0;
-    if (ok) {
+    bool fused = fsum != nullptr;
+    if (fused) {
+        int any = 0;
+        for (int g = threadIdx.x; g < G; g += 256) any |= fflags[g];
+        fused = !__syncthreads_or(any);
+    }
+    if (ok && fused) {
+        const double* ps = fsum + int64_t(k) * D + d;
+        const int32_t* pc = fcnt + k;
+        const int64_t sstride = int64_t(K) * D;
+        int s = q;
+        for (; s + 28 < G; s += 32) {
+            double t[8];
+            int32_t c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                t[u] = ps[(s + 4 * u) * sstride];
+                c[u] = pc[int64_t(s + 4 * u) * K];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                sum += t[u];
+                n += c[u];
+            }
+        }
+        for (; s < G; s += 4) {
+            sum += ps[s * sstride];
+            n += pc[int64_t(s) * K];
+        }
+    } else if (ok) {
         const float* ps = part_sum + int64_t(k) * DPAD + d;
         const int32_t* pc = part_cnt + k;
         const int64_t sstride = int64_t(K) * DPAD;
@@ -214,13 +253,42 @@ int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32
     const size_t lds = size_t(g.KR + 1) * 32 * sizeof(float) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
                        size_t(UPD_HALVES) * (64 + 8) * sizeof(int2);
     hipLaunchKernelGGL(update_partial_kernel, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
-                       D, ldx, labels, K, g.KR, g.rows_per_chunk, w.part_sum, w.part_cnt, dpad);
+                       D, ldx, labels, K, g.KR, g.rows_per_chunk, w.part_sum, w.part_cnt, dpad,
+                       static_cast<const int32_t*>(nullptr), 0);
     int rc = check_launch("update_partial_kernel");
     if (rc) return rc;
     const int64_t tot = int64_t(K) * D;
     const int nb = int((tot + 63) / 64);
     hipLaunchKernelGGL(update_finalize_kernel, dim3(nb), dim3(256), 0, st, w.part_sum, w.part_cnt,
-                       g.S, K, D, dpad, C_new, ldcn, counts, C_old, w.shift_part);
+                       g.S, K, D, dpad, C_new, ldcn, counts, C_old, w.shift_part,
+                       static_cast<const double*>(nullptr), static_cast<const int32_t*>(nullptr),
+                       static_cast<const int32_t*>(nullptr), 0);
+    rc = check_launch("update_finalize_kernel");
+    if (rc || !C_old) return rc;
+    hipLaunchKernelGGL(shift_final_kernel, dim3(1), dim3(256), 0, st, w.shift_part, nb, shift);
+    return check_launch("shift_final_kernel");
+}
+
+// Second half of the one-sweep MFMA step: the two-pass update gated by the flags of the fused kernel
+// (normally every workgroup returns at once), then the finalize that reads whichever partials hold.
+int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                        int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                        int fgrid, const float* C_old, float* shift, hipStream_t st) {
+    const UpdateGeom g = update_geom(N, D, K);
+    const int dpad = g.J * 32;
+    const size_t lds = size_t(g.KR + 1) * 32 * sizeof(float) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
+                       size_t(UPD_HALVES) * (64 + 8) * sizeof(int2);
+    hipLaunchKernelGGL(update_partial_kernel, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
+                       D, ldx, labels, K, g.KR, g.rows_per_chunk, w.part_sum, w.part_cnt, dpad,
+                       static_cast<const int32_t*>(w.fflags), fgrid);
+    int rc = check_launch("update_partial_kernel");
+    if (rc) return rc;
+    const int64_t tot = int64_t(K) * D;
+    const int nb = int((tot + 63) / 64);
+    hipLaunchKernelGGL(update_finalize_kernel, dim3(nb), dim3(256), 0, st, w.part_sum, w.part_cnt,
+                       g.S, K, D, dpad, C_new, ldcn, counts, C_old, w.shift_part,
+                       static_cast<const double*>(w.fsum), static_cast<const int32_t*>(w.fcnt),
+                       static_cast<const int32_t*>(w.fflags), fgrid);
     rc = check_launch("update_finalize_kernel");
     if (rc || !C_old) return rc;
     hipLaunchKernelGGL(shift_final_kernel, dim3(1), dim3(256), 0, st, w.shift_part, nb, shift);

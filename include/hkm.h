@@ -77,7 +77,9 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
 /*
  * One Lloyd iteration: labels against C, C_new = per-cluster means, *shift = sum((C - C_new)^2)
  * (fp32 value, device scalar), optional *sse = sum_i min_d2[i] (device scalar; NULL to skip).
- * C and C_new are K x D with leading dimension D.
+ * C and C_new are K x D with leading dimension D.  shift (and sse) may also point to pinned,
+ * device-accessible host memory: the finishing kernel then delivers the scalar itself and no copy
+ * sits between two steps on the stream.
  * Replaces the loop body of heat/cluster/kmeans.py:131-143 (KMeans.fit).
  */
 int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
@@ -151,6 +153,10 @@ int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_s
 /* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "mfma_resident",
  * "mfma_tiled", "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
 const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K);
+
+/* Same for hkm_lloyd_step_f32: "lloyd_small" and "lloyd_mfma_resident" read X once per step (labels and
+ * per-cluster sums in one kernel); every other shape runs "<assign kernel>+update" (two reads of X). */
+const char* hkm_lloyd_kernel_name(int64_t N, int32_t D, int32_t K);
 
 #ifdef __cplusplus
 }

@@ -159,7 +159,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) >= 15
+    assert len(names) >= 16
     for name in names:
         assert hasattr(lib, name), name
         assert name in _native.SIGNATURES, f"{name} has no ctypes signature"
@@ -178,6 +178,10 @@ def test_workspace_and_kernel_selection():
     assert _native.assign_kernel_name(10_000_000, 32, 256) == "mfma_resident"
     assert _native.assign_kernel_name(1 << 20, 64, 1024) == "mfma_tiled"
     assert _native.assign_kernel_name(2_000_000, 512, 1024) == "mfma_stream"
+    assert _native.lloyd_kernel_name(200_000_000, 3, 8) == "lloyd_small"
+    assert _native.lloyd_kernel_name(10_000_000, 32, 256) == "lloyd_mfma_resident"
+    assert _native.lloyd_kernel_name(10_000_000, 64, 512) == "mfma_tiled+update"  # accumulators exceed LDS
+    assert _native.lloyd_kernel_name(2_000_000, 512, 1024) == "mfma_stream+update"
 
 
 def test_argument_validation_happens_on_the_host():

@@ -167,6 +167,77 @@ def test_lloyd_step_matches_oracle_and_is_deterministic(cuda, n, d, k):
     assert orc.rel_err_scalar(float(sse), ref_sse) <= 1e-4
 
 
+def _step_and_two_pass(xs, cs, dev):
+    """One hkm_lloyd_step_f32 and, from the same inputs, hkm_assign_f32 + hkm_update_f32."""
+    n, k = xs.shape[0], cs.shape[0]
+    ws = _native.Workspace(dev)
+    c_step = torch.empty_like(cs)
+    lab_step = torch.empty((n,), dtype=torch.int32, device=dev)
+    shift = torch.empty((), device=dev)
+    _native.lloyd_step(xs, cs, c_step, lab_step, shift, None, ws)
+    lab2 = torch.empty_like(lab_step)
+    _native.assign(xs, cs, lab2, None, ws)
+    c2 = torch.empty_like(cs)
+    cnt2 = torch.empty((k,), dtype=torch.int64, device=dev)
+    _native.update(xs, lab2, c2, cnt2, ws)
+    torch.cuda.synchronize()
+    return c_step, lab_step, shift, c2, lab2, cnt2
+
+
+# shapes of the one-sweep MFMA step (16 < D <= 64, centroids + fp64 accumulators fit in LDS):
+# ragged N, K not a multiple of 32, D not a multiple of 4 (scalar loads), every padded width
+@pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (40000, 30, 100),
+                                   (70001, 40, 129), (30000, 64, 128), (768, 17, 5), (100, 48, 7)])
+def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
+    print(f"one-sweep n={n} d={d} k={k}", flush=True)
+    x, _ = _data(n, d, k, seed=5 * n + d)
+    x[::97] = 0.0  # all-zero rows only count
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(4))[:k]].contiguous()
+    xs, cs = x.to(cuda), c0.to(cuda)
+    c_step, lab_step, shift, c2, lab2, cnt2 = _step_and_two_pass(xs, cs, cuda)
+    assert torch.equal(lab_step, lab2)
+    assert orc.rel_err_centers(c_step.cpu(), c2.cpu()) <= 1e-6
+    # the fp64 sums of the one-sweep step are exact up to 2^-29 per row: compare with fp64 directly
+    ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab2.cpu().long(), x.double())
+    ref = (ref / cnt2.cpu().clamp(min=1).double().unsqueeze(1)).float()
+    assert (c_step.cpu() - ref).abs().max() <= 2e-7 * float(x.abs().max())
+    again = _step_and_two_pass(xs, cs, cuda)
+    assert torch.equal(again[0], c_step) and torch.equal(again[2], shift)
+
+
+def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
+    # Row magnitudes spread over 2^60 (or rows holding inf / NaN) break the condition under which the
+    # fp64 LDS sums are independent of the order of additions: the step must then produce exactly
+    # what assign + update produce (their fp32 partials, fixed order), run after run.
+    n, d, k = 60000, 32, 64
+    x, _ = _data(n, d, k, seed=77)
+    g = torch.Generator().manual_seed(2)
+    scale = torch.pow(2.0, torch.randint(-30, 31, (n, 1), generator=g).float())
+    for variant in ("wide", "nonfinite"):
+        xv = x * scale if variant == "wide" else x.clone()
+        if variant == "nonfinite":
+            xv[5, 3] = float("inf")
+            xv[4000, 0] = float("nan")
+        c0 = xv[torch.randperm(n, generator=g)[:k]].contiguous()
+        c0 = torch.nan_to_num(c0, nan=0.0, posinf=1.0, neginf=-1.0)
+        xs, cs = xv.to(cuda), c0.to(cuda)
+        c_step, lab_step, shift, c2, lab2, _ = _step_and_two_pass(xs, cs, cuda)
+        assert torch.equal(lab_step, lab2)
+        assert torch.equal(c_step.isnan(), c2.isnan())
+        assert torch.equal(torch.nan_to_num(c_step), torch.nan_to_num(c2)), variant
+        again = _step_and_two_pass(xs, cs, cuda)
+        assert torch.equal(torch.nan_to_num(again[0]), torch.nan_to_num(c_step))
+    # moderate spread (2^+-3) stays on the exact path: the result is the fp64 mean, which the fp32
+    # partials of the two-pass update only approximate
+    xv = x * torch.pow(2.0, torch.randint(-3, 4, (n, 1), generator=g).float())
+    c0 = xv[torch.randperm(n, generator=g)[:k]].contiguous()
+    c_step, lab_step, _, c2, lab2, cnt2 = _step_and_two_pass(xv.to(cuda), c0.to(cuda), cuda)
+    ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab2.cpu().long(), xv.double())
+    ref = (ref / cnt2.cpu().clamp(min=1).double().unsqueeze(1)).float()
+    assert (c_step.cpu() - ref).abs().max() <= 2e-7 * float(xv.abs().max())
+
+
 def test_shift_and_functional_value(cuda):
     g = torch.Generator().manual_seed(9)
     a, b = torch.randn((37, 19), generator=g), torch.randn((37, 19), generator=g)
