@@ -18,7 +18,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "li
 _lib: Optional[ctypes.CDLL] = None
 
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
-WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE = 1, 2, 3, 4
+WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN = 1, 2, 3, 4, 8
 
 # name -> (restype, argtypes); must list every symbol declared in include/hkm.h
 SIGNATURES = {
@@ -43,6 +43,13 @@ SIGNATURES = {
     "hkm_sample_select_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_void_p, ctypes.c_float, c_void_p,
                                              c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_label_counts_i64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
+    "hkm_assign_l1_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                         c_void_p, c_void_p, c_void_p]),
+    "hkm_closest_rows_l1_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                               c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_update_median_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
+                                             c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p,
+                                             c_size_t, c_void_p]),
     "hkm_widen_labels_i64": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
 }
 
@@ -223,6 +230,41 @@ def label_counts(labels32: torch.Tensor, k: int, counts: torch.Tensor) -> None:
     if counts.numel() != k:
         raise ValueError(f"counts has {counts.numel()} elements, expected {k}")
     check(load().hkm_label_counts_i64(_ptr(labels32), labels32.numel(), k, _ptr(counts), _stream()))
+
+
+def assign_l1(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_dist: Optional[torch.Tensor]) -> None:
+    """labels[i] = argmin_k sum|x_i - c_k| (Manhattan), optional minimum distance."""
+    _require_gpu(x, c, labels, min_dist)
+    n, d = x.shape
+    k = c.shape[0]
+    check(load().hkm_assign_l1_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
+                                   c.stride(0) if k > 1 else d, _ptr(labels), _ptr(min_dist), _stream()))
+
+
+def closest_rows_l1(x: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, dist: Optional[torch.Tensor],
+                    ws: Workspace) -> None:
+    """idx[m] = row of x closest to q[m] in the Manhattan metric (first index on ties)."""
+    _require_gpu(x, q, idx, dist)
+    n, d = x.shape
+    m = q.shape[0]
+    buf = ws.get(workspace_bytes(n, d, m, WS_MEDIAN))
+    check(load().hkm_closest_rows_l1_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(q), m,
+                                         q.stride(0) if m > 1 else d, _ptr(idx), _ptr(dist), _ptr(buf),
+                                         buf.numel(), _stream()))
+
+
+def update_median(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, ws: Workspace,
+                  fallback_rows: Optional[torch.Tensor] = None, c_old: Optional[torch.Tensor] = None,
+                  counts: Optional[torch.Tensor] = None, lower: bool = False, skip_zero_rows: bool = False) -> None:
+    """Per-cluster, per-coordinate median (see hkm_update_median_f32 in include/hkm.h)."""
+    _require_gpu(x, labels, c_new, fallback_rows, c_old, counts)
+    n, d = x.shape
+    k = c_new.shape[0]
+    buf = ws.get(workspace_bytes(n, d, k, WS_MEDIAN))
+    check(load().hkm_update_median_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k,
+                                       _ptr(fallback_rows), _ptr(c_old), _ptr(c_new),
+                                       c_new.stride(0) if k > 1 else d, _ptr(counts), 1 if lower else 0,
+                                       1 if skip_zero_rows else 0, _ptr(buf), buf.numel(), _stream()))
 
 
 def widen_labels(labels32: torch.Tensor, out64: torch.Tensor) -> None:

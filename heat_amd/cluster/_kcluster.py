@@ -84,6 +84,10 @@ class _KCluster(ClusteringMixin, BaseEstimator):
             t = t.contiguous()
         return t
 
+    def _manhattan_metric(self) -> bool:
+        """True for the estimators constructed with the Manhattan metric (KMedians, KMedoids)."""
+        return type(self).__name__ in ("KMedians", "KMedoids")
+
     @staticmethod
     def _check_split(x: DNDarray) -> None:
         # the reference raises this from cdist (heat/spatial/distance.py:386-390)
@@ -137,7 +141,10 @@ class _KCluster(ClusteringMixin, BaseEstimator):
                     clusterer = BatchParallelKMeans(n_clusters=self.n_clusters, init="k-means++", max_iter=100,
                                                     random_state=self.random_state)
                 elif self._p == 1:
-                    raise NotImplementedError("BatchParallelKMedians is not built in heat_amd")
+                    from .batchparallelclustering import BatchParallelKMedians
+
+                    clusterer = BatchParallelKMedians(n_clusters=self.n_clusters, init="k-medians++", max_iter=100,
+                                                      random_state=self.random_state)
                 else:
                     raise ValueError("Batch parallel initialization only implemented for KMeans and KMedians")
                 clusterer.fit(x)
@@ -244,7 +251,14 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         ws = self._workspace(dev)
         lab32 = torch.empty((n,), dtype=torch.int32, device=dev)
         min_d2 = torch.empty((n,), dtype=torch.float32, device=dev) if eval_functional_value else None
-        _native.assign(xt, ct, lab32, min_d2, ws)
+        if self._manhattan_metric():
+            # k-medians / k-medoids: fused sum|x - c| + argmin; the functional is the squared 2-norm of
+            # the minimum distances, so they are squared before the same reduction
+            _native.assign_l1(xt, ct, lab32, min_d2)
+            if min_d2 is not None:
+                min_d2.mul_(min_d2)
+        else:
+            _native.assign(xt, ct, lab32, min_d2, ws)
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         _native.widen_labels(lab32, lab64)
         if eval_functional_value:

@@ -22,11 +22,12 @@ from ..core.dndarray import DNDarray
 from ._sampling import DeviceSampler
 
 
-def _dist_to_row(x: torch.Tensor, row: torch.Tensor) -> torch.Tensor:
-    """Euclidean distance sqrt(sum((x_i - row)^2)) of every row of x to one row (direct form: exactly
-    zero for the row itself, which a quadratic expansion does not guarantee)."""
+def _dist_to_row(x: torch.Tensor, row: torch.Tensor, p: int) -> torch.Tensor:
+    """Distance of every row of x to one row: sqrt(sum((x_i - row)^2)) for p = 2 (direct form: exactly
+    zero for the row itself, which a quadratic expansion does not guarantee), sum|x_i - row| for p = 1."""
     out = torch.empty((x.shape[0], 1), dtype=torch.float32, device=x.device)
-    _native.pairwise(x, row.reshape(1, -1).contiguous(), out, _native.METRIC_EUCLID)
+    _native.pairwise(x, row.reshape(1, -1).contiguous(), out,
+                     _native.METRIC_MANHATTAN if p == 1 else _native.METRIC_EUCLID)
     return out.view(-1)
 
 
@@ -35,22 +36,20 @@ def _initialize_plus_plus(x: torch.Tensor, n_clusters: int, p: int, sampler, wei
     """
     k-means++ seeding as heat/cluster/batchparallelclustering.py:22-46 does it: the first centre
     uniformly, every further one with probability proportional to ``weights * distance`` (the plain
-    distance to the closest centre chosen so far, not its square).  More than ``max_samples`` rows
+    p-norm distance to the closest centre chosen so far, not its square).  More than ``max_samples`` rows
     are subsampled first because a categorical draw is limited to 2**24 categories.  The reference
     recomputes the distances to all chosen centres in every step; the running minimum kept here is
     the same number and needs one N x 1 distance column per step.
     """
-    if p != 2:
-        raise NotImplementedError("only the Euclidean (p=2) seeding is built")
     if x.shape[0] > max_samples:
         sub = torch.tensor([sampler.randint(x.shape[0]) for _ in range(max_samples)], device=x.device)
         x = x[sub].contiguous()
     idxs = [sampler.randint(x.shape[0])]
-    dist = _dist_to_row(x, x[idxs[0]])
+    dist = _dist_to_row(x, x[idxs[0]], p)
     for i in range(1, n_clusters):
         idxs.append(sampler.multinomial(weights * dist))
         if i + 1 < n_clusters:
-            dist = torch.minimum(dist, _dist_to_row(x, x[idxs[-1]]))
+            dist = torch.minimum(dist, _dist_to_row(x, x[idxs[-1]], p))
     return x[torch.tensor(idxs, device=x.device)]
 
 
@@ -59,10 +58,10 @@ def _kmex(x: torch.Tensor, p: int, n_clusters: int, init: Union[str, torch.Tenso
     """
     Lloyd iteration on a local matrix (heat/cluster/batchparallelclustering.py:49-88): an empty
     cluster KEEPS its centre (unlike KMeans._update_centroids), the loop stops when
-    ``allclose(centers, previous, atol=tol)`` (rtol 1e-5).  Returns (centers, iterations run).
+    ``allclose(centers, previous, atol=tol)`` (rtol 1e-5).  p = 1 is k-medians: Manhattan assignment
+    and ``torch.median``, i.e. the LOWER middle value of every coordinate.  Any other p runs as p = 2,
+    like the reference.  Returns (centers, iterations run).
     """
-    if p != 2:
-        raise NotImplementedError("only p=2 (k-means) is built")
     _native._require_gpu(x)
     ws = ws or _native.Workspace(x.device)
     sampler = sampler or DeviceSampler(x.device)
@@ -82,9 +81,14 @@ def _kmex(x: torch.Tensor, p: int, n_clusters: int, init: Union[str, torch.Tenso
     means = torch.empty_like(centers)
     it = 0
     for it in range(max_iter):
-        _native.assign(x, centers, lab, None, ws)
-        _native.update(x, lab, means, counts, ws)
-        new = torch.where(counts.unsqueeze(1) > 0, means, centers)
+        if p == 1:
+            _native.assign_l1(x, centers, lab, None)
+            new = torch.empty_like(centers)
+            _native.update_median(x, lab, new, ws, c_old=centers.contiguous(), lower=True)
+        else:
+            _native.assign(x, centers, lab, None, ws)
+            _native.update(x, lab, means, counts, ws)
+            new = torch.where(counts.unsqueeze(1) > 0, means, centers)
         done = bool(torch.allclose(new, centers, atol=tol))
         centers = new
         if done:
@@ -190,18 +194,22 @@ class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
             raise ValueError(
                 f"input needs to have {self._cluster_centers.shape[1]} features, but has {x.shape[1]}"
             )
-        if self._p != 2:
-            raise NotImplementedError("only p=2 (k-means) is built")
         xt = self._local_f32(x)
         if self._ws is None or self._ws.device != xt.device:
             self._ws = _native.Workspace(xt.device)
         n = xt.shape[0]
         lab = torch.empty((n, 1), dtype=torch.int32, device=xt.device)
         d2 = torch.empty((n,), dtype=torch.float32, device=xt.device)
-        _native.assign(xt, self._cluster_centers.larray, lab.view(-1), d2, self._ws)
         fv = torch.empty((), dtype=torch.float32, device=xt.device)
-        # ||x - C[labels]||_F ** 2 = sum of the squared distances to the closest centre
-        _native.functional_value(d2, fv, self._ws)
+        if self._p == 1:
+            # sum of the Manhattan distances to the closest centre: min_dist_sum adds sqrt(v), so it is
+            # fed the squared distances
+            _native.assign_l1(xt, self._cluster_centers.larray, lab.view(-1), d2)
+            _native.min_dist_sum(d2.mul_(d2), fv, self._ws)
+        else:
+            # ||x - C[labels]||_F ** 2 = sum of the squared distances to the closest centre
+            _native.assign(xt, self._cluster_centers.larray, lab.view(-1), d2, self._ws)
+            _native.functional_value(d2, fv, self._ws)
         self._functional_value = fv.item()
         return DNDarray(lab, (n, 1), types.int32, x.split, x.device, x.comm, x.balanced)
 
@@ -222,5 +230,25 @@ class BatchParallelKMeans(_BatchParallelKCluster):
         else:
             raise ValueError(f"init must be 'k-means++' or 'random', but was {init}")
         super().__init__(p=2, n_clusters=n_clusters, init=_init, max_iter=max_iter, tol=tol,
+                         random_state=random_state, n_procs_to_merge=n_procs_to_merge)
+        self.init = init
+
+
+class BatchParallelKMedians(_BatchParallelKCluster):
+    """Batch-parallel k-medians (heat/cluster/batchparallelclustering.py:400-458)."""
+
+    def __init__(self, n_clusters: int = 8, init: str = "k-medians++", max_iter: int = 300, tol: float = 1e-4,
+                 random_state: Optional[int] = None, n_procs_to_merge: Optional[int] = None):  # noqa: D107
+        if not isinstance(init, str):
+            raise TypeError(f"init must be str, but was {type(init)}")
+        if init == "k-medians++":
+            _init = "++"
+        elif init == "random":
+            raise NotImplementedError(
+                "random initialization for batch parallel k-medians is currently not supported due to instable behaviour of the algorithm. Use init='k-medians++' instead."
+            )
+        else:
+            raise ValueError(f"init must be 'k-medians++' or 'random', but was {init}")
+        super().__init__(p=1, n_clusters=n_clusters, init=_init, max_iter=max_iter, tol=tol,
                          random_state=random_state, n_procs_to_merge=n_procs_to_merge)
         self.init = init

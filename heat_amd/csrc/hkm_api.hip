@@ -87,6 +87,33 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
     return w;
 }
 
+MedianWorkspace carve_median(void* base, int64_t N, int32_t D, int32_t K) {
+    MedianWorkspace w;
+    memset(&w, 0, sizeof(w));
+    char* p = static_cast<char*>(base);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* r = p ? p + off : nullptr;
+        off += align_up(bytes, 256);
+        return r;
+    };
+    const size_t n = size_t(N < 1 ? 1 : N), kd = size_t(K) * D;
+    w.eff = reinterpret_cast<int32_t*>(take(n * sizeof(int32_t)));
+    w.perm = reinterpret_cast<int32_t*>(take(n * sizeof(int32_t)));
+    w.counts = reinterpret_cast<int64_t*>(take(size_t(K) * sizeof(int64_t)));
+    w.offsets = reinterpret_cast<int64_t*>(take((size_t(K) + 1) * sizeof(int64_t)));
+    w.chunk_start = reinterpret_cast<int32_t*>(take((size_t(K) + 1) * sizeof(int32_t)));
+    w.cursor = reinterpret_cast<int32_t*>(take(size_t(K) * sizeof(int32_t)));
+    w.prefix = reinterpret_cast<unsigned*>(take(kd * sizeof(unsigned)));
+    w.rank = reinterpret_cast<int64_t*>(take(kd * sizeof(int64_t)));
+    w.eqcnt = reinterpret_cast<unsigned*>(take(kd * sizeof(unsigned)));
+    w.next = reinterpret_cast<unsigned*>(take(kd * sizeof(unsigned)));
+    w.hist = reinterpret_cast<unsigned*>(take(kd * 256 * sizeof(unsigned)));
+    w.keys = reinterpret_cast<unsigned long long*>(take(size_t(K) * sizeof(unsigned long long)));
+    w.total = off;
+    return w;
+}
+
 static int check_matrix(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
     if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);
     if (reinterpret_cast<uintptr_t>(p) & 3u) return fail(HKM_EINVAL, "%s is not 4-byte aligned", name);
@@ -144,6 +171,7 @@ const char* hkm_last_error(void) { return g_err; }
 
 size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags) {
     if (N < 0 || D < 1 || K < 1) return 0;
+    if (flags == HKM_WS_MEDIAN) return carve_median(nullptr, N, D, K).total;
     return carve(nullptr, N, D, K, flags).total;
 }
 
@@ -295,6 +323,55 @@ int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* c
     if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
     if ((N > 0 && !labels) || !counts) return fail(HKM_EINVAL, "NULL pointer argument");
     return launch_label_counts(labels, N, K, counts, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_assign_l1_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                      int64_t ldc, int32_t* labels, float* min_dist, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C", C, K, D, ldc))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (N == 0) return HKM_OK;
+    return launch_assign_l1(X, N, D, ldx, C, K, ldc, labels, min_dist, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_closest_rows_l1_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* Q, int32_t M,
+                            int64_t ldq, int64_t* idx, float* dist, void* ws, size_t ws_bytes,
+                            void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, M);
+    if (rc) return rc;
+    if (N < 1) return fail(HKM_EINVAL, "N = %lld: there is no closest row in an empty matrix", (long long)N);
+    if (N > 0xfffffffeLL) return fail(HKM_EUNSUPPORTED, "N = %lld exceeds 32-bit row indices", (long long)N);
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("Q", Q, M, D, ldq))) return rc;
+    if (!idx) return fail(HKM_EINVAL, "idx is NULL");
+    const size_t need = carve_median(nullptr, N, D, M).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const MedianWorkspace w = carve_median(ws, N, D, M);
+    return launch_closest_rows_l1(X, N, D, ldx, Q, M, ldq, idx, dist, w.keys, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_update_median_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                          const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
+                          int64_t* counts, int32_t mode, int32_t skip_zero_rows, void* ws, size_t ws_bytes,
+                          void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if (N > 0x7ffffffeLL) return fail(HKM_EUNSUPPORTED, "N = %lld exceeds 31-bit row indices", (long long)N);
+    if (mode != 0 && mode != 1) return fail(HKM_EINVAL, "mode = %d must be 0 (mean of the middles) or 1 (lower middle)", mode);
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C_new", C_new, K, D, ldcn))) return rc;
+    if (C_old && (rc = check_matrix("C_old", C_old, K, D, D))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    const size_t need = carve_median(nullptr, N, D, K).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const MedianWorkspace w = carve_median(ws, N, D, K);
+    return launch_update_median(X, N, D, ldx, labels, K, fallback_rows, C_old, C_new, ldcn, counts, mode,
+                                skip_zero_rows, w, static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,

@@ -64,6 +64,24 @@ static const int SMALL_MAX_GRID = 2048;
 static const int FUSED_MAX_GRID = 512;
 Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags);
 
+// scratch of the per-cluster median (hkm_l1.hip)
+struct MedianWorkspace {
+    int32_t* eff;          // [N] label, or -1 for a row left out
+    int32_t* perm;         // [N] row indices grouped by cluster
+    int64_t* counts;       // [K]
+    int64_t* offsets;      // [K + 1]
+    int32_t* chunk_start;  // [K + 1]
+    int32_t* cursor;       // [K]
+    unsigned* prefix;      // [K * D]
+    int64_t* rank;         // [K * D]
+    unsigned* eqcnt;       // [K * D]
+    unsigned* next;        // [K * D]
+    unsigned* hist;        // [K * D * 256]
+    unsigned long long* keys;  // [K] merge keys of the closest-row search
+    size_t total;
+};
+MedianWorkspace carve_median(void* base, int64_t N, int32_t D, int32_t K);
+
 // ---- launchers (one per .hip file) ------------------------------------------------------------
 int launch_norms(const float* C, int32_t K, int32_t D, int64_t ldc, float* cn, int32_t kpad,
                  hipStream_t st);
@@ -109,6 +127,15 @@ int launch_select(const float* d2, const float* u, int64_t N, const float* cost,
                   int64_t* idx, int64_t cap, int64_t* count, double* red, hipStream_t st);
 int launch_label_counts(const int32_t* labels, int64_t N, int32_t K, int64_t* counts,
                         hipStream_t st);
+int launch_assign_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                     int64_t ldc, int32_t* labels, float* min_dist, hipStream_t st);
+int launch_closest_rows_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* Qm,
+                           int32_t M, int64_t ldq, int64_t* idx, float* dist,
+                           unsigned long long* keys, hipStream_t st);
+int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                         int32_t K, const int64_t* fallback_rows, const float* C_old, float* C_new,
+                         int64_t ldcn, int64_t* counts_out, int32_t mode, int32_t skip_zero_rows,
+                         const MedianWorkspace& w, hipStream_t st);
 int launch_widen(const int32_t* in, int64_t N, int64_t* out, hipStream_t st);
 
 int num_cus();

@@ -42,6 +42,7 @@ extern "C" {
 #define HKM_WS_UPDATE 2
 #define HKM_WS_LLOYD 3 /* assign + update */
 #define HKM_WS_SSE 4   /* add when hkm_lloyd_step_f32 is called with sse != NULL (N floats of scratch) */
+#define HKM_WS_MEDIAN 8 /* on its own: scratch of hkm_update_median_f32 / hkm_closest_rows_l1_f32 */
 
 /* Library version: major*10000 + minor*100 + patch. */
 int hkm_version(void);
@@ -146,6 +147,35 @@ int hkm_sample_select_f32(const float* min_d2, const float* u, int64_t N, const 
                           size_t ws_bytes, void* hip_stream);
 int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* counts,
                          void* hip_stream);
+
+/*
+ * Manhattan-metric siblings for k-medians / k-medoids (heat/cluster/kmedians.py:60-106,
+ * heat/cluster/kmedoids.py:57-115, heat/cluster/batchparallelclustering.py:49-97 with p = 1).
+ *
+ * hkm_assign_l1_f32: labels[i] = argmin_k sum_d |x_id - c_kd| (first index on ties), min_dist[i] = that
+ *   minimum (may be NULL); the N x K matrix of manhattan(x, c) (heat/spatial/distance.py:106-133) is
+ *   never written.  Replaces _KCluster._assign_to_cluster with the Manhattan metric.
+ * hkm_closest_rows_l1_f32: idx[m] = argmin_i sum_d |x_id - q_md| over ALL rows of X (first index on
+ *   ties), dist[m] = that distance (may be NULL): the snap of a median to the closest sample of
+ *   kmedoids.py:91-106.  ws needs hkm_workspace_bytes(N, D, M, HKM_WS_MEDIAN) bytes.
+ * hkm_update_median_f32: C_new[k][d] = median over {i : labels[i] == k} of x_id.
+ *   mode 0: percentile 50 with linear interpolation as heat/core/statistics.py computes it on the
+ *           float64 `x * selection`: the middle value, or lo + (hi - lo) * 0.5 in fp64 rounded to fp32;
+ *   mode 1: the lower of the two middle values (torch.median, batchparallelclustering.py:77).
+ *   skip_zero_rows != 0 leaves out rows that are entirely zero, as kmedians.py:93-96 does.
+ *   An empty cluster takes the data row fallback_rows[k] (int64[K] device array) if that pointer is
+ *   given, else keeps C_old[k] if given, else becomes a zero row.  counts (int64[K]) may be NULL.
+ *   ws needs hkm_workspace_bytes(N, D, K, HKM_WS_MEDIAN) bytes.
+ */
+int hkm_assign_l1_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                      int64_t ldc, int32_t* labels, float* min_dist, void* hip_stream);
+int hkm_closest_rows_l1_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* Q, int32_t M,
+                            int64_t ldq, int64_t* idx, float* dist, void* ws, size_t ws_bytes,
+                            void* hip_stream);
+int hkm_update_median_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                          const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
+                          int64_t* counts, int32_t mode, int32_t skip_zero_rows, void* ws, size_t ws_bytes,
+                          void* hip_stream);
 
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);

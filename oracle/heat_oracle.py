@@ -45,6 +45,13 @@ Pins (what each function is checked against, see tests/test_oracle_pins.py):
   rule and the allclose stop of ``_kmex``, and recovery of well-separated blobs.  **Parity unpinned**
   for the random draws themselves: the reference takes them from Heat's counter-based generator and
   from torch's unseeded global generator, and stores no seeded result anywhere.
+* manhattan / assign_l1 / heat_median_axis0 / update_medians / kmedians_fit / kmedoids_fit: the
+  known answers of ``tests/spatial/test_distances.py:20-23,42-48,67-73`` (ones vs zeros, D=4 -> 4.0;
+  X vs X -> 0), scipy's cityblock distances, ``numpy.median`` and a python sort, hand-made cases for
+  the dropped all-zero rows and the empty-cluster restart, brute force for the medoid (a data row, at
+  minimal Manhattan distance from the median), K = 1 closed form (the coordinate-wise median after
+  one iteration), and the reference's own assertion that every medoid is a data point
+  (``tests/cluster/test_kmedoids.py:44-48``).  End-to-end numbers: parity unpinned, as for KMeans.
 """
 
 from __future__ import annotations
@@ -501,38 +508,41 @@ def centroid_sampling_helper(x: torch.Tensor, centroids: torch.Tensor, oversampl
     return centroids
 
 
-def initialize_plus_plus(x: torch.Tensor, n_clusters: int, sampler, weights=1.0) -> torch.Tensor:
-    """Follows heat/cluster/batchparallelclustering.py:22-46 (p = 2, no subsampling)."""
+def initialize_plus_plus(x: torch.Tensor, n_clusters: int, sampler, weights=1.0, p: int = 2) -> torch.Tensor:
+    """Follows heat/cluster/batchparallelclustering.py:22-46 (no subsampling)."""
     idxs = torch.zeros(n_clusters, dtype=torch.long)
     idxs[0] = sampler.randint(x.shape[0])
     for i in range(1, n_clusters):
-        dist = torch.cdist(x, x[idxs[:i]], p=2)
+        dist = torch.cdist(x, x[idxs[:i]], p=p)
         dist = torch.min(dist, dim=1)[0]
         idxs[i] = sampler.multinomial(weights * dist)
     return x[idxs]
 
 
 def kmex(x: torch.Tensor, n_clusters: int, init, max_iter: int, tol: float, sampler=None,
-         weights=1.0) -> Tuple[torch.Tensor, int]:
-    """Follows heat/cluster/batchparallelclustering.py:49-88 (p = 2)."""
+         weights=1.0, p: int = 2) -> Tuple[torch.Tensor, int]:
+    """Follows heat/cluster/batchparallelclustering.py:49-88 (p = 2: means, p = 1: torch.median)."""
     if isinstance(init, torch.Tensor):
         if init.shape != (n_clusters, x.shape[1]):
             raise ValueError("if a torch tensor, init must have shape (n_clusters, n_features).")
         centers = init.clone()
     elif init == "++":
-        centers = initialize_plus_plus(x, n_clusters, sampler, weights)
+        centers = initialize_plus_plus(x, n_clusters, sampler, weights, p)
     elif init == "random":
         centers = x[torch.tensor([sampler.randint(x.shape[0]) for _ in range(n_clusters)])]
     else:
         raise ValueError("init must be a torch tensor with initial centers, string '++', or 'random'.")
     it = 0
     for it in range(max_iter):
-        dist = torch.cdist(x, centers, p=2)
+        dist = torch.cdist(x, centers, p=p)
         labels = torch.argmin(dist, dim=1)
         centers_old = centers.clone()
         for i in range(n_clusters):
             if (labels == i).any():
-                centers[i] = torch.mean(x[labels == i], dim=0)
+                if p == 1:
+                    centers[i] = torch.median(x[labels == i], dim=0)[0]
+                else:
+                    centers[i] = torch.mean(x[labels == i], dim=0)
         if torch.allclose(centers, centers_old, atol=tol):
             break
     return centers, it + 1
@@ -568,3 +578,113 @@ def kmeans_parallel_init(x: torch.Tensor, n_clusters: int, oversampling: float, 
     info = {"init_idx": init_idx, "init_cost": float(init_cost), "num_iters": num_iters,
             "candidates": centroids, "weights": weights, "kmex_iters": n_it, "oversampling": oversampling}
     return centers, info
+
+
+# --------------------------------------------------------------------------------------------------
+# k-medians / k-medoids (Manhattan metric)
+# --------------------------------------------------------------------------------------------------
+def manhattan(x: torch.Tensor, y: torch.Tensor, expand: bool = False) -> torch.Tensor:
+    """heat/spatial/distance.py:106-133: torch.cdist(p=1), or the broadcast form with ``expand``."""
+    if expand:
+        return torch.sum(torch.abs(x.unsqueeze(1) - y.unsqueeze(0)), dim=2)
+    return torch.cdist(x, y, p=1)
+
+
+def assign_l1(x: torch.Tensor, centers: torch.Tensor, chunk: int = 1 << 12) -> Tuple[torch.Tensor, torch.Tensor]:
+    """_KCluster._assign_to_cluster with the metric of KMedians / KMedoids (manhattan, expand=True);
+    returns labels (N, 1) int64 and the minimum distances (N,)."""
+    labs, mins = [], []
+    for i0 in range(0, x.shape[0], chunk):
+        v, i = torch.min(manhattan(x[i0 : i0 + chunk], centers, expand=True), dim=1, keepdim=True)
+        labs.append(i)
+        mins.append(v.view(-1))
+    return torch.cat(labs), torch.cat(mins)
+
+
+def heat_median_axis0(a: torch.Tensor) -> torch.Tensor:
+    """
+    ht.median(a, axis=0) = percentile 50 with linear interpolation, heat/core/statistics.py:1460-1718:
+    sort, index q/100 * (n - 1) as a float32 tensor, floors + (ceils - floors) * fraction in the
+    (float64, see update_medians) dtype of the data.
+    """
+    n = a.shape[0]
+    sorted_a, _ = torch.sort(a, dim=0)
+    perc = torch.tensor(50) / 100 * (n - 1)
+    lo, hi = sorted_a[perc.floor().type(torch.int)], sorted_a[perc.ceil().type(torch.int)]
+    return lo + (hi - lo) * (perc - perc.floor())
+
+
+def update_medians(x: torch.Tensor, labels: torch.Tensor, centers: torch.Tensor, sampler,
+                   snap_to_sample: bool = False) -> torch.Tensor:
+    """
+    KMedians._update_centroids (heat/cluster/kmedians.py:60-118) and, with ``snap_to_sample``,
+    KMedoids._update_centroids (heat/cluster/kmedoids.py:57-115).  ``x * selection`` is float64
+    (heat/core/types.py promotes float32 * int64), rows whose absolute sum is zero are dropped, an
+    empty cluster restarts at a random row, the result is stored into the float32 centres.
+    """
+    new_centers = centers.clone()
+    k = centers.shape[0]
+    for i in range(k):
+        selection = (labels == i).to(torch.int64)
+        assigned = x.to(torch.float64) * selection
+        rows = assigned.abs().sum(dim=1) != 0
+        clean = assigned[rows]
+        if clean.shape[0] == 0:
+            new_centers[i, :] = x[sampler.randint(x.shape[0])]
+        else:
+            median = heat_median_axis0(clean).reshape(1, -1)
+            if snap_to_sample:
+                dist = manhattan(x.to(torch.float64), median, expand=True)
+                idx = int(torch.argmin(dist, dim=0))
+                new_centers[i, :] = x[idx]
+            else:
+                new_centers[i : i + 1, :] = median.to(centers.dtype)
+    return new_centers
+
+
+def kmedians_fit(x: torch.Tensor, init_centers: torch.Tensor, max_iter: int, tol: Optional[float], sampler):
+    """KMedians.fit with explicit initial centroids (heat/cluster/kmedians.py:120-147)."""
+    centers = init_centers.clone()
+    n_iter, labels, inertia = 0, None, None
+    for _ in range(max_iter):
+        n_iter += 1
+        labels, _d = assign_l1(x, centers)
+        new_centers = update_medians(x, labels, centers, sampler)
+        inertia = ((centers - new_centers) ** 2).sum()
+        centers = new_centers.clone()
+        if tol is not None and bool(inertia <= tol):
+            break
+    return {"cluster_centers": centers, "labels": labels, "inertia": inertia, "n_iter": n_iter}
+
+
+def kmedoids_fit(x: torch.Tensor, init_centers: torch.Tensor, max_iter: int, sampler):
+    """KMedoids.fit with explicit initial centroids (heat/cluster/kmedoids.py:117-156)."""
+    centers = init_centers.clone()
+    n_iter, labels = 0, None
+    for _ in range(max_iter):
+        n_iter += 1
+        labels, _d = assign_l1(x, centers)
+        new_centers = update_medians(x, labels, centers, sampler, snap_to_sample=True)
+        if torch.equal(centers, new_centers):
+            break
+        centers = new_centers.clone()
+    return {"cluster_centers": centers, "labels": labels, "n_iter": n_iter}
+
+
+def label_agreement_l1(x: torch.Tensor, centers: torch.Tensor, lab_a: torch.Tensor, lab_b: torch.Tensor,
+                       rel_gap: float = 1e-5) -> dict:
+    """Like label_agreement for the Manhattan metric: a difference is excused when both chosen
+    centres lie within rel_gap * best + D * eps32 * (|x|_1 + |c|_1) of the best fp64 distance."""
+    a, b = lab_a.view(-1).long(), lab_b.view(-1).long()
+    diff = torch.nonzero(a != b).view(-1)
+    out = {"n": int(a.numel()), "n_diff": int(diff.numel()), "n_unexcused": 0,
+           "agreement": 1.0 - diff.numel() / max(1, a.numel())}
+    if diff.numel():
+        xd = x[diff].double()
+        d = (xd.unsqueeze(1) - centers.double().unsqueeze(0)).abs().sum(2)
+        best = d.min(1).values
+        mag = xd.abs().sum(1) + centers.double().abs().sum(1).max()
+        tol = rel_gap * best + x.shape[1] * 1.2e-7 * mag
+        da, db = d.gather(1, a[diff].view(-1, 1)).view(-1), d.gather(1, b[diff].view(-1, 1)).view(-1)
+        out["n_unexcused"] = int(((da - best > tol) | (db - best > tol)).sum())
+    return out

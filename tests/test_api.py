@@ -159,7 +159,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) >= 16
+    assert len(names) >= 19
     for name in names:
         assert hasattr(lib, name), name
         assert name in _native.SIGNATURES, f"{name} has no ctypes signature"
@@ -230,6 +230,20 @@ def test_argument_validation_happens_on_the_host():
     assert lib.hkm_sample_select_f32(good, good, 8, good, 2.0, good, 4, None, ws, big, None) == _native.HKM_EINVAL
     assert lib.hkm_label_counts_i64(good, 8, 0, good, None) == _native.HKM_EINVAL
     assert lib.hkm_label_counts_i64(None, 8, 4, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_l1_f32(None, 10, 3, 3, good, 8, 3, good, None, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_l1_f32(good, 10, 3, 2, good, 8, 3, good, None, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_l1_f32(good, 10, 3, 3, good, 8, 3, None, None, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_l1_f32(good, 0, 3, 3, good, 8, 3, None, None, None) == _native.HKM_OK
+    assert lib.hkm_closest_rows_l1_f32(good, 0, 3, 3, good, 2, 3, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert "empty" in err()
+    assert lib.hkm_closest_rows_l1_f32(good, 10, 3, 3, good, 2, 3, None, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_closest_rows_l1_f32(good, 10, 3, 3, good, 2, 3, good, None, ws, 16, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_update_median_f32(good, 10, 3, 3, good, 4, None, None, good, 3, None, 2, 0, ws, big, None) == _native.HKM_EINVAL
+    assert "mode" in err()
+    assert lib.hkm_update_median_f32(good, 10, 3, 3, None, 4, None, None, good, 3, None, 0, 0, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_update_median_f32(good, 10, 3, 3, good, 4, None, None, good, 2, None, 0, 0, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_update_median_f32(good, 10, 3, 3, good, 4, None, None, good, 3, None, 0, 0, ws, 64, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_update_median_f32(good, 1 << 31, 3, 3, good, 4, None, None, good, 3, None, 0, 0, ws, big, None) == _native.HKM_EUNSUPPORTED
     assert lib.hkm_functional_value_f32(good, -1, good, ws, big, None) == _native.HKM_EINVAL
     # zero-sized problems succeed without touching the device
     assert lib.hkm_widen_labels_i64(good, 0, good, None) == _native.HKM_OK
@@ -277,3 +291,31 @@ def test_batchparallel_kmeans_surface():
         ht.cluster.BatchParallelKMeans(n_clusters=2).fit(ht.array(torch.rand(16, 2), split=0))
     with pytest.raises(RuntimeError):
         ht.cluster.KMeans(n_clusters=2, init="probability_based").fit(ht.array(torch.rand(16, 2), split=0))
+
+
+def test_manhattan_estimators_surface():
+    # tests/cluster/test_kmedians.py / test_kmedoids.py of the reference: protocol and parameters
+    kmed = ht.cluster.KMedians()
+    assert ht.is_estimator(kmed) and ht.is_clusterer(kmed)
+    assert kmed.get_params() == {"n_clusters": 8, "init": "random", "max_iter": 300, "tol": 1e-4, "random_state": None}
+    kmedoid = ht.cluster.KMedoids()
+    assert ht.is_estimator(kmedoid) and ht.is_clusterer(kmedoid)
+    params = kmedoid.get_params()
+    assert params == {"n_clusters": 8, "init": "random", "max_iter": 300, "random_state": None}
+    params["n_clusters"] = 10
+    kmedoid.set_params(**params)
+    assert kmedoid.n_clusters == 10 and kmedoid.tol == 0.0
+    assert ht.cluster.KMedians(init="kmedians++").init == "probability_based"
+    assert ht.cluster.KMedoids(init="kmedoids++").init == "probability_based"
+    bp = ht.cluster.BatchParallelKMedians()
+    assert bp.get_params()["init"] == "k-medians++" and bp._p == 1
+    with pytest.raises(NotImplementedError):
+        ht.cluster.BatchParallelKMedians(init="random")
+    with pytest.raises(ValueError):
+        ht.cluster.BatchParallelKMedians(init="k-means++")
+    host = ht.array(torch.rand(16, 2), split=0)
+    for est in (ht.cluster.KMedians(n_clusters=2), ht.cluster.KMedoids(n_clusters=2),
+                ht.cluster.BatchParallelKMedians(n_clusters=2)):
+        with pytest.raises(RuntimeError):  # host data is refused, never computed on the CPU
+            est.fit(host)
+    assert _native.workspace_bytes(1000, 4, 8, _native.WS_MEDIAN) > 8 * 4 * 256 * 4

@@ -334,3 +334,80 @@ def test_kmeans_parallel_init_composition():
     tiny = torch.ones((50, 2))
     with pytest.raises(ValueError):
         orc.kmeans_parallel_init(tiny, 3, 2.0, 1.0, 10, 1e-4, orc.CpuSampler(0))
+
+
+# ---- k-medians / k-medoids ------------------------------------------------------------------------
+def test_manhattan_known_answers_and_scipy():
+    from scipy.spatial.distance import cdist as sp_cdist
+
+    X, Y = torch.ones((8, 4)), torch.zeros((8, 4))
+    for expand in (False, True):  # tests/spatial/test_distances.py:20-23,42-48,67-73
+        assert torch.equal(orc.manhattan(X, X, expand), torch.zeros((8, 8)))
+        assert torch.equal(orc.manhattan(X, Y, expand), torch.full((8, 8), 4.0))
+    g = torch.Generator().manual_seed(3)
+    a, b = torch.randn((50, 7), generator=g), torch.randn((20, 7), generator=g)
+    ref = torch.from_numpy(sp_cdist(a.double().numpy(), b.double().numpy(), metric="cityblock"))
+    for expand in (False, True):
+        assert torch.allclose(orc.manhattan(a, b, expand).double(), ref, rtol=1e-5, atol=1e-5)
+    lab, dmin = orc.assign_l1(a, b)
+    assert lab.shape == (50, 1) and torch.equal(lab.view(-1), ref.argmin(1))
+    assert torch.allclose(dmin.double(), ref.min(1).values, rtol=1e-5)
+
+
+def test_heat_median_is_numpy_median():
+    g = torch.Generator().manual_seed(8)
+    for n in (1, 2, 3, 10, 11, 64):
+        a = torch.randn((n, 5), generator=g, dtype=torch.float64)
+        assert np.allclose(orc.heat_median_axis0(a).numpy(), np.median(a.numpy(), axis=0), rtol=0, atol=1e-15)
+    a = torch.tensor([[1.0], [7.0], [3.0], [5.0]], dtype=torch.float64)
+    assert float(orc.heat_median_axis0(a)) == 4.0  # mean of the two middle values 3 and 5
+    assert float(orc.heat_median_axis0(a[:3])) == 3.0
+
+
+def test_update_medians_rules():
+    x = torch.tensor([[1.0, 10.0], [2.0, 30.0], [0.0, 0.0], [4.0, 20.0], [100.0, 100.0], [0.0, 0.0]])
+    lab = torch.tensor([0, 0, 0, 0, 1, 2]).view(-1, 1)
+    c_old = torch.zeros((3, 2))
+    smp = _RecordingSampler(0, first=4)
+    c = orc.update_medians(x, lab, c_old, smp)
+    # cluster 0: the all-zero row 2 is dropped -> median of {1, 2, 4} and {10, 30, 20}
+    assert torch.equal(c[0], torch.tensor([2.0, 20.0]))
+    assert torch.equal(c[1], x[4])
+    # cluster 2 holds only an all-zero row -> treated as empty -> restart at the drawn row (4)
+    assert torch.equal(c[2], x[4])
+    # even count: mean of the middles, computed in float64 and rounded once
+    x2 = torch.tensor([[1.0], [2.0], [1e-8], [3.0]])
+    c2 = orc.update_medians(x2, torch.zeros((4, 1), dtype=torch.long), torch.zeros((1, 1)), smp)
+    assert float(c2[0, 0]) == np.float32((1.0 + 2.0) / 2)
+    # medoid: a data row, at minimal Manhattan distance from the median among ALL rows
+    g = torch.Generator().manual_seed(4)
+    xs = torch.randn((200, 3), generator=g)
+    labs = torch.randint(0, 4, (200, 1), generator=g)
+    med = orc.update_medians(xs, labs, torch.zeros((4, 3)), smp)
+    snap = orc.update_medians(xs, labs, torch.zeros((4, 3)), smp, snap_to_sample=True)
+    for k in range(4):
+        d = (xs.double() - med[k].double()).abs().sum(1)
+        assert bool((xs == snap[k]).all(1).any())
+        assert float((snap[k].double() - med[k].double()).abs().sum()) <= float(d.min()) + 1e-6
+
+
+def test_kmedians_and_kmedoids_closed_forms():
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((301, 4), generator=g) + 3.0
+    smp = orc.CpuSampler(0)
+    # K = 1: one iteration lands on the coordinate-wise median, the second finds no movement
+    r = orc.kmedians_fit(x, x[:1].clone(), 10, 0.0, smp)
+    assert r["n_iter"] == 2 and torch.allclose(r["cluster_centers"][0], x.median(0).values)
+    r = orc.kmedoids_fit(x, x[:1].clone(), 10, smp)
+    d = (x - x.median(0).values).abs().sum(1)
+    assert torch.equal(r["cluster_centers"][0], x[int(d.argmin())])
+    # two far blobs: medians of the blobs, every point with its blob
+    x2 = torch.cat([x, x + 50.0])
+    r = orc.kmedians_fit(x2, x2[[0, 301]].clone(), 10, 0.0, smp)
+    assert torch.allclose(r["cluster_centers"][0], x.median(0).values)
+    assert torch.allclose(r["cluster_centers"][1], (x + 50.0).median(0).values)
+    assert torch.equal(r["labels"].view(-1), torch.cat([torch.zeros(301), torch.ones(301)]).long())
+    # k-medians flavour of the local Lloyd helper: lower median, empty cluster keeps its centre
+    far = torch.cat([x2[[0, 301]], torch.full((1, 4), 1e4)])
+    c, _ = orc.kmex(x2, 3, far.clone(), 20, 1e-4, p=1)
+    assert torch.equal(c[2], far[2]) and torch.equal(c[0], torch.median(x, dim=0)[0])
