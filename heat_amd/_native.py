@@ -18,7 +18,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "li
 _lib: Optional[ctypes.CDLL] = None
 
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
-WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN = 1, 2, 3, 4, 8
+WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64 = 1, 2, 3, 4, 8, 16
 
 # name -> (restype, argtypes); must list every symbol declared in include/hkm.h
 SIGNATURES = {
@@ -50,6 +50,16 @@ SIGNATURES = {
     "hkm_update_median_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                              c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p,
                                              c_size_t, c_void_p]),
+    "hkm_assign_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                      c_void_p, c_void_p, c_void_p]),
+    "hkm_update_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
+                                      c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_lloyd_step_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_shift_f64": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
+    "hkm_functional_value_f64": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_pairwise_f64": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
+                                        c_void_p, c_int64, c_int32, ctypes.c_double, c_void_p]),
     "hkm_widen_labels_i64": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
 }
 
@@ -133,11 +143,23 @@ def lloyd_kernel_name(n: int, d: int, k: int) -> str:
     return load().hkm_lloyd_kernel_name(n, d, k).decode()
 
 
+def _is_f64(*tensors: Optional[torch.Tensor]) -> bool:
+    """True if the floating-point operands are float64 (all of them must then be)."""
+    kinds = {t.dtype for t in tensors if t is not None and t.dtype in (torch.float32, torch.float64)}
+    if len(kinds) > 1:
+        raise TypeError("float32 and float64 operands cannot be mixed")
+    return kinds == {torch.float64}
+
+
 def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optional[torch.Tensor],
            ws: Workspace) -> None:
     _require_gpu(x, c, labels, min_d2)
     n, d = x.shape
     k = c.shape[0]
+    if _is_f64(x, c, min_d2):
+        check(load().hkm_assign_f64(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
+                                    c.stride(0) if k > 1 else d, _ptr(labels), _ptr(min_d2), _stream()))
+        return
     need = workspace_bytes(n, d, k, WS_ASSIGN)
     buf = ws.get(need)
     check(load().hkm_assign_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k, c.stride(0) if k > 1 else d,
@@ -149,6 +171,11 @@ def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: O
     _require_gpu(x, labels, c_new, counts)
     n, d = x.shape
     k = c_new.shape[0]
+    if _is_f64(x, c_new):
+        buf = ws.get(workspace_bytes(n, d, k, WS_UPDATE | WS_F64))
+        check(load().hkm_update_f64(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k, _ptr(c_new),
+                                    c_new.stride(0) if k > 1 else d, _ptr(counts), _ptr(buf), buf.numel(), _stream()))
+        return
     need = workspace_bytes(n, d, k, WS_UPDATE)
     buf = ws.get(need)
     check(load().hkm_update_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k, _ptr(c_new),
@@ -164,6 +191,12 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: to
         raise RuntimeError("shift must live on the GPU or in pinned host memory")
     n, d = x.shape
     k = c.shape[0]
+    if _is_f64(x, c, c_new, shift, sse):
+        flags = WS_LLOYD | WS_F64 | (WS_SSE if sse is not None else 0)
+        buf = ws.get(workspace_bytes(n, d, k, flags))
+        check(load().hkm_lloyd_step_f64(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
+                                        _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
+        return
     flags = WS_LLOYD | (WS_SSE if sse is not None else 0)
     need = workspace_bytes(n, d, k, flags)
     buf = ws.get(need)
@@ -174,6 +207,9 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: to
 def shift(c_old: torch.Tensor, c_new: torch.Tensor, out: torch.Tensor) -> None:
     _require_gpu(c_old, c_new, out)
     k, d = c_old.shape
+    if _is_f64(c_old, c_new, out):
+        check(load().hkm_shift_f64(_ptr(c_old), _ptr(c_new), k, d, _ptr(out), _stream()))
+        return
     check(load().hkm_shift_f32(_ptr(c_old), _ptr(c_new), k, d, _ptr(out), _stream()))
 
 
@@ -182,6 +218,9 @@ def functional_value(min_d2: torch.Tensor, out: torch.Tensor, ws: Workspace) -> 
     n = min_d2.numel()
     need = workspace_bytes(n, 1, 1, WS_ASSIGN)
     buf = ws.get(need)
+    if _is_f64(min_d2, out):
+        check(load().hkm_functional_value_f64(_ptr(min_d2), n, _ptr(out), _ptr(buf), buf.numel(), _stream()))
+        return
     check(load().hkm_functional_value_f32(_ptr(min_d2), n, _ptr(out), _ptr(buf), buf.numel(), _stream()))
 
 
@@ -200,6 +239,11 @@ def pairwise(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, metric: int, s
     _require_gpu(x, y, out)
     m, d = x.shape
     nn = y.shape[0]
+    if _is_f64(x, y, out):
+        check(load().hkm_pairwise_f64(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn,
+                                      y.stride(0) if nn > 1 else d, d, _ptr(out), out.stride(0) if m > 1 else nn,
+                                      metric, float(sigma), _stream()))
+        return
     check(load().hkm_pairwise_f32(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn,
                                   y.stride(0) if nn > 1 else d, d, _ptr(out), out.stride(0) if m > 1 else nn,
                                   metric, float(sigma), _stream()))

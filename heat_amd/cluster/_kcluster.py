@@ -37,6 +37,7 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         self._inertia = None
         self._n_iter = None
         self._p = None
+        self._l1_metric = False
         self._ws = None
 
     # ---- read-only results (heat/cluster/_kcluster.py:63-98) -----------------------------------
@@ -68,25 +69,34 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         return self._ws
 
     @staticmethod
-    def _local_f32(x: DNDarray) -> torch.Tensor:
-        """The local tensor as a row-major float32 matrix (ints are widened as the reference's
-        promote(X, C, float32) does; float64 is outside the float32 kernels)."""
+    def _local_f32(x: DNDarray, like: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The local tensor as a row-major matrix in the compute dtype: float32, or float64 where the
+        reference's promote(X, C, float32) gives float64 (float64 and int64 data).  ``like`` forces the
+        dtype of another operand (centroids follow the data)."""
         t = x.larray
         if t.dim() != 2:
             raise NotImplementedError("Only 2D data matrices are currently supported")
-        if t.dtype == torch.float64 or types.promote_types(x.dtype, types.float32) is not types.float32:
-            raise NotImplementedError(
-                f"the gfx950 kernels compute in float32; input dtype {x.dtype.__name__} promotes to float64"
-            )
-        if t.dtype != torch.float32:
-            t = t.to(torch.float32)
+        want = torch.float64 if types.promote_types(x.dtype, types.float32) is types.float64 else torch.float32
+        if like is not None:
+            want = like.dtype
+        if t.dtype != want:
+            t = t.to(want)
         if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
             t = t.contiguous()
         return t
 
+    def _local_f32_only(self, x: DNDarray) -> torch.Tensor:
+        """The local matrix for the kernels that exist in float32 only (Manhattan metric, medians)."""
+        t = self._local_f32(x)
+        if t.dtype != torch.float32:
+            raise NotImplementedError(
+                f"{type(self).__name__} is built for float32 data; {x.dtype.__name__} input promotes to float64"
+            )
+        return t
+
     def _manhattan_metric(self) -> bool:
-        """True for the estimators constructed with the Manhattan metric (KMedians, KMedoids)."""
-        return type(self).__name__ in ("KMedians", "KMedoids")
+        """True for the estimators constructed with the Manhattan metric (KMedians, KMedoids set it)."""
+        return self._l1_metric
 
     @staticmethod
     def _check_split(x: DNDarray) -> None:
@@ -130,7 +140,8 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         elif isinstance(self.init, str) and self.init == "probability_based":
             if x.split is None or x.split == 0:
                 cent = self._kmeans_parallel(x, oversampling, iter_multiplier)
-                self._cluster_centers = DNDarray(cent, tuple(cent.shape), types.float32, None, x.device, x.comm, True)
+                self._cluster_centers = DNDarray(cent, tuple(cent.shape), types.canonical_heat_type(cent.dtype), None,
+                                                 x.device, x.comm, True)
             else:
                 raise NotImplementedError("Not implemented for other splitting-axes")
         elif isinstance(self.init, str) and self.init == "batchparallel":
@@ -176,12 +187,13 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         n = xt.shape[0]
         dev = xt.device
         lab = torch.empty((n,), dtype=torch.int32, device=dev)
-        d2 = torch.empty((n,), dtype=torch.float32, device=dev)
+        dmin = torch.empty((n,), dtype=xt.dtype, device=dev)
         cost = torch.empty((), dtype=torch.float32, device=dev)
         count = torch.zeros((), dtype=torch.int64, device=dev)
         idx = torch.empty((max(1024, int(16 * oversampling)),), dtype=torch.int64, device=dev)
         for _ in range(num_iters):
-            _native.assign(xt, centroids, lab, d2, ws)
+            _native.assign(xt, centroids, lab, dmin, ws)
+            d2 = dmin if dmin.dtype == torch.float32 else dmin.float()  # the draw itself runs in float32
             _native.min_dist_sum(d2, cost, ws)
             u = sampler.uniform(n)
             _native.sample_select(d2, u, cost, oversampling, idx, count, ws)
@@ -205,10 +217,10 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         first = sampler.randint(max(n - 1, 1))
         init_centroids = xt[first : first + 1].clone()
         lab = torch.empty((n,), dtype=torch.int32, device=dev)
-        d2 = torch.empty((n,), dtype=torch.float32, device=dev)
+        dmin = torch.empty((n,), dtype=xt.dtype, device=dev)
         cost = torch.empty((), dtype=torch.float32, device=dev)
-        _native.assign(xt, init_centroids, lab, d2, ws)
-        _native.min_dist_sum(d2, cost, ws)
+        _native.assign(xt, init_centroids, lab, dmin, ws)
+        _native.min_dist_sum(dmin if dmin.dtype == torch.float32 else dmin.float(), cost, ws)
         init_cost = float(cost.item())
         # the order of magnitude of the initial cost sets the number of rounds (_kcluster.py:172-175);
         # all rows equal gives cost 0, where the reference fails in int(-inf): one round instead
@@ -243,14 +255,16 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         """
         self._check_split(x)
         xt = self._local_f32(x)
-        ct = self._local_f32(self._cluster_centers)
+        if self._manhattan_metric() and xt.dtype != torch.float32:
+            raise NotImplementedError("the Manhattan-metric kernels cover float32 data only")
+        ct = self._local_f32(self._cluster_centers, like=xt)
         if xt.shape[1] != ct.shape[1]:
             raise ValueError("Inputs must have same shape[1]")
         dev = xt.device
         n = xt.shape[0]
         ws = self._workspace(dev)
         lab32 = torch.empty((n,), dtype=torch.int32, device=dev)
-        min_d2 = torch.empty((n,), dtype=torch.float32, device=dev) if eval_functional_value else None
+        min_d2 = torch.empty((n,), dtype=xt.dtype, device=dev) if eval_functional_value else None
         if self._manhattan_metric():
             # k-medians / k-medoids: fused sum|x - c| + argmin; the functional is the squared 2-norm of
             # the minimum distances, so they are squared before the same reduction
@@ -262,9 +276,10 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         _native.widen_labels(lab32, lab64)
         if eval_functional_value:
-            fv = torch.empty((), dtype=torch.float32, device=dev)
+            fv = torch.empty((), dtype=xt.dtype, device=dev)
             _native.functional_value(min_d2, fv, ws)
-            self._functional_value = DNDarray(fv, (), types.float32, None, x.device, x.comm, True)
+            self._functional_value = DNDarray(fv, (), types.canonical_heat_type(xt.dtype), None, x.device, x.comm,
+                                              True)
         return DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
 
     def _update_centroids(self, x: DNDarray, matching_centroids: DNDarray):

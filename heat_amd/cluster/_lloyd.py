@@ -28,7 +28,7 @@ class LloydLoop:
         self.ws = ws
         self.c = [c0.clone(), torch.empty_like(c0), torch.empty_like(c0)]
         self.lab = [torch.empty((xt.shape[0],), dtype=torch.int32, device=dev) for _ in range(2)]
-        self.shift_host = torch.zeros((2,), dtype=torch.float32, pin_memory=True)
+        self.shift_host = torch.zeros((2,), dtype=xt.dtype, pin_memory=True)
         self.ev = [torch.cuda.Event(), torch.cuda.Event()]
         self.enqueued = 0  # steps handed to the stream
         self.done = 0      # steps whose results count

@@ -25,7 +25,7 @@ from ._sampling import DeviceSampler
 def _dist_to_row(x: torch.Tensor, row: torch.Tensor, p: int) -> torch.Tensor:
     """Distance of every row of x to one row: sqrt(sum((x_i - row)^2)) for p = 2 (direct form: exactly
     zero for the row itself, which a quadratic expansion does not guarantee), sum|x_i - row| for p = 1."""
-    out = torch.empty((x.shape[0], 1), dtype=torch.float32, device=x.device)
+    out = torch.empty((x.shape[0], 1), dtype=x.dtype, device=x.device)
     _native.pairwise(x, row.reshape(1, -1).contiguous(), out,
                      _native.METRIC_MANHATTAN if p == 1 else _native.METRIC_EUCLID)
     return out.view(-1)
@@ -68,7 +68,7 @@ def _kmex(x: torch.Tensor, p: int, n_clusters: int, init: Union[str, torch.Tenso
     if isinstance(init, torch.Tensor):
         if init.shape != (n_clusters, x.shape[1]):
             raise ValueError("if a torch tensor, init must have shape (n_clusters, n_features).")
-        centers = init.to(torch.float32).contiguous()
+        centers = init.to(x.dtype).contiguous()
     elif init == "++":
         centers = _initialize_plus_plus(x, n_clusters, p, sampler, weights, ws=ws)
     elif init == "random":
@@ -153,11 +153,13 @@ class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
         seed = None if self.random_state is None else self.random_state + rank
         return DeviceSampler(device, seed)
 
-    @staticmethod
-    def _local_f32(x: DNDarray) -> torch.Tensor:
+    def _local_f32(self, x: DNDarray) -> torch.Tensor:
+        """Local rows in the compute dtype: float64 stays float64 for k-means, everything else float32."""
         t = x.larray
         if t.dtype == torch.float64:
-            raise NotImplementedError("the gfx950 kernels compute in float32; float64 input is not supported")
+            if self._p == 1:
+                raise NotImplementedError("the Manhattan-metric kernels cover float32 data only")
+            return t.contiguous()
         if t.dtype != torch.float32:
             t = t.to(torch.float32)
         return t.contiguous()
@@ -175,8 +177,8 @@ class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
             self._ws = _native.Workspace(xt.device)
         centers, n_iter = _kmex(xt, self._p, self.n_clusters, self._init, self.max_iter, self.tol,
                                 self._make_sampler(xt.device, x.comm.rank), ws=self._ws)
-        self._cluster_centers = DNDarray(centers, (self.n_clusters, x.shape[1]), types.float32, None, x.device,
-                                         x.comm, True)
+        self._cluster_centers = DNDarray(centers, (self.n_clusters, x.shape[1]),
+                                         types.canonical_heat_type(centers.dtype), None, x.device, x.comm, True)
         self._n_iter = n_iter
         return self
 
@@ -199,16 +201,16 @@ class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
             self._ws = _native.Workspace(xt.device)
         n = xt.shape[0]
         lab = torch.empty((n, 1), dtype=torch.int32, device=xt.device)
-        d2 = torch.empty((n,), dtype=torch.float32, device=xt.device)
-        fv = torch.empty((), dtype=torch.float32, device=xt.device)
+        d2 = torch.empty((n,), dtype=xt.dtype, device=xt.device)
+        fv = torch.empty((), dtype=xt.dtype, device=xt.device)
         if self._p == 1:
             # sum of the Manhattan distances to the closest centre: min_dist_sum adds sqrt(v), so it is
             # fed the squared distances
-            _native.assign_l1(xt, self._cluster_centers.larray, lab.view(-1), d2)
+            _native.assign_l1(xt, self._cluster_centers.larray.to(xt.dtype), lab.view(-1), d2)
             _native.min_dist_sum(d2.mul_(d2), fv, self._ws)
         else:
             # ||x - C[labels]||_F ** 2 = sum of the squared distances to the closest centre
-            _native.assign(xt, self._cluster_centers.larray, lab.view(-1), d2, self._ws)
+            _native.assign(xt, self._cluster_centers.larray.to(xt.dtype), lab.view(-1), d2, self._ws)
             _native.functional_value(d2, fv, self._ws)
         self._functional_value = fv.item()
         return DNDarray(lab, (n, 1), types.int32, x.split, x.device, x.comm, x.balanced)

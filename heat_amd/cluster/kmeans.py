@@ -56,9 +56,9 @@ class KMeans(_KCluster):
         xt = self._local_f32(x)
         lab = matching_centroids.larray.reshape(-1).to(torch.int32)
         k = self.n_clusters
-        c_new = torch.empty((k, xt.shape[1]), dtype=torch.float32, device=xt.device)
+        c_new = torch.empty((k, xt.shape[1]), dtype=xt.dtype, device=xt.device)
         _native.update(xt, lab, c_new, None, self._workspace(xt.device))
-        return DNDarray(c_new, tuple(c_new.shape), types.float32, None, x.device, x.comm, True)
+        return DNDarray(c_new, tuple(c_new.shape), types.canonical_heat_type(xt.dtype), None, x.device, x.comm, True)
 
     def fit(self, x: DNDarray, oversampling: float = 2, iter_multiplier: float = 1) -> "KMeans":
         """
@@ -79,7 +79,7 @@ class KMeans(_KCluster):
         k = self.n_clusters
         # the reference evaluates ``inertia <= tol`` on the host every iteration (kmeans.py:143); the
         # loop keeps the next step enqueued while the host looks at the shift of the current one
-        loop = LloydLoop(xt, self._local_f32(self._cluster_centers), self._workspace(dev))
+        loop = LloydLoop(xt, self._local_f32(self._cluster_centers, like=xt), self._workspace(dev))
         self._n_iter = loop.run(self.max_iter, self.tol)
         if self._n_iter == 0:
             raise ValueError(f"max_iter must be positive, but was {self.max_iter}")
@@ -87,7 +87,8 @@ class KMeans(_KCluster):
 
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         _native.widen_labels(lab32, lab64)
-        self._cluster_centers = DNDarray(c_cur, (k, d), types.float32, None, x.device, x.comm, True)
-        self._inertia = DNDarray(shift.clone(), (), types.float32, None, x.device, x.comm, True)
+        ftype = types.canonical_heat_type(xt.dtype)
+        self._cluster_centers = DNDarray(c_cur, (k, d), ftype, None, x.device, x.comm, True)
+        self._inertia = DNDarray(shift.clone(), (), ftype, None, x.device, x.comm, True)
         self._labels = DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
         return self

@@ -34,6 +34,7 @@ class KMedians(_KCluster):
             random_state=random_state,
         )
         self._p = 1
+        self._l1_metric = True
 
     def _median_step(self, xt: torch.Tensor, lab32: torch.Tensor, centers: torch.Tensor, sampler) -> torch.Tensor:
         """
@@ -50,9 +51,9 @@ class KMedians(_KCluster):
         return c_new
 
     def _update_centroids(self, x: DNDarray, matching_centroids: DNDarray) -> DNDarray:
-        xt = self._local_f32(x)
+        xt = self._local_f32_only(x)
         lab = matching_centroids.larray.reshape(-1).to(torch.int32)
-        c_new = self._median_step(xt, lab, self._local_f32(self._cluster_centers), self._make_sampler(xt.device))
+        c_new = self._median_step(xt, lab, self._local_f32(self._cluster_centers, like=xt), self._make_sampler(xt.device))
         return DNDarray(c_new, tuple(c_new.shape), types.float32, None, x.device, x.comm, True)
 
     def fit(self, x: DNDarray, oversampling: float = 2, iter_multiplier: float = 1) -> "KMedians":
@@ -62,11 +63,11 @@ class KMedians(_KCluster):
         self._initialize_cluster_centers(x, oversampling, iter_multiplier)
         self._n_iter = 0
         self._check_split(x)
-        xt = self._local_f32(x)
+        xt = self._local_f32_only(x)
         dev = xt.device
         n, d = xt.shape
         sampler = self._make_sampler(dev)
-        centers = self._local_f32(self._cluster_centers).clone()
+        centers = self._local_f32(self._cluster_centers, like=xt).clone()
         lab32 = torch.empty((n,), dtype=torch.int32, device=dev)
         shift = torch.zeros((), dtype=torch.float32, device=dev)
         if self.max_iter <= 0:

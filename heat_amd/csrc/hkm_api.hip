@@ -68,21 +68,24 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         if (assign_kind(D, K) == ASSIGN_MFMA_STREAM)
             w.keys = reinterpret_cast<unsigned long long*>(take(size_t(N < 1 ? 1 : N) * sizeof(unsigned long long)));
     }
-    if ((flags & HKM_WS_UPDATE) && small_eligible(D, K))
+    if ((flags & HKM_WS_UPDATE) && !(flags & HKM_WS_F64) && small_eligible(D, K))
         w.small_part = reinterpret_cast<double*>(take(size_t(SMALL_MAX_GRID) * (size_t(K) * (D + 1) + 1) * sizeof(double)));
     if (flags & HKM_WS_UPDATE) {
-        const UpdateGeom g = update_geom(N, D, K);
-        w.part_sum = reinterpret_cast<float*>(take(size_t(g.S) * K * g.J * 32 * sizeof(float)));
+        const size_t elem = (flags & HKM_WS_F64) ? sizeof(double) : sizeof(float);
+        const UpdateGeom g = update_geom(N, D, K, int32_t(elem));
+        w.part_sum = reinterpret_cast<float*>(take(size_t(g.S) * K * g.J * 32 * elem));
         w.part_cnt = reinterpret_cast<int32_t*>(take(size_t(g.S) * K * sizeof(int32_t)));
         w.counts = reinterpret_cast<int64_t*>(take(size_t(K) * sizeof(int64_t)));
         w.shift_part = reinterpret_cast<double*>(take((size_t(K) * D / 64 + 1) * sizeof(double)));
     }
-    if ((flags & HKM_WS_LLOYD) == HKM_WS_LLOYD && fused_eligible(D, K)) {
+    if ((flags & HKM_WS_LLOYD) == HKM_WS_LLOYD && !(flags & HKM_WS_F64) && fused_eligible(D, K)) {
         w.fsum = reinterpret_cast<double*>(take(size_t(FUSED_MAX_GRID) * K * D * sizeof(double)));
         w.fcnt = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * K * sizeof(int32_t)));
         w.fflags = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * sizeof(int32_t)));
     }
-    if (flags & HKM_WS_SSE) w.min_d2 = reinterpret_cast<float*>(take(size_t(N < 1 ? 1 : N) * sizeof(float)));
+    if (flags & HKM_WS_SSE)
+        w.min_d2 = reinterpret_cast<float*>(
+            take(size_t(N < 1 ? 1 : N) * ((flags & HKM_WS_F64) ? sizeof(double) : sizeof(float))));
     w.total = off;
     return w;
 }
@@ -323,6 +326,107 @@ int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* c
     if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
     if ((N > 0 && !labels) || !counts) return fail(HKM_EINVAL, "NULL pointer argument");
     return launch_label_counts(labels, N, K, counts, static_cast<hipStream_t>(hip_stream));
+}
+
+// ---- float64 data -----------------------------------------------------------------------------
+static int check_matrix64(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
+    if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);
+    if (reinterpret_cast<uintptr_t>(p) & 7u) return fail(HKM_EINVAL, "%s is not 8-byte aligned", name);
+    if (ld < cols) return fail(HKM_EINVAL, "leading dimension of %s (%lld) < columns (%d)", name, (long long)ld, cols);
+    return HKM_OK;
+}
+
+int hkm_assign_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, int32_t K,
+                   int64_t ldc, int32_t* labels, double* min_d2, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix64("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix64("C", C, K, D, ldc))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (N == 0) return HKM_OK;
+    return launch_assign_f64(X, N, D, ldx, C, K, ldc, labels, min_d2, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                   double* C_new, int64_t ldcn, int64_t* counts, void* ws, size_t ws_bytes,
+                   void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix64("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix64("C_new", C_new, K, D, ldcn))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    const int32_t flags = HKM_WS_UPDATE | HKM_WS_F64;
+    const size_t need = carve(nullptr, N, D, K, flags).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const Workspace w = carve(ws, N, D, K, flags);
+    return launch_update_f64(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, nullptr, nullptr,
+                             static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_lloyd_step_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, double* C_new,
+                       int32_t K, int32_t* labels, double* shift, double* sse, void* ws, size_t ws_bytes,
+                       void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix64("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix64("C", C, K, D, D))) return rc;
+    if ((rc = check_matrix64("C_new", C_new, K, D, D))) return rc;
+    if (C == C_new) return fail(HKM_EINVAL, "C and C_new must not alias");
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (!shift) return fail(HKM_EINVAL, "shift is NULL");
+    const int32_t flags = HKM_WS_LLOYD | HKM_WS_F64 | (sse ? HKM_WS_SSE : 0);
+    const size_t need = carve(nullptr, N, D, K, flags).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const Workspace w = carve(ws, N, D, K, flags);
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    double* md = sse ? reinterpret_cast<double*>(w.min_d2) : nullptr;
+    if (N > 0 && (rc = launch_assign_f64(X, N, D, ldx, C, K, D, labels, md, st))) return rc;
+    if ((rc = launch_update_f64(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
+    if (sse) rc = launch_sum_min_d2_f64(md, N, sse, w.red, 1, st);
+    return rc;
+}
+
+int hkm_shift_f64(const double* C_old, const double* C_new, int32_t K, int32_t D, double* shift,
+                  void* hip_stream) {
+    g_err[0] = 0;
+    if (K < 1 || D < 1) return fail(HKM_EINVAL, "K = %d and D = %d must be >= 1", K, D);
+    if (!C_old || !C_new || !shift) return fail(HKM_EINVAL, "NULL pointer argument");
+    return launch_shift_f64(C_old, C_new, K, D, shift, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_functional_value_f64(const double* min_d2, int64_t N, double* out, void* ws, size_t ws_bytes,
+                             void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (!min_d2 || !out) return fail(HKM_EINVAL, "NULL pointer argument");
+    const size_t need = carve(nullptr, N, 1, 1, HKM_WS_ASSIGN).total;
+    int rc = check_ws(ws, ws_bytes, need);
+    if (rc) return rc;
+    const Workspace w = carve(ws, N, 1, 1, HKM_WS_ASSIGN);
+    return launch_sum_min_d2_f64(min_d2, N, out, w.red, 2, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, int64_t Nn, int64_t ldy,
+                     int32_t D, double* out, int64_t ldo, int32_t metric, double sigma, void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 0 || Nn < 0) return fail(HKM_EINVAL, "negative row count (M = %lld, Nn = %lld)", (long long)M, (long long)Nn);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    if (metric < HKM_METRIC_EUCLID_QE || metric > HKM_METRIC_MANHATTAN) return fail(HKM_EINVAL, "unknown metric %d", metric);
+    const bool gaussian = metric == HKM_METRIC_GAUSS_QE || metric == HKM_METRIC_GAUSS;
+    if (gaussian && !(sigma > 0.0)) return fail(HKM_EINVAL, "sigma = %g must be > 0", sigma);
+    int rc;
+    if ((rc = check_matrix64("X", X, M, D, ldx))) return rc;
+    if ((rc = check_matrix64("Y", Y, Nn, D, ldy))) return rc;
+    if (!out) return fail(HKM_EINVAL, "out is NULL");
+    if (ldo < Nn) return fail(HKM_EINVAL, "leading dimension of out (%lld) < columns (%lld)", (long long)ldo, (long long)Nn);
+    if (M == 0 || Nn == 0) return HKM_OK;
+    const int form = (metric == HKM_METRIC_EUCLID_QE || metric == HKM_METRIC_GAUSS_QE) ? 0
+                     : (metric == HKM_METRIC_MANHATTAN ? 2 : 1);
+    return launch_cdist_f64(X, M, ldx, Y, Nn, ldy, D, out, ldo, form, gaussian ? 0 : 1,
+                            gaussian ? 1.0 / (2.0 * sigma * sigma) : 0.0, static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_assign_l1_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,

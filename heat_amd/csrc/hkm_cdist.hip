@@ -13,15 +13,24 @@ static constexpr int CD_KC = 16;  // feature chunk
 
 // METRIC: 0 = quadratic expansion (squared, optional sqrt), 1 = direct sum((x-y)^2) (optional sqrt),
 //         2 = sum |x-y|;  gauss != 0 applies exp(-d2 * gauss) to the squared distance instead of sqrt
-template <int METRIC>
-__global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X, int64_t M,
-                                                    int64_t ldx, const float* __restrict__ Y,
+__device__ __forceinline__ float cd_sqrt(float v) { return sqrtf(v); }
+__device__ __forceinline__ double cd_sqrt(double v) { return sqrt(v); }
+__device__ __forceinline__ float cd_exp(float v) { return expf(v); }
+__device__ __forceinline__ double cd_exp(double v) { return exp(v); }
+__device__ __forceinline__ float cd_abs(float v) { return fabsf(v); }
+__device__ __forceinline__ double cd_abs(double v) { return fabs(v); }
+__device__ __forceinline__ float cd_fma(float a, float b, float c) { return fmaf(a, b, c); }
+__device__ __forceinline__ double cd_fma(double a, double b, double c) { return fma(a, b, c); }
+
+template <typename T, int METRIC>
+__global__ __launch_bounds__(256) void cdist_kernel(const T* __restrict__ X, int64_t M,
+                                                    int64_t ldx, const T* __restrict__ Y,
                                                     int64_t Nn, int64_t ldy, int D,
-                                                    float* __restrict__ out, int64_t ldo,
-                                                    int sqrt_flag, float gauss, int64_t tiles_n) {
-    __shared__ float sX[CD_KC][CD_T + 4];
-    __shared__ float sY[CD_KC][CD_T + 4];
-    __shared__ float sXn[CD_T], sYn[CD_T];
+                                                    T* __restrict__ out, int64_t ldo,
+                                                    int sqrt_flag, T gauss, int64_t tiles_n) {
+    __shared__ T sX[CD_KC][CD_T + 4];
+    __shared__ T sY[CD_KC][CD_T + 4];
+    __shared__ T sXn[CD_T], sYn[CD_T];
     const int tid = threadIdx.x;
     const int64_t tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
     const int64_t i0 = tm * CD_T, j0 = tn * CD_T;
@@ -32,20 +41,20 @@ __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X,
         const int r = is_x ? tid : tid - CD_T;
         const int64_t g = (is_x ? i0 : j0) + r;
         const int64_t lim = is_x ? M : Nn;
-        float s = 0.f;
+        T s = T(0);
         if (g < lim) {
-            const float* row = is_x ? X + g * ldx : Y + g * ldy;
-            for (int d = 0; d < D; ++d) s = fmaf(row[d], row[d], s);
+            const T* row = is_x ? X + g * ldx : Y + g * ldy;
+            for (int d = 0; d < D; ++d) s = cd_fma(row[d], row[d], s);
         }
         (is_x ? sXn : sYn)[r] = s;
     }
 
     const int tx = tid & 15, ty = tid >> 4;
-    float acc[4][4];
+    T acc[4][4];
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
+        for (int b = 0; b < 4; ++b) acc[a][b] = T(0);
 
     // staging role: element (row lr, feature lk) of both tiles, 4 passes of 16 rows
     const int lk = tid & 15, lr = tid >> 4;
@@ -56,13 +65,13 @@ __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X,
             const int r = lr + 16 * q;
             const int d = d0 + lk;
             const int64_t gi = i0 + r, gj = j0 + r;
-            sX[lk][r] = (gi < M && d < D) ? X[gi * ldx + d] : 0.f;
-            sY[lk][r] = (gj < Nn && d < D) ? Y[gj * ldy + d] : 0.f;
+            sX[lk][r] = (gi < M && d < D) ? X[gi * ldx + d] : T(0);
+            sY[lk][r] = (gj < Nn && d < D) ? Y[gj * ldy + d] : T(0);
         }
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < CD_KC; ++k) {
-            float xa[4], yb[4];
+            T xa[4], yb[4];
 #pragma unroll
             for (int a = 0; a < 4; ++a) xa[a] = sX[k][ty * 4 + a];
 #pragma unroll
@@ -72,12 +81,12 @@ __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X,
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     if (METRIC == 0) {
-                        acc[a][b] = fmaf(xa[a], yb[b], acc[a][b]);
+                        acc[a][b] = cd_fma(xa[a], yb[b], acc[a][b]);
                     } else if (METRIC == 1) {
-                        const float df = xa[a] - yb[b];
-                        acc[a][b] = fmaf(df, df, acc[a][b]);
+                        const T df = xa[a] - yb[b];
+                        acc[a][b] = cd_fma(df, df, acc[a][b]);
                     } else {
-                        acc[a][b] += fabsf(xa[a] - yb[b]);
+                        acc[a][b] += cd_abs(xa[a] - yb[b]);
                     }
                 }
         }
@@ -88,39 +97,52 @@ __global__ __launch_bounds__(256) void cdist_kernel(const float* __restrict__ X,
     for (int a = 0; a < 4; ++a) {
         const int64_t gi = i0 + ty * 4 + a;
         if (gi >= M) continue;
-        const float xn = sXn[ty * 4 + a];
+        const T xn = sXn[ty * 4 + a];
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int64_t gj = j0 + tx * 4 + b;
             if (gj >= Nn) continue;
-            float d = acc[a][b];
+            T d = acc[a][b];
             if (METRIC == 0) {
-                d = fmaf(-2.0f, d, xn + sYn[tx * 4 + b]);
-                d = fmaxf(d, 0.0f);
+                d = cd_fma(T(-2), d, xn + sYn[tx * 4 + b]);
+                d = d > T(0) ? d : (d != d ? d : T(0));  // clamp at 0, NaN passes through
             }
             if (METRIC != 2) {
-                if (gauss != 0.f) d = expf(-d * gauss);
-                else if (sqrt_flag) d = sqrtf(d);
+                if (gauss != T(0)) d = cd_exp(-d * gauss);
+                else if (sqrt_flag) d = cd_sqrt(d);
             }
             out[gi * ldo + gj] = d;
         }
     }
 }
 
-int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
-                 int32_t D, float* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, float gauss,
-                 hipStream_t st) {
+template <typename T>
+static int launch_cdist_t(const T* X, int64_t M, int64_t ldx, const T* Y, int64_t Nn, int64_t ldy,
+                          int32_t D, T* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, T gauss,
+                          hipStream_t st) {
     const int64_t tiles_m = (M + CD_T - 1) / CD_T, tiles_n = (Nn + CD_T - 1) / CD_T;
     const int64_t total = tiles_m * tiles_n;
     if (total > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "cdist: %lld tiles exceed the grid limit", (long long)total);
-#define HKM_GO(MET)                                                                              \
-    hipLaunchKernelGGL(cdist_kernel<MET>, dim3((unsigned)total), dim3(256), 0, st, X, M, ldx, Y, Nn, \
+#define HKM_GO(MET)                                                                                      \
+    hipLaunchKernelGGL((cdist_kernel<T, MET>), dim3((unsigned)total), dim3(256), 0, st, X, M, ldx, Y, Nn, \
                        ldy, D, out, ldo, sqrt_flag, gauss, tiles_n)
     if (metric == 0) HKM_GO(0);
     else if (metric == 1) HKM_GO(1);
     else HKM_GO(2);
 #undef HKM_GO
     return check_launch("cdist_kernel");
+}
+
+int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                 int32_t D, float* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, float gauss,
+                 hipStream_t st) {
+    return launch_cdist_t<float>(X, M, ldx, Y, Nn, ldy, D, out, ldo, metric, sqrt_flag, gauss, st);
+}
+
+int launch_cdist_f64(const double* X, int64_t M, int64_t ldx, const double* Y, int64_t Nn, int64_t ldy,
+                     int32_t D, double* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, double gauss,
+                     hipStream_t st) {
+    return launch_cdist_t<double>(X, M, ldx, Y, Nn, ldy, D, out, ldo, metric, sqrt_flag, gauss, st);
 }
 
 }  // namespace hkm

@@ -41,7 +41,7 @@ struct UpdateGeom {
     int32_t Z;               // number of cluster ranges
     int32_t KR;              // clusters per range (LDS accumulator rows)
 };
-UpdateGeom update_geom(int64_t N, int32_t D, int32_t K);
+UpdateGeom update_geom(int64_t N, int32_t D, int32_t K, int32_t elem = 4);
 
 // ---- workspace layout --------------------------------------------------------------------------
 struct Workspace {
@@ -116,6 +116,18 @@ int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, co
 int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                   const float* C_old, float* shift, hipStream_t st);
+int launch_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                      int32_t K, double* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                      const double* C_old, double* shift, hipStream_t st);
+int launch_shift_f64(const double* C_old, const double* C_new, int32_t K, int32_t D, double* shift,
+                     hipStream_t st);
+int launch_sum_min_d2_f64(const double* v, int64_t N, double* out, double* red, int mode,
+                          hipStream_t st);
+int launch_assign_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, int32_t K,
+                      int64_t ldc, int32_t* labels, double* min_d2, hipStream_t st);
+int launch_cdist_f64(const double* X, int64_t M, int64_t ldx, const double* Y, int64_t Nn, int64_t ldy,
+                     int32_t D, double* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, double gauss,
+                     hipStream_t st);
 int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
                  hipStream_t st);
 int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, int mode,

@@ -20,10 +20,11 @@ static constexpr int UPD_THREADS = 256;
 static constexpr int UPD_HALVES = 8;
 static constexpr int UPD_KR_MAX = 448;  // (448 + 1) x (32 x 4 + 4) B + 4.6 KB of row lists = 63.9 KB of LDS (64 KB dynamic limit)
 
-UpdateGeom update_geom(int64_t N, int32_t D, int32_t K) {
+UpdateGeom update_geom(int64_t N, int32_t D, int32_t K, int32_t elem) {
     UpdateGeom g;
+    const int kr_max = elem == 8 ? UPD_KR_MAX / 2 : UPD_KR_MAX;  // fp64 accumulator rows are twice as wide
     g.J = (D + 31) / 32;
-    g.Z = (K + UPD_KR_MAX - 1) / UPD_KR_MAX;
+    g.Z = (K + kr_max - 1) / kr_max;
     g.KR = (K + g.Z - 1) / g.Z;
     // aim at ~1024 workgroups overall; keep fp32 runs <= 32768 rows and chunks >= 1024 rows
     int64_t want_s = 1024 / (int64_t(g.J) * g.Z);
@@ -38,9 +39,10 @@ UpdateGeom update_geom(int64_t N, int32_t D, int32_t K) {
     return g;
 }
 
+template <typename T>
 __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
-    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const int32_t* __restrict__ labels,
-    int K, int KR, int64_t rows_per_chunk, float* __restrict__ part_sum,
+    const T* __restrict__ X, int64_t N, int D, int64_t ldx, const int32_t* __restrict__ labels,
+    int K, int KR, int64_t rows_per_chunk, T* __restrict__ part_sum,
     int32_t* __restrict__ part_cnt, int DPAD, const int32_t* __restrict__ gate, int ngate) {
     // behind the one-sweep MFMA step this pass only runs if some workgroup there raised its flag
     if (gate) {
@@ -50,16 +52,16 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
     }
     constexpr int U = 4;          // rows per half-wave and pass
     constexpr int LIST = 64 + U;  // a batch has 64 rows; room for the padding to a multiple of U
-    extern __shared__ __align__(16) float lds[];
-    float* acc = lds;                                                 // [KR + 1][32], last row = sink
-    int32_t* cnt = reinterpret_cast<int32_t*>(lds + (KR + 1) * 32);   // [KR + 1]
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T* acc = reinterpret_cast<T*>(lds_raw);                           // [KR + 1][32], last row = sink
+    int32_t* cnt = reinterpret_cast<int32_t*>(acc + (KR + 1) * 32);   // [KR + 1]
     int2* lists = reinterpret_cast<int2*>(cnt + ((KR + 1 + 1) & ~1)); // [8 half-waves][LIST]
     const int tid = threadIdx.x;
     const int s = blockIdx.x, j = blockIdx.y, z = blockIdx.z;
     const int kbase = z * KR;
     const int kend = min(K, kbase + KR);
 
-    for (int i = tid; i < (KR + 1) * 32; i += UPD_THREADS) acc[i] = 0.f;
+    for (int i = tid; i < (KR + 1) * 32; i += UPD_THREADS) acc[i] = T(0);
     for (int i = tid; i < KR + 1; i += UPD_THREADS) cnt[i] = 0;
     __syncthreads();
 
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
     const bool count_here = (c == 0) && (j == 0);
     const int64_t r_begin = int64_t(s) * rows_per_chunk;
     const int64_t r_end = min(N, r_begin + rows_per_chunk);
-    const float* xcol = X + (col_ok ? col : 0);
+    const T* xcol = X + (col_ok ? col : 0);
 
     int lab_next = -1;
     if (r_begin + lane < r_end) lab_next = labels[r_begin + lane];
@@ -103,21 +105,21 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
 
         for (int t = 0; t < npad; t += U) {
             int2 e[U];
-            float xv[U];
+            T xv[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) e[u] = my_list[t + u];
 #pragma unroll
             for (int u = 0; u < U; ++u) xv[u] = xcol[(base + e[u].x) * ldx];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                acc[e[u].y * 32 + c] += col_ok ? xv[u] : 0.f;
+                acc[e[u].y * 32 + c] += col_ok ? xv[u] : T(0);
                 if (count_here) cnt[e[u].y] += 1;
             }
         }
     }
     __syncthreads();
 
-    float* ps = part_sum + (int64_t(s) * K + kbase) * DPAD + j * 32;
+    T* ps = part_sum + (int64_t(s) * K + kbase) * DPAD + j * 32;
     for (int i = tid; i < (kend - kbase) * 32; i += UPD_THREADS) {
         const int k = i >> 5, cc = i & 31;
         ps[int64_t(k) * DPAD + cc] = acc[k * 32 + cc];
@@ -132,10 +134,11 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
 // lane order.  The order depends only on S.
 // With fsum != NULL the partials of the one-sweep MFMA step ([G][K][D] fp64, [G][K] counts) are used
 // unless one of its workgroups raised its flag; then the fp32 partials of pass 1 are.
+template <typename T>
 __global__ __launch_bounds__(256) void update_finalize_kernel(
-    const float* __restrict__ part_sum, const int32_t* __restrict__ part_cnt, int S, int K, int D,
-    int DPAD, float* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts,
-    const float* __restrict__ C_old, double* __restrict__ shift_part,
+    const T* __restrict__ part_sum, const int32_t* __restrict__ part_cnt, int S, int K, int D,
+    int DPAD, T* __restrict__ C_new, int64_t ldcn, int64_t* __restrict__ counts,
+    const T* __restrict__ C_old, double* __restrict__ shift_part,
     const double* __restrict__ fsum, const int32_t* __restrict__ fcnt,
     const int32_t* __restrict__ fflags, int G) {
     __shared__ double ssum[4][64];
@@ -177,12 +180,12 @@ __global__ __launch_bounds__(256) void update_finalize_kernel(
             n += pc[int64_t(s) * K];
         }
     } else if (ok) {
-        const float* ps = part_sum + int64_t(k) * DPAD + d;
+        const T* ps = part_sum + int64_t(k) * DPAD + d;
         const int32_t* pc = part_cnt + k;
         const int64_t sstride = int64_t(K) * DPAD;
         int s = q;
         for (; s + 28 < S; s += 32) {
-            float t[8];
+            T t[8];
             int32_t c[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
@@ -208,11 +211,11 @@ __global__ __launch_bounds__(256) void update_finalize_kernel(
         n = scnt[0][e] + scnt[1][e] + scnt[2][e] + scnt[3][e];
         // the reference's count passes through fp32 (clamp of an int64 tensor with a float bound)
         const double cnt = double(float(n < 1 ? 1 : n));
-        const float cnew = float(sum / cnt);
+        const T cnew = T(sum / cnt);
         C_new[int64_t(k) * ldcn + d] = cnew;
         if (d == 0 && counts) counts[k] = n;
         if (C_old) {
-            const float df = C_old[int64_t(k) * D + d] - cnew;  // square taken in fp32 (kmeans.py:141)
+            const T df = C_old[int64_t(k) * D + d] - cnew;  // square taken in the data type (kmeans.py:141)
             ssq[e] = double(df * df);
         }
     }
@@ -229,8 +232,9 @@ __global__ __launch_bounds__(256) void update_finalize_kernel(
 }
 
 // one workgroup adds the per-block shares in block order
+template <typename T>
 __global__ __launch_bounds__(256) void shift_final_kernel(const double* __restrict__ part, int nb,
-                                                          float* __restrict__ out) {
+                                                          T* __restrict__ out) {
     __shared__ double sh[256];
     const int per = (nb + 255) / 256;
     double acc = 0.0;
@@ -241,32 +245,47 @@ __global__ __launch_bounds__(256) void shift_final_kernel(const double* __restri
     if (threadIdx.x == 0) {
         double t = 0.0;
         for (int i = 0; i < 256; ++i) t += sh[i];
-        *out = float(t);
+        *out = T(t);
     }
 }
 
-int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
-                  int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
-                  const float* C_old, float* shift, hipStream_t st) {
-    const UpdateGeom g = update_geom(N, D, K);
+template <typename T>
+static int launch_update_t(const T* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                           int32_t K, T* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                           const T* C_old, T* shift, hipStream_t st) {
+    const UpdateGeom g = update_geom(N, D, K, int32_t(sizeof(T)));
     const int dpad = g.J * 32;
-    const size_t lds = size_t(g.KR + 1) * 32 * sizeof(float) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
+    const size_t lds = size_t(g.KR + 1) * 32 * sizeof(T) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
                        size_t(UPD_HALVES) * (64 + 8) * sizeof(int2);
-    hipLaunchKernelGGL(update_partial_kernel, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
-                       D, ldx, labels, K, g.KR, g.rows_per_chunk, w.part_sum, w.part_cnt, dpad,
+    T* part = reinterpret_cast<T*>(w.part_sum);
+    hipLaunchKernelGGL(update_partial_kernel<T>, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
+                       D, ldx, labels, K, g.KR, g.rows_per_chunk, part, w.part_cnt, dpad,
                        static_cast<const int32_t*>(nullptr), 0);
     int rc = check_launch("update_partial_kernel");
     if (rc) return rc;
     const int64_t tot = int64_t(K) * D;
     const int nb = int((tot + 63) / 64);
-    hipLaunchKernelGGL(update_finalize_kernel, dim3(nb), dim3(256), 0, st, w.part_sum, w.part_cnt,
-                       g.S, K, D, dpad, C_new, ldcn, counts, C_old, w.shift_part,
-                       static_cast<const double*>(nullptr), static_cast<const int32_t*>(nullptr),
-                       static_cast<const int32_t*>(nullptr), 0);
+    hipLaunchKernelGGL(update_finalize_kernel<T>, dim3(nb), dim3(256), 0, st, static_cast<const T*>(part),
+                       static_cast<const int32_t*>(w.part_cnt), g.S, K, D, dpad, C_new, ldcn, counts, C_old,
+                       w.shift_part, static_cast<const double*>(nullptr),
+                       static_cast<const int32_t*>(nullptr), static_cast<const int32_t*>(nullptr), 0);
     rc = check_launch("update_finalize_kernel");
     if (rc || !C_old) return rc;
-    hipLaunchKernelGGL(shift_final_kernel, dim3(1), dim3(256), 0, st, w.shift_part, nb, shift);
+    hipLaunchKernelGGL(shift_final_kernel<T>, dim3(1), dim3(256), 0, st, static_cast<const double*>(w.shift_part),
+                       nb, shift);
     return check_launch("shift_final_kernel");
+}
+
+int launch_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                      int32_t K, double* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                      const double* C_old, double* shift, hipStream_t st) {
+    return launch_update_t<double>(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, C_old, shift, st);
+}
+
+int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                  int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                  const float* C_old, float* shift, hipStream_t st) {
+    return launch_update_t<float>(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, C_old, shift, st);
 }
 
 // Second half of the one-sweep MFMA step: the two-pass update gated by the flags of the fused kernel
@@ -274,24 +293,25 @@ int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32
 int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                         int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                         int fgrid, const float* C_old, float* shift, hipStream_t st) {
-    const UpdateGeom g = update_geom(N, D, K);
+    const UpdateGeom g = update_geom(N, D, K, 4);
     const int dpad = g.J * 32;
     const size_t lds = size_t(g.KR + 1) * 32 * sizeof(float) + size_t((g.KR + 2) & ~1) * sizeof(int32_t) +
                        size_t(UPD_HALVES) * (64 + 8) * sizeof(int2);
-    hipLaunchKernelGGL(update_partial_kernel, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
+    hipLaunchKernelGGL(update_partial_kernel<float>, dim3(g.S, g.J, g.Z), dim3(UPD_THREADS), lds, st, X, N,
                        D, ldx, labels, K, g.KR, g.rows_per_chunk, w.part_sum, w.part_cnt, dpad,
                        static_cast<const int32_t*>(w.fflags), fgrid);
     int rc = check_launch("update_partial_kernel");
     if (rc) return rc;
     const int64_t tot = int64_t(K) * D;
     const int nb = int((tot + 63) / 64);
-    hipLaunchKernelGGL(update_finalize_kernel, dim3(nb), dim3(256), 0, st, w.part_sum, w.part_cnt,
-                       g.S, K, D, dpad, C_new, ldcn, counts, C_old, w.shift_part,
-                       static_cast<const double*>(w.fsum), static_cast<const int32_t*>(w.fcnt),
-                       static_cast<const int32_t*>(w.fflags), fgrid);
+    hipLaunchKernelGGL(update_finalize_kernel<float>, dim3(nb), dim3(256), 0, st,
+                       static_cast<const float*>(w.part_sum), static_cast<const int32_t*>(w.part_cnt), g.S, K,
+                       D, dpad, C_new, ldcn, counts, C_old, w.shift_part, static_cast<const double*>(w.fsum),
+                       static_cast<const int32_t*>(w.fcnt), static_cast<const int32_t*>(w.fflags), fgrid);
     rc = check_launch("update_finalize_kernel");
     if (rc || !C_old) return rc;
-    hipLaunchKernelGGL(shift_final_kernel, dim3(1), dim3(256), 0, st, w.shift_part, nb, shift);
+    hipLaunchKernelGGL(shift_final_kernel<float>, dim3(1), dim3(256), 0, st,
+                       static_cast<const double*>(w.shift_part), nb, shift);
     return check_launch("shift_final_kernel");
 }
 
@@ -313,26 +333,37 @@ __device__ __forceinline__ double block_sum_fixed(double v, double* sh) {
     return r;
 }
 
-__global__ __launch_bounds__(256) void shift_kernel(const float* __restrict__ a,
-                                                    const float* __restrict__ b, int64_t n,
-                                                    float* __restrict__ out) {
+__device__ __forceinline__ float hkm_sqrt(float v) { return sqrtf(v); }
+__device__ __forceinline__ double hkm_sqrt(double v) { return sqrt(v); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void shift_kernel(const T* __restrict__ a,
+                                                    const T* __restrict__ b, int64_t n,
+                                                    T* __restrict__ out) {
     __shared__ double sh[256];
     double acc = 0.0;
     for (int64_t i = threadIdx.x; i < n; i += 256) {
-        const float d = a[i] - b[i];
+        const T d = a[i] - b[i];
         acc += double(d * d);
     }
     const double t = block_sum_fixed(acc, sh);
-    if (threadIdx.x == 0) *out = float(t);
+    if (threadIdx.x == 0) *out = T(t);
 }
 
 int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
                  hipStream_t st) {
-    hipLaunchKernelGGL(shift_kernel, dim3(1), dim3(256), 0, st, C_old, C_new, int64_t(K) * D, shift);
+    hipLaunchKernelGGL(shift_kernel<float>, dim3(1), dim3(256), 0, st, C_old, C_new, int64_t(K) * D, shift);
     return check_launch("shift_kernel");
 }
 
-__global__ __launch_bounds__(256) void sum_partial_kernel(const float* __restrict__ v, int64_t n,
+int launch_shift_f64(const double* C_old, const double* C_new, int32_t K, int32_t D, double* shift,
+                     hipStream_t st) {
+    hipLaunchKernelGGL(shift_kernel<double>, dim3(1), dim3(256), 0, st, C_old, C_new, int64_t(K) * D, shift);
+    return check_launch("shift_kernel");
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sum_partial_kernel(const T* __restrict__ v, int64_t n,
                                                           int64_t per_block, int mode,
                                                           double* __restrict__ red) {
     __shared__ double sh[256];
@@ -340,12 +371,12 @@ __global__ __launch_bounds__(256) void sum_partial_kernel(const float* __restric
     const int64_t b1 = min(n, b0 + per_block);
     double acc = 0.0;
     for (int64_t i = b0 + threadIdx.x; i < b1; i += 256) {
-        float x = v[i];
+        T x = v[i];
         if (mode == 2) {
-            const float r = sqrtf(x);
+            const T r = hkm_sqrt(x);
             x = r * r;
         } else if (mode == 3) {
-            x = sqrtf(x);
+            x = hkm_sqrt(x);
         }
         acc += double(x);
     }
@@ -353,33 +384,43 @@ __global__ __launch_bounds__(256) void sum_partial_kernel(const float* __restric
     if (threadIdx.x == 0) red[blockIdx.x] = t;
 }
 
+template <typename T>
 __global__ __launch_bounds__(256) void sum_final_kernel(const double* __restrict__ red, int nb,
-                                                        int mode, float* __restrict__ out) {
+                                                        int mode, T* __restrict__ out) {
     __shared__ double sh[256];
     double acc = 0.0;
     for (int i = threadIdx.x; i < nb; i += 256) acc += red[i];
     const double t = block_sum_fixed(acc, sh);
     if (threadIdx.x == 0) {
-        float f = float(t);
+        T f = T(t);
         if (mode == 2) {
-            const float r = sqrtf(f);
+            const T r = hkm_sqrt(f);
             f = r * r;
         }
         *out = f;
     }
 }
 
-int launch_sum_min_d2(const float* v, int64_t N, float* out, double* red, int mode,
-                      hipStream_t st) {
+template <typename T>
+static int launch_sum_t(const T* v, int64_t N, T* out, double* red, int mode, hipStream_t st) {
     int nb = int((N + 65535) / 65536);
     if (nb < 1) nb = 1;
     if (nb > RED_SLOTS) nb = RED_SLOTS;
     const int64_t per_block = (N + nb - 1) / nb;
-    hipLaunchKernelGGL(sum_partial_kernel, dim3(nb), dim3(256), 0, st, v, N, per_block, mode, red);
+    hipLaunchKernelGGL(sum_partial_kernel<T>, dim3(nb), dim3(256), 0, st, v, N, per_block, mode, red);
     int rc = check_launch("sum_partial_kernel");
     if (rc) return rc;
-    hipLaunchKernelGGL(sum_final_kernel, dim3(1), dim3(256), 0, st, red, nb, mode, out);
+    hipLaunchKernelGGL(sum_final_kernel<T>, dim3(1), dim3(256), 0, st, static_cast<const double*>(red), nb, mode,
+                       out);
     return check_launch("sum_final_kernel");
+}
+
+int launch_sum_min_d2(const float* v, int64_t N, float* out, double* red, int mode, hipStream_t st) {
+    return launch_sum_t<float>(v, N, out, red, mode, st);
+}
+
+int launch_sum_min_d2_f64(const double* v, int64_t N, double* out, double* red, int mode, hipStream_t st) {
+    return launch_sum_t<double>(v, N, out, red, mode, st);
 }
 
 __global__ void widen_kernel(const int32_t* __restrict__ in, int64_t n, int64_t* __restrict__ out) {

@@ -1,6 +1,7 @@
 """
 Pairwise distances with the interface of heat/spatial/distance.py:136-206 (``cdist``, ``rbf``,
-``manhattan``), backed by the hkm_pairwise_f32 kernel, computed in float32 on one rank.
+``manhattan``), backed by the hkm_pairwise_f32 / hkm_pairwise_f64 kernels on one rank, in the
+dtype the reference's promote(X, Y, float32) gives.
 """
 
 from __future__ import annotations
@@ -50,15 +51,15 @@ def _check_inputs(X: DNDarray, Y: Optional[DNDarray]):
 
 
 def _as_f32_matrix(a: DNDarray, promoted) -> torch.Tensor:
+    """The local matrix in the promoted dtype (float32 or float64), row-major."""
     t = a.larray
     if t.dim() != 2:
         raise NotImplementedError("Only 2D data matrices are currently supported")
-    if promoted is not types.float32:
-        raise NotImplementedError(
-            f"the gfx950 kernels compute in float32; inputs promote to {promoted.__name__}"
-        )
-    if t.dtype != torch.float32:
-        t = t.to(torch.float32)
+    if promoted not in (types.float32, types.float64):
+        raise NotImplementedError(f"inputs promote to {promoted.__name__}, which the kernels do not cover")
+    want = torch.float64 if promoted is types.float64 else torch.float32
+    if t.dtype != want:
+        t = t.to(want)
     if t.stride(-1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
         t = t.contiguous()
     return t
@@ -75,16 +76,16 @@ def _pairwise(X: DNDarray, Y: Optional[DNDarray], metric: int, sigma: float = 1.
     y = x if Y is None else _as_f32_matrix(Y, promoted)
     if x.shape[1] != y.shape[1]:
         raise ValueError("Inputs must have same shape[1]")
-    out = torch.empty((x.shape[0], y.shape[0]), dtype=torch.float32, device=x.device)
+    out = torch.empty((x.shape[0], y.shape[0]), dtype=x.dtype, device=x.device)
     _native.pairwise(x, y, out, metric, sigma)
-    return DNDarray(out, tuple(out.shape), types.float32, split, X.device, X.comm, True)
+    return DNDarray(out, tuple(out.shape), promoted, split, X.device, X.comm, True)
 
 
 def cdist(X: DNDarray, Y: Optional[DNDarray] = None, quadratic_expansion: bool = False) -> DNDarray:
     """
     Euclidean distance between all rows of ``X`` (m x f) and ``Y`` (n x f): an (m, n) DNDarray of
     square-rooted distances in promote(X, Y, float32), ``split = X.split`` (1 when only ``Y`` is
-    split).  ``Y=None`` means ``Y = X``.  Computed in float32.
+    split).  ``Y=None`` means ``Y = X``.
 
     ``quadratic_expansion=True``: |x-y|^2 = |x|^2 + |y|^2 - 2xy clamped at 0 (the metric KMeans
     uses); ``False``: sum((x-y)^2) directly (heat/spatial/distance.py:136-156).

@@ -43,6 +43,7 @@ extern "C" {
 #define HKM_WS_LLOYD 3 /* assign + update */
 #define HKM_WS_SSE 4   /* add when hkm_lloyd_step_f32 is called with sse != NULL (N floats of scratch) */
 #define HKM_WS_MEDIAN 8 /* on its own: scratch of hkm_update_median_f32 / hkm_closest_rows_l1_f32 */
+#define HKM_WS_F64 16   /* add for the *_f64 entry points (partials and scratch are doubles) */
 
 /* Library version: major*10000 + minor*100 + patch. */
 int hkm_version(void);
@@ -176,6 +177,32 @@ int hkm_update_median_f32(const float* X, int64_t N, int32_t D, int64_t ldx, con
                           const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
                           int64_t* counts, int32_t mode, int32_t skip_zero_rows, void* ws, size_t ws_bytes,
                           void* hip_stream);
+
+/*
+ * float64 data.  The reference keeps float64 inputs in float64 through the same op sequence
+ * (promote(X, Y, float32), heat/spatial/distance.py:392-403; heat/cluster/kmeans.py:76-148), so these
+ * mirror the *_f32 entry points of the same name with double operands: quadratic-expansion distance +
+ * argmin, deterministic per-cluster mean (sums in fp64, count through fp32 as in the reference), one
+ * Lloyd iteration, centroid shift, clustering functional, full pairwise matrices.  Pointers must be
+ * 8-byte aligned; workspaces are sized with HKM_WS_F64 added to the flags (hkm_update_f64:
+ * HKM_WS_UPDATE | HKM_WS_F64, hkm_lloyd_step_f64: HKM_WS_LLOYD | HKM_WS_F64 [| HKM_WS_SSE],
+ * hkm_functional_value_f64: as the f32 one).  Labels stay int32.  These run on the fp64 vector ALU
+ * and read X twice per iteration; they are not the tuned path.
+ */
+int hkm_assign_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, int32_t K,
+                   int64_t ldc, int32_t* labels, double* min_d2, void* hip_stream);
+int hkm_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                   double* C_new, int64_t ldcn, int64_t* counts, void* ws, size_t ws_bytes,
+                   void* hip_stream);
+int hkm_lloyd_step_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, double* C_new,
+                       int32_t K, int32_t* labels, double* shift, double* sse, void* ws, size_t ws_bytes,
+                       void* hip_stream);
+int hkm_shift_f64(const double* C_old, const double* C_new, int32_t K, int32_t D, double* shift,
+                  void* hip_stream);
+int hkm_functional_value_f64(const double* min_d2, int64_t N, double* out, void* ws, size_t ws_bytes,
+                             void* hip_stream);
+int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, int64_t Nn, int64_t ldy,
+                     int32_t D, double* out, int64_t ldo, int32_t metric, double sigma, void* hip_stream);
 
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);

@@ -97,7 +97,7 @@ def test_cdist_exceptions():
         ht.spatial.cdist(ht.ones((4, 4)), Z, quadratic_expansion=True)
     with pytest.raises(ValueError):
         ht.spatial.cdist(ht.ones((4, 4)), ht.ones((4, 5)), quadratic_expansion=True)
-    with pytest.raises(NotImplementedError):  # float64 is outside the float32 kernels
+    with pytest.raises(RuntimeError):  # float64 has kernels of its own, but host data is still refused
         ht.spatial.cdist(ht.ones((4, 4), dtype=ht.float64), quadratic_expansion=True)
     with pytest.raises(NotImplementedError):
         ht.spatial.rbf(X)
@@ -159,7 +159,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) >= 19
+    assert len(names) >= 25
     for name in names:
         assert hasattr(lib, name), name
         assert name in _native.SIGNATURES, f"{name} has no ctypes signature"
@@ -221,6 +221,14 @@ def test_argument_validation_happens_on_the_host():
     assert lib.hkm_pairwise_f32(good, 4, 3, good, 4, 3, 3, good, 4, _native.METRIC_GAUSS, 0.0, None) == _native.HKM_EINVAL
     assert "sigma" in err()
     assert lib.hkm_widen_labels_i64(None, 4, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_assign_f64(P(4100), 10, 3, 3, good, 8, 3, good, None, None) == _native.HKM_EINVAL
+    assert "8-byte" in err()
+    assert lib.hkm_assign_f64(good, 10, 3, 2, good, 8, 3, good, None, None) == _native.HKM_EINVAL
+    assert lib.hkm_update_f64(good, 10, 3, 3, good, 8, good, 3, None, ws, 8, None) == _native.HKM_EWORKSPACE
+    assert lib.hkm_lloyd_step_f64(good, 10, 3, 3, good, good, 8, good, good, None, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_shift_f64(None, good, 8, 3, good, None) == _native.HKM_EINVAL
+    assert lib.hkm_functional_value_f64(good, -1, good, ws, big, None) == _native.HKM_EINVAL
+    assert lib.hkm_pairwise_f64(good, 4, 3, good, 4, 3, 3, good, 4, 9, 1.0, None) == _native.HKM_EINVAL
     assert lib.hkm_min_dist_sum_f32(good, -1, good, ws, big, None) == _native.HKM_EINVAL
     assert lib.hkm_min_dist_sum_f32(good, 8, good, None, 0, None) == _native.HKM_EWORKSPACE
     assert lib.hkm_sample_select_f32(good, good, 8, good, 0.0, good, 4, good, ws, big, None) == _native.HKM_EINVAL

@@ -1,0 +1,118 @@
+"""
+float64 data through the same estimators: the reference keeps float64 (and int64) inputs in float64
+through its op sequence (promote(X, Y, float32), heat/spatial/distance.py:392-403), so results are
+compared with the float64 oracle: labels equal except at ties of 1e-12 relative, centroids, shift and
+functional value within 1e-12 relative, repeated runs bit-identical.
+"""
+import numpy as np
+import pytest
+import torch
+
+import heat_amd as ht
+from heat_amd import _native
+from heat_amd.utils import synthetic
+from oracle import heat_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _data(n, d, k, seed, spread=3.0):
+    g = torch.Generator().manual_seed(seed)
+    c = torch.randn((k, d), generator=g, dtype=torch.float64) * spread
+    x = c[torch.randint(0, k, (n,), generator=g)] + torch.randn((n, d), generator=g, dtype=torch.float64)
+    return x.contiguous(), c.contiguous()
+
+
+@pytest.mark.parametrize("n,d,k", [(1, 3, 8), (3000, 3, 8), (5000, 32, 256), (999, 17, 1), (1300, 50, 37),
+                                   (700, 130, 70), (2000, 64, 1030)])
+def test_assign_and_update_f64(cuda, n, d, k):
+    print(f"f64 n={n} d={d} k={k}", flush=True)
+    x, c = _data(n, d, k, seed=n + d + k)
+    xg, cg = x.to(cuda), c.to(cuda)
+    ws = _native.Workspace(cuda)
+    lab = torch.full((n,), -7, dtype=torch.int32, device=cuda)
+    md = torch.full((n,), -1.0, dtype=torch.float64, device=cuda)
+    _native.assign(xg, cg, lab, md, ws)
+    ref_lab, _ = orc.assign_to_cluster_literal(x, c)
+    d2 = orc.brute_force_d2(x, c)
+    got = d2.gather(1, lab.cpu().long().view(-1, 1)).view(-1)
+    best = d2.min(1).values
+    scale = (x ** 2).sum(1) + (c ** 2).sum(1).max()
+    assert torch.all(got - best <= 1e-12 * scale)  # same centroid, or a tie at float64 resolution
+    assert float((lab.cpu().long() == ref_lab.view(-1)).float().mean()) >= 0.999
+    assert torch.all((md.cpu() - best).abs() <= 1e-12 * scale)
+    # update from those labels
+    c_new = torch.empty_like(cg)
+    cnt = torch.empty((k,), dtype=torch.int64, device=cuda)
+    _native.update(xg, lab, c_new, cnt, ws)
+    ref_c, ref_cnt = orc.update_centroids_fast(x, lab.cpu().long().view(-1, 1), k, out_dtype=torch.float64)
+    assert torch.equal(cnt.cpu(), ref_cnt.view(-1).long())
+    assert orc.rel_err_centers(c_new.cpu(), ref_c) <= 1e-12
+    # one step, twice: identical, and consistent with its parts
+    outs = []
+    for _ in range(2):
+        c2 = torch.empty_like(cg)
+        lab2 = torch.empty_like(lab)
+        shift = torch.empty((), dtype=torch.float64, device=cuda)
+        sse = torch.empty((), dtype=torch.float64, device=cuda)
+        _native.lloyd_step(xg, cg, c2, lab2, shift, sse, ws)
+        outs.append((c2.cpu(), lab2.cpu(), shift.cpu(), sse.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert torch.equal(outs[0][0], c_new.cpu()) and torch.equal(outs[0][1], lab.cpu())
+    ref_shift = float(((c - outs[0][0]) ** 2).sum())
+    assert abs(float(outs[0][2]) - ref_shift) <= 1e-12 * max(ref_shift, 1e-300)
+    assert abs(float(outs[0][3]) - float(best.sum())) <= 1e-10 * float(best.sum()) + 1e-12 * float(scale.sum())
+
+
+def test_kmeans_fit_predict_f64_matches_oracle(cuda):
+    w = synthetic.config1(0.3)
+    x, init = w.x.double(), w.init.double()
+    ref = orc.kmeans_fit(x, init, 15, 0.0, literal=True)
+    km = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(init.to(cuda)), max_iter=15, tol=0.0)
+    km.fit(ht.array(x.to(cuda), split=0))
+    assert km.cluster_centers_.dtype is ht.float64 and km.cluster_centers_.larray.dtype == torch.float64
+    assert km.n_iter_ == ref["n_iter"]
+    assert orc.rel_err_centers(km.cluster_centers_.larray.cpu(), ref["cluster_centers"]) <= 1e-10
+    assert torch.equal(km.labels_.larray.cpu(), ref["labels"])
+    assert abs(float(km.inertia_.larray) - float(ref["inertia"])) <= 1e-9 * max(float(ref["inertia"]), 1e-30)
+    pred = km.predict(ht.array(x.to(cuda), split=0))
+    ref_lab, ref_fv = orc.predict(x, ref["cluster_centers"])
+    assert torch.equal(pred.larray.cpu(), ref_lab)
+    assert abs(float(km.functional_value_.larray) - float(ref_fv)) <= 1e-10 * float(ref_fv)
+    # int64 data promote to float64 like the reference's promote(int64, float32)
+    xi = (x * 10).round().long()
+    km = ht.cluster.KMeans(n_clusters=w.k, init="random", max_iter=5, random_state=3).fit(ht.array(xi.to(cuda), split=0))
+    assert km.cluster_centers_.larray.dtype == torch.float64
+
+
+def test_spatial_f64_and_other_estimators(cuda):
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn((130, 9), generator=g, dtype=torch.float64)
+    b = torch.randn((70, 9), generator=g, dtype=torch.float64)
+    A, B = ht.array(a.to(cuda), split=0), ht.array(b.to(cuda))
+    for qe in (False, True):
+        d = ht.spatial.cdist(A, B, quadratic_expansion=qe)
+        assert d.dtype is ht.float64 and torch.allclose(d.larray.cpu(), torch.cdist(a, b), rtol=1e-9, atol=1e-9)
+        r = ht.spatial.rbf(A, B, sigma=1.5, quadratic_expansion=qe)
+        assert torch.allclose(r.larray.cpu(), torch.exp(-torch.cdist(a, b) ** 2 / (2 * 1.5 ** 2)), rtol=1e-9, atol=1e-12)
+    m = ht.spatial.manhattan(A, B)
+    assert torch.allclose(m.larray.cpu(), torch.cdist(a, b, p=1), rtol=1e-12)
+    # mixed float32 / float64 promote to float64 (heat/spatial/distance.py:392-403)
+    d = ht.spatial.cdist(A, ht.array(b.float().to(cuda)), quadratic_expansion=True)
+    assert d.dtype is ht.float64
+    # the reference's float64 datasets (tests/cluster/test_kmeans.py:125-134, test_batchparallelclustering.py:90)
+    data = synthetic.spherical_dataset(20, 1.0, 4.0, torch.float64, seed=1)
+    xs = ht.array(data.to(cuda), split=0)
+    for init in ("kmeans++", "batchparallel", "random"):
+        km = ht.cluster.KMeans(n_clusters=4, init=init, random_state=1).fit(xs)
+        assert km.cluster_centers_.shape == (4, 3) and km.cluster_centers_.dtype is ht.float64
+    bp = ht.cluster.BatchParallelKMeans(n_clusters=4, random_state=1).fit(xs)
+    assert bp.cluster_centers_.dtype is ht.float64
+    lab = bp.predict(xs)
+    c = bp.cluster_centers_.larray.cpu()
+    fv = float(((data - c[lab.larray.view(-1).cpu().long()]) ** 2).sum())
+    assert abs(bp.functional_value_ - fv) <= 1e-9 * fv
+    for est in (ht.cluster.KMedians, ht.cluster.KMedoids, ht.cluster.BatchParallelKMedians):
+        with pytest.raises(NotImplementedError):  # Manhattan-metric kernels: float32 only
+            est(n_clusters=4).fit(xs)
