@@ -135,8 +135,89 @@ __global__ void l1_unpack_rows_kernel(const unsigned long long* __restrict__ key
     if (dist) dist[i] = __uint_as_float(unsigned(k >> 32));
 }
 
+// Narrow rows (D <= 16): one point per lane in registers, the centroids in LDS read as wave-wide
+// broadcasts, k ascending with a strict '<' so the first index wins ties.  Bound by streaming X.
+static constexpr int L1S_THREADS = 256;
+static constexpr int L1S_LDS_FLOATS = 8192;
+
+template <int D>
+__global__ __launch_bounds__(L1S_THREADS) void l1_assign_small_kernel(
+    const float* __restrict__ X, int64_t N, int64_t ldx, const float* __restrict__ C, int K, int64_t ldc,
+    int32_t* __restrict__ labels, float* __restrict__ min_dist, int ktile, int64_t nbatches) {
+    __shared__ float sC[L1S_LDS_FLOATS];
+    const int tid = threadIdx.x;
+    const int nkt = (K + ktile - 1) / ktile;
+    auto stage = [&](int kt) {
+        const int k0 = kt * ktile;
+        const int kn = min(ktile, K - k0);
+        for (int i = tid; i < kn * D; i += L1S_THREADS) {
+            const int r = i / D, c = i - r * D;
+            sC[i] = C[int64_t(k0 + r) * ldc + c];
+        }
+        __syncthreads();
+        return kn;
+    };
+    int kn = 0;
+    if (nkt == 1) kn = stage(0);
+    for (int64_t b = blockIdx.x; b < nbatches; b += gridDim.x) {
+        const int64_t i = b * L1S_THREADS + tid;
+        const int64_t ir = i < N ? i : N - 1;
+        float x[D];
+        const float* xp = X + ir * ldx;
+#pragma unroll
+        for (int d = 0; d < D; ++d) x[d] = xp[d];
+        float m = HKM_INF;
+        int mi = 0;
+        for (int kt = 0; kt < nkt; ++kt) {
+            if (nkt > 1) {
+                __syncthreads();
+                kn = stage(kt);
+            }
+            const int k0 = kt * ktile;
+#pragma unroll 4
+            for (int k = 0; k < kn; ++k) {
+                const float* c = sC + k * D;
+                float dist = fabsf(x[0] - c[0]);
+#pragma unroll
+                for (int d = 1; d < D; ++d) dist += fabsf(x[d] - c[d]);
+                if (dist < m) {
+                    m = dist;
+                    mi = k0 + k;
+                }
+            }
+        }
+        if (i < N) {
+            labels[i] = mi;
+            if (min_dist) min_dist[i] = m;
+        }
+    }
+}
+
+template <int D>
+static int launch_l1_small_t(const float* X, int64_t N, int64_t ldx, const float* C, int32_t K, int64_t ldc,
+                             int32_t* labels, float* min_dist, hipStream_t st) {
+    const int ktile = L1S_LDS_FLOATS / D;
+    const int64_t nbatches = (N + L1S_THREADS - 1) / L1S_THREADS;
+    int64_t grid = int64_t(num_cus()) * 8;
+    if (grid > nbatches) grid = nbatches;
+    hipLaunchKernelGGL(l1_assign_small_kernel<D>, dim3((unsigned)grid), dim3(L1S_THREADS), 0, st, X, N, ldx, C, K,
+                       ldc, labels, min_dist, ktile, nbatches);
+    return check_launch("l1_assign_small_kernel");
+}
+
 int launch_assign_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                      int64_t ldc, int32_t* labels, float* min_dist, hipStream_t st) {
+    // narrow rows and few centroids: the 64 x 64 tile would be mostly padding
+    if (D <= 16 && int64_t(K) * D <= 1024) {
+#define HKM_CASE(d) \
+    case d:         \
+        return launch_l1_small_t<d>(X, N, ldx, C, K, ldc, labels, min_dist, st);
+        switch (D) {
+            HKM_CASE(1) HKM_CASE(2) HKM_CASE(3) HKM_CASE(4) HKM_CASE(5) HKM_CASE(6) HKM_CASE(7) HKM_CASE(8)
+            HKM_CASE(9) HKM_CASE(10) HKM_CASE(11) HKM_CASE(12) HKM_CASE(13) HKM_CASE(14) HKM_CASE(15) HKM_CASE(16)
+        }
+#undef HKM_CASE
+    }
     const int64_t tiles = (N + L1_T - 1) / L1_T;
     if (tiles > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "assign_l1: too many row tiles");
     hipLaunchKernelGGL(l1_argmin_kernel, dim3((unsigned)tiles, 1), dim3(256), 0, st, X, N, ldx, C,

@@ -102,7 +102,9 @@ def test_assign_strided_rows(cuda):
 
 
 UPDATE_SHAPES = [(1000, 3, 8), (5000, 8, 16), (4096, 32, 256), (3000, 64, 100), (70000, 20, 33),
-                 (900, 512, 130), (2500, 130, 1030), (100000, 32, 7)]
+                 (900, 512, 130), (2500, 130, 1030), (100000, 32, 7),
+                 # wide rows (D >= 128, D % 4 == 0): 128-column slices, several cluster ranges
+                 (30000, 128, 50), (20000, 132, 500), (6000, 512, 1024), (777, 256, 3)]
 
 
 @pytest.mark.parametrize("n,d,k", UPDATE_SHAPES)
