@@ -168,7 +168,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 100; }
+int hkm_version(void) { return 200; }
 
 const char* hkm_last_error(void) { return g_err; }
 

@@ -228,6 +228,45 @@ def test_config4_full_size_properties(cuda):
     _full_size_properties(synthetic.config4(), cuda, iters=2)
 
 
+def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
+    """KMeans.fit keeps the next step enqueued while the host reads the shift of the current one; when
+    the tolerance is met the extra step must leave no trace: same iteration count, centroids, labels and
+    inertia as a loop that only launches a step after looking at the previous shift."""
+    from heat_amd import _native
+    from heat_amd.cluster._lloyd import LloydLoop
+
+    w = synthetic.config1(0.5)
+    x = w.x.to(cuda)
+    for tol in (1e-1, 1e-3, 0.0, None):
+        ws = _native.Workspace(cuda)
+        c_cur = w.init.to(cuda).clone()
+        c_nxt = torch.empty_like(c_cur)
+        lab = torch.empty((x.shape[0],), dtype=torch.int32, device=cuda)
+        shift = torch.empty((), device=cuda)
+        n_seq = 0
+        for _ in range(40):
+            n_seq += 1
+            _native.lloyd_step(x, c_cur, c_nxt, lab, shift, None, ws)
+            c_cur, c_nxt = c_nxt, c_cur
+            if tol is not None and float(shift) <= tol:
+                break
+        km = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(cuda)), max_iter=40, tol=tol)
+        km.fit(ht.array(x, split=0))
+        assert km.n_iter_ == n_seq, (tol, km.n_iter_, n_seq)
+        assert torch.equal(km.cluster_centers_.larray, c_cur)
+        assert torch.equal(km.labels_.larray.view(-1), lab.long())
+        assert float(km.inertia_.larray) == float(shift)
+    assert n_seq == 40  # tol=None never stops early
+    # a loop can be driven in pieces (the benchmark does): 3 + 4 steps == 7 steps
+    a = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
+    assert a.run(3, -1.0) == 3 and a.run(4, -1.0) == 4
+    b = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
+    assert b.run(7, None) == 7
+    assert torch.equal(a.centers, b.centers) and torch.equal(a.labels, b.labels)
+    with pytest.raises(ValueError):
+        ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(cuda)), max_iter=0).fit(ht.array(x, split=0))
+
+
 def test_random_init_and_fit_predict(cuda):
     w = synthetic.config1(0.2)
     x = ht.array(w.x.to(cuda), split=0)
