@@ -182,7 +182,7 @@ def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: O
                                 c_new.stride(0) if k > 1 else d, _ptr(counts), _ptr(buf), buf.numel(), _stream()))
 
 
-def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: torch.Tensor,
+def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],
                shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace) -> None:
     _require_gpu(x, c, c_new, labels, sse)
     if not (shift.is_cuda or shift.is_pinned()):

@@ -7,8 +7,11 @@ host waits for the shift of step i: if the loop goes on (the usual case) the GPU
 stops the extra step is simply not used -- it writes to buffers the results of step i do not live
 in (three centroid buffers, two label buffers, two shift scalars in rotation).  The shift scalars
 live in pinned host memory and are written by the finishing kernel itself, so no copy-engine
-operation sits between two steps on the stream.  The values returned are exactly those of the
-sequential loop.
+operation sits between two steps on the stream.  For the narrow shapes whose step is one sweep of a
+vector kernel (D <= 8), writing N labels is a quarter of the step's memory traffic, so the steps run
+without storing labels and those of the last iteration are computed once, on demand, against the
+centroids that iteration started from -- the same kernel code, hence the same bits.  The values
+returned are exactly those of the sequential loop.
 """
 
 from __future__ import annotations
@@ -27,7 +30,11 @@ class LloydLoop:
         self.x = xt
         self.ws = ws
         self.c = [c0.clone(), torch.empty_like(c0), torch.empty_like(c0)]
-        self.lab = [torch.empty((xt.shape[0],), dtype=torch.int32, device=dev) for _ in range(2)]
+        n, d = xt.shape
+        self.lazy_labels = xt.dtype == torch.float32 and _native.lloyd_kernel_name(n, d, c0.shape[0]) == "lloyd_small"
+        nbuf = 1 if self.lazy_labels else 2
+        self.lab = [torch.empty((n,), dtype=torch.int32, device=dev) for _ in range(nbuf)]
+        self._lab_of = -1  # iteration whose labels self.lab[0] holds (lazy mode)
         self.shift_host = torch.zeros((2,), dtype=xt.dtype, pin_memory=True)
         self.ev = [torch.cuda.Event(), torch.cuda.Event()]
         self.enqueued = 0  # steps handed to the stream
@@ -35,8 +42,8 @@ class LloydLoop:
 
     def _enqueue(self) -> None:
         j = self.enqueued
-        _native.lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3], self.lab[j % 2], self.shift_host[j % 2],
-                           None, self.ws)
+        _native.lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3], None if self.lazy_labels else self.lab[j % 2],
+                           self.shift_host[j % 2], None, self.ws)
         self.ev[j % 2].record()
         self.enqueued = j + 1
 
@@ -68,7 +75,14 @@ class LloydLoop:
 
     @property
     def labels(self) -> torch.Tensor:
-        return self.lab[(self.done - 1) % 2]
+        """int32 labels of the last iteration that counts (against the centroids it started from)."""
+        i = self.done - 1
+        if not self.lazy_labels:
+            return self.lab[i % 2]
+        if self._lab_of != i:
+            _native.assign(self.x, self.c[i % 3], self.lab[0], None, self.ws)
+            self._lab_of = i
+        return self.lab[0]
 
     @property
     def last_shift(self) -> torch.Tensor:

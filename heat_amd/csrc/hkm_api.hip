@@ -243,7 +243,8 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     if ((rc = check_matrix("C", C, K, D, D))) return rc;
     if ((rc = check_matrix("C_new", C_new, K, D, D))) return rc;
     if (C == C_new) return fail(HKM_EINVAL, "C and C_new must not alias");
-    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (!labels && N > 0 && !small_eligible(D, K))
+        return fail(HKM_EINVAL, "labels is NULL (only the one-sweep small-D step can run without storing labels)");
     if (!shift) return fail(HKM_EINVAL, "shift is NULL");
     const int32_t flags = HKM_WS_LLOYD | (sse ? HKM_WS_SSE : 0);
     const size_t need = carve(nullptr, N, D, K, flags).total;

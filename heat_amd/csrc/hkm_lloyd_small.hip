@@ -206,18 +206,22 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             scan_centroids<D, PPT, true>(sC, 0, K, x, xn, m, mi);
         }
 
+        // labels == NULL: the caller only wants the sums (a fit needs the labels of its last
+        // iteration only and can recompute those)
         if constexpr (!GUARD) {
-            if constexpr (PPT == 4) {
-                *reinterpret_cast<int4*>(labels + i0) = make_int4(mi[0], mi[1], mi[2], mi[3]);
-            } else {
-                *reinterpret_cast<int2*>(labels + i0) = make_int2(mi[0], mi[1]);
+            if (labels) {
+                if constexpr (PPT == 4) {
+                    *reinterpret_cast<int4*>(labels + i0) = make_int4(mi[0], mi[1], mi[2], mi[3]);
+                } else {
+                    *reinterpret_cast<int2*>(labels + i0) = make_int2(mi[0], mi[1]);
+                }
             }
         }
 #pragma unroll
         for (int p = 0; p < PPT; ++p) {
             const bool ok = !GUARD || i0 + p < N;
             if (ok) {
-                if (GUARD) labels[i0 + p] = mi[p];
+                if (GUARD && labels) labels[i0 + p] = mi[p];
                 if (WANT_MIN) min_d2[i0 + p] = m[p];
                 if (WANT_SSE) sse += double(m[p]);
             } else {
