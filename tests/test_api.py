@@ -327,3 +327,25 @@ def test_manhattan_estimators_surface():
         with pytest.raises(RuntimeError):  # host data is refused, never computed on the CPU
             est.fit(host)
     assert _native.workspace_bytes(1000, 4, 8, _native.WS_MEDIAN) > 8 * 4 * 256 * 4
+
+
+def test_load_csv():
+    # the reference's clustering tests start from ht.load(<iris.csv>, sep=";", split=...)
+    import os
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "iris.csv")
+    a = ht.load(path, sep=";", split=0)
+    assert a.shape == (150, 4) and a.dtype is ht.float32 and a.split == 0
+    assert np.allclose(a.larray.numpy(), IRIS)
+    b = ht.load_csv(path, sep=";", header_lines=10, dtype=ht.float64, split=1)
+    assert b.shape == (140, 4) and b.dtype is ht.float64 and b.split == 1
+    with pytest.raises(TypeError):
+        ht.load_csv(12)
+    with pytest.raises(TypeError):
+        ht.load_csv(path, sep=3)
+    with pytest.raises(TypeError):
+        ht.load_csv(path, header_lines="3")
+    with pytest.raises(ValueError):
+        ht.load("data.txt")
+    with pytest.raises(RuntimeError):
+        ht.load("data.h5")
