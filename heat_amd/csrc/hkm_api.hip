@@ -2,6 +2,7 @@
 // Nothing here allocates device memory or synchronises; every entry point only enqueues kernels.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "hkm_common.h"
@@ -78,6 +79,11 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         w.counts = reinterpret_cast<int64_t*>(take(size_t(K) * sizeof(int64_t)));
         w.shift_part = reinterpret_cast<double*>(take((size_t(K) * D / 64 + 1) * sizeof(double)));
     }
+    if ((flags & HKM_WS_UPDATE) && sorted_update_eligible(K)) {
+        const int32_t elem = (flags & HKM_WS_F64) ? 8 : 4;
+        w.srt = carve_sorted(p ? p + off : nullptr, N, D, K, elem);
+        off += align_up(w.srt.total, 256);
+    }
     if ((flags & HKM_WS_LLOYD) == HKM_WS_LLOYD && !(flags & HKM_WS_F64) && fused_eligible(D, K)) {
         w.fsum = reinterpret_cast<double*>(take(size_t(FUSED_MAX_GRID) * K * D * sizeof(double)));
         w.fcnt = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * K * sizeof(int32_t)));
@@ -115,6 +121,31 @@ MedianWorkspace carve_median(void* base, int64_t N, int32_t D, int32_t K) {
     w.keys = reinterpret_cast<unsigned long long*>(take(size_t(K) * sizeof(unsigned long long)));
     w.total = off;
     return w;
+}
+
+// the two-pass update: stable sort + segmented sums where its per-wave cursors fit in LDS, the
+// list-based kernels otherwise.  HKM_UPDATE_LISTS=1 in the environment (looked up per call) forces
+// the latter: the one-sweep MFMA step falls back to exactly those kernels, and tests compare the two.
+static bool use_sorted_update(int32_t K) {
+    const char* e = getenv("HKM_UPDATE_LISTS");
+    const bool forced_lists = e && e[0] == '1';
+    return sorted_update_eligible(K) && !forced_lists;
+}
+
+static int do_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                     float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w, const float* C_old,
+                     float* shift, hipStream_t st) {
+    if (use_sorted_update(K))
+        return launch_update_sorted(X, N, D, ldx, labels, K, C_new, ldcn, counts, w.srt, C_old, shift, st);
+    return launch_update(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, C_old, shift, st);
+}
+
+static int do_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                         double* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
+                         const double* C_old, double* shift, hipStream_t st) {
+    if (use_sorted_update(K))
+        return launch_update_sorted_f64(X, N, D, ldx, labels, K, C_new, ldcn, counts, w.srt, C_old, shift, st);
+    return launch_update_f64(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, C_old, shift, st);
 }
 
 static int check_matrix(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
@@ -229,8 +260,8 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
     const size_t need = carve(nullptr, N, D, K, HKM_WS_UPDATE).total;
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const Workspace w = carve(ws, N, D, K, HKM_WS_UPDATE);
-    return launch_update(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, nullptr, nullptr,
-                         static_cast<hipStream_t>(hip_stream));
+    return do_update(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, nullptr, nullptr,
+                     static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
@@ -265,7 +296,7 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
             return rc;
     } else {
         if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;
-        if ((rc = launch_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
+        if ((rc = do_update(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
     }
     if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
     return rc;
@@ -362,8 +393,8 @@ int hkm_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int
     const size_t need = carve(nullptr, N, D, K, flags).total;
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const Workspace w = carve(ws, N, D, K, flags);
-    return launch_update_f64(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, nullptr, nullptr,
-                             static_cast<hipStream_t>(hip_stream));
+    return do_update_f64(X, N, D, ldx, labels, K, C_new, ldcn, counts, w, nullptr, nullptr,
+                         static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_lloyd_step_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, double* C_new,
@@ -385,7 +416,7 @@ int hkm_lloyd_step_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
     double* md = sse ? reinterpret_cast<double*>(w.min_d2) : nullptr;
     if (N > 0 && (rc = launch_assign_f64(X, N, D, ldx, C, K, D, labels, md, st))) return rc;
-    if ((rc = launch_update_f64(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
+    if ((rc = do_update_f64(X, N, D, ldx, labels, K, C_new, D, nullptr, w, C, shift, st))) return rc;
     if (sse) rc = launch_sum_min_d2_f64(md, N, sse, w.red, 1, st);
     return rc;
 }

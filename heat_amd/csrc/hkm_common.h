@@ -43,6 +43,20 @@ struct UpdateGeom {
 };
 UpdateGeom update_geom(int64_t N, int32_t D, int32_t K, int32_t elem = 4);
 
+// scratch of the sorted update (hkm_update_sorted.hip)
+struct SortedWorkspace {
+    int32_t* blk_cnt;      // [blocks][K] label counts of every block, then positions inside the cluster's segment
+    int64_t* counts;       // [K]
+    int64_t* offsets;      // [K + 1]
+    int32_t* chunk_start;  // [K + 1]
+    int32_t* perm;         // [N] row indices grouped by cluster, ascending inside a cluster
+    void* part;            // [chunks][D padded to 32] partial sums (float or double)
+    double* shift_part;
+    size_t total;
+};
+SortedWorkspace carve_sorted(void* base, int64_t N, int32_t D, int32_t K, int32_t elem);
+bool sorted_update_eligible(int32_t K);
+
 // ---- workspace layout --------------------------------------------------------------------------
 struct Workspace {
     float* cn;          // squared centroid norms, padded to a multiple of 128 with +inf
@@ -57,6 +71,7 @@ struct Workspace {
     double* fsum;       // [FUSED_MAX_GRID][K][D] fp64 partial sums of the one-sweep MFMA step
     int32_t* fcnt;      // [FUSED_MAX_GRID][K]
     int32_t* fflags;    // [FUSED_MAX_GRID] 1 = this workgroup's sums may depend on the addition order
+    SortedWorkspace srt; // scratch of the sorted update (with the UPDATE flag, K <= 4096)
     size_t total;
 };
 static const int RED_SLOTS = 2048;
@@ -116,6 +131,12 @@ int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, co
 int launch_update(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                   int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                   const float* C_old, float* shift, hipStream_t st);
+int launch_update_sorted(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                         float* C_new, int64_t ldcn, int64_t* counts, const SortedWorkspace& w,
+                         const float* C_old, float* shift, hipStream_t st);
+int launch_update_sorted_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
+                             int32_t K, double* C_new, int64_t ldcn, int64_t* counts,
+                             const SortedWorkspace& w, const double* C_old, double* shift, hipStream_t st);
 int launch_update_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                       int32_t K, double* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                       const double* C_old, double* shift, hipStream_t st);

@@ -107,9 +107,14 @@ UPDATE_SHAPES = [(1000, 3, 8), (5000, 8, 16), (4096, 32, 256), (3000, 64, 100), 
                  (30000, 128, 50), (20000, 132, 500), (6000, 512, 1024), (777, 256, 3)]
 
 
-@pytest.mark.parametrize("n,d,k", UPDATE_SHAPES)
-def test_update_matches_oracle(cuda, n, d, k):
-    print(f"update n={n} d={d} k={k}", flush=True)
+@pytest.mark.parametrize("path", ["sorted", "lists"])
+@pytest.mark.parametrize("n,d,k", UPDATE_SHAPES + [(20000, 5, 5000)])
+def test_update_matches_oracle(cuda, n, d, k, path, monkeypatch):
+    # two implementations of hkm_update_f32: stable sort + segmented sums (default up to K = 4096) and
+    # the list-based kernels (larger K, and the fallback of the one-sweep MFMA step)
+    print(f"update n={n} d={d} k={k} path={path}", flush=True)
+    if path == "lists":
+        monkeypatch.setenv("HKM_UPDATE_LISTS", "1")
     g = torch.Generator().manual_seed(n + k)
     x = torch.randn((n, d), generator=g) * 4 + 1
     lab = torch.randint(0, k, (n,), generator=g)
@@ -118,6 +123,9 @@ def test_update_matches_oracle(cuda, n, d, k):
     cnt = torch.full((k,), -1, dtype=torch.int64, device=cuda)
     _native.update(x.to(cuda), lab.to(torch.int32).to(cuda), c_new, cnt, _native.Workspace(cuda))
     torch.cuda.synchronize()
+    again = torch.empty_like(c_new)
+    _native.update(x.to(cuda), lab.to(torch.int32).to(cuda), again, None, _native.Workspace(cuda))
+    assert torch.equal(again, c_new), "two runs must be bit-identical"
     ref, ref_cnt = orc.update_centroids_fast(x, lab.view(-1, 1), k)
     assert torch.equal(cnt.cpu(), ref_cnt)
     assert int(cnt.sum()) == n
@@ -169,8 +177,20 @@ def test_lloyd_step_matches_oracle_and_is_deterministic(cuda, n, d, k):
     assert orc.rel_err_scalar(float(sse), ref_sse) <= 1e-4
 
 
-def _step_and_two_pass(xs, cs, dev):
-    """One hkm_lloyd_step_f32 and, from the same inputs, hkm_assign_f32 + hkm_update_f32."""
+def _step_and_two_pass(xs, cs, dev, lists=False):
+    """One hkm_lloyd_step_f32 and, from the same inputs, hkm_assign_f32 + hkm_update_f32 (``lists``:
+    with the list-based update kernels, which are also what the one-sweep step falls back to)."""
+    import os
+
+    if lists:
+        os.environ["HKM_UPDATE_LISTS"] = "1"
+    try:
+        return _step_and_two_pass_impl(xs, cs, dev)
+    finally:
+        os.environ.pop("HKM_UPDATE_LISTS", None)
+
+
+def _step_and_two_pass_impl(xs, cs, dev):
     n, k = xs.shape[0], cs.shape[0]
     ws = _native.Workspace(dev)
     c_step = torch.empty_like(cs)
@@ -224,11 +244,11 @@ def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
         c0 = xv[torch.randperm(n, generator=g)[:k]].contiguous()
         c0 = torch.nan_to_num(c0, nan=0.0, posinf=1.0, neginf=-1.0)
         xs, cs = xv.to(cuda), c0.to(cuda)
-        c_step, lab_step, shift, c2, lab2, _ = _step_and_two_pass(xs, cs, cuda)
+        c_step, lab_step, shift, c2, lab2, _ = _step_and_two_pass(xs, cs, cuda, lists=True)
         assert torch.equal(lab_step, lab2)
         assert torch.equal(c_step.isnan(), c2.isnan())
         assert torch.equal(torch.nan_to_num(c_step), torch.nan_to_num(c2)), variant
-        again = _step_and_two_pass(xs, cs, cuda)
+        again = _step_and_two_pass(xs, cs, cuda, lists=True)
         assert torch.equal(torch.nan_to_num(again[0]), torch.nan_to_num(c_step))
     # moderate spread (2^+-3) stays on the exact path: the result is the fp64 mean, which the fp32
     # partials of the two-pass update only approximate
