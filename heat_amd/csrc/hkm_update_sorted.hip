@@ -22,7 +22,7 @@
 namespace hkm {
 
 static constexpr int SRT_R = 2048;      // rows of one cluster per segmented-sum workgroup
-static constexpr int SRT_MAXBLK = 1024;  // blocks of the grouping passes
+static constexpr int SRT_MAXBLK = 4096;  // blocks of the grouping passes (one wave each)
 static constexpr int SRT_MAXK = 4096;    // per-wave LDS cursors: 4 waves x K x 4 B <= 64 KB
 
 bool sorted_update_eligible(int32_t K) { return K <= SRT_MAXK; }
