@@ -52,35 +52,42 @@ __device__ __forceinline__ void merge_halves(float& m, int& mi) {
 //
 // On this hardware every VALU instruction takes issue time away from the fp32 MFMA pipe (there is no
 // co-execution), so the epilogue is kept to three VALU instructions per distance:
-//   * the norms ride along in the contraction: LDS row k holds [-2*c_k (zero-padded to DP), |c_k|^2,
-//     1] and the point operand is extended by [1, |x|^2], so the accumulator IS
-//     (|x|^2 + |c|^2) - 2 x.c.  The extra step goes first, i.e. the accumulator starts at the rounded
-//     sum of the two norms like the reference's x_norm + y_norm, and scaling by -2 is exact;
+//   * LDS row k holds -2*c_k (zero-padded to DP; scaling by -2 is exact) and a separate LDS array the
+//     squared norms |c_k|^2; the accumulators of a block START at the norms of their centroid rows
+//     (the C operand of the first MFMA, four 16-byte LDS reads, no vector instruction), so they end
+//     as |c|^2 - 2 x.c.  |x|^2 is the same for every centroid: it is added to the minimum only;
 //   * the clamp at 0 is applied lazily: only if some running minimum went negative (a point that
 //     coincides with a centroid up to rounding) the tile is rescanned with the clamp on every value;
 //   * per value: compare, select index, select value (see resident_scan).  The lane-half term of the
 //     index is added once per tile.
 // ------------------------------------------------------------------------------------------------
-// One centroid block (32 rows) against the wave's PB point blocks: 1 + DP/2 MFMAs per point block.
-template <int DP, int PB>
-__device__ __forceinline__ void resident_block(const float* arow, int h, const floatx4 (&b)[PB][DP / 8],
-                                               const float (&baug)[PB], floatx16 (&acc)[PB]) {
-    constexpr int NJ = DP / 8;
-    const float aaug = arow[DP + h];
+// One centroid block (32 rows) against the wave's PB point blocks: DP/2 MFMAs per point block.  The
+// accumulators start at the squared norms of the lane's 16 centroid rows (cn16 points at the norm of
+// row 4*h of the block; rows 8g + 4h .. 8g + 4h + 3 belong to accumulator elements 4g .. 4g + 3), so
+// they end as |c|^2 - 2 x.c: the distance without the term |x|^2, which is the same for every centroid.
+__device__ __forceinline__ floatx16 load_cn16(const float* cn16) {
+    floatx16 c0;
 #pragma unroll
-    for (int pb = 0; pb < PB; ++pb) {
-        floatx16 z;
+    for (int g = 0; g < 4; ++g) {
+        const floatx4 t = ld4(cn16 + 8 * g);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) z[v] = 0.f;
-        acc[pb] = MFMA32(aaug, baug[pb], z);
+        for (int q = 0; q < 4; ++q) c0[4 * g + q] = t[q];
     }
+    return c0;
+}
+
+template <int DP, int PB>
+__device__ __forceinline__ void resident_block(const float* arow, const floatx16& c0, int h,
+                                               const floatx4 (&b)[PB][DP / 8], floatx16 (&acc)[PB]) {
+    constexpr int NJ = DP / 8;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const floatx4 a = ld4(arow + h * (DP / 2) + 4 * j);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int pb = 0; pb < PB; ++pb) acc[pb] = MFMA32(a[t], b[pb][j][t], acc[pb]);
+            for (int pb = 0; pb < PB; ++pb)
+                acc[pb] = (j == 0 && t == 0) ? MFMA32(a[t], b[pb][j][t], c0) : MFMA32(a[t], b[pb][j][t], acc[pb]);
     }
 }
 
@@ -89,9 +96,9 @@ __device__ __forceinline__ void resident_block(const float* arow, int h, const f
 // block.  Strict '<' everywhere keeps the first index on ties.  CLAMP applies max(., 0) to every
 // value (the rescan of a tile whose lazy minimum came out negative).
 template <int DP, int PB, bool CLAMP>
-__device__ __forceinline__ void resident_scan(const float* sC, int ncb, int p, int h,
+__device__ __forceinline__ void resident_scan(const float* sC, const float* sCn, int ncb, int p, int h,
                                               const floatx4 (&b)[PB][DP / 8],
-                                              const float (&baug)[PB], float (&m)[PB],
+                                              const float (&xn)[PB], float (&m)[PB],
                                               int (&mi)[PB]) {
     constexpr int LDC = DP + 4;
 #pragma unroll
@@ -99,18 +106,23 @@ __device__ __forceinline__ void resident_scan(const float* sC, int ncb, int p, i
         m[pb] = HKM_INF;
         mi[pb] = 0;
     }
+    // the norms of the next block are requested before the current block's MFMAs
+    floatx16 c0 = load_cn16(sCn + 4 * h);
     for (int cb = 0; cb < ncb; ++cb) {
         floatx16 acc[PB];
-        resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, h, b, baug, acc);
+        const floatx16 c0n = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
+        resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, c0, h, b, acc);
+        c0 = c0n;
         const int kb = cb * 32;
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
-            float bm = CLAMP ? fmaxf(acc[pb][0], 0.0f) : acc[pb][0];
+            // CLAMP: the full distance (|x|^2 + (|c|^2 - 2 x.c)) clamped at 0, as the reference orders them
+            float bm = CLAMP ? fmaxf(acc[pb][0] + xn[pb], 0.0f) : acc[pb][0];
             int bi = 0;
 #pragma unroll
             for (int v = 1; v < 16; ++v) {
                 float d = acc[pb][v];
-                if (CLAMP) d = fmaxf(d, 0.0f);
+                if (CLAMP) d = fmaxf(d + xn[pb], 0.0f);
                 const bool lt = d < bm;
                 bi = lt ? 8 * (v >> 2) + (v & 3) : bi;
                 bm = lt ? d : bm;
@@ -119,6 +131,11 @@ __device__ __forceinline__ void resident_scan(const float* sC, int ncb, int p, i
             mi[pb] = lt ? kb + bi : mi[pb];
             m[pb] = lt ? bm : m[pb];
         }
+    }
+    // without CLAMP the minimum still lacks |x|^2
+    if (!CLAMP) {
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) m[pb] += xn[pb];
     }
 }
 
@@ -130,7 +147,8 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     constexpr int LDC = DP + 4;  // row: DP scaled coordinates, |c|^2, 1, 2 pad; also keeps 16-B reads conflict-free
     constexpr int NJ = DP / 8;   // 16-byte groups per lane-half
     const int KP = (K + 31) & ~31;
-    float* sC = lds;  // [KP][LDC]
+    float* sC = lds;              // [KP][LDC]
+    float* sCn = lds + KP * LDC;  // [KP] squared norms
     const int tid = threadIdx.x;
 
     for (int i = tid; i < KP * DP; i += 256) {
@@ -144,8 +162,7 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
             const float* c = C + int64_t(r) * ldc;
             for (int d = 0; d < D; ++d) s = fmaf(c[d], c[d], s);
         }
-        sC[r * LDC + DP] = s;
-        sC[r * LDC + DP + 1] = 1.0f;
+        sCn[r] = s;
     }
     __syncthreads();
 
@@ -171,7 +188,7 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
         floatx4 b[PB][NJ];
-        float baug[PB], m[PB];
+        float xn[PB], m[PB];
         int mi[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
@@ -182,16 +199,15 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 #pragma unroll
                 for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
             }
-            const float xn = s + __shfl_xor(s, 32);
-            baug[pb] = h ? xn : 1.0f;  // pairs with [|c|^2, 1] of the centroid row
+            xn[pb] = s + __shfl_xor(s, 32);
         }
         if (tile + gridDim.x < ntiles) fetch(tile + gridDim.x);
 
-        resident_scan<DP, PB, false>(sC, ncb, p, h, b, baug, m, mi);
+        resident_scan<DP, PB, false>(sC, sCn, ncb, p, h, b, xn, m, mi);
         bool neg = false;
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) neg |= m[pb] < 0.f;
-        if (__any(neg)) resident_scan<DP, PB, true>(sC, ncb, p, h, b, baug, m, mi);
+        if (__any(neg)) resident_scan<DP, PB, true>(sC, sCn, ncb, p, h, b, xn, m, mi);
 
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
@@ -236,7 +252,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
     constexpr int NJ = DP / 8;
     const int KP = (K + 31) & ~31;
     float* sC = lds;                                              // [KP][LDC]
-    double* sA = reinterpret_cast<double*>(lds + KP * LDC);       // [K][LDA]
+    float* sCn = lds + KP * LDC;                                  // [KP] squared norms
+    double* sA = reinterpret_cast<double*>(sCn + KP);             // [K][LDA]
     int* sN = reinterpret_cast<int*>(sA + size_t(K) * LDA);       // [K] counts, then Emin, Emax
     const int tid = threadIdx.x, nthr = blockDim.x;
 
@@ -251,8 +268,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
             const float* c = C + int64_t(r) * ldc;
             for (int d = 0; d < D; ++d) s = fmaf(c[d], c[d], s);
         }
-        sC[r * LDC + DP] = s;
-        sC[r * LDC + DP + 1] = 1.0f;
+        sCn[r] = s;
     }
     for (int i = tid; i < K * LDA; i += nthr) sA[i] = 0.0;
     for (int i = tid; i < K; i += nthr) sN[i] = 0;
@@ -285,7 +301,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t row0 = tile * tile_rows + wave * (PB * 32);
         floatx4 b[PB][NJ];
-        float baug[PB], xnr[PB], m[PB];
+        float xnr[PB], m[PB];
         int mi[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
@@ -297,15 +313,14 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
                 for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
             }
             xnr[pb] = s + __shfl_xor(s, 32);
-            baug[pb] = h ? xnr[pb] : 1.0f;
         }
         if (tile + gridDim.x < ntiles) fetch(tile + gridDim.x);
 
-        resident_scan<DP, PB, false>(sC, ncb, p, h, b, baug, m, mi);
+        resident_scan<DP, PB, false>(sC, sCn, ncb, p, h, b, xnr, m, mi);
         bool neg = false;
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) neg |= m[pb] < 0.f;
-        if (__any(neg)) resident_scan<DP, PB, true>(sC, ncb, p, h, b, baug, m, mi);
+        if (__any(neg)) resident_scan<DP, PB, true>(sC, sCn, ncb, p, h, b, xnr, m, mi);
 
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
@@ -358,8 +373,10 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
 // resident kernel (a wave keeps its 32*PB points in B-operand registers for the whole feature range
 // and scans centroid blocks), but the centroids pass through LDS in tiles of 128 rows, double
 // buffered; all 256 threads fetch the next tile while the current one is scanned, one barrier per
-// tile (every 4*(1+DP/2)*PB MFMAs per wave).  The running (min, argmin) is carried across tiles, so
-// the clamp is applied eagerly here.  Squared centroid norms come from global memory.
+// tile (every 4*(DP/2)*PB MFMAs per wave).  The running (min, argmin) is carried across tiles and the
+// clamp at 0 is applied to the final minimum: where several centroids coincide with a point up to
+// rounding (several negative values) the most negative one wins instead of the first -- a tie at the
+// resolution of the formula.  Squared centroid norms come from global memory.
 // ------------------------------------------------------------------------------------------------
 template <int DP, int PB, bool VEC>
 __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
@@ -398,20 +415,18 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
     if (nsteps > 0) issue(0);
 
     floatx4 b[PB][NJ];
-    float baug[PB], m[PB];
+    float xn[PB], m[PB];
     int mi[PB];
 
     for (int64_t it = 0; it < nsteps; ++it) {
-        float* sC = lds + (it & 1) * (TC * LDC);
+        float* sC = lds + (it & 1) * (TC * LDC + TC);
+        float* sCn = sC + TC * LDC;
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
             const int g = tid + 256 * q;
             *reinterpret_cast<floatx4*>(sC + (g / GPR) * LDC + (g % GPR) * 4) = -2.0f * pc[q];
         }
-        if (tid < TC) {
-            sC[tid * LDC + DP] = pcn;
-            sC[tid * LDC + DP + 1] = 1.0f;
-        }
+        if (tid < TC) sCn[tid] = pcn;
         __syncthreads();
 
         const int64_t cur_tile = tile;
@@ -436,8 +451,7 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
 #pragma unroll
                     for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
                 }
-                const float xn = s + __shfl_xor(s, 32);
-                baug[pb] = h ? xn : 1.0f;
+                xn[pb] = s + __shfl_xor(s, 32);
                 m[pb] = HKM_INF;
                 mi[pb] = 0;
             }
@@ -446,15 +460,16 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
 #pragma unroll 1
         for (int cb = 0; cb < TC / 32; ++cb) {
             floatx16 acc[PB];
-            resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, h, b, baug, acc);
+            const floatx16 c0 = load_cn16(sCn + cb * 32 + 4 * h);
+            resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, c0, h, b, acc);
             const int kb = cur_ct * TC + cb * 32;
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
-                float bm = fmaxf(acc[pb][0], 0.0f);
+                float bm = acc[pb][0];
                 int bi = 0;
 #pragma unroll
                 for (int v = 1; v < 16; ++v) {
-                    const float d = fmaxf(acc[pb][v], 0.0f);
+                    const float d = acc[pb][v];
                     const bool lt = d < bm;
                     bi = lt ? 8 * (v >> 2) + (v & 3) : bi;
                     bm = lt ? d : bm;
@@ -468,7 +483,8 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
         if (cur_ct == nct - 1) {
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
-                float mm = m[pb];
+                // the distance gets its |x|^2 and the clamp at 0 here, once per point
+                float mm = fmaxf(m[pb] + xn[pb], 0.0f);
                 int ii = mi[pb] + 4 * h;
                 merge_halves(mm, ii);
                 const int64_t r = row0 + pb * 32 + p;
@@ -487,7 +503,7 @@ static int launch_tiled_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
                           hipStream_t st) {
     constexpr int PB = 2;
     const int64_t ntiles = (N + 4 * PB * 32 - 1) / (4 * PB * 32);
-    const size_t lds = size_t(2) * 128 * (DP + 4) * sizeof(float);
+    const size_t lds = size_t(2) * 128 * (DP + 5) * sizeof(float);
     auto kern = assign_mfma_tiled_kernel<DP, PB, VEC>;
     int64_t grid = int64_t(num_cus()) * 2;
     if (grid > ntiles) grid = ntiles;
@@ -536,7 +552,7 @@ static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, 
 size_t fused_lds_bytes(int32_t D, int32_t K) {
     const size_t kp = (size_t(K) + 31) / 32 * 32;
     const int dp = resident_dp(D);
-    return kp * (dp + 4) * sizeof(float) + size_t(K) * (dp + 1) * sizeof(double) + (size_t(K) + 4) * sizeof(int);
+    return kp * (dp + 5) * sizeof(float) + size_t(K) * (dp + 1) * sizeof(double) + (size_t(K) + 4) * sizeof(int);
 }
 
 int fused_grid(int64_t N) {

@@ -30,7 +30,7 @@ AssignKind assign_kind(int32_t D, int32_t K);
 static inline int resident_dp(int32_t D) { return D <= 24 ? 24 : D <= 32 ? 32 : D <= 48 ? 48 : 64; }
 static inline size_t resident_lds_bytes(int32_t D, int32_t K) {
     size_t kp = (size_t(K) + 31) / 32 * 32;
-    return kp * (resident_dp(D) + 4) * sizeof(float);
+    return kp * (resident_dp(D) + 5) * sizeof(float);  // rows of DP + 4 floats, plus the squared norms
 }
 
 // ---- geometry of the deterministic update ----------------------------------------------------
