@@ -15,6 +15,19 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 namespace hkm {
 
+#ifdef __HIPCC__
+// Orders a wave's LDS accesses across its lanes for the COMPILER: seen from one lane, a store and a
+// later load of another lane's address have no dependence, so without this a load may be merged with
+// an earlier one or moved across the store.  The hardware runs one wave's LDS operations in order,
+// so nothing is emitted.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+#endif
+
+
 // ---- error plumbing (hkm_api.hip) -----------------------------------------------------------
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);

@@ -1,12 +1,13 @@
 // One-sweep Lloyd step for small feature counts (D <= 8) and small K*(D+1): X is read from HBM
 // exactly once per iteration (4D bytes per point) and only the labels are written (4 bytes).
 //
-// Assignment: a lane owns PPT consecutive points in registers; centroids and their squared norms
-// sit in LDS and are read as wave-wide broadcasts; d2 = (|x|^2 + |c|^2) - 2 x.c exactly in the
-// reference's evaluation order (heat/spatial/distance.py:59-64), first index wins ties
-// (torch.min, heat/core/statistics.py:177).  The clamp at 0 is applied lazily: a negative minimum
-// (a point that coincides with a centroid up to rounding) triggers a rescan with the clamp applied
-// to every candidate, so the result equals clamping first.
+// Assignment: a lane owns PPT consecutive points in registers; the centroids (scaled by -2, which is
+// exact) and their squared norms sit in LDS and are read as wave-wide broadcasts.  The quadratic
+// expansion of heat/spatial/distance.py:59-64, d2 = |x|^2 + |c|^2 - 2 x.c, is evaluated as a chain of
+// D fused multiply-adds that starts at |c|^2; |x|^2, the same for every centroid, is added to the
+// minimum only.  First index wins ties (torch.min, heat/core/statistics.py:177).  The clamp at 0 is
+// applied lazily: a negative minimum (a point that coincides with a centroid up to rounding)
+// triggers a rescan with the clamp applied to every candidate, so the result equals clamping first.
 //
 // Update (heat/cluster/kmeans.py:76-103) without atomics, two strategies with a fixed summation order:
 //   K*(D+1) <= 48: every lane owns a private fp32 column per (cluster, coordinate) in LDS and adds
@@ -25,7 +26,11 @@
 
 namespace hkm {
 
-__device__ __forceinline__ floatx4 ldg4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
+// stream: the matrix is larger than the last-level cache, so its lines are not worth keeping there
+__device__ __forceinline__ floatx4 ldg4(const float* p, bool stream) {
+    const floatx4* q = reinterpret_cast<const floatx4*>(p);
+    return stream ? __builtin_nontemporal_load(q) : *q;
+}
 
 template <int D>
 struct SmallCfg {
@@ -82,11 +87,11 @@ __device__ __forceinline__ void scan_centroids(const float* sC, int k0, int k1,
         }
 #pragma unroll
         for (int p = 0; p < PPT; ++p) {
-            float dot = x[p][0] * c[0];
+            // c holds -2*c_k and |c_k|^2: the chain ends as |c|^2 - 2 x.c, D instructions per distance
+            float dist = fmaf(x[p][0], c[0], c[D]);
 #pragma unroll
-            for (int d = 1; d < D; ++d) dot = fmaf(x[p][d], c[d], dot);
-            float dist = fmaf(-2.0f, dot, xn[p] + c[D]);
-            if (CLAMP) dist = fmaxf(dist, 0.0f);
+            for (int d = 1; d < D; ++d) dist = fmaf(x[p][d], c[d], dist);
+            if (CLAMP) dist = fmaxf(dist + xn[p], 0.0f);
             mi[p] = dist < m[p] ? k : mi[p];
             m[p] = fminf(m[p], dist);
         }
@@ -108,6 +113,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     float* sC = lds;  // [K][SC]
     const int slots = K * (D + 1);
     constexpr bool ACCUM = ACC != 0;
+    const bool stream = (vec & 2) != 0;
     float* stage = lds + ((K * SC + 3) & ~3);                        // [NW][NV*64*4] transpose buffer
     float* after = stage + NW * NV * 256;
     double* wacc_all = reinterpret_cast<double*>(after);             // ACC==2: [NW][slots]
@@ -119,7 +125,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 
     for (int i = tid; i < K * SC; i += T) {
         const int r = i / SC, c = i - r * SC;
-        sC[i] = c < D ? C[int64_t(r) * ldc + c] : 0.f;
+        sC[i] = c < D ? C[int64_t(r) * ldc + c] : 0.f;  // scaled by -2 once the norms are taken
     }
     if (ACC == 2)
         for (int i = tid; i < NW * slots; i += T) wacc_all[i] = 0.0;
@@ -131,12 +137,14 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
         for (int d = 0; d < D; ++d) s = __fadd_rn(s, __fmul_rn(sC[r * SC + d], sC[r * SC + d]));
         sC[r * SC + D] = s;
+#pragma unroll
+        for (int d = 0; d < D; ++d) sC[r * SC + d] *= -2.0f;  // exact
     }
     __syncthreads();
 
     double sse = 0.0;
     const int64_t groups = (N + PPT - 1) / PPT;
-    const int64_t full = vec ? N / PPT : 0;  // groups served by the 16-byte vector path
+    const int64_t full = (vec & 1) ? N / PPT : 0;  // groups served by the 16-byte vector path
     const int64_t stride = int64_t(gridDim.x) * T;
 
     // ACC == 1: the additions of a round are deferred to the NEXT round and interleaved with its
@@ -194,9 +202,13 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             rmw_write(2, r);
             rmw_read(3, r);
         }
+        // |x|^2 is the same for every centroid: it joins the minimum only
         bool neg = false;
 #pragma unroll
-        for (int p = 0; p < PPT; ++p) neg |= (m[p] < 0.f);
+        for (int p = 0; p < PPT; ++p) {
+            m[p] += xn[p];
+            neg |= (m[p] < 0.f);
+        }
         if (__any(neg)) {
 #pragma unroll
             for (int p = 0; p < PPT; ++p) {
@@ -280,7 +292,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         for (int f = 0; f < PF; ++f) {
             if (base + f * stride + T <= full) {
 #pragma unroll
-                for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + f * rstride + v * 256);
+                for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + f * rstride + v * 256, stream);
             }
         }
         // The loop is unrolled PF times so that each round's buffer is a fixed set of registers: a
@@ -291,12 +303,17 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             for (int f = 0; f < PF; ++f) {
                 if (more) {
                     float x[PPT][D];
+                    // lanes exchange data through the wave's buffer: the fences tell the compiler
+                    // that other lanes read what this lane wrote (and wrote what it reads); the
+                    // hardware runs a wave's LDS operations in order
+                    wave_lds_sync();
 #pragma unroll
                     for (int v = 0; v < NV; ++v)
                         *reinterpret_cast<floatx4*>(wstage + v * 256 + lane * 4) = nxt[f][v];
+                    wave_lds_sync();
                     if (base + PF * stride + T <= full) {
 #pragma unroll
-                        for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + PF * rstride + v * 256);
+                        for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + PF * rstride + v * 256, stream);
                     }
                     wsrc += rstride;
 #pragma unroll
@@ -445,7 +462,9 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     const size_t lds = size_t((K * SC + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * NV * 256 * sizeof(float) +
                        (acc_mode == 2 ? size_t(SMALL_T / 64) * slots * sizeof(double)
                         : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float) : 0);
-    const int vec = (ldx == D) && aligned16(X) && aligned16(labels);
+    // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads
+    const int vec = ((ldx == D) && aligned16(X) && aligned16(labels) ? 1 : 0) |
+                    (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0);
 #define HKM_GO(A, M, S)                                                                             \
     hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S>), dim3(grid), dim3(SMALL_T), lds, st, X, N, ldx, \
                        C, K, ldc, labels, min_d2, part, vec)

@@ -102,6 +102,7 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
         const int npad = (nmax + U - 1) / U * U;
         if (lane < npad - n0) list0[n0 + lane] = make_int2(0, KR);
         if (lane < npad - n1) list1[n1 + lane] = make_int2(0, KR);
+        wave_lds_sync();  // the lists are read by other lanes than those that wrote them
 
         for (int t = 0; t < npad; t += U) {
             int2 e[U];
@@ -116,6 +117,7 @@ __global__ __launch_bounds__(UPD_THREADS) void update_partial_kernel(
                 if (count_here) cnt[e[u].y] += 1;
             }
         }
+        wave_lds_sync();  // the next batch overwrites the lists
     }
     __syncthreads();
 

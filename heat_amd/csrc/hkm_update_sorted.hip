@@ -42,11 +42,13 @@ __global__ __launch_bounds__(256) void srt_count_kernel(const int32_t* __restric
     int* cnt = lcnt + wave * K;
     for (int k = lane; k < K; k += 64) cnt[k] = 0;
     if (b >= nblk) return;
+    wave_lds_sync();
     const int64_t r0 = int64_t(b) * blk_rows, r1 = min(N, r0 + blk_rows);
     for (int64_t r = r0 + lane; r < r1; r += 64) {
         const int l = labels[r];
         if (l >= 0 && l < K) atomicAdd(&cnt[l], 1);
     }
+    wave_lds_sync();
     for (int k = lane; k < K; k += 64) blk_cnt[int64_t(b) * K + k] = cnt[k];
 }
 
@@ -93,6 +95,7 @@ __global__ __launch_bounds__(256) void srt_scatter_kernel(const int32_t* __restr
     const int64_t r0 = int64_t(b) * blk_rows, r1 = min(N, r0 + blk_rows);
     const unsigned long long lt = (1ull << lane) - 1ull;
     for (int64_t base = r0; base < r1; base += 64) {
+        wave_lds_sync();  // the cursors other lanes advanced in the previous batch
         const int64_t r = base + lane;
         int l = r < r1 ? labels[r] : -1;
         const bool ok = l >= 0 && l < K;
