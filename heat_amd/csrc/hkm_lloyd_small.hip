@@ -98,8 +98,29 @@ __device__ __forceinline__ void scan_centroids(const float* sC, int k0, int k1,
     }
 }
 
+// The same scan with the centroids in registers that are uniform over the wave (KT rows, those
+// beyond K hold |c|^2 = +inf and never win): no LDS reads and no loop in the round.
+template <int D, int PPT, int KT, bool CLAMP>
+__device__ __forceinline__ void scan_centroids_reg(const float (&cs)[KT][D + 1], int k0, int k1,
+                                                   const float (&x)[PPT][D], const float (&xn)[PPT],
+                                                   float (&m)[PPT], int (&mi)[PPT]) {
+#pragma unroll
+    for (int k = k0; k < k1; ++k) {
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            float dist = fmaf(x[p][0], cs[k][0], cs[k][D]);
+#pragma unroll
+            for (int d = 1; d < D; ++d) dist = fmaf(x[p][d], cs[k][d], dist);
+            if (CLAMP) dist = fmaxf(dist + xn[p], 0.0f);
+            mi[p] = dist < m[p] ? k : mi[p];
+            m[p] = fminf(m[p], dist);
+        }
+    }
+}
+
 // ACC: 0 = labels only, 1 = per-lane private LDS columns, 2 = DPP wave tree + per-wave fp64 rows
-template <int D, int ACC, bool WANT_MIN, bool WANT_SSE>
+// KT: 0 = centroids read from LDS in a loop over K; otherwise K <= KT and they sit in registers
+template <int D, int ACC, bool WANT_MIN, bool WANT_SSE, int KT>
 __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const float* __restrict__ X, int64_t N, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2,
@@ -141,6 +162,19 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         for (int d = 0; d < D; ++d) sC[r * SC + d] *= -2.0f;  // exact
     }
     __syncthreads();
+
+    // KT > 0: one copy of the centroid table per wave, in scalar registers
+    constexpr int KR = KT > 0 ? KT : 1;
+    float cs[KR][D + 1];
+    if (KT > 0) {
+#pragma unroll
+        for (int k = 0; k < KR; ++k)
+#pragma unroll
+            for (int d = 0; d <= D; ++d) {
+                const float v = k < K ? sC[k * SC + d] : (d == D ? HKM_INF : 0.f);
+                cs[k][d] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+            }
+    }
 
     double sse = 0.0;
     const int64_t groups = (N + PPT - 1) / PPT;
@@ -187,17 +221,19 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             m[p] = HKM_INF;
             mi[p] = 0;
         }
-        const int kh = K >> 1;
+        const int kh = KT > 0 ? KT / 2 : K >> 1;
         if (ACC == 1 && PPT == 4) {
             rmw_write(0, r);
             rmw_read(1, r);
         }
-        scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
+        if constexpr (KT > 0) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
+        else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
         if (ACC == 1) {
             rmw_write(PPT == 4 ? 1 : 0, r);
             rmw_read(PPT == 4 ? 2 : 1, r);
         }
-        scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
+        if constexpr (KT > 0) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
+        else scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
         if (ACC == 1 && PPT == 4) {
             rmw_write(2, r);
             rmw_read(3, r);
@@ -215,7 +251,8 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 m[p] = HKM_INF;
                 mi[p] = 0;
             }
-            scan_centroids<D, PPT, true>(sC, 0, K, x, xn, m, mi);
+            if constexpr (KT > 0) scan_centroids_reg<D, PPT, KR, true>(cs, 0, KR, x, xn, m, mi);
+            else scan_centroids<D, PPT, true>(sC, 0, K, x, xn, m, mi);
         }
 
         // labels == NULL: the caller only wants the sums (a fit needs the labels of its last
@@ -465,9 +502,18 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads
     const int vec = ((ldx == D) && aligned16(X) && aligned16(labels) ? 1 : 0) |
                     (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0);
-#define HKM_GO(A, M, S)                                                                             \
-    hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S>), dim3(grid), dim3(SMALL_T), lds, st, X, N, ldx, \
-                       C, K, ldc, labels, min_d2, part, vec)
+    // the register-resident centroid table: K <= 8 rows of at most 5 values
+    constexpr int KT8 = D <= 4 ? 8 : 0;
+    const bool reg = KT8 > 0 && K <= KT8;
+#define HKM_GO(A, M, S)                                                                                  \
+    do {                                                                                                 \
+        if (reg)                                                                                         \
+            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, KT8>), dim3(grid), dim3(SMALL_T), lds, st, X, \
+                               N, ldx, C, K, ldc, labels, min_d2, part, vec);                            \
+        else                                                                                             \
+            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, 0>), dim3(grid), dim3(SMALL_T), lds, st, X, \
+                               N, ldx, C, K, ldc, labels, min_d2, part, vec);                            \
+    } while (0)
     if (acc_mode == 1) {
         if (want_sse) HKM_GO(1, false, true);
         else HKM_GO(1, false, false);
