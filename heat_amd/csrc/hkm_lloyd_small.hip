@@ -41,13 +41,27 @@ struct SmallCfg {
 
 bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
 static constexpr int SMALL_T = 256;
+// LDS of one workgroup; acc_mode as in the kernel (0 labels only, 1 lane columns, 2 wave rows)
+static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
+    const int ppt = (D % 2 == 0) ? 2 : 4;
+    const int sc = (D + 1 + 3) / 4 * 4, nv = ppt * D / 4, slots = K * (D + 1);
+    return size_t((K * sc + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) +
+           (acc_mode == 2 ? size_t(SMALL_T / 64) * slots * sizeof(double)
+            : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float) : 0);
+}
+static int small_acc_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : 2; }
+
 int small_grid(int64_t N, int32_t D, int32_t K) {
-    (void)K;
     const int ppt = (D % 2 == 0) ? 2 : 4;
     const int64_t groups = (N + ppt - 1) / ppt;
-    // one group per lane until 4 workgroups per CU are reached, then grid-stride
+    // one group per lane until every CU holds as many workgroups as fit (4 by registers, fewer if the
+    // accumulating variant's LDS says so: a grid beyond that would run in two uneven batches), then
+    // grid-stride
     int64_t want = (groups + SMALL_T - 1) / SMALL_T;
-    int64_t cap = int64_t(num_cus()) * 4;
+    int64_t per_cu = int64_t(160 * 1024) / int64_t(small_lds_bytes(D, K, small_acc_mode(D, K)));
+    if (per_cu > 4) per_cu = 4;
+    if (per_cu < 1) per_cu = 1;
+    int64_t cap = int64_t(num_cus()) * per_cu;
     if (cap > SMALL_MAX_GRID) cap = SMALL_MAX_GRID;
     if (want > cap) want = cap;
     if (want < 1) want = 1;
@@ -490,15 +504,10 @@ template <int D>
 static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C, int32_t K,
                           int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
                           int grid, hipStream_t st) {
-    constexpr int SC = SmallCfg<D>::SC;
     const bool accum = mode & 1, want_sse = mode & 2, want_min = min_d2 != nullptr;
-    constexpr int NV = SmallCfg<D>::PPT * D / 4;
-    const int slots = K * (D + 1);
     // per-lane LDS columns while they fit (slots * 1 KB), the DPP tree otherwise
-    const int acc_mode = !accum ? 0 : (slots <= 48 ? 1 : 2);
-    const size_t lds = size_t((K * SC + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * NV * 256 * sizeof(float) +
-                       (acc_mode == 2 ? size_t(SMALL_T / 64) * slots * sizeof(double)
-                        : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float) : 0);
+    const int acc_mode = !accum ? 0 : small_acc_mode(D, K);
+    const size_t lds = small_lds_bytes(D, K, acc_mode);
     // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads
     const int vec = ((ldx == D) && aligned16(X) && aligned16(labels) ? 1 : 0) |
                     (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0);
