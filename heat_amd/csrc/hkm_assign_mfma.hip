@@ -632,8 +632,8 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
 // threads one chunk ahead and staged through double-buffered LDS (row stride 36 floats keeps the
 // 16-byte operand reads conflict-free).  After the last chunk one more MFMA adds
 // (-|c|^2/2) * 1 + 1 * (-|x|^2/2), so the accumulator is minus half the squared distance (squared
-// centroid norms come from global memory, padded with +inf; |x|^2 is accumulated from the point
-// operand on the way).
+// centroid norms come from global memory, padded with +inf; |x|^2 is accumulated by the staging
+// threads from the registers they stage and combined once per tile).
 //
 // Work items are laid out so that the workgroups of one XCD (workgroup b runs on XCD b % 8) work on
 // the SAME few point tiles at the same time, one centroid tile each: a point tile is then read from
@@ -694,6 +694,7 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     __shared__ __align__(16) float sB[2][TP * LDS_LD];
     __shared__ float sM[2][TP];
     __shared__ int sI[2][TP];
+    __shared__ float sXn[TP];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wp = wave & 1, wc = wave >> 1;  // this wave: points [64 wp, +64), centroids [64 wc, +64)
@@ -712,26 +713,58 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     const int sr = tid >> 3;         // staging: rows sr + 32 q (q = 0..3) of both panels
     const int sc = (tid & 7) * 4;    // column group
 
-    floatx4 pa[4], pb_[4];
-    auto issue = [&](int64_t xt, int ct, int dc) {
+    // Addresses of a chunk's loads are (workgroup-uniform panel base, advanced by scalar arithmetic)
+    // + (a per-thread byte offset that only changes with the tile): no vector instruction per chunk.
+    // Rows beyond K or N are clamped to the last valid row (a padding centroid has |c|^2 = +inf and
+    // never wins; a padding point is never stored).
+    const float* baseA = C;
+    const float* baseB = X;
+    unsigned offA[4], offB[4];
+    auto set_tile = [&](int64_t xt, int ct) {
+        baseA = C + int64_t(ct) * TC * ldc;
+        baseB = X + xt * TP * ldx;
+        const int lastA = K - 1 - ct * TC;
+        const int64_t lastB = N - 1 - xt * TP;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int rc = ct * TC + sr + 32 * q;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if (rc < K) v = load_row4<VEC>(C + int64_t(rc) * ldc, dc * DC + sc, D);
-            pa[q] = v;
-            int64_t rp = xt * TP + sr + 32 * q;
-            rp = rp < N ? rp : N - 1;
-            pb_[q] = load_row4<VEC>(X + rp * ldx, dc * DC + sc, D);
+            const int r = sr + 32 * q;
+            const int ra = r < lastA ? r : lastA;
+            const int rb = r < lastB ? r : int(lastB);
+            offA[q] = unsigned((int64_t(ra) * ldc + sc) * 4);
+            offB[q] = unsigned((int64_t(rb) * ldx + sc) * 4);
+        }
+    };
+    floatx4 pa[4], pb_[4];
+    auto issue = [&](int dc) {
+        const float* a = baseA + dc * DC;
+        const float* bq = baseB + dc * DC;
+        if (VEC && dc * DC + DC <= D) {  // whole chunk inside the rows: unconditional 16-byte loads
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                pa[q] = *reinterpret_cast<const floatx4*>(reinterpret_cast<const char*>(a) + offA[q]);
+                pb_[q] = *reinterpret_cast<const floatx4*>(reinterpret_cast<const char*>(bq) + offB[q]);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                // offsets hold the column group; load_row4 wants the row start and the column
+                pa[q] = load_row4<VEC>(reinterpret_cast<const float*>(reinterpret_cast<const char*>(a) + offA[q]) - sc - dc * DC,
+                                       dc * DC + sc, D);
+                pb_[q] = load_row4<VEC>(reinterpret_cast<const float*>(reinterpret_cast<const char*>(bq) + offB[q]) - sc - dc * DC,
+                                        dc * DC + sc, D);
+            }
         }
     };
 
     int64_t xi = 0;  // index of the point tile within this workgroup's sequence
     int ci = 0, dc = 0;
-    if (nsteps > 0) issue(xt0, ct0, 0);
+    if (nsteps > 0) {
+        set_tile(xt0, ct0);
+        issue(0);
+    }
 
     floatx16 acc[PB][CB];
-    float xs[PB] = {0.f, 0.f};
+    float xsq[4] = {0.f, 0.f, 0.f, 0.f};  // |x|^2 of staging rows sr + 32 q over this thread's column group
 
     for (int64_t it = 0; it < nsteps; ++it) {
         const int buf = int(it & 1);
@@ -739,6 +772,8 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         for (int q = 0; q < 4; ++q) {
             *reinterpret_cast<floatx4*>(&sA[buf][(sr + 32 * q) * LDS_LD + sc]) = pa[q];
             *reinterpret_cast<floatx4*>(&sB[buf][(sr + 32 * q) * LDS_LD + sc]) = pb_[q];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) xsq[q] = fmaf(pb_[q][t], pb_[q][t], xsq[q]);
         }
         __syncthreads();
 
@@ -750,13 +785,13 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
                 ci = 0;
                 ++xi;
             }
+            if (it + 1 < nsteps) set_tile(xt0 + xi * xstep, ct0 + ci * W);
         }
-        if (it + 1 < nsteps) issue(xt0 + xi * xstep, ct0 + ci * W, dc);
+        if (it + 1 < nsteps) issue(dc);
 
         if (cur_dc == 0) {
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
-                xs[pb] = 0.f;
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
@@ -770,11 +805,7 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         for (int pb = 0; pb < PB; ++pb) {
             const float* brow = &sB[buf][(wp * 64 + pb * 32 + p) * LDS_LD + h * 16];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                b[pb][j] = ld4(brow + 4 * j);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) xs[pb] = fmaf(b[pb][j][t], b[pb][j][t], xs[pb]);
-            }
+            for (int j = 0; j < 4; ++j) b[pb][j] = ld4(brow + 4 * j);
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
@@ -791,11 +822,22 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
         }
 
         if (cur_dc == ndc - 1) {
+            // squared norms of the tile's points: the eight threads that staged a row add their parts
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v = xsq[q];
+                v += __shfl_xor(v, 1);
+                v += __shfl_xor(v, 2);
+                v += __shfl_xor(v, 4);
+                if ((tid & 7) == 0) sXn[sr + 32 * q] = v;
+                xsq[q] = 0.f;
+            }
+            __syncthreads();
             float m[PB];
             int mi[PB];
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) {
-                const float xn = xs[pb] + __shfl_xor(xs[pb], 32);
+                const float xn = sXn[wp * 64 + pb * 32 + p];
                 const float baug = h ? -0.5f * xn : 1.0f;
                 m[pb] = -HKM_INF;
                 mi[pb] = 0;
