@@ -51,15 +51,16 @@ __device__ __forceinline__ void merge_halves(float& m, int& mi) {
 // B-operand registers.  No barrier inside the tile loop.
 //
 // On this hardware every VALU instruction takes issue time away from the fp32 MFMA pipe (there is no
-// co-execution), so the epilogue is kept to three VALU instructions per distance:
+// co-execution), so the epilogue is kept to fewer than three VALU instructions per distance:
 //   * LDS row k holds -2*c_k (zero-padded to DP; scaling by -2 is exact) and a separate LDS array the
 //     squared norms |c_k|^2; the accumulators of a block START at the norms of their centroid rows
 //     (the C operand of the first MFMA, four 16-byte LDS reads, no vector instruction), so they end
 //     as |c|^2 - 2 x.c.  |x|^2 is the same for every centroid: it is added to the minimum only;
 //   * the clamp at 0 is applied lazily: only if some running minimum went negative (a point that
 //     coincides with a centroid up to rounding) the tile is rescanned with the clamp on every value;
-//   * per value: compare, select index, select value (see resident_scan).  The lane-half term of the
-//     index is added once per tile.
+//   * per block of 16 values a tree of three-input minima; only if that improves the running minimum
+//     the position is looked up by equality (see block_argmin).  The lane-half term of the index is
+//     added once per tile.
 // ------------------------------------------------------------------------------------------------
 // One centroid block (32 rows) against the wave's PB point blocks: DP/2 MFMAs per point block.  The
 // accumulators start at the squared norms of the lane's 16 centroid rows (cn16 points at the norm of
@@ -91,10 +92,36 @@ __device__ __forceinline__ void resident_block(const float* arow, const floatx16
     }
 }
 
-// Scan of all centroid blocks: per distance compare, select index, select value; the block-local
-// first minimum (candidate indices are small literals) is merged into the running minimum once per
-// block.  Strict '<' everywhere keeps the first index on ties.  CLAMP applies max(., 0) to every
-// value (the rescan of a tile whose lazy minimum came out negative).
+// Minimum and first argmin over the 16 distances a lane holds of one centroid block, merged into the
+// running (m, mi).  The minimum is a tree of three-input minima (8 instructions, no dependence on
+// compare results); only lanes whose block minimum improves the running one look for its position,
+// by equality from the last register down so that the first one wins -- independent compares, then a
+// chain of selects with literal indices.  Strict '<' keeps the earlier block on ties.  NaNs never win.
+__device__ __forceinline__ void block_argmin(const floatx16& d, int kb, float& m, int& mi) {
+    const float t0 = fminf(fminf(d[0], d[1]), d[2]);
+    const float t1 = fminf(fminf(d[3], d[4]), d[5]);
+    const float t2 = fminf(fminf(d[6], d[7]), d[8]);
+    const float t3 = fminf(fminf(d[9], d[10]), d[11]);
+    const float t4 = fminf(fminf(d[12], d[13]), d[14]);
+    const float bm = fminf(fminf(fminf(t0, t1), t2), fminf(fminf(t3, t4), d[15]));
+    if (bm < m) {
+        // all compares first (each into its own scalar register pair), then the selects: a select
+        // right behind the compare it consumes would wait for it
+        bool e[15];
+#pragma unroll
+        for (int v = 0; v < 15; ++v) e[v] = d[v] == bm;
+        __builtin_amdgcn_sched_barrier(0);
+        int bi = 8 * (15 >> 2) + (15 & 3);
+#pragma unroll
+        for (int v = 14; v >= 0; --v) bi = e[v] ? 8 * (v >> 2) + (v & 3) : bi;
+        mi = kb + bi;
+        m = bm;
+    }
+}
+
+// Scan of all centroid blocks.  CLAMP applies max(. + |x|^2, 0) to every value (the rescan of a tile
+// whose lazy minimum came out negative).  Two blocks per trip: the squared norms of a block are
+// requested one block ahead into registers that then serve, in place, as an accumulator.
 template <int DP, int PB, bool CLAMP>
 __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn, int ncb, int p, int h,
                                               const floatx4 (&b)[PB][DP / 8],
@@ -106,30 +133,26 @@ __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn,
         m[pb] = HKM_INF;
         mi[pb] = 0;
     }
-    // the norms of the next block are requested before the current block's MFMAs
-    floatx16 c0 = load_cn16(sCn + 4 * h);
-    for (int cb = 0; cb < ncb; ++cb) {
+    auto one_block = [&](int cb, const floatx16& c0) {
         floatx16 acc[PB];
-        const floatx16 c0n = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
         resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, c0, h, b, acc);
-        c0 = c0n;
-        const int kb = cb * 32;
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
-            // CLAMP: the full distance (|x|^2 + (|c|^2 - 2 x.c)) clamped at 0, as the reference orders them
-            float bm = CLAMP ? fmaxf(acc[pb][0] + xn[pb], 0.0f) : acc[pb][0];
-            int bi = 0;
+            if (CLAMP) {
+                // the full distance (|x|^2 + (|c|^2 - 2 x.c)) clamped at 0, as the reference orders them
 #pragma unroll
-            for (int v = 1; v < 16; ++v) {
-                float d = acc[pb][v];
-                if (CLAMP) d = fmaxf(d + xn[pb], 0.0f);
-                const bool lt = d < bm;
-                bi = lt ? 8 * (v >> 2) + (v & 3) : bi;
-                bm = lt ? d : bm;
+                for (int v = 0; v < 16; ++v) acc[pb][v] = fmaxf(acc[pb][v] + xn[pb], 0.0f);
             }
-            const bool lt = bm < m[pb];
-            mi[pb] = lt ? kb + bi : mi[pb];
-            m[pb] = lt ? bm : m[pb];
+            block_argmin(acc[pb], cb * 32, m[pb], mi[pb]);
+        }
+    };
+    floatx16 ca = load_cn16(sCn + 4 * h);
+    for (int cb = 0; cb < ncb; cb += 2) {
+        const floatx16 cb1 = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
+        one_block(cb, ca);
+        if (cb + 1 < ncb) {
+            ca = load_cn16(sCn + (cb + 2 < ncb ? cb + 2 : cb + 1) * 32 + 4 * h);
+            one_block(cb + 1, cb1);
         }
     }
     // without CLAMP the minimum still lacks |x|^2
@@ -464,20 +487,7 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
             resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, c0, h, b, acc);
             const int kb = cur_ct * TC + cb * 32;
 #pragma unroll
-            for (int pb = 0; pb < PB; ++pb) {
-                float bm = acc[pb][0];
-                int bi = 0;
-#pragma unroll
-                for (int v = 1; v < 16; ++v) {
-                    const float d = acc[pb][v];
-                    const bool lt = d < bm;
-                    bi = lt ? 8 * (v >> 2) + (v & 3) : bi;
-                    bm = lt ? d : bm;
-                }
-                const bool lt = bm < m[pb];
-                mi[pb] = lt ? kb + bi : mi[pb];
-                m[pb] = lt ? bm : m[pb];
-            }
+            for (int pb = 0; pb < PB; ++pb) block_argmin(acc[pb], kb, m[pb], mi[pb]);
         }
 
         if (cur_ct == nct - 1) {
