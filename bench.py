@@ -99,6 +99,61 @@ def bench_kmedians(args, w, x, t_gen) -> int:
     return 0
 
 
+def bench_cdist(args, w, x, t_gen) -> int:
+    """The public full-matrix ht.spatial.cdist(X, Y, quadratic_expansion=True) on rows of the c2 data:
+    X = the first 32768 rows, Y = the next 32768 rows (D = 64), a 4.29 GB matrix of sqrt distances per
+    step, written into one resident output buffer through the C ABI.  flops = 2 M N D."""
+    import torch
+
+    from heat_amd import _native
+
+    if args.config != "c2":
+        print("--estimator cdist runs on the c2 data", file=sys.stderr)
+        return 2
+    m = nn = min(32768, x.shape[0] // 2)
+    d = x.shape[1]
+    xa, ya = x[:m], x[m:m + nn]
+    out = torch.empty((m, nn), dtype=torch.float32, device=x.device)
+
+    def step():
+        _native.pairwise(xa, ya, out, _native.METRIC_EUCLID_QE)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ev = []
+    for _ in range(args.steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step()
+        e1.record()
+        torch.cuda.synchronize()
+        ev.append(e0.elapsed_time(e1))
+    kern_ms = sum(ev) / len(ev)
+    flops = 2.0 * m * nn * d
+    out_bytes = 4.0 * m * nn
+    res = {
+        "metric": "cdist GFLOP/s", "value": round(flops * args.steps / elapsed / 1e9, 1), "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32",
+        "data": f"synthetic (seed {w.seed}, generated on CPU in {t_gen:.1f} s, resident in HBM before timing)",
+        "config": {"workload": f"cdist_full_m{m}_n{nn}_d{d}", "M": m, "N": nn, "D": d, "scale": args.scale},
+        "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 3), "peak": 157.3,
+                     "unit": "TFLOP/s", "frac": round(flops / (kern_ms * 1e-3) / 1e12 / 157.3, 4),
+                     "hbm_frac": round(out_bytes / (kern_ms * 1e-3) / 8e12, 4),
+                     "kernel": "cdist_mfma", "kernel_ms": round(kern_ms, 4), "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(res))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,8 +162,9 @@ def main() -> int:
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink N (testing only; invalidates the figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians"],
-                    help="kmedians: the Manhattan-metric sibling on the same data (not the headline metric)")
+    ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians", "cdist"],
+                    help="kmedians: the Manhattan-metric sibling on the same data; cdist: the full-matrix "
+                         "public cdist on rows of c2 (neither is the headline metric)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
@@ -140,6 +196,8 @@ def main() -> int:
     ev_ms = []
     if args.estimator == "kmedians":
         return bench_kmedians(args, w, x, t_gen)
+    if args.estimator == "cdist":
+        return bench_cdist(args, w, x, t_gen)
     if args.config == "c2":
         # assignment only: labels + min squared distance
         y = w.y.to(dev)

@@ -35,19 +35,9 @@ __global__ __launch_bounds__(256) void cdist_kernel(const T* __restrict__ X, int
     const int64_t tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
     const int64_t i0 = tm * CD_T, j0 = tn * CD_T;
 
-    // squared norms of the tile's rows / columns, each summed in feature order
-    if (tid < 2 * CD_T) {
-        const bool is_x = tid < CD_T;
-        const int r = is_x ? tid : tid - CD_T;
-        const int64_t g = (is_x ? i0 : j0) + r;
-        const int64_t lim = is_x ? M : Nn;
-        T s = T(0);
-        if (g < lim) {
-            const T* row = is_x ? X + g * ldx : Y + g * ldy;
-            for (int d = 0; d < D; ++d) s = cd_fma(row[d], row[d], s);
-        }
-        (is_x ? sXn : sYn)[r] = s;
-    }
+    // squared norms of the tile's rows / columns (quadratic expansion only), each summed in feature
+    // order from the staged chunks: thread r < 64 owns row r of the X tile, thread 64 + r row r of Y
+    T nrm = T(0);
 
     const int tx = tid & 15, ty = tid >> 4;
     T acc[4][4];
@@ -69,6 +59,12 @@ __global__ __launch_bounds__(256) void cdist_kernel(const T* __restrict__ X, int
             sY[lk][r] = (gj < Nn && d < D) ? Y[gj * ldy + d] : T(0);
         }
         __syncthreads();
+        if (METRIC == 0 && tid < 2 * CD_T) {
+            const T(*tile)[CD_T + 4] = tid < CD_T ? sX : sY;
+            const int r = tid & (CD_T - 1);
+#pragma unroll
+            for (int k = 0; k < CD_KC; ++k) nrm = cd_fma(tile[k][r], tile[k][r], nrm);
+        }
 #pragma unroll
         for (int k = 0; k < CD_KC; ++k) {
             T xa[4], yb[4];
@@ -91,13 +87,16 @@ __global__ __launch_bounds__(256) void cdist_kernel(const T* __restrict__ X, int
                 }
         }
     }
-    __syncthreads();
+    if (METRIC == 0) {
+        if (tid < 2 * CD_T) (tid < CD_T ? sXn : sYn)[tid & (CD_T - 1)] = nrm;
+        __syncthreads();
+    }
 
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
         const int64_t gi = i0 + ty * 4 + a;
         if (gi >= M) continue;
-        const T xn = sXn[ty * 4 + a];
+        const T xn = METRIC == 0 ? sXn[ty * 4 + a] : T(0);
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const int64_t gj = j0 + tx * 4 + b;
@@ -136,6 +135,9 @@ static int launch_cdist_t(const T* X, int64_t M, int64_t ldx, const T* Y, int64_
 int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                  int32_t D, float* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, float gauss,
                  hipStream_t st) {
+    // the quadratic expansion is a matrix product: matrix cores from 16 features on
+    if (metric == 0 && cdist_mfma_eligible(M, Nn, D, ldx, ldy, ldo))
+        return launch_cdist_mfma(X, M, ldx, Y, Nn, ldy, D, out, ldo, sqrt_flag, gauss, st);
     return launch_cdist_t<float>(X, M, ldx, Y, Nn, ldy, D, out, ldo, metric, sqrt_flag, gauss, st);
 }
 

@@ -166,6 +166,9 @@ int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, f
                  hipStream_t st);
 int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, int mode,
                       hipStream_t st);
+bool cdist_mfma_eligible(int64_t M, int64_t Nn, int32_t D, int64_t ldx, int64_t ldy, int64_t ldo);
+int launch_cdist_mfma(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
+                      int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, float gauss, hipStream_t st);
 int launch_cdist(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                  int32_t D, float* out, int64_t ldo, int32_t metric, int32_t sqrt_flag, float gauss,
                  hipStream_t st);
