@@ -296,6 +296,60 @@ def test_cdist_known_answers_and_oracle(cuda):
         assert float((out.cpu().double() - bf).abs().max()) <= 1e-3
 
 
+@pytest.mark.parametrize("m,n,d", [(300, 257, 40), (129, 1, 64), (1000, 700, 100), (128, 128, 32), (5, 3, 18),
+                                   (200, 333, 16), (64, 513, 130)])
+def test_cdist_matrix_core_path(cuda, m, n, d):
+    """Quadratic-expansion full matrices from 16 features on take the matrix-core kernel: ragged tiles,
+    feature counts that are no multiple of the chunk or of 4, strided rows, every epilogue."""
+    g = torch.Generator().manual_seed(m * 7 + n * 3 + d)
+    a, b = torch.randn((m, d), generator=g) * 3, torch.randn((n, d), generator=g) * 3
+    scale = float((a.double() ** 2).sum(1).max() + (b.double() ** 2).sum(1).max())
+    ref = orc.quadratic_expand(a, b)
+    bf = orc.brute_force_d2(a, b)
+    ag, bg = a.to(cuda), b.to(cuda)
+    out = torch.full((m, n + 5), -7.0, device=cuda)[:, :n]  # strided output, guard columns behind it
+    _native.cdist(ag, bg, out, sqrt=False)
+    assert float((out.cpu() - ref).abs().max()) <= 2e-6 * scale
+    assert float(out.min()) >= 0.0
+    assert torch.all(out._base[:, n:] == -7.0), "stores beyond the last column"
+    _native.pairwise(ag, bg, out, _native.METRIC_EUCLID_QE)
+    assert float((out.cpu().double() ** 2 - bf).abs().max()) <= 4e-6 * scale
+    _native.pairwise(ag, bg, out, _native.METRIC_GAUSS_QE, 2.5)
+    want = torch.exp(-bf / (2 * 2.5 ** 2))
+    assert float((out.cpu().double() - want).abs().max()) <= 1e-5 + 4e-6 * scale / (2 * 2.5 ** 2)
+    # strided inputs (rows embedded in wider matrices, 16-byte alignment lost for odd strides)
+    wide_a = torch.zeros((m, d + 3), device=cuda)
+    wide_a[:, 1:d + 1] = ag
+    wide_b = torch.zeros((n, d + 8), device=cuda)
+    wide_b[:, 4:d + 4] = bg
+    dense = torch.empty((m, n), device=cuda)
+    _native.cdist(wide_a[:, 1:d + 1], wide_b[:, 4:d + 4], dense, sqrt=False)
+    assert float((dense.cpu() - ref).abs().max()) <= 2e-6 * scale
+    # X against itself: symmetric to rounding, diagonal zero within the resolution of the formula
+    sq = torch.empty((m, m), device=cuda)
+    _native.cdist(ag, ag, sq, sqrt=False)
+    assert float(sq.diagonal().abs().max()) <= 2e-6 * scale
+    assert float((sq - sq.T).abs().max()) <= 2e-6 * scale
+    # NaN rows pass through the clamp
+    a2 = ag.clone()
+    a2[0, 0] = float("nan")
+    _native.cdist(a2, bg, dense, sqrt=True)
+    assert bool(torch.isnan(dense[0]).all()) and not bool(torch.isnan(dense[1:]).any())
+
+
+def test_cdist_matrix_core_known_answers(cuda):
+    # the reference's known answers (tests/spatial/test_distances.py:16-58) at a width that takes the
+    # matrix-core kernel: ones against zeros -> sqrt(D), a matrix against itself -> 0, exactly
+    for d in (16, 36, 64):
+        X, Y = torch.ones((40, d), device=cuda), torch.zeros((150, d), device=cuda)
+        out = torch.empty((40, 150), device=cuda)
+        _native.cdist(X, Y, out, sqrt=True)
+        assert torch.equal(out.cpu(), torch.full((40, 150), float(d)).sqrt())
+        sq = torch.empty((40, 40), device=cuda)
+        _native.cdist(X, X, sq, sqrt=True)
+        assert torch.equal(sq.cpu(), torch.zeros((40, 40)))
+
+
 def test_widen_and_empty_inputs(cuda):
     lab = torch.tensor([3, 0, 2147483647, 5], dtype=torch.int32, device=cuda)
     out = torch.empty((4,), dtype=torch.int64, device=cuda)
