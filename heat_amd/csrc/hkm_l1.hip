@@ -267,24 +267,37 @@ __device__ __forceinline__ float from_key(unsigned k) {
 // eff[i] = labels[i] if the row takes part in the medians, else -1.  With skip_zero a row whose
 // entries are all zero is left out, as the reference drops the rows of `x * selection` that sum to
 // zero in absolute value (heat/cluster/kmedians.py:93-96).
+// LPR lanes share a row (a power of two <= 32, about the feature count: no idle lanes on narrow data).
+template <int LPR>
 __global__ __launch_bounds__(256) void med_eff_label_kernel(const float* __restrict__ X, int64_t N,
                                                             int D, int64_t ldx,
                                                             const int32_t* __restrict__ labels, int K,
-                                                            int skip_zero, int32_t* __restrict__ eff) {
-    const int lane = threadIdx.x & 31;
-    const int64_t row = (int64_t(blockIdx.x) * 256 + threadIdx.x) >> 5;
-    if (row >= N) return;  // whole 32-lane groups leave together
-    bool nz = !skip_zero;
-    if (skip_zero) {
-        const float* xr = X + row * ldx;
-        for (int d = lane; d < D; d += 32) nz |= (xr[d] != 0.f);
+                                                            int32_t* __restrict__ eff) {
+    constexpr int RPG = 8;  // rows per lane group: that many independent loads in flight per lane
+    const int sub = threadIdx.x & (LPR - 1);
+    const int64_t row0 = ((int64_t(blockIdx.x) * 256 + threadIdx.x) / LPR) * RPG;
+    int nz[RPG];
+#pragma unroll
+    for (int u = 0; u < RPG; ++u) nz[u] = 0;
+    for (int d = sub; d < D; d += LPR) {
+        float v[RPG];
+#pragma unroll
+        for (int u = 0; u < RPG; ++u) v[u] = row0 + u < N ? X[(row0 + u) * ldx + d] : 0.f;
+#pragma unroll
+        for (int u = 0; u < RPG; ++u) nz[u] |= (v[u] != 0.f);
     }
-    const unsigned long long m = __ballot(nz);
-    const int half = (threadIdx.x & 63) >> 5;
-    const bool any = ((m >> (32 * half)) & 0xffffffffull) != 0;
-    if (lane == 0) {
-        const int l = labels[row];
-        eff[row] = (l >= 0 && l < K && any) ? l : -1;
+#pragma unroll
+    for (int u = 0; u < RPG; ++u) {
+#pragma unroll
+        for (int w = 1; w < LPR; w <<= 1) nz[u] |= __shfl_xor(nz[u], w);
+    }
+    // lane u of the group stores row u
+#pragma unroll
+    for (int u = 0; u < RPG; ++u) {
+        if ((LPR >= RPG ? sub == u : sub == 0) && row0 + u < N) {
+            const int l = labels[row0 + u];
+            eff[row0 + u] = (l >= 0 && l < K && nz[u]) ? l : -1;
+        }
     }
 }
 
@@ -427,8 +440,10 @@ __global__ __launch_bounds__(256) void med_pass_kernel(const float* __restrict__
     int run_bin = -1;
     unsigned run_len = 0;
     if (ok) {
-        for (int64_t r = r0 + rl; r < r1; r += rstep) {
-            const unsigned key = to_key(X[int64_t(perm[r]) * ldx + d]);
+        // eight rows in flight per lane: the gather is latency-bound otherwise
+        constexpr int UF = 8;
+        int64_t r = r0 + rl;
+        auto consume = [&](unsigned key) {
             if (MODE == 0) {
                 // bytes above `shift + 8` must equal the prefix (nothing to compare in the first pass)
                 const bool match = pass == 0 || (key >> (shift + 8)) == pf;
@@ -445,7 +460,18 @@ __global__ __launch_bounds__(256) void med_pass_kernel(const float* __restrict__
             } else if (key > pf) {
                 best = min(best, key);
             }
+        };
+        for (; r + int64_t(UF - 1) * rstep < r1; r += int64_t(UF) * rstep) {
+            int row[UF];
+            float v[UF];
+#pragma unroll
+            for (int u = 0; u < UF; ++u) row[u] = perm[r + int64_t(u) * rstep];
+#pragma unroll
+            for (int u = 0; u < UF; ++u) v[u] = X[int64_t(row[u]) * ldx + d];
+#pragma unroll
+            for (int u = 0; u < UF; ++u) consume(to_key(v[u]));
         }
+        for (; r < r1; r += rstep) consume(to_key(X[int64_t(perm[r]) * ldx + d]));
         if (MODE == 0 && run_len) atomicAdd(&lh[col][run_bin], run_len);
         if (MODE == 1 && best != 0xffffffffu) atomicMin(&lmin[col], best);
     }
@@ -551,10 +577,18 @@ int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, cons
     int rc;
     const int32_t* eff = labels;
     if (N > 0 && skip_zero_rows) {
-        const int64_t blocks = (N * 32 + 255) / 256;
+        const int lpr = D <= 2 ? 1 : D <= 6 ? 4 : D <= 12 ? 8 : D <= 24 ? 16 : 32;
+        const int64_t blocks = ((N + 7) / 8 * lpr + 255) / 256;  // 8 rows per lane group
         if (blocks > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "update_median: N too large");
-        hipLaunchKernelGGL(med_eff_label_kernel, dim3((unsigned)blocks), dim3(256), 0, st, X, N, D, ldx,
-                           labels, K, 1, w.eff);
+#define HKM_EFF(L)                                                                                         \
+    hipLaunchKernelGGL(med_eff_label_kernel<L>, dim3((unsigned)blocks), dim3(256), 0, st, X, N, D, ldx, labels, \
+                       K, w.eff)
+        if (lpr == 1) HKM_EFF(1);
+        else if (lpr == 4) HKM_EFF(4);
+        else if (lpr == 8) HKM_EFF(8);
+        else if (lpr == 16) HKM_EFF(16);
+        else HKM_EFF(32);
+#undef HKM_EFF
         if ((rc = check_launch("med_eff_label_kernel"))) return rc;
         eff = w.eff;
     }
