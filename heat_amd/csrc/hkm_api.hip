@@ -169,6 +169,14 @@ static int check_ws(void* ws, size_t ws_bytes, size_t need) {
     return HKM_OK;
 }
 
+// HKM_PRODUCTS=bf16x3 in the environment (looked up per call) evaluates the cross term of the
+// resident matrix-core kernels with three-way split bf16 operands instead of fp32 MFMAs
+// (hkm_assign_split.hip).  Off by default: the default path computes every product in fp32.
+static bool use_split_products() {
+    const char* e = getenv("HKM_PRODUCTS");
+    return e && strcmp(e, "bf16x3") == 0;
+}
+
 static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                      int64_t ldc, int32_t* labels, float* min_d2, const Workspace& w,
                      hipStream_t st) {
@@ -179,6 +187,8 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
                 return launch_small(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, 0, st);
             return launch_assign_valu(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_RESIDENT:
+            if (use_split_products() && split_eligible(D, K, false))
+                return launch_split_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, nullptr, nullptr, st);
             return launch_assign_mfma_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_TILED: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
@@ -289,10 +299,16 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     }
     if (fused_eligible(D, K) && N > 0) {
         // one sweep over X on the matrix cores: labels + fp64 per-cluster sums in LDS
-        if ((rc = launch_lloyd_mfma_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum,
-                                             w.fcnt, w.fflags, st)))
-            return rc;
-        if ((rc = launch_update_fused(X, N, D, ldx, labels, K, C_new, D, nullptr, w, fused_grid(N), C, shift, st)))
+        const bool split = use_split_products() && split_eligible(D, K, true);
+        if (split)
+            rc = launch_split_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum, w.fcnt,
+                                       w.fflags, st);
+        else
+            rc = launch_lloyd_mfma_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum,
+                                            w.fcnt, w.fflags, st);
+        if (rc) return rc;
+        if ((rc = launch_update_fused(X, N, D, ldx, labels, K, C_new, D, nullptr, w,
+                                      split ? split_fused_grid(N) : fused_grid(N), C, shift, st)))
             return rc;
     } else {
         if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;

@@ -166,6 +166,11 @@ int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, f
                  hipStream_t st);
 int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, int mode,
                       hipStream_t st);
+bool split_eligible(int32_t D, int32_t K, bool fused);
+int split_fused_grid(int64_t N);
+int launch_split_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                          int64_t ldc, int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt,
+                          int32_t* flags, hipStream_t st);
 bool cdist_mfma_eligible(int64_t M, int64_t Nn, int32_t D, int64_t ldx, int64_t ldy, int64_t ldo);
 int launch_cdist_mfma(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,
                       int32_t D, float* out, int64_t ldo, int32_t sqrt_flag, float gauss, hipStream_t st);
