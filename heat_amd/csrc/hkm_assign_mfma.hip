@@ -840,6 +840,9 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
                               int32_t K, int64_t ldc, const float* cn, unsigned long long* keys,
                               int32_t* labels, float* min_d2, hipStream_t st) {
     const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
+    // per-thread offsets inside a 128-row tile are 32-bit byte offsets
+    if (ldx >= (int64_t(1) << 22) || ldc >= (int64_t(1) << 22))
+        return fail(HKM_EUNSUPPORTED, "assign_mfma_stream: leading dimension of 2^22 elements or more");
     const int64_t ntiles = (N + 127) / 128;
     const StreamPlan pl = stream_plan(N, D, K);
     int64_t fgrid = (N + 255) / 256;
