@@ -69,14 +69,51 @@ __device__ __forceinline__ floatx16 split_products(const uintx4 (&cs)[3][NS], co
     return acc;
 }
 
-// Scan of all centroid blocks for PB = 2 point blocks.  CLAMP applies max(. + |x|^2, 0) to every
-// value (the rescan of a tile whose lazy minimum came out negative).
+// block_argmin without its branch, so that it can share a basic block with matrix instructions: the
+// position is looked up unconditionally and taken if the block minimum improves the running one
+__device__ __forceinline__ void block_argmin_flat(const floatx16& d, int kb, float& m, int& mi) {
+    const float t0 = fminf(fminf(d[0], d[1]), d[2]);
+    const float t1 = fminf(fminf(d[3], d[4]), d[5]);
+    const float t2 = fminf(fminf(d[6], d[7]), d[8]);
+    const float t3 = fminf(fminf(d[9], d[10]), d[11]);
+    const float t4 = fminf(fminf(d[12], d[13]), d[14]);
+    const float bm = fminf(fminf(fminf(t0, t1), t2), fminf(fminf(t3, t4), d[15]));
+    int bi = 8 * (15 >> 2) + (15 & 3);
+#pragma unroll
+    for (int v = 14; v >= 0; --v) bi = (d[v] == bm) ? 8 * (v >> 2) + (v & 3) : bi;
+    const bool lt = bm < m;
+    mi = lt ? kb + bi : mi;
+    m = lt ? bm : m;
+}
+
+// asks the scheduler to order the region that ends here as N groups of one matrix instruction
+// followed by VALU vector instructions
+template <int N, int VALU>
+__device__ __forceinline__ void interleave_mfma_valu() {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Scan of all centroid blocks for PB = 2 point blocks as a software pipeline.  A wave issues in
+// order, and the bf16 matrix core runs concurrently with the vector ALU only for what is issued
+// between its instructions, so the vector instructions of one argmin scan are placed BETWEEN the
+// matrix instructions of the next product block (about four per matrix instruction):
+//   phase B of block cb:   products (cb, point block 1)   with the scan of (cb, point block 0)
+//   phase A of block cb+1: products (cb+1, point block 0) with the scan of (cb, point block 1)
+// CLAMP applies max(. + |x|^2, 0) to every value (the rescan of a tile whose lazy minimum came out
+// negative).
 template <int DP, bool CLAMP>
 __device__ __forceinline__ void split_scan(const __bf16* planes, int plane_stride, const float* sCn, int ncb, int p,
                                            int h, const uintx4 (&xs)[2][3][DP / 16], const float (&xn)[2],
                                            float (&m)[2], int (&mi)[2]) {
     constexpr int LDB = split_ldb(DP);
     constexpr int NS = DP / 16;
+    constexpr int NM = 6 * NS;
+    constexpr int VPM = CLAMP ? 7 : 4;  // vector instructions per matrix instruction
 #pragma unroll
     for (int pb = 0; pb < 2; ++pb) {
         m[pb] = HKM_INF;
@@ -90,31 +127,37 @@ __device__ __forceinline__ void split_scan(const __bf16* planes, int plane_strid
             for (int s = 0; s < NS; ++s)
                 cs[part][s] = *reinterpret_cast<const uintx4*>(planes + part * plane_stride + row_off + 8 * s);
     };
-    // operands of the next block are requested before the current block's products
-    uintx4 cs[3][NS], csn[3][NS];
+    auto scan = [&](floatx16& acc, int pb, int kb) {
+        if (CLAMP) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = fmaxf(acc[v] + xn[pb], 0.0f);
+        }
+        block_argmin_flat(acc, kb, m[pb], mi[pb]);
+    };
+    uintx4 cs[3][NS];
     load_cs(0, cs);
     floatx16 c0 = load_cn16(sCn + 4 * h);
-    for (int cb = 0; cb < ncb; ++cb) {
-        const int nb = cb + 1 < ncb ? cb + 1 : cb;
-        load_cs(nb, csn);
-        const floatx16 c0n = load_cn16(sCn + nb * 32 + 4 * h);
-        floatx16 acc[2];
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb) acc[pb] = split_products<NS>(cs, xs[pb], c0);
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb) {
-            if (CLAMP) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[pb][v] = fmaxf(acc[pb][v] + xn[pb], 0.0f);
-            }
-            block_argmin(acc[pb], cb * 32, m[pb], mi[pb]);
-        }
-#pragma unroll
-        for (int part = 0; part < 3; ++part)
-#pragma unroll
-            for (int s = 0; s < NS; ++s) cs[part][s] = csn[part][s];
-        c0 = c0n;
+    floatx16 acc0 = split_products<NS>(cs, xs[0], c0);  // prologue: (block 0, point block 0)
+    __builtin_amdgcn_sched_barrier(0);
+    floatx16 acc1;
+    // (no branch inside the loop body: the scheduler orders one basic block at a time)
+    for (int cb = 0; cb + 1 < ncb; ++cb) {
+        // phase B of block cb
+        acc1 = split_products<NS>(cs, xs[1], c0);
+        scan(acc0, 0, cb * 32);
+        interleave_mfma_valu<NM, VPM>();
+        // phase A of block cb + 1
+        load_cs(cb + 1, cs);
+        c0 = load_cn16(sCn + (cb + 1) * 32 + 4 * h);
+        acc0 = split_products<NS>(cs, xs[0], c0);
+        scan(acc1, 1, cb * 32);
+        interleave_mfma_valu<NM, VPM>();
     }
+    // last block: phase B, then the scan that has nothing left to hide behind
+    acc1 = split_products<NS>(cs, xs[1], c0);
+    scan(acc0, 0, (ncb - 1) * 32);
+    interleave_mfma_valu<NM, VPM>();
+    scan(acc1, 1, (ncb - 1) * 32);
     if (!CLAMP) {
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) m[pb] += xn[pb];
