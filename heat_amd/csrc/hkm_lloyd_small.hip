@@ -9,11 +9,15 @@
 // applied lazily: a negative minimum (a point that coincides with a centroid up to rounding)
 // triggers a rescan with the clamp applied to every candidate, so the result equals clamping first.
 //
-// Update (heat/cluster/kmeans.py:76-103) without atomics, two strategies with a fixed summation order:
+// Update (heat/cluster/kmeans.py:76-103) without atomics, three strategies with a fixed summation order:
 //   K*(D+1) <= 48: every lane owns a private fp32 column per (cluster, coordinate) in LDS and adds
 //     its own points in program order; the read-add-write round trips of a round are deferred to the
 //     next round and interleaved with its arithmetic.  At the end lanes' columns are added in a fixed
 //     fp64 tree.
+//   otherwise, K <= 32: the sums are a matrix product, (one-hot labels)^T x [X, 1], evaluated on the
+//     fp32 matrix cores with v_mfma_f32_16x16x4_f32 over the wave's points of the round (read back from
+//     the staging buffer); the fp32 accumulators move into the wave's private fp64 row in LDS every
+//     eight rounds.
 //   otherwise: for every cluster k and coordinate d the wavefront forms
 //     sum over lanes of [label == k] * x_d with a fixed DPP tree (row shifts, then row broadcasts;
 //     the total lands in lane 63) and lane 63 adds it to the wave's private fp64 row in LDS.
@@ -41,15 +45,20 @@ struct SmallCfg {
 
 bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
 static constexpr int SMALL_T = 256;
-// LDS of one workgroup; acc_mode as in the kernel (0 labels only, 1 lane columns, 2 wave rows)
+// LDS of one workgroup; acc_mode as in the kernel (0 labels only, 1 lane columns, 2 wave rows by the
+// DPP tree, 3 wave rows by the matrix cores)
 static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
     const int sc = (D + 1 + 3) / 4 * 4, nv = ppt * D / 4, slots = K * (D + 1);
     return size_t((K * sc + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) +
-           (acc_mode == 2 ? size_t(SMALL_T / 64) * slots * sizeof(double)
-            : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float) : 0);
+           (acc_mode == 2   ? size_t(SMALL_T / 64) * slots * sizeof(double)
+            : acc_mode == 3 ? size_t(SMALL_T / 64) * (slots * sizeof(double) + 64 * ppt * sizeof(int))
+            : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float)
+                            : 0);
 }
-static int small_acc_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : 2; }
+// per-lane LDS columns while they fit (slots * 1 KB), the matrix-core product up to 32 clusters, the
+// DPP tree otherwise
+static int small_acc_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : K <= 32 ? 3 : 2; }
 
 int small_grid(int64_t N, int32_t D, int32_t K) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
@@ -132,7 +141,8 @@ __device__ __forceinline__ void scan_centroids_reg(const float (&cs)[KT][D + 1],
     }
 }
 
-// ACC: 0 = labels only, 1 = per-lane private LDS columns, 2 = DPP wave tree + per-wave fp64 rows
+// ACC: 0 = labels only, 1 = per-lane private LDS columns, 2 = DPP wave tree + per-wave fp64 rows,
+//      3 = matrix-core product (one-hot labels x points) + per-wave fp64 rows
 // KT: 0 = centroids read from LDS in a loop over K; otherwise K <= KT and they sit in registers
 template <int D, int ACC, bool WANT_MIN, bool WANT_SSE, int KT>
 __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
@@ -156,13 +166,14 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     double* wacc = wacc_all + wave * slots;
+    int* wlab = reinterpret_cast<int*>(wacc_all + NW * slots) + wave * (64 * PPT);  // ACC==3: [4][16*PPT]
     float* wstage = stage + wave * NV * 256;
 
     for (int i = tid; i < K * SC; i += T) {
         const int r = i / SC, c = i - r * SC;
         sC[i] = c < D ? C[int64_t(r) * ldc + c] : 0.f;  // scaled by -2 once the norms are taken
     }
-    if (ACC == 2)
+    if (ACC == 2 || ACC == 3)
         for (int i = tid; i < NW * slots; i += T) wacc_all[i] = 0.0;
     if (ACC == 1)
         for (int i = tid; i < (slots + D + 1) * T; i += T) cols[i] = 0.f;
@@ -177,10 +188,13 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     }
     __syncthreads();
 
-    // KT > 0: one copy of the centroid table per wave, in scalar registers
-    constexpr int KR = KT > 0 ? KT : 1;
+    // 0 < KT <= 8: one copy of the centroid table per wave, in scalar registers
+    // KT = 16 / 32 (ACC == 3 only): one / two blocks of 16 clusters in the matrix-core accumulation
+    constexpr bool REGC = KT > 0 && KT <= 8;
+    constexpr int KR = REGC ? KT : 1;
+    constexpr int MB = KT == 32 ? 2 : 1;
     float cs[KR][D + 1];
-    if (KT > 0) {
+    if (REGC) {
 #pragma unroll
         for (int k = 0; k < KR; ++k)
 #pragma unroll
@@ -218,6 +232,26 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         for (int d = 0; d <= D; ++d) cols[pcol[p] + d * T] = r[d] + px[p][d];
     };
 
+    // ACC == 3: fp32 accumulators of the matrix-core product (lane: cluster rows 4*(lane/16) + r of
+    // block mb, column lane%16), moved into the wave's fp64 row every eight rounds (1024 points at
+    // most in fp32) -- every (cluster, column) has one owner, so plain read-add-write.
+    floatx4 macc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) macc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    int since_flush = 0;
+    auto flush_macc = [&]() {
+        const int col = lane & 15;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 16 * mb + 4 * (lane >> 4) + r;
+                if (row < K && col <= D) wacc[row * (D + 1) + col] += double(macc[mb][r]);
+                macc[mb][r] = 0.f;
+            }
+        since_flush = 0;
+    };
+
     // label + accumulate one group of PPT points held in registers.  Executed by ALL lanes of the
     // wave (the DPP tree needs them); GUARD: rows >= N contribute nothing and store nothing.
     auto process = [&](int64_t i0, const float (&x)[PPT][D], auto guard_tag) {
@@ -235,18 +269,18 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             m[p] = HKM_INF;
             mi[p] = 0;
         }
-        const int kh = KT > 0 ? KT / 2 : K >> 1;
+        const int kh = REGC ? KT / 2 : K >> 1;
         if (ACC == 1 && PPT == 4) {
             rmw_write(0, r);
             rmw_read(1, r);
         }
-        if constexpr (KT > 0) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
+        if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
         else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
         if (ACC == 1) {
             rmw_write(PPT == 4 ? 1 : 0, r);
             rmw_read(PPT == 4 ? 2 : 1, r);
         }
-        if constexpr (KT > 0) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
+        if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
         else scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
         if (ACC == 1 && PPT == 4) {
             rmw_write(2, r);
@@ -265,7 +299,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 m[p] = HKM_INF;
                 mi[p] = 0;
             }
-            if constexpr (KT > 0) scan_centroids_reg<D, PPT, KR, true>(cs, 0, KR, x, xn, m, mi);
+            if constexpr (REGC) scan_centroids_reg<D, PPT, KR, true>(cs, 0, KR, x, xn, m, mi);
             else scan_centroids<D, PPT, true>(sC, 0, K, x, xn, m, mi);
         }
 
@@ -301,6 +335,42 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 for (int d = 0; d < D; ++d) px[p][d] = x[p][d];
                 px[p][D] = 1.0f;
             }
+        }
+        if (ACC == 3) {
+            // Per-cluster sums as a matrix product on the fp32 matrix cores: (one-hot labels, 16 x 4
+            // points) x (4 points x [coordinates, 1]) per v_mfma_f32_16x16x4_f32, accumulated over the
+            // wave's 64*PPT points of the round.  The points are read back from the wave's staging
+            // buffer (row q = point q of the round), the labels go through LDS transposed so that a
+            // lane fetches those of four steps at once.
+            constexpr int G = 16 * PPT;  // MFMA steps per round
+#pragma unroll
+            for (int p = 0; p < PPT; ++p) {
+                const int q = lane * PPT + p;
+                wlab[(q & 3) * G + (q >> 2)] = mi[p];  // -1 for rows beyond N: matches no cluster
+            }
+            wave_lds_sync();
+            const int kk = lane >> 4, col = lane & 15;
+            const float bconst = col == D ? 1.0f : 0.0f;
+            const int cread = col < D ? col : D - 1;  // lanes of the padding columns read a valid address
+#pragma unroll
+            for (int g4 = 0; g4 < G; g4 += 4) {
+                const int4 lb = *reinterpret_cast<const int4*>(wlab + kk * G + g4);
+                const int lbs[4] = {lb.x, lb.y, lb.z, lb.w};
+                float bv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) bv[u] = wstage[(4 * (g4 + u) + kk) * D + cread];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const float bval = col < D ? bv[u] : bconst;
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        const float a = lbs[u] == col + 16 * mb ? 1.0f : 0.0f;
+                        macc[mb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bval, macc[mb], 0, 0, 0);
+                    }
+                }
+            }
+            wave_lds_sync();  // the next round overwrites the staging buffer and the labels
+            if (++since_flush == 8) flush_macc();
         }
         if (ACC == 2) {
             for (int k = 0; k < K; ++k) {
@@ -391,6 +461,15 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
             for (int d = 0; d < D; ++d) x[p][d] = X[r * ldx + d];
         }
+        if (ACC == 3) {
+            // the matrix-core accumulation reads the round's points from the staging buffer
+            wave_lds_sync();
+#pragma unroll
+            for (int p = 0; p < PPT; ++p)
+#pragma unroll
+                for (int d = 0; d < D; ++d) wstage[(lane * PPT + p) * D + d] = x[p][d];
+            wave_lds_sync();
+        }
         process(i0, x, std::true_type{});
     }
 
@@ -403,10 +482,11 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             rmw_write(p, r);
         }
     }
+    if (ACC == 3) flush_macc();
     if (ACCUM || WANT_SSE) {
         __syncthreads();
         double* prow = part + int64_t(blockIdx.x) * (slots + 1);
-        if (ACC == 2) {
+        if (ACC == 2 || ACC == 3) {
             for (int s = tid; s < slots; s += T) {
                 double v = 0.0;
 #pragma unroll
@@ -516,7 +596,13 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     const bool reg = KT8 > 0 && K <= KT8;
 #define HKM_GO(A, M, S)                                                                                  \
     do {                                                                                                 \
-        if (reg)                                                                                         \
+        if (A == 3 && K > 16)                                                                            \
+            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A == 3 ? 32 : 0>), dim3(grid), dim3(SMALL_T), lds, \
+                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec);                     \
+        else if (A == 3)                                                                                 \
+            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A == 3 ? 16 : 0>), dim3(grid), dim3(SMALL_T), lds, \
+                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec);                     \
+        else if (reg)                                                                                    \
             hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, KT8>), dim3(grid), dim3(SMALL_T), lds, st, X, \
                                N, ldx, C, K, ldc, labels, min_d2, part, vec);                            \
         else                                                                                             \
@@ -529,6 +615,9 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     } else if (acc_mode == 2) {
         if (want_sse) HKM_GO(2, false, true);
         else HKM_GO(2, false, false);
+    } else if (acc_mode == 3) {
+        if (want_sse) HKM_GO(3, false, true);
+        else HKM_GO(3, false, false);
     } else {
         if (want_min) HKM_GO(0, true, false);
         else HKM_GO(0, false, false);
