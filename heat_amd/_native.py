@@ -204,6 +204,33 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Op
                                     _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
 
 
+def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],
+                       shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace):
+    """The same call as :func:`lloyd_step` with every argument converted once: returns a function
+    without arguments that enqueues the step on the stream that was current when it was prepared.
+    For loops that issue thousands of steps on small problems, where building the argument list costs
+    as much as the step.  The tensors are kept alive by the returned function."""
+    _require_gpu(x, c, c_new, labels, sse)
+    if not (shift.is_cuda or shift.is_pinned()):
+        raise RuntimeError("shift must live on the GPU or in pinned host memory")
+    n, d = x.shape
+    k = c.shape[0]
+    f64 = _is_f64(x, c, c_new, shift, sse)
+    flags = WS_LLOYD | (WS_F64 if f64 else 0) | (WS_SSE if sse is not None else 0)
+    buf = ws.get(workspace_bytes(n, d, k, flags))
+    fn = load().hkm_lloyd_step_f64 if f64 else load().hkm_lloyd_step_f32
+    args = (_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k, _ptr(labels), _ptr(shift),
+            _ptr(sse), _ptr(buf), buf.numel(), _stream())
+    keep = (x, c, c_new, labels, shift, sse, buf)
+
+    def enqueue(_fn=fn, _args=args, _keep=keep) -> None:
+        rc = _fn(*_args)
+        if rc != HKM_OK:
+            raise HkmError(rc, last_error())
+
+    return enqueue
+
+
 def shift(c_old: torch.Tensor, c_new: torch.Tensor, out: torch.Tensor) -> None:
     _require_gpu(c_old, c_new, out)
     k, d = c_old.shape

@@ -39,11 +39,19 @@ class LloydLoop:
         self.ev = [torch.cuda.Event(), torch.cuda.Event()]
         self.enqueued = 0  # steps handed to the stream
         self.done = 0      # steps whose results count
+        self._plans = {}   # prepared calls, one per rotation of the buffers (and stream)
 
     def _enqueue(self) -> None:
         j = self.enqueued
-        _native.lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3], None if self.lazy_labels else self.lab[j % 2],
-                           self.shift_host[j % 2], None, self.ws)
+        key = (j % 6, torch.cuda.current_stream().cuda_stream)
+        plan = self._plans.get(key)
+        if plan is None:
+            # the argument list of a step only depends on which buffers of the rotation it uses
+            plan = _native.prepare_lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3],
+                                              None if self.lazy_labels else self.lab[j % 2],
+                                              self.shift_host[j % 2], None, self.ws)
+            self._plans[key] = plan
+        plan()
         self.ev[j % 2].record()
         self.enqueued = j + 1
 

@@ -533,10 +533,10 @@ __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
     const int tid = threadIdx.x;
     const int slots = K * (D + 1);
     const int nslot = slots + 1;  // last = sum of min d2
-    const int J = 1024 / spad;
+    const int J = 1024 / spad;  // spad = nslot: as many row groups as fit the workgroup
     const int s = tid % spad, j = tid / spad;
     double v = 0.0;
-    if (s < nslot && (s < slots || have_sse)) {
+    if (j < J && s < nslot && (s < slots || have_sse)) {
         int g = j;
         for (; g + 7 * J < G; g += 8 * J) {
             double t[8];
@@ -549,7 +549,7 @@ __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
     }
     strided[tid] = v;
     __syncthreads();
-    if (j == 0 && s < nslot) {
+    if (j == 0 && s < nslot) {  // (threads of j == 0 are tid < spad)
         double t = 0.0;
         for (int q = 0; q < J; ++q) t += strided[q * spad + s];
         tot[s] = t;
@@ -645,8 +645,7 @@ int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float*
 int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, const float* C_old,
                           float* C_new, int64_t ldcn, int64_t* counts, float* shift, float* sse,
                           hipStream_t st) {
-    int spad = 1;
-    while (spad < K * (D + 1) + 1) spad <<= 1;  // <= 256 because K*(D+1) <= 240
+    const int spad = K * (D + 1) + 1;  // <= 241 because K*(D+1) <= 240
     hipLaunchKernelGGL(lloyd_small_finalize_kernel, dim3(1), dim3(1024), 0, st, part, grid, K, D,
                        C_old, C_new, ldcn, counts, shift, sse, sse ? 1 : 0, spad);
     return check_launch("lloyd_small_finalize_kernel");
