@@ -268,7 +268,9 @@ __device__ __forceinline__ float from_key(unsigned k) {
 // entries are all zero is left out, as the reference drops the rows of `x * selection` that sum to
 // zero in absolute value (heat/cluster/kmedians.py:93-96).
 // LPR lanes share a row (a power of two <= 32, about the feature count: no idle lanes on narrow data).
-template <int LPR>
+// VEC: rows are read in 16-byte groups (X 16-byte aligned, ldx % 4 == 0, D % 4 == 0; LPR then counts
+// lanes per row of D / 4 groups).
+template <int LPR, bool VEC>
 __global__ __launch_bounds__(256) void med_eff_label_kernel(const float* __restrict__ X, int64_t N,
                                                             int D, int64_t ldx,
                                                             const int32_t* __restrict__ labels, int K,
@@ -279,12 +281,26 @@ __global__ __launch_bounds__(256) void med_eff_label_kernel(const float* __restr
     int nz[RPG];
 #pragma unroll
     for (int u = 0; u < RPG; ++u) nz[u] = 0;
-    for (int d = sub; d < D; d += LPR) {
-        float v[RPG];
+    if (VEC) {
+        const int ng = D >> 2;
+        for (int g = sub; g < ng; g += LPR) {
+            float4 v[RPG];
 #pragma unroll
-        for (int u = 0; u < RPG; ++u) v[u] = row0 + u < N ? X[(row0 + u) * ldx + d] : 0.f;
+            for (int u = 0; u < RPG; ++u)
+                v[u] = row0 + u < N ? *reinterpret_cast<const float4*>(X + (row0 + u) * ldx + 4 * g)
+                                    : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int u = 0; u < RPG; ++u) nz[u] |= (v[u] != 0.f);
+            for (int u = 0; u < RPG; ++u)
+                nz[u] |= (v[u].x != 0.f) | (v[u].y != 0.f) | (v[u].z != 0.f) | (v[u].w != 0.f);
+        }
+    } else {
+        for (int d = sub; d < D; d += LPR) {
+            float v[RPG];
+#pragma unroll
+            for (int u = 0; u < RPG; ++u) v[u] = row0 + u < N ? X[(row0 + u) * ldx + d] : 0.f;
+#pragma unroll
+            for (int u = 0; u < RPG; ++u) nz[u] |= (v[u] != 0.f);
+        }
     }
 #pragma unroll
     for (int u = 0; u < RPG; ++u) {
@@ -490,43 +506,61 @@ __global__ __launch_bounds__(256) void med_pass_kernel(const float* __restrict__
     }
 }
 
-// one thread per (cluster, coordinate): walk the 256 bins to the one that holds the wanted rank,
-// extend the prefix by that byte, make the rank relative to the bin, and clear the bins
+// one wave per (cluster, coordinate): find the bin that holds the wanted rank (each lane owns four
+// consecutive bins, an exclusive scan over the lanes gives their first rank), extend the prefix by
+// that byte, make the rank relative to the bin, and clear the bins
 __global__ __launch_bounds__(256) void med_pick_kernel(unsigned* __restrict__ hist_g, int64_t KD, int D,
                                                        const int64_t* __restrict__ counts, int pass,
                                                        unsigned* __restrict__ prefix,
                                                        int64_t* __restrict__ rank,
                                                        unsigned* __restrict__ eqcnt,
                                                        unsigned* __restrict__ next_g) {
-    const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
-    if (i >= KD) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t i = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (i >= KD) return;  // whole waves leave together
     const int64_t n = counts[i / D];
-    unsigned* h = hist_g + i * 256;
-    if (pass == 0) {
-        rank[i] = n > 0 ? (n - 1) / 2 : 0;
-        prefix[i] = 0;
-        next_g[i] = 0xffffffffu;
+    uint4* h4 = reinterpret_cast<uint4*>(hist_g + i * 256) + lane;
+    const uint4 c = *h4;
+    *h4 = make_uint4(0u, 0u, 0u, 0u);
+    int64_t want = pass == 0 ? (n > 0 ? (n - 1) / 2 : 0) : rank[i];
+    const unsigned pf = pass == 0 ? 0u : prefix[i];
+    // exclusive scan of the lanes' totals (bins are 32-bit counts of at most 2^31 rows)
+    const unsigned tot = c.x + c.y + c.z + c.w;
+    unsigned incl = tot;
+#pragma unroll
+    for (int w = 1; w < 64; w <<= 1) {
+        const unsigned o = __shfl_up(incl, w);
+        if (lane >= w) incl += o;
     }
-    int64_t want = rank[i];
-    int digit = 0;
+    const int64_t first = int64_t(incl) - tot;  // rank of this lane's first element
+    const unsigned cs[4] = {c.x, c.y, c.z, c.w};
+    int digit = -1;
     unsigned in_bin = 0;
-    bool found = false;
-    for (int b = 0; b < 256; ++b) {
-        const unsigned c = h[b];
-        h[b] = 0;
-        if (!found) {
-            if (want < int64_t(c)) {
-                digit = b;
-                in_bin = c;
-                found = true;
-            } else {
-                want -= c;
-            }
+    int64_t rel = 0, lo = first;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        if (digit < 0 && want >= lo && want < lo + int64_t(cs[q])) {
+            digit = 4 * lane + q;
+            in_bin = cs[q];
+            rel = want - lo;
         }
+        lo += cs[q];
     }
-    prefix[i] = (prefix[i] << 8) | unsigned(digit);
-    rank[i] = found ? want : 0;
-    eqcnt[i] = in_bin;
+    const unsigned long long who = __ballot(digit >= 0);
+    if (who == 0) {
+        // nothing holds the rank (an empty cluster): digit 0, as a walk over empty bins ends
+        if (lane == 0) {
+            prefix[i] = pf << 8;
+            rank[i] = 0;
+            eqcnt[i] = 0;
+            if (pass == 0) next_g[i] = 0xffffffffu;
+        }
+    } else if (digit >= 0) {
+        prefix[i] = (pf << 8) | unsigned(digit);
+        rank[i] = rel;
+        eqcnt[i] = in_bin;
+        if (pass == 0) next_g[i] = 0xffffffffu;
+    }
 }
 
 // mode 0: the reference's median (percentile 50, linear): lower middle for an odd count, for an even
@@ -577,12 +611,20 @@ int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, cons
     int rc;
     const int32_t* eff = labels;
     if (N > 0 && skip_zero_rows) {
-        const int lpr = D <= 2 ? 1 : D <= 6 ? 4 : D <= 12 ? 8 : D <= 24 ? 16 : 32;
+        const bool vec = aligned16(X) && (ldx % 4 == 0) && (D % 4 == 0);
+        const int units = vec ? D / 4 : D;  // loads per row
+        const int lpr = units <= 2 ? 1 : units <= 6 ? 4 : units <= 12 ? 8 : units <= 24 ? 16 : 32;
         const int64_t blocks = ((N + 7) / 8 * lpr + 255) / 256;  // 8 rows per lane group
         if (blocks > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "update_median: N too large");
-#define HKM_EFF(L)                                                                                         \
-    hipLaunchKernelGGL(med_eff_label_kernel<L>, dim3((unsigned)blocks), dim3(256), 0, st, X, N, D, ldx, labels, \
-                       K, w.eff)
+#define HKM_EFF(L)                                                                                             \
+    do {                                                                                                       \
+        if (vec)                                                                                               \
+            hipLaunchKernelGGL((med_eff_label_kernel<L, true>), dim3((unsigned)blocks), dim3(256), 0, st, X, N, D, \
+                               ldx, labels, K, w.eff);                                                         \
+        else                                                                                                   \
+            hipLaunchKernelGGL((med_eff_label_kernel<L, false>), dim3((unsigned)blocks), dim3(256), 0, st, X, N, D, \
+                               ldx, labels, K, w.eff);                                                         \
+    } while (0)
         if (lpr == 1) HKM_EFF(1);
         else if (lpr == 4) HKM_EFF(4);
         else if (lpr == 8) HKM_EFF(8);
@@ -621,7 +663,7 @@ int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, cons
                                w.perm, w.offsets, w.chunk_start, K, pass, cl, w.prefix, w.hist, w.next);
             if ((rc = check_launch("med_pass_kernel<0>"))) return rc;
         }
-        hipLaunchKernelGGL(med_pick_kernel, dim3(kd_blocks), dim3(256), 0, st, w.hist, KD, D, w.counts, pass,
+        hipLaunchKernelGGL(med_pick_kernel, dim3((unsigned)((KD + 3) / 4)), dim3(256), 0, st, w.hist, KD, D, w.counts, pass,
                            w.prefix, w.rank, w.eqcnt, w.next);
         if ((rc = check_launch("med_pick_kernel"))) return rc;
     }
