@@ -836,9 +836,242 @@ __global__ __launch_bounds__(256) void assign_mfma_stream_kernel(
     }
 }
 
+// The same kernel with the cross term evaluated from three-way split bf16 operands on the bf16 matrix
+// cores (opt-in, see hkm_assign_split.hip for the arithmetic): the staging threads split the fp32
+// values they fetched and store three bf16 planes per panel.
+template <bool VEC>
+__global__ __launch_bounds__(256) void assign_split_stream_kernel(
+    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, const float* __restrict__ cn, unsigned long long* __restrict__ keys, int64_t ntiles,
+    int nct, int ndc, int W, int PG) {
+    constexpr int PB = 2, CB = 2, TP = 128, TC = 128, DC = 32, LDB = DC + 8;
+    // three bf16 planes per panel, one buffer (two barriers per chunk; two workgroups per CU overlap)
+    __shared__ __align__(16) __bf16 sA[3][TC * LDB];
+    __shared__ __align__(16) __bf16 sB[3][TP * LDB];
+    __shared__ float sM[2][TP];
+    __shared__ int sI[2][TP];
+    __shared__ float sXn[TP];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wp = wave & 1, wc = wave >> 1;  // this wave: points [64 wp, +64), centroids [64 wc, +64)
+    const int p = lane & 31, h = lane >> 5;
+
+    // items of this workgroup: item q = (point tile xt0 + 8 PG (q / cpw), centroid tile ct0 + W (q % cpw))
+    const int xcd = blockIdx.x & 7, l = blockIdx.x >> 3;
+    const bool spread = nct <= W;  // one centroid tile per workgroup, PG point tiles in flight
+    const int ct0 = spread ? l % nct : l;
+    const int64_t xt0 = xcd + 8 * int64_t(spread ? l / nct : 0);
+    const int cpw = spread ? 1 : (nct - l + W - 1) / W;
+    const int64_t xstep = 8 * int64_t(PG);
+    const int64_t nx = xt0 < ntiles ? (ntiles - xt0 + xstep - 1) / xstep : 0;
+    const int64_t nsteps = nx * cpw * ndc;
+
+    const int sr = tid >> 3;         // staging: rows sr + 32 q (q = 0..3) of both panels
+    const int sc = (tid & 7) * 4;    // column group
+
+    // Addresses of a chunk's loads are (workgroup-uniform panel base, advanced by scalar arithmetic)
+    // + (a per-thread byte offset that only changes with the tile): no vector instruction per chunk.
+    // Rows beyond K or N are clamped to the last valid row (a padding centroid has |c|^2 = +inf and
+    // never wins; a padding point is never stored).
+    const float* baseA = C;
+    const float* baseB = X;
+    unsigned offA[4], offB[4];
+    auto set_tile = [&](int64_t xt, int ct) {
+        baseA = C + int64_t(ct) * TC * ldc;
+        baseB = X + xt * TP * ldx;
+        const int lastA = K - 1 - ct * TC;
+        const int64_t lastB = N - 1 - xt * TP;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int r = sr + 32 * q;
+            const int ra = r < lastA ? r : lastA;
+            const int rb = r < lastB ? r : int(lastB);
+            offA[q] = unsigned((int64_t(ra) * ldc + sc) * 4);
+            offB[q] = unsigned((int64_t(rb) * ldx + sc) * 4);
+        }
+    };
+    floatx4 pa[4], pb_[4];
+    auto issue = [&](int dc) {
+        const float* a = baseA + dc * DC;
+        const float* bq = baseB + dc * DC;
+        if (VEC && dc * DC + DC <= D) {  // whole chunk inside the rows: unconditional 16-byte loads
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                pa[q] = *reinterpret_cast<const floatx4*>(reinterpret_cast<const char*>(a) + offA[q]);
+                pb_[q] = *reinterpret_cast<const floatx4*>(reinterpret_cast<const char*>(bq) + offB[q]);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                // offsets hold the column group; load_row4 wants the row start and the column
+                pa[q] = load_row4<VEC>(reinterpret_cast<const float*>(reinterpret_cast<const char*>(a) + offA[q]) - sc - dc * DC,
+                                       dc * DC + sc, D);
+                pb_[q] = load_row4<VEC>(reinterpret_cast<const float*>(reinterpret_cast<const char*>(bq) + offB[q]) - sc - dc * DC,
+                                        dc * DC + sc, D);
+            }
+        }
+    };
+
+    int64_t xi = 0;  // index of the point tile within this workgroup's sequence
+    int ci = 0, dc = 0;
+    if (nsteps > 0) {
+        set_tile(xt0, ct0);
+        issue(0);
+    }
+
+    floatx16 acc[PB][CB];
+    float xsq[4] = {0.f, 0.f, 0.f, 0.f};  // |x|^2 of staging rows sr + 32 q over this thread's column group
+
+    for (int64_t it = 0; it < nsteps; ++it) {
+        if (it > 0) __syncthreads();  // the previous chunk's operands have been read
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            unsigned a1[2], a2[2], a3[2], b1[2], b2[2], b3[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                split_pair(pa[q][2 * e], pa[q][2 * e + 1], a1[e], a2[e], a3[e]);
+                split_pair(pb_[q][2 * e], pb_[q][2 * e + 1], b1[e], b2[e], b3[e]);
+            }
+            const int o = (sr + 32 * q) * LDB + sc;
+            *reinterpret_cast<uint2*>(&sA[0][o]) = make_uint2(a1[0], a1[1]);
+            *reinterpret_cast<uint2*>(&sA[1][o]) = make_uint2(a2[0], a2[1]);
+            *reinterpret_cast<uint2*>(&sA[2][o]) = make_uint2(a3[0], a3[1]);
+            *reinterpret_cast<uint2*>(&sB[0][o]) = make_uint2(b1[0], b1[1]);
+            *reinterpret_cast<uint2*>(&sB[1][o]) = make_uint2(b2[0], b2[1]);
+            *reinterpret_cast<uint2*>(&sB[2][o]) = make_uint2(b3[0], b3[1]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) xsq[q] = fmaf(pb_[q][t], pb_[q][t], xsq[q]);
+        }
+        __syncthreads();
+
+        const int64_t cur_xt = xt0 + xi * xstep;
+        const int cur_ct = ct0 + ci * W, cur_dc = dc;
+        if (++dc == ndc) {
+            dc = 0;
+            if (++ci == cpw) {
+                ci = 0;
+                ++xi;
+            }
+            if (it + 1 < nsteps) set_tile(xt0 + xi * xstep, ct0 + ci * W);
+        }
+        if (it + 1 < nsteps) issue(dc);
+
+        if (cur_dc == 0) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[pb][cb][v] = 0.f;
+            }
+        }
+
+        // k-step s of the bf16 MFMA covers features 16 s .. 16 s + 15 of the chunk, 8 per lane-half;
+        // the six partial products per (centroid block, point block), smallest first
+        uintx4 xb[PB][3][2];
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+            for (int part = 0; part < 3; ++part)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+                    xb[pb][part][s2] = *reinterpret_cast<const uintx4*>(
+                        &sB[part][(wp * 64 + pb * 32 + p) * LDB + 16 * s2 + 8 * h]);
+        constexpr int XP[6] = {2, 0, 1, 1, 0, 0};
+        constexpr int CP[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            uintx4 ca[3][2];
+#pragma unroll
+            for (int part = 0; part < 3; ++part)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+                    ca[part][s2] = *reinterpret_cast<const uintx4*>(
+                        &sA[part][(wc * 64 + cb * 32 + p) * LDB + 16 * s2 + 8 * h]);
+#pragma unroll
+            for (int t = 0; t < 6; ++t)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                    for (int pb = 0; pb < PB; ++pb)
+                        acc[pb][cb] = MFMA_BF16(as_bf16x8(ca[CP[t]][s2]), as_bf16x8(xb[pb][XP[t]][s2]), acc[pb][cb]);
+        }
+
+        if (cur_dc == ndc - 1) {
+            // squared norms of the tile's points: the eight threads that staged a row add their parts
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v = xsq[q];
+                v += __shfl_xor(v, 1);
+                v += __shfl_xor(v, 2);
+                v += __shfl_xor(v, 4);
+                if ((tid & 7) == 0) sXn[sr + 32 * q] = v;
+                xsq[q] = 0.f;
+            }
+            __syncthreads();
+            float m[PB];
+            int mi[PB];
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                const float xn = sXn[wp * 64 + pb * 32 + p];
+                const float baug = h ? -0.5f * xn : 1.0f;
+                m[pb] = -HKM_INF;
+                mi[pb] = 0;
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const int kb = cur_ct * TC + wc * 64 + cb * 32;
+                    const float aaug = h ? 1.0f : -0.5f * cn[kb + p];
+                    // g = x.c - |c|^2/2 - |x|^2/2 = -d2/2 (halving is exact): the nearest centroid has
+                    // the LARGEST g; the clamp of d2 at 0 is a clamp of g at 0 from above
+                    const floatx16 g16 = MFMA32(aaug, baug, acc[pb][cb]);
+                    float bm = fminf(g16[0], 0.0f);
+                    int bi = 0;
+#pragma unroll
+                    for (int v = 1; v < 16; ++v) {
+                        const float g = fminf(g16[v], 0.0f);
+                        const bool gt = g > bm;
+                        bi = gt ? 8 * (v >> 2) + (v & 3) : bi;
+                        bm = gt ? g : bm;
+                    }
+                    const bool gt = bm > m[pb];
+                    mi[pb] = gt ? kb + bi : mi[pb];
+                    m[pb] = gt ? bm : m[pb];
+                }
+                // merge lane halves, then the two waves that cover the same points
+                mi[pb] += 4 * h;
+                // back to the squared distance (+inf if every g was NaN or -inf); the "+ 0" turns a
+                // -0.0 into +0.0, whose bit pattern is the smallest key
+                m[pb] = -2.0f * m[pb] + 0.0f;
+                merge_halves(m[pb], mi[pb]);
+                if (h == 0) {
+                    sM[wc][wp * 64 + pb * 32 + p] = m[pb];
+                    sI[wc][wp * 64 + pb * 32 + p] = mi[pb];
+                }
+            }
+            __syncthreads();
+            if (tid < TP) {
+                float m0 = sM[0][tid];
+                int i0 = sI[0][tid];
+                const float m1 = sM[1][tid];
+                const int i1 = sI[1][tid];
+                if (m1 < m0 || (m1 == m0 && i1 < i0)) {
+                    m0 = m1;
+                    i0 = i1;
+                }
+                const int64_t r = cur_xt * TP + tid;
+                if (r < N && m0 < HKM_INF) {
+                    const unsigned long long key =
+                        (static_cast<unsigned long long>(__float_as_uint(m0)) << 32) | unsigned(i0);
+                    atomicMin(keys + r, key);
+                }
+            }
+        }
+    }
+}
+
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                               int32_t K, int64_t ldc, const float* cn, unsigned long long* keys,
-                              int32_t* labels, float* min_d2, hipStream_t st) {
+                              int32_t* labels, float* min_d2, bool split, hipStream_t st) {
     const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
     // per-thread offsets inside a 128-row tile are 32-bit byte offsets
     if (ldx >= (int64_t(1) << 22) || ldc >= (int64_t(1) << 22))
@@ -851,7 +1084,13 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
     hipLaunchKernelGGL(fill_keys_kernel, dim3((unsigned)fgrid), dim3(256), 0, st, keys, N);
     int rc = check_launch("fill_keys_kernel");
     if (rc) return rc;
-    if (vec)
+    if (split && vec)
+        hipLaunchKernelGGL(assign_split_stream_kernel<true>, dim3(pl.grid), dim3(256), 0, st, X, N, D, ldx,
+                           C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
+    else if (split)
+        hipLaunchKernelGGL(assign_split_stream_kernel<false>, dim3(pl.grid), dim3(256), 0, st, X, N, D, ldx,
+                           C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
+    else if (vec)
         hipLaunchKernelGGL(assign_mfma_stream_kernel<true>, dim3(pl.grid), dim3(256), 0, st, X, N, D, ldx,
                            C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
     else

@@ -22,33 +22,8 @@
 
 namespace hkm {
 
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
-
-#define MFMA_BF16(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
-
 static constexpr int SPLIT_QBITS = 28;
 static constexpr int SPLIT_FUSED_THREADS = 512;  // 2 waves per SIMD: room for the split operands without spills
-
-// two fp32 values -> their bf16 roundings packed in one register (element 0 in the low half)
-__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
-    const floatx2 v = {a, b};
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
-}
-__device__ __forceinline__ float bf16_lo(unsigned u) { return __uint_as_float(u << 16); }
-__device__ __forceinline__ float bf16_hi(unsigned u) { return __uint_as_float(u & 0xffff0000u); }
-
-// three-way split of a pair; p1, p2, p3 receive the packed parts
-__device__ __forceinline__ void split_pair(float a, float b, unsigned& p1, unsigned& p2, unsigned& p3) {
-    p1 = pack_bf16(a, b);
-    const float ra = a - bf16_lo(p1), rb = b - bf16_hi(p1);
-    p2 = pack_bf16(ra, rb);
-    p3 = pack_bf16(ra - bf16_lo(p2), rb - bf16_hi(p2));
-}
-
-__device__ __forceinline__ bf16x8 as_bf16x8(const uintx4& u) { return __builtin_bit_cast(bf16x8, u); }
 
 // LDS row stride of a centroid plane in bf16 elements: 16 bytes of padding keep the 16-byte operand
 // reads of 16 consecutive lanes on different banks

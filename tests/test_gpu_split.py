@@ -52,6 +52,30 @@ def test_split_assign_matches_oracle(cuda, split_products, n, d, k):
     assert torch.all((md.double() - d2).abs() <= 2e-5 * scale + 1e-6)
 
 
+# wide rows (D > 64): the 2-D streaming kernel, whose staging threads split the panels
+@pytest.mark.parametrize("n,d,k", [(1500, 100, 70), (900, 512, 130), (513, 130, 1030), (300, 65, 3)])
+def test_split_streaming_assign_matches_oracle(cuda, split_products, n, d, k):
+    assert _native.assign_kernel_name(n, d, k) == "mfma_stream"
+    x, c = _data(n, d, k, seed=n + d + k)
+    xs, cs = x.to(cuda), c.to(cuda)
+    ws = _native.Workspace(cuda)
+    out = []
+    for _ in range(2):
+        lab = torch.full((n,), -7, dtype=torch.int32, device=cuda)
+        md = torch.full((n,), -1.0, device=cuda)
+        _native.assign(xs, cs, lab, md, ws)
+        out.append((lab.cpu(), md.cpu()))
+    assert torch.equal(out[0][0], out[1][0]) and torch.equal(out[0][1], out[1][1])
+    lab, md = out[0]
+    ref_lab, _ = orc.assign_to_cluster_literal(x, c)
+    assert lab.min() >= 0 and lab.max() < k
+    rep = orc.label_agreement(x, c, lab, ref_lab)
+    assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.999, rep
+    scale = (x.double() ** 2).sum(1) + (c.double() ** 2).sum(1).max()
+    d2 = orc.brute_force_d2(x, c).min(dim=1).values
+    assert torch.all((md.double() - d2).abs() <= 2e-5 * scale + 1e-6)
+
+
 def test_split_products_are_as_accurate_as_fp32_products(cuda, monkeypatch):
     """min_d2 of both paths against fp64 on data with large norms and small distances (the hard case
     for the quadratic expansion): the split path's error must stay within 1.5x the fp32 path's."""
@@ -131,5 +155,5 @@ def test_split_path_is_off_by_default_and_only_covers_its_shapes(cuda, monkeypat
             res.append((lab.cpu(), md.cpu()))
         assert torch.equal(res[0][0], res[2][0]) and torch.equal(res[0][1], res[2][1])
         if d != 32:
-            assert torch.equal(res[0][1], res[1][1])
+            assert torch.equal(res[0][1], res[1][1])  # tiled (D = 64) and narrow shapes have no split variant
     monkeypatch.delenv("HKM_PRODUCTS", raising=False)
