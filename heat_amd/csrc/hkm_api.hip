@@ -193,7 +193,7 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
         case ASSIGN_MFMA_TILED: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
             if (rc) return rc;
-            return launch_assign_mfma_tiled(X, N, D, ldx, C, K, ldc, w.cn, labels, min_d2, st);
+            return launch_assign_mfma_tiled(X, N, D, ldx, C, K, ldc, w.cn, labels, min_d2, use_split_products(), st);
         }
         default: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);

@@ -440,6 +440,171 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
     }
 }
 
+// The tiled kernel with the cross term from three-way split bf16 operands on the bf16 matrix cores
+// (opt-in, arithmetic as in hkm_assign_split.hip).  The threads that stage a centroid tile split the
+// fp32 values they fetched into three bf16 planes (one LDS buffer, two barriers per tile; two
+// workgroups per CU overlap); a wave splits its points once per point tile and keeps the parts in
+// registers.  DP is a multiple of 16 here (whole k-steps of the bf16 MFMA).
+template <int DP, bool VEC>
+__global__ __launch_bounds__(256) void assign_split_tiled_kernel(
+    const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
+    int64_t ldc, const float* __restrict__ cn, int32_t* __restrict__ labels,
+    float* __restrict__ min_d2, int64_t ntiles) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    constexpr int PB = 2;
+    constexpr int LDB = DP + 8;             // row stride of a plane in bf16 elements
+    constexpr int NJ = DP / 8;
+    constexpr int NS = DP / 16;             // k-steps
+    constexpr int TC = 128;                 // centroid rows per LDS tile
+    constexpr int GPR = DP / 4;             // 16-byte groups of fp32 per row
+    constexpr int NQ = TC * GPR / 256;      // groups per thread and tile
+    constexpr int PLANE = TC * LDB;         // bf16 elements per plane
+    __bf16* planes = reinterpret_cast<__bf16*>(lds_raw);                       // [3][TC][LDB]
+    float* sCn = reinterpret_cast<float*>(lds_raw + size_t(3) * PLANE * 2);    // [TC]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int p = lane & 31, h = lane >> 5;
+    const int nct = (K + TC - 1) / TC;
+    const int64_t my_tiles = (ntiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const int64_t nsteps = my_tiles * nct;
+
+    floatx4 pc[NQ];
+    float pcn = 0.f;
+    auto issue = [&](int ct) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int g = tid + 256 * q;
+            const int r = ct * TC + g / GPR, c = (g % GPR) * 4;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (r < K) v = load_row4<VEC>(C + int64_t(r) * ldc, c, D);
+            pc[q] = v;
+        }
+        if (tid < TC) pcn = cn[ct * TC + tid];  // padded with +inf beyond K
+    };
+
+    int64_t tile = blockIdx.x;
+    int ct = 0;
+    if (nsteps > 0) issue(0);
+
+    uintx4 xs[PB][3][NS];
+    float xn[PB], m[PB];
+    int mi[PB];
+
+    for (int64_t it = 0; it < nsteps; ++it) {
+        if (it > 0) __syncthreads();  // the previous tile's operands have been read
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+            const int g = tid + 256 * q;
+            unsigned a1[2], a2[2], a3[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+                split_pair(-2.0f * pc[q][2 * e], -2.0f * pc[q][2 * e + 1], a1[e], a2[e], a3[e]);
+            const int o = (g / GPR) * LDB + (g % GPR) * 4;
+            *reinterpret_cast<uint2*>(planes + o) = make_uint2(a1[0], a1[1]);
+            *reinterpret_cast<uint2*>(planes + PLANE + o) = make_uint2(a2[0], a2[1]);
+            *reinterpret_cast<uint2*>(planes + 2 * PLANE + o) = make_uint2(a3[0], a3[1]);
+        }
+        if (tid < TC) sCn[tid] = pcn;
+        __syncthreads();
+
+        const int64_t cur_tile = tile;
+        const int cur_ct = ct;
+        if (++ct == nct) {
+            ct = 0;
+            tile += gridDim.x;
+        }
+        if (it + 1 < nsteps) issue(ct);
+
+        const int64_t row0 = cur_tile * (4 * PB * 32) + wave * (PB * 32);
+        if (cur_ct == 0) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                int64_t r = row0 + pb * 32 + p;
+                r = r < N ? r : N - 1;
+                const float* xr = X + r * ldx;
+                float s = 0.f;
+                floatx4 b[NJ];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    b[j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) s = fmaf(b[j][t], b[j][t], s);
+                }
+                xn[pb] = s + __shfl_xor(s, 32);
+#pragma unroll
+                for (int st = 0; st < NS; ++st)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const floatx4 g = b[2 * st + (q >> 1)];
+                        unsigned p1, p2, p3;
+                        split_pair(g[2 * (q & 1)], g[2 * (q & 1) + 1], p1, p2, p3);
+                        xs[pb][0][st][q] = p1;
+                        xs[pb][1][st][q] = p2;
+                        xs[pb][2][st][q] = p3;
+                    }
+                m[pb] = HKM_INF;
+                mi[pb] = 0;
+            }
+        }
+
+        constexpr int XP[6] = {2, 0, 1, 1, 0, 0};
+        constexpr int CP[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll 1
+        for (int cb = 0; cb < TC / 32; ++cb) {
+            const floatx16 c0 = load_cn16(sCn + cb * 32 + 4 * h);
+            uintx4 cs[3][NS];
+#pragma unroll
+            for (int part = 0; part < 3; ++part)
+#pragma unroll
+                for (int st = 0; st < NS; ++st)
+                    cs[part][st] = *reinterpret_cast<const uintx4*>(planes + part * PLANE + (cb * 32 + p) * LDB +
+                                                                   h * (DP / 2) + 8 * st);
+            floatx16 acc[PB];
+#pragma unroll
+            for (int t = 0; t < 6; ++t)
+#pragma unroll
+                for (int st = 0; st < NS; ++st)
+#pragma unroll
+                    for (int pb = 0; pb < PB; ++pb)
+                        acc[pb] = (t == 0 && st == 0)
+                                      ? MFMA_BF16(as_bf16x8(cs[CP[t]][st]), as_bf16x8(xs[pb][XP[t]][st]), c0)
+                                      : MFMA_BF16(as_bf16x8(cs[CP[t]][st]), as_bf16x8(xs[pb][XP[t]][st]), acc[pb]);
+            const int kb = cur_ct * TC + cb * 32;
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) block_argmin(acc[pb], kb, m[pb], mi[pb]);
+        }
+
+        if (cur_ct == nct - 1) {
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb) {
+                float mm = fmaxf(m[pb] + xn[pb], 0.0f);
+                int ii = mi[pb] + 4 * h;
+                merge_halves(mm, ii);
+                const int64_t r = row0 + pb * 32 + p;
+                if (h == 0 && r < N) {
+                    labels[r] = ii;
+                    if (min_d2) min_d2[r] = mm;
+                }
+            }
+        }
+    }
+}
+
+template <int DP, bool VEC>
+static int launch_split_tiled_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                                int32_t K, int64_t ldc, const float* cn, int32_t* labels, float* min_d2,
+                                hipStream_t st) {
+    constexpr int PB = 2;
+    const int64_t ntiles = (N + 4 * PB * 32 - 1) / (4 * PB * 32);
+    const size_t lds = size_t(3) * 128 * (DP + 8) * 2 + 128 * sizeof(float);
+    auto kern = assign_split_tiled_kernel<DP, VEC>;
+    int64_t grid = int64_t(num_cus()) * 2;
+    if (grid > ntiles) grid = ntiles;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc, cn, labels,
+                       min_d2, ntiles);
+    return check_launch("assign_split_tiled_kernel");
+}
+
 template <int DP, bool VEC>
 static int launch_tiled_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                           int32_t K, int64_t ldc, const float* cn, int32_t* labels, float* min_d2,
@@ -462,8 +627,17 @@ static int launch_tiled_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
 
 int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
-                             float* min_d2, hipStream_t st) {
+                             float* min_d2, bool split, hipStream_t st) {
     const bool vec = aligned16(X) && aligned16(C) && (ldx % 4 == 0) && (ldc % 4 == 0) && (D % 4 == 0);
+    if (split) {
+        const int sdp = D <= 32 ? 32 : D <= 48 ? 48 : 64;  // whole k-steps of 16
+#define HKM_SCASE(d)                                                                                    \
+    case d:                                                                                             \
+        return vec ? launch_split_tiled_t<d, true>(X, N, D, ldx, C, K, ldc, cn, labels, min_d2, st)     \
+                   : launch_split_tiled_t<d, false>(X, N, D, ldx, C, K, ldc, cn, labels, min_d2, st);
+        switch (sdp) { HKM_SCASE(32) HKM_SCASE(48) HKM_SCASE(64) }
+#undef HKM_SCASE
+    }
     const int dp = resident_dp(D);
 #define HKM_CASE(d)                                                                              \
     case d:                                                                                      \

@@ -120,7 +120,7 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
                                 hipStream_t st);
 int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                              int32_t K, int64_t ldc, const float* cn, int32_t* labels,
-                             float* min_d2, hipStream_t st);
+                             float* min_d2, bool split, hipStream_t st);
 int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                               int32_t K, int64_t ldc, const float* cn, unsigned long long* keys,
                               int32_t* labels, float* min_d2, bool split, hipStream_t st);

@@ -22,11 +22,11 @@
  *   - all reductions use a fixed order: the same inputs give bit-identical outputs on every run.
  *
  * Environment (looked up on every call, nothing is cached)
- *   HKM_PRODUCTS=bf16x3   hkm_assign_f32 / hkm_lloyd_step_f32, shapes with 16 < D <= 32 whose centroids
- *                         fit in LDS, and shapes with D > 64: the cross term x.c is evaluated on the
- *                         bf16 matrix cores from operands split three ways (six partial products, fp32
- *                         accumulation) instead of fp32 matrix instructions.  Same error bound per
- *                         product as fp32, 1.3x to 1.5x the throughput.  Off by default.
+ *   HKM_PRODUCTS=bf16x3   hkm_assign_f32 / hkm_lloyd_step_f32, every shape with D > 16 except those with
+ *                         32 < D <= 64 whose centroids fit in LDS: the cross term x.c is evaluated on
+ *                         the bf16 matrix cores from operands split three ways (six partial products,
+ *                         fp32 accumulation) instead of fp32 matrix instructions.  Same error bound per
+ *                         product as fp32, 1.3x to 1.7x the throughput.  Off by default.
  *   HKM_UPDATE_LISTS=1    hkm_update_f32 and the two-pass part of hkm_lloyd_step_f32 use the list-based
  *                         kernels instead of the sort-based ones (a testing aid).
  */

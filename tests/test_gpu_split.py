@@ -52,10 +52,12 @@ def test_split_assign_matches_oracle(cuda, split_products, n, d, k):
     assert torch.all((md.double() - d2).abs() <= 2e-5 * scale + 1e-6)
 
 
-# wide rows (D > 64): the 2-D streaming kernel, whose staging threads split the panels
-@pytest.mark.parametrize("n,d,k", [(1500, 100, 70), (900, 512, 130), (513, 130, 1030), (300, 65, 3)])
-def test_split_streaming_assign_matches_oracle(cuda, split_products, n, d, k):
-    assert _native.assign_kernel_name(n, d, k) == "mfma_stream"
+# wide rows (D > 64): the 2-D streaming kernel, whose staging threads split the panels; 16 < D <= 64 with
+# more centroids than LDS holds: the tiled kernel, whose staging threads split the centroid tiles
+@pytest.mark.parametrize("n,d,k", [(1500, 100, 70), (900, 512, 130), (513, 130, 1030), (300, 65, 3),
+                                   (2048, 64, 1024), (3000, 64, 300), (700, 33, 500), (1300, 50, 437), (5000, 20, 900)])
+def test_split_streaming_and_tiled_assign_match_oracle(cuda, split_products, n, d, k):
+    assert _native.assign_kernel_name(n, d, k) in ("mfma_stream", "mfma_tiled")
     x, c = _data(n, d, k, seed=n + d + k)
     xs, cs = x.to(cuda), c.to(cuda)
     ws = _native.Workspace(cuda)
@@ -139,7 +141,7 @@ def test_split_path_is_off_by_default_and_only_covers_its_shapes(cuda, monkeypat
     """Without the environment variable nothing changes; with it, shapes outside 16 < D <= 32 keep the
     fp32 kernels (same bits as without)."""
     monkeypatch.delenv("HKM_PRODUCTS", raising=False)
-    for n, d, k in ((3000, 64, 100), (2000, 8, 16), (4096, 32, 256)):
+    for n, d, k in ((3000, 64, 100), (2000, 8, 16), (4096, 32, 256)):  # resident D=64, narrow, resident D=32
         x, c = _data(n, d, k, seed=1)
         xs, cs = x.to(cuda), c.to(cuda)
         ws = _native.Workspace(cuda)
@@ -155,5 +157,5 @@ def test_split_path_is_off_by_default_and_only_covers_its_shapes(cuda, monkeypat
             res.append((lab.cpu(), md.cpu()))
         assert torch.equal(res[0][0], res[2][0]) and torch.equal(res[0][1], res[2][1])
         if d != 32:
-            assert torch.equal(res[0][1], res[1][1])  # tiled (D = 64) and narrow shapes have no split variant
+            assert torch.equal(res[0][1], res[1][1])  # resident shapes wider than 32 and narrow ones have no split variant
     monkeypatch.delenv("HKM_PRODUCTS", raising=False)
