@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0
 PEAK_FP32_MFMA_TFLOPS = 157.3
 # configs that are bound by the fp32 matrix pipe; the others stream X from HBM
 MFMA_BOUND = {"c2", "c3", "c4"}
-CPU_SAMPLE_DIV = {"c1": 1, "c2": 16, "c3": 32, "c4": 256, "c5": 128}
+CPU_SAMPLE_DIV = {"c1": 1, "c2": 16, "c3": 16, "c4": 256, "c5": 128}
 
 
 def bench_kmedians(args, w, x, t_gen) -> int:
