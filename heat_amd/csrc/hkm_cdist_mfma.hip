@@ -24,31 +24,43 @@ static constexpr int CM_LD = CM_DC + 4;
 
 __device__ __forceinline__ floatx4 cm_ld4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
 
-// FULL: the tile lies inside the matrix (no guards on the stores); EPI: 0 squared distance, 1 sqrt,
-// 2 exp(-d2 * gauss)
+// Correctly rounded square root of t = 0, +inf, NaN or any finite t >= 2^-96: the hardware square root
+// (1 ulp) followed by a two-sided test of its neighbours against the exact residual.  Equal to sqrtf
+// on every such input (checked exhaustively on the device; the first disagreement lies below 2^-104,
+// where the residual underflows) at half of its instruction count: no range scaling, no class test.
+// Zero, infinity and NaN fall through because every comparison against a NaN residual is false.
+__device__ __forceinline__ float cm_sqrt_rn(float t) {
+    const float s = __builtin_amdgcn_sqrtf(t);
+    const float sd = __uint_as_float(__float_as_uint(s) - 1u), su = __uint_as_float(__float_as_uint(s) + 1u);
+    const float ed = fmaf(-sd, s, t), eu = fmaf(-su, s, t);
+    float r = ed <= 0.f ? sd : s;
+    r = eu > 0.f ? su : r;
+    return r;
+}
+
+// FULL: the tile lies inside the matrix (no guards on the stores); EPI: 0 squared distance, 1 sqrt with
+// the short form above, 2 exp(-d2 * gauss), 3 sqrt by the library routine (any input)
 template <bool FULL, int EPI>
-__device__ __forceinline__ void cm_store_tile(const floatx16 (&acc)[2][2], const float* sXn, const float* sYn,
-                                              float* __restrict__ out_tile, int64_t ldo, int wx, int wy, int p,
-                                              int h, int rows_left, int cols_left, float gauss) {
+__device__ __forceinline__ void cm_store_values(const floatx16 (&acc)[2][2], float* __restrict__ out_tile,
+                                                int64_t ldo, int wx, int wy, int p, int h, int rows_left,
+                                                int cols_left, float gauss) {
     // byte offset of this lane inside the tile, without the block / register terms (those are uniform)
     const unsigned lane_off = unsigned(((wx * 64 + 4 * h) * ldo + wy * 64 + p) * 4);
-    const float yn[2] = {sYn[wy * 64 + p], sYn[wy * 64 + 32 + p]};
 #pragma unroll
     for (int xb = 0; xb < 2; ++xb)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             // rows 8g + 4h .. + 3 of the block: registers 4g .. 4g + 3
             const int r0 = wx * 64 + xb * 32 + 8 * g + 4 * h;
-            const floatx4 xn4 = cm_ld4(sXn + r0);
             float d[4][2];
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
                 for (int yb = 0; yb < 2; ++yb) {
-                    float t = fmaf(-2.0f, acc[xb][yb][4 * g + q], xn4[q] + yn[yb]);
-                    t = t > 0.0f ? t : (t != t ? t : 0.0f);  // clamp at 0, NaN passes through
+                    float t = acc[xb][yb][4 * g + q];
                     if (EPI == 2) t = expf(-t * gauss);
-                    else if (EPI == 1) t = sqrtf(t);
+                    else if (EPI == 1) t = cm_sqrt_rn(t);
+                    else if (EPI == 3) t = sqrtf(t);
                     d[q][yb] = t;
                 }
 #pragma unroll
@@ -62,8 +74,50 @@ __device__ __forceinline__ void cm_store_tile(const floatx16 (&acc)[2][2], const
         }
 }
 
+template <bool FULL, int EPI>
+__device__ __forceinline__ void cm_store_tile(floatx16 (&acc)[2][2], const float* sXn, const float* sYn,
+                                              float* __restrict__ out_tile, int64_t ldo, int wx, int wy, int p,
+                                              int h, int rows_left, int cols_left, float gauss) {
+    // squared distances in place, in the reference's order: (|x|^2 + |y|^2) first, then - 2 x.y, then
+    // the clamp at 0.  A NaN passes through (NaN < 0 is false); the value is never -0 (the sum of
+    // the norms is never -0), so the comparison form equals clamp(min=0) on every input.
+    const float yn[2] = {sYn[wy * 64 + p], sYn[wy * 64 + 32 + p]};
+#pragma unroll
+    for (int xb = 0; xb < 2; ++xb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const floatx4 xn4 = cm_ld4(sXn + wx * 64 + xb * 32 + 8 * g + 4 * h);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int yb = 0; yb < 2; ++yb) {
+                    const float t = fmaf(-2.0f, acc[xb][yb][4 * g + q], xn4[q] + yn[yb]);
+                    acc[xb][yb][4 * g + q] = t < 0.0f ? 0.0f : t;
+                }
+        }
+    if (EPI == 1) {
+        // the short square root covers 0 and everything from 2^-96 up; a wave whose smallest POSITIVE
+        // value lies below takes the library routine for its whole sub-tile.  As unsigned integers
+        // (bits - 1) orders the non-negative floats with zero moved to the top, so one integer
+        // minimum tree finds the smallest positive value (a NaN sits above every finite value).
+        unsigned m = 0xffffffffu;
+#pragma unroll
+        for (int xb = 0; xb < 2; ++xb)
+#pragma unroll
+            for (int yb = 0; yb < 2; ++yb)
+#pragma unroll
+                for (int v = 0; v < 16; v += 2)
+                    m = min(m, min(__float_as_uint(acc[xb][yb][v]) - 1u, __float_as_uint(acc[xb][yb][v + 1]) - 1u));
+        if (__builtin_amdgcn_ballot_w64(m < 0x0f800000u - 1u) != 0) {  // some 0 < t < 2^-96 in the wave
+            cm_store_values<FULL, 3>(acc, out_tile, ldo, wx, wy, p, h, rows_left, cols_left, gauss);
+            return;
+        }
+    }
+    cm_store_values<FULL, EPI>(acc, out_tile, ldo, wx, wy, p, h, rows_left, cols_left, gauss);
+}
+
 template <bool VEC, int EPI>
-__global__ __launch_bounds__(256) void cdist_mfma_kernel(const float* __restrict__ X, int64_t M, int64_t ldx,
+__global__ __launch_bounds__(256, 2) void cdist_mfma_kernel(const float* __restrict__ X, int64_t M, int64_t ldx,
                                                          const float* __restrict__ Y, int64_t Nn, int64_t ldy,
                                                          int D, float* __restrict__ out, int64_t ldo,
                                                          float gauss, int64_t tiles_n, int64_t total, int ndc) {
@@ -138,12 +192,8 @@ __global__ __launch_bounds__(256) void cdist_mfma_kernel(const float* __restrict
     int dc = 0;
     floatx16 acc[2][2];
     float xsq[4] = {0.f, 0.f, 0.f, 0.f}, ysq[4] = {0.f, 0.f, 0.f, 0.f};
-    if (nsteps > 0) {
-        set_tile(tile);
-        issue(0);
-    }
-    for (int64_t it = 0; it < nsteps; ++it) {
-        const int buf = int(it & 1);
+    // registers of the chunk in flight -> LDS buffer `buf`, squared norms accumulated on the way
+    auto stage = [&](int buf) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             *reinterpret_cast<floatx4*>(&sA[buf][(sr + 32 * q) * CM_LD + sc]) = pa[q];
@@ -154,16 +204,39 @@ __global__ __launch_bounds__(256) void cdist_mfma_kernel(const float* __restrict
                 ysq[q] = fmaf(pb[q][t], pb[q][t], ysq[q]);
             }
         }
+    };
+    if (nsteps > 0) {
+        set_tile(tile);
+        issue(0);
+        if (my_tiles >= 16) {
+            // Stagger the start.  Workgroups launched together would run their store phases together:
+            // the matrix cores idle while the whole chip stores, and the memory system idles while it
+            // computes.  Sixteen start phases across one tile period (about 10 000 cycles per chunk
+            // with two workgroups sharing a CU) spread the stores evenly over time; workgroups b and
+            // b + 256, which tend to share a CU, start half a period apart.  Costs at most one tile
+            // time of the my_tiles a workgroup processes.
+            const int phase = (((blockIdx.x >> 3) & 7) + 8 * ((blockIdx.x >> 8) & 1)) & 15;
+            for (int i = 0; i < phase * ndc; ++i) __builtin_amdgcn_s_sleep(10);  // 640 cycles each
+        }
+        stage(0);
+    }
+    // One barrier per step: it publishes the chunk staged at the end of the previous step and retires
+    // every read of the other buffer.  The chunk of the NEXT step is requested right after it and moved
+    // to LDS after this step's MFMAs -- before a tile's results are stored, so that no wait for loaded
+    // data ever has those stores ahead of it in the memory queue (loads and stores share one counter).
+    for (int64_t it = 0; it < nsteps; ++it) {
+        const int buf = int(it & 1);
         __syncthreads();
 
         const int64_t cur_tile = tile;
         const int cur_dc = dc;
+        const bool more = it + 1 < nsteps;
         if (++dc == ndc) {
             dc = 0;
             tile += gridDim.x;
-            if (it + 1 < nsteps) set_tile(tile);
+            if (more) set_tile(tile);
         }
-        if (it + 1 < nsteps) issue(dc);
+        if (more) issue(dc);
 
         if (cur_dc == 0) {
 #pragma unroll
@@ -195,8 +268,10 @@ __global__ __launch_bounds__(256) void cdist_mfma_kernel(const float* __restrict
             }
         }
 
-        if (cur_dc == ndc - 1) {
-            // squared norms of the tile's rows of X and Y: the eight threads that staged a row add their parts
+        const bool last = cur_dc == ndc - 1;
+        if (last) {
+            // squared norms of the tile's rows of X and Y: the eight threads that staged a row add their
+            // parts (the previous tile's readers of sXn / sYn are behind this step's barrier)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 float vx = xsq[q], vy = ysq[q];
@@ -213,6 +288,9 @@ __global__ __launch_bounds__(256) void cdist_mfma_kernel(const float* __restrict
                 xsq[q] = 0.f;
                 ysq[q] = 0.f;
             }
+        }
+        if (more) stage(buf ^ 1);
+        if (last) {
             __syncthreads();
             const int64_t i0 = (cur_tile / tiles_n) * CM_T, j0 = (cur_tile % tiles_n) * CM_T;
             float* out_tile = out + i0 * ldo + j0;

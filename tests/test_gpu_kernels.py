@@ -337,6 +337,36 @@ def test_cdist_matrix_core_path(cuda, m, n, d):
     assert bool(torch.isnan(dense[0]).all()) and not bool(torch.isnan(dense[1:]).any())
 
 
+@pytest.mark.parametrize("scale", [1.0, 1e-3, 1e-15, 1e-18, 1e-22])
+def test_cdist_matrix_core_sqrt_is_correctly_rounded(cuda, scale):
+    """The kernel's square root is the correctly rounded one at every magnitude: the short form for
+    ordinary values, the library routine for sub-tiles that hold positive values below 2^-96
+    (squared distances of rows scaled by 1e-15 and less, denormals included), zeros on the diagonal,
+    infinities and NaN.  Checked against the square root, taken in float64 by numpy and rounded to
+    float32 (innocuous double rounding: 53 >= 2 * 24 + 2 bits), of the kernel's own squared output --
+    not against torch's CPU square root, which goes through a vector math library that is only
+    accurate to an ulp on some hosts."""
+    m, n, d = 300, 260, 48
+    g = torch.Generator().manual_seed(int(-torch.log10(torch.tensor(scale))) + 5)
+    a, b = torch.randn((m, d), generator=g) * scale, torch.randn((n, d), generator=g) * scale
+    b[:100] = a[:100]  # exact zeros
+    a[200:, :] *= 1e6 / scale if scale < 1e-10 else 1.0  # ordinary and tiny values in one matrix
+    a[299, 0] = float("inf")
+    b[259, 1] = float("nan")
+    ag, bg = a.to(cuda), b.to(cuda)
+    sq = torch.empty((m, n), device=cuda)
+    rt = torch.empty((m, n), device=cuda)
+    _native.cdist(ag, bg, sq, sqrt=False)
+    _native.cdist(ag, bg, rt, sqrt=True)
+    with np.errstate(invalid="ignore"):
+        want = torch.from_numpy(np.sqrt(sq.cpu().numpy().astype(np.float64)).astype(np.float32))
+    got = rt.cpu()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    assert torch.equal(got[~nan].view(torch.int32), want[~nan].view(torch.int32))
+    assert int((sq[:100, :100].diagonal() == 0).sum()) > 0 or scale >= 1e-3
+
+
 def test_cdist_matrix_core_known_answers(cuda):
     # the reference's known answers (tests/spatial/test_distances.py:16-58) at a width that takes the
     # matrix-core kernel: ones against zeros -> sqrt(D), a matrix against itself -> 0, exactly
