@@ -24,20 +24,6 @@ static constexpr int CM_LD = CM_DC + 4;
 
 __device__ __forceinline__ floatx4 cm_ld4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
 
-// Correctly rounded square root of t = 0, +inf, NaN or any finite t >= 2^-96: the hardware square root
-// (1 ulp) followed by a two-sided test of its neighbours against the exact residual.  Equal to sqrtf
-// on every such input (checked exhaustively on the device; the first disagreement lies below 2^-104,
-// where the residual underflows) at half of its instruction count: no range scaling, no class test.
-// Zero, infinity and NaN fall through because every comparison against a NaN residual is false.
-__device__ __forceinline__ float cm_sqrt_rn(float t) {
-    const float s = __builtin_amdgcn_sqrtf(t);
-    const float sd = __uint_as_float(__float_as_uint(s) - 1u), su = __uint_as_float(__float_as_uint(s) + 1u);
-    const float ed = fmaf(-sd, s, t), eu = fmaf(-su, s, t);
-    float r = ed <= 0.f ? sd : s;
-    r = eu > 0.f ? su : r;
-    return r;
-}
-
 // FULL: the tile lies inside the matrix (no guards on the stores); EPI: 0 squared distance, 1 sqrt with
 // the short form above, 2 exp(-d2 * gauss), 3 sqrt by the library routine (any input)
 template <bool FULL, int EPI>
@@ -59,7 +45,7 @@ __device__ __forceinline__ void cm_store_values(const floatx16 (&acc)[2][2], flo
                 for (int yb = 0; yb < 2; ++yb) {
                     float t = acc[xb][yb][4 * g + q];
                     if (EPI == 2) t = expf(-t * gauss);
-                    else if (EPI == 1) t = cm_sqrt_rn(t);
+                    else if (EPI == 1) t = sqrt_rn_short(t);
                     else if (EPI == 3) t = sqrtf(t);
                     d[q][yb] = t;
                 }
@@ -107,8 +93,8 @@ __device__ __forceinline__ void cm_store_tile(floatx16 (&acc)[2][2], const float
             for (int yb = 0; yb < 2; ++yb)
 #pragma unroll
                 for (int v = 0; v < 16; v += 2)
-                    m = min(m, min(__float_as_uint(acc[xb][yb][v]) - 1u, __float_as_uint(acc[xb][yb][v + 1]) - 1u));
-        if (__builtin_amdgcn_ballot_w64(m < 0x0f800000u - 1u) != 0) {  // some 0 < t < 2^-96 in the wave
+                    m = min(m, min(sqrt_short_key(acc[xb][yb][v]), sqrt_short_key(acc[xb][yb][v + 1])));
+        if (__builtin_amdgcn_ballot_w64(m < SQRT_SHORT_KEY_LIMIT) != 0) {  // some 0 < t < 2^-96 in the wave
             cm_store_values<FULL, 3>(acc, out_tile, ldo, wx, wy, p, h, rows_left, cols_left, gauss);
             return;
         }
