@@ -99,6 +99,61 @@ def bench_kmedians(args, w, x, t_gen) -> int:
     return 0
 
 
+def bench_init(args, w, x, t_gen) -> int:
+    """The k-means|| initialiser (KMeans(init="probability_based"), heat/cluster/_kcluster.py:146-247) on
+    the workload's data: a "step" is one complete initialisation -- the sampling rounds (one fused
+    distance + minimum launch against the round's new candidates, a reduction, an ordered selection),
+    the weights of the candidates and their k-means++ reclustering.  oversampling = 20 (with the
+    reference's default of 2 fewer candidates than clusters come out for K = 256 and the reference
+    restarts with 20 itself).  The rounds are bound by reading X once each: algorithmic bytes per step
+    = (rounds + 2) * N * 4 D (initial cost, one read per round but the last, the final assignment)."""
+    import warnings
+
+    import torch
+
+    import heat_amd as ht
+
+    if w.init is None:
+        print("--estimator init needs a clustering workload (not c2)", file=sys.stderr)
+        return 2
+    n, d = x.shape
+    k = w.k
+    xd = ht.array(x, split=0)
+
+    def step(seed):
+        km = ht.cluster.KMeans(n_clusters=k, init="probability_based", random_state=seed)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            km._initialize_cluster_centers(xd, 20, 1)
+        return km
+
+    for i in range(min(args.warmup, 5)):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        km = step(100 + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    nrounds = int(km._init_rounds)  # int(ln(initial cost)) of the last seed
+    alg = (nrounds + 2) * n * 4.0 * d
+    ms = elapsed / args.steps * 1e3
+    out = {
+        "metric": "k-means|| initialisation points/s", "value": round(n * args.steps / elapsed, 1), "unit": "points/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": min(args.warmup, 5), "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": f"synthetic (seed {w.seed}, generated on CPU in {t_gen:.1f} s, resident in HBM before timing)",
+        "config": {"workload": w.name, "estimator": "KMeans(init=probability_based)", "N": n, "D": d, "K": k,
+                   "oversampling": 20, "rounds": nrounds, "scale": args.scale},
+        "roofline": {"bound": "hbm", "achieved": round(alg / (ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(alg / (ms * 1e-3) / 8e12, 4), "kernel": "whole initialisation (host-timed)",
+                     "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+    return 0
+
+
 def bench_cdist(args, w, x, t_gen) -> int:
     """The public full-matrix ht.spatial.cdist(X, Y, quadratic_expansion=True) on rows of the c2 data:
     X = the first 32768 rows, Y = the next 32768 rows (D = 64), a 4.29 GB matrix of sqrt distances per
@@ -162,9 +217,9 @@ def main() -> int:
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink N (testing only; invalidates the figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians", "cdist"],
+    ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians", "cdist", "init"],
                     help="kmedians: the Manhattan-metric sibling on the same data; cdist: the full-matrix "
-                         "public cdist on rows of c2 (neither is the headline metric)")
+                         "public cdist on rows of c2; init: the k-means|| initialiser (none is the headline metric)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
@@ -198,6 +253,8 @@ def main() -> int:
         return bench_kmedians(args, w, x, t_gen)
     if args.estimator == "cdist":
         return bench_cdist(args, w, x, t_gen)
+    if args.estimator == "init":
+        return bench_init(args, w, x, t_gen)
     if args.config == "c2":
         # assignment only: labels + min squared distance
         y = w.y.to(dev)

@@ -43,6 +43,8 @@ SIGNATURES = {
     "hkm_sample_select_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_void_p, ctypes.c_float, c_void_p,
                                              c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_label_counts_i64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
+    "hkm_seed_plus_plus_f32": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_int32, c_void_p,
+                                              c_int32, c_int32, c_void_p, c_void_p]),
     "hkm_assign_l1_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                          c_void_p, c_void_p, c_void_p]),
     "hkm_closest_rows_l1_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
@@ -301,6 +303,25 @@ def label_counts(labels32: torch.Tensor, k: int, counts: torch.Tensor) -> None:
     if counts.numel() != k:
         raise ValueError(f"counts has {counts.numel()} elements, expected {k}")
     check(load().hkm_label_counts_i64(_ptr(labels32), labels32.numel(), k, _ptr(counts), _stream()))
+
+
+SEED_MAX_ROWS = 16384  # HKM_SEED_MAX_ROWS
+
+
+def seed_plus_plus(x: torch.Tensor, weights: Optional[torch.Tensor], first: int, u: torch.Tensor, k: int, p: int,
+                   idx: torch.Tensor) -> None:
+    """k-means++ seeding of at most SEED_MAX_ROWS rows in one launch (see hkm_seed_plus_plus_f32 in
+    include/hkm.h): idx[0] = first, idx[j] drawn by inverse CDF from u[j - 1]; -1 where no row has mass."""
+    _require_gpu(x, weights, u, idx)
+    m, d = x.shape
+    if idx.numel() != k or idx.dtype != torch.int64:
+        raise ValueError("idx must hold k int64 entries")
+    if u.numel() < k - 1 or u.dtype != torch.float32:
+        raise ValueError("u must hold k - 1 float32 numbers")
+    if weights is not None and (weights.numel() != m or weights.dtype != torch.float32 or not weights.is_contiguous()):
+        raise ValueError("weights must be a contiguous float32 vector with one entry per row")
+    check(load().hkm_seed_plus_plus_f32(_ptr(x), m, d, x.stride(0) if m > 1 else d, _ptr(weights), int(first),
+                                        _ptr(u), k, p, _ptr(idx), _stream()))
 
 
 def assign_l1(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_dist: Optional[torch.Tensor]) -> None:

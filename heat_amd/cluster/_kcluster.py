@@ -177,22 +177,28 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         return DeviceSampler(device, self.random_state)
 
     def _centroid_sampling_helper(self, xt: torch.Tensor, centroids: torch.Tensor, oversampling: float,
-                                  num_iters: int, sampler, ws) -> torch.Tensor:
+                                  num_iters: int, sampler, ws, dmin: Optional[torch.Tensor] = None) -> torch.Tensor:
         """
         ``num_iters`` rounds of: distance of every row to its closest current candidate, then every
         row joins the candidates with probability ``oversampling * distance / sum(distance)``
-        (heat/cluster/_kcluster.py:283-350).  One fused distance+argmin launch, one reduction and one
-        ordered selection per round; only the number of new candidates comes back to the host.
+        (heat/cluster/_kcluster.py:283-350).  ``dmin``, if given, holds the squared distances to the
+        closest of the candidates passed in (it is overwritten).  The reference recomputes the distances to ALL
+        candidates in every round; the minimum over a grown set is the minimum of the old minimum and
+        the distances to the new members, so a round here costs one fused distance+argmin launch
+        against the handful of NEW candidates, one elementwise minimum, one reduction and one ordered
+        selection; only the number of new candidates comes back to the host.
         """
         n = xt.shape[0]
         dev = xt.device
         lab = torch.empty((n,), dtype=torch.int32, device=dev)
-        dmin = torch.empty((n,), dtype=xt.dtype, device=dev)
+        if dmin is None:
+            dmin = torch.empty((n,), dtype=xt.dtype, device=dev)
+            _native.assign(xt, centroids, lab, dmin, ws)
+        dnew = torch.empty_like(dmin)
         cost = torch.empty((), dtype=torch.float32, device=dev)
         count = torch.zeros((), dtype=torch.int64, device=dev)
         idx = torch.empty((max(1024, int(16 * oversampling)),), dtype=torch.int64, device=dev)
-        for _ in range(num_iters):
-            _native.assign(xt, centroids, lab, dmin, ws)
+        for it in range(num_iters):
             d2 = dmin if dmin.dtype == torch.float32 else dmin.float()  # the draw itself runs in float32
             _native.min_dist_sum(d2, cost, ws)
             u = sampler.uniform(n)
@@ -201,7 +207,13 @@ class _KCluster(ClusteringMixin, BaseEstimator):
             if c > idx.numel():
                 idx = torch.empty((c,), dtype=torch.int64, device=dev)
                 _native.sample_select(d2, u, cost, oversampling, idx, count, ws)
-            centroids = torch.cat((centroids, xt[idx[:c]]), dim=0)
+            if c == 0:
+                continue
+            fresh = xt[idx[:c]]
+            centroids = torch.cat((centroids, fresh), dim=0)
+            if it + 1 < num_iters:
+                _native.assign(xt, fresh, lab, dnew, ws)
+                torch.minimum(dmin, dnew, out=dmin)
         return centroids
 
     def _kmeans_parallel(self, x: DNDarray, oversampling: float, iter_multiplier: float) -> torch.Tensor:
@@ -225,7 +237,9 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         # the order of magnitude of the initial cost sets the number of rounds (_kcluster.py:172-175);
         # all rows equal gives cost 0, where the reference fails in int(-inf): one round instead
         num_iters = max(1, int(iter_multiplier * math.log(init_cost))) if init_cost > 0.0 else 1
-        centroids = self._centroid_sampling_helper(xt, init_centroids, oversampling, num_iters, sampler, ws)
+        self._init_rounds = num_iters
+        centroids = self._centroid_sampling_helper(xt, init_centroids, oversampling, num_iters, sampler, ws,
+                                                   dmin.clone())
         if centroids.shape[0] <= self.n_clusters:
             warnings.warn(
                 f"Oversampling={oversampling} is too low for data set."
@@ -233,7 +247,7 @@ class _KCluster(ClusteringMixin, BaseEstimator):
                 UserWarning,
             )
             oversampling = 10 * oversampling
-            centroids = self._centroid_sampling_helper(xt, init_centroids, oversampling, num_iters, sampler, ws)
+            centroids = self._centroid_sampling_helper(xt, init_centroids, oversampling, num_iters, sampler, ws, dmin)
         if centroids.shape[0] <= self.n_clusters:
             raise ValueError(
                 f"The parameter oversampling={oversampling} and/or iter_multiplier={iter_multiplier} "

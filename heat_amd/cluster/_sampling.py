@@ -18,6 +18,9 @@ import torch
 
 
 class DeviceSampler:
+    # the k-means++ seeding of a small row set may take all its draws at once, as uniform numbers
+    fused_seeding = True
+
     def __init__(self, device: torch.device, seed: Optional[int] = None):
         self.device = torch.device(device)
         self._gen = torch.Generator(device=self.device)
@@ -37,3 +40,7 @@ class DeviceSampler:
     def multinomial(self, weights: torch.Tensor) -> int:
         """One index drawn with probability proportional to ``weights`` (non-negative, not all zero)."""
         return int(torch.multinomial(weights, 1, generator=self._gen).item())
+
+    def multinomial_on_device(self, weights: torch.Tensor) -> torch.Tensor:
+        """The same draw as :meth:`multinomial`, left on the device as a 0-d int64 tensor."""
+        return torch.multinomial(weights, 1, generator=self._gen).reshape(())

@@ -37,20 +37,40 @@ def _initialize_plus_plus(x: torch.Tensor, n_clusters: int, p: int, sampler, wei
     k-means++ seeding as heat/cluster/batchparallelclustering.py:22-46 does it: the first centre
     uniformly, every further one with probability proportional to ``weights * distance`` (the plain
     p-norm distance to the closest centre chosen so far, not its square).  More than ``max_samples`` rows
-    are subsampled first because a categorical draw is limited to 2**24 categories.  The reference
+    are subsampled first because a categorical draw is limited to 2**24 categories.  Up to
+    ``_native.SEED_MAX_ROWS`` float32 rows with a sampler that allows it (``fused_seeding``) are seeded by
+    one kernel launch that draws by inverse CDF from one uniform number per centre.  The reference
     recomputes the distances to all chosen centres in every step; the running minimum kept here is
     the same number and needs one N x 1 distance column per step.
     """
     if x.shape[0] > max_samples:
         sub = torch.tensor([sampler.randint(x.shape[0]) for _ in range(max_samples)], device=x.device)
         x = x[sub].contiguous()
+    if (getattr(sampler, "fused_seeding", False) and x.dtype == torch.float32 and x.shape[0] <= _native.SEED_MAX_ROWS
+            and p in (1, 2)):
+        # a small row set (the candidates of k-means||): all draws in one launch, from one uniform number each
+        w = None
+        if isinstance(weights, torch.Tensor):
+            w = weights.to(device=x.device, dtype=torch.float32).contiguous()
+        elif float(weights) != 1.0:
+            w = torch.full((x.shape[0],), float(weights), dtype=torch.float32, device=x.device)
+        first = sampler.randint(x.shape[0])
+        u = sampler.uniform(max(n_clusters - 1, 1))
+        idx = torch.empty((n_clusters,), dtype=torch.int64, device=x.device)
+        _native.seed_plus_plus(x.contiguous() if x.stride(1) != 1 else x, w, first, u, n_clusters, p, idx)
+        if bool((idx < 0).any()):
+            raise RuntimeError("invalid multinomial distribution (sum of probabilities <= 0)")
+        return x[idx]
+    # the drawn indices stay on the device where the sampler can leave them there: a draw only feeds
+    # the gather of the next centre, and reading each one back would stall the queue n_clusters times
+    draw = getattr(sampler, "multinomial_on_device", None) or sampler.multinomial
     idxs = [sampler.randint(x.shape[0])]
     dist = _dist_to_row(x, x[idxs[0]], p)
     for i in range(1, n_clusters):
-        idxs.append(sampler.multinomial(weights * dist))
+        idxs.append(draw(weights * dist))
         if i + 1 < n_clusters:
-            dist = torch.minimum(dist, _dist_to_row(x, x[idxs[-1]], p))
-    return x[torch.tensor(idxs, device=x.device)]
+            dist = torch.minimum(dist, _dist_to_row(x, x[idxs[-1]].reshape(-1), p))
+    return x[torch.stack([torch.as_tensor(i, device=x.device).reshape(()) for i in idxs])]
 
 
 def _kmex(x: torch.Tensor, p: int, n_clusters: int, init: Union[str, torch.Tensor], max_iter: int, tol: float,

@@ -376,6 +376,20 @@ int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* c
     return launch_label_counts(labels, N, K, counts, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_seed_plus_plus_f32(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
+                           const float* u, int32_t K, int32_t p, int64_t* idx, void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 1 || M > HKM_SEED_MAX_ROWS)
+        return fail(HKM_EINVAL, "M = %d outside 1..%d", M, HKM_SEED_MAX_ROWS);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
+    if (ldx < D) return fail(HKM_EINVAL, "leading dimension of X (%lld) < columns (%d)", (long long)ldx, D);
+    if (first < 0 || first >= M) return fail(HKM_EINVAL, "first = %d outside 0..%d", first, M - 1);
+    if (p != 1 && p != 2) return fail(HKM_EINVAL, "p = %d must be 1 or 2", p);
+    if (!X || !idx || (K > 1 && !u)) return fail(HKM_EINVAL, "NULL pointer argument");
+    return launch_seed_plus_plus(X, M, D, ldx, w, first, u, K, p, idx, static_cast<hipStream_t>(hip_stream));
+}
+
 // ---- float64 data -----------------------------------------------------------------------------
 static int check_matrix64(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
     if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);

@@ -199,6 +199,8 @@ int launch_select(const float* d2, const float* u, int64_t N, const float* cost,
                   int64_t* idx, int64_t cap, int64_t* count, double* red, hipStream_t st);
 int launch_label_counts(const int32_t* labels, int64_t N, int32_t K, int64_t* counts,
                         hipStream_t st);
+int launch_seed_plus_plus(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
+                          const float* u, int32_t K, int32_t p, int64_t* idx, hipStream_t st);
 int launch_assign_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                      int64_t ldc, int32_t* labels, float* min_dist, hipStream_t st);
 int launch_closest_rows_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* Qm,

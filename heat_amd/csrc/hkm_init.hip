@@ -18,13 +18,22 @@ __global__ __launch_bounds__(256) void select_count_kernel(const float* __restri
                                                            const float* __restrict__ u, int64_t n,
                                                            int64_t per_block,
                                                            const float* __restrict__ cost, float os,
-                                                           long long* __restrict__ block_cnt) {
+                                                           long long* __restrict__ block_cnt, bool vec) {
     __shared__ int sh[256];
     const float denom = fmaxf(*cost, 1e-12f);
     const int64_t b0 = int64_t(blockIdx.x) * per_block;
     const int64_t b1 = min(n, b0 + per_block);
     int c = 0;
-    for (int64_t i = b0 + threadIdx.x; i < b1; i += 256) c += selected(d2[i], u[i], os, denom) ? 1 : 0;
+    int64_t i0 = b0;
+    if (vec) {  // both arrays 16-byte aligned, per_block a multiple of 1024: whole 16-byte groups
+        for (; i0 + 1024 <= b1; i0 += 1024) {
+            const float4 a = *reinterpret_cast<const float4*>(d2 + i0 + threadIdx.x * 4);
+            const float4 b = *reinterpret_cast<const float4*>(u + i0 + threadIdx.x * 4);
+            c += (selected(a.x, b.x, os, denom) ? 1 : 0) + (selected(a.y, b.y, os, denom) ? 1 : 0) +
+                 (selected(a.z, b.z, os, denom) ? 1 : 0) + (selected(a.w, b.w, os, denom) ? 1 : 0);
+        }
+    }
+    for (int64_t i = i0 + threadIdx.x; i < b1; i += 256) c += selected(d2[i], u[i], os, denom) ? 1 : 0;
     sh[threadIdx.x] = c;
     __syncthreads();
     for (int w = 128; w > 0; w >>= 1) {
@@ -67,8 +76,12 @@ __global__ __launch_bounds__(256) void select_write_kernel(const float* __restri
                                                            int64_t per_block,
                                                            const float* __restrict__ cost, float os,
                                                            const long long* __restrict__ block_off,
+                                                           const long long* __restrict__ count, int nb,
                                                            int64_t* __restrict__ idx, int64_t cap) {
     __shared__ int wave_cnt[4];
+    // a block without a selected row (nearly all of them: a round selects a handful of rows) is done
+    const long long mine = (int(blockIdx.x) + 1 < nb ? block_off[blockIdx.x + 1] : *count) - block_off[blockIdx.x];
+    if (mine == 0) return;
     const float denom = fmaxf(*cost, 1e-12f);
     const int64_t b0 = int64_t(blockIdx.x) * per_block;
     const int64_t b1 = min(n, b0 + per_block);
@@ -99,20 +112,25 @@ __global__ __launch_bounds__(256) void select_write_kernel(const float* __restri
 
 int launch_select(const float* d2, const float* u, int64_t N, const float* cost, float os,
                   int64_t* idx, int64_t cap, int64_t* count, double* red, hipStream_t st) {
-    int nb = int((N + 16383) / 16384);
+    // short blocks: the few blocks that hold a selected row walk their range in dependent steps of 256
+    // rows in the write pass and set its duration
+    int nb = int((N + 2047) / 2048);
     if (nb < 1) nb = 1;
     if (nb > RED_SLOTS) nb = RED_SLOTS;
     int64_t per_block = (N + nb - 1) / nb;
-    per_block = (per_block + 255) / 256 * 256;
+    per_block = (per_block + 1023) / 1024 * 1024;
+    nb = int((N + per_block - 1) / per_block);
+    if (nb < 1) nb = 1;
     long long* bc = reinterpret_cast<long long*>(red);
-    hipLaunchKernelGGL(select_count_kernel, dim3(nb), dim3(256), 0, st, d2, u, N, per_block, cost, os, bc);
+    const bool vec = aligned16(d2) && aligned16(u);
+    hipLaunchKernelGGL(select_count_kernel, dim3(nb), dim3(256), 0, st, d2, u, N, per_block, cost, os, bc, vec);
     int rc = check_launch("select_count_kernel");
     if (rc) return rc;
     hipLaunchKernelGGL(select_scan_kernel, dim3(1), dim3(256), 0, st, bc, nb,
                        reinterpret_cast<long long*>(count));
     if ((rc = check_launch("select_scan_kernel"))) return rc;
     hipLaunchKernelGGL(select_write_kernel, dim3(nb), dim3(256), 0, st, d2, u, N, per_block, cost, os,
-                       bc, idx, cap);
+                       bc, reinterpret_cast<const long long*>(count), nb, idx, cap);
     return check_launch("select_write_kernel");
 }
 
@@ -163,6 +181,121 @@ int launch_label_counts(const int32_t* labels, int64_t N, int32_t K, int64_t* co
     hipLaunchKernelGGL(label_hist_kernel, dim3((unsigned)nb), dim3(256), 0, st, labels, N, per_block, K,
                        reinterpret_cast<unsigned long long*>(counts));
     return check_launch("label_hist_kernel");
+}
+
+// ---- k-means++ seeding of a small row set in one launch ------------------------------------------
+// heat/cluster/batchparallelclustering.py:22-46 on the candidates of k-means|| (a few hundred to a few
+// thousand rows): K - 1 sequential categorical draws with probability proportional to
+// weight * (distance to the closest centre chosen so far).  Issued from the host, every draw is a
+// dozen launches of a few hundred threads; here one workgroup keeps the running distances in
+// registers and does a draw in a few microseconds:
+//   * thread t owns the rows [t R, (t + 1) R), R = ceil(M / 1024) <= SEED_RPT, so thread order is row order;
+//   * the distance of a row to the newest centre is the direct form, summed in feature order and
+//     followed by the correctly rounded square root (p = 2) or sum |x - c| (p = 1): the same numbers
+//     hkm_pairwise_f32 returns for that column;
+//   * weight * distance is formed in fp32, as the host code would, and scanned in fp64 in row order
+//     (sequential inside a thread, shuffle scan across a wave, wave totals through LDS);
+//   * draw k picks the first row whose inclusive prefix exceeds u[k - 1] * total (inverse CDF).  A row
+//     with weight * distance = 0 -- in particular every centre already chosen -- cannot be picked.
+// total <= 0 (every row coincides with a chosen centre, or all weights are zero) has no valid
+// distribution: the remaining entries of idx are set to -1.
+static constexpr int SEED_THREADS = 1024;
+static constexpr int SEED_RPT = HKM_SEED_MAX_ROWS / SEED_THREADS;
+
+template <int P>
+__device__ __forceinline__ float seed_row_dist(const float* __restrict__ x, const float* __restrict__ c, int D) {
+    float acc = 0.f;
+    for (int f = 0; f < D; ++f) {
+        const float df = x[f] - c[f];
+        acc = P == 1 ? acc + fabsf(df) : fmaf(df, df, acc);
+    }
+    return P == 1 ? acc : sqrtf(acc);
+}
+
+template <int P>
+__global__ __launch_bounds__(SEED_THREADS) void seed_plus_plus_kernel(const float* __restrict__ X, int M, int D,
+                                                                      int64_t ldx, const float* __restrict__ w,
+                                                                      int first, const float* __restrict__ u, int K,
+                                                                      long long* __restrict__ idx) {
+    __shared__ double s_wave[SEED_THREADS / 64];
+    __shared__ int s_pick, s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int R = (M + SEED_THREADS - 1) / SEED_THREADS;
+    const int r0 = tid * R;
+    float dist[SEED_RPT], wt[SEED_RPT];
+#pragma unroll
+    for (int r = 0; r < SEED_RPT; ++r) {
+        dist[r] = 0.f;
+        wt[r] = (r < R && r0 + r < M) ? (w ? w[r0 + r] : 1.0f) : 0.f;
+    }
+    int cur = first;
+    if (tid == 0) idx[0] = first;
+    for (int k = 1; k < K; ++k) {
+        // running distance to the closest chosen centre, and this thread's share of the mass
+        const float* c = X + int64_t(cur) * ldx;
+        double mine = 0.0;
+#pragma unroll
+        for (int r = 0; r < SEED_RPT; ++r)
+            if (r < R && r0 + r < M) {
+                const float d = seed_row_dist<P>(X + int64_t(r0 + r) * ldx, c, D);
+                dist[r] = k == 1 ? d : fminf(dist[r], d);
+                mine += double(wt[r] * dist[r]);
+            }
+        // inclusive scan over the threads, in thread (= row) order
+        double incl = mine;
+#pragma unroll
+        for (int s = 1; s < 64; s <<= 1) {
+            const double o = __shfl_up(incl, s);
+            if (lane >= s) incl += o;
+        }
+        if (tid == 0) {
+            s_pick = 0x7fffffff;
+            s_last = -1;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        double before = 0.0, total = 0.0;
+#pragma unroll
+        for (int v = 0; v < SEED_THREADS / 64; ++v) {
+            if (v < wave) before += s_wave[v];
+            total += s_wave[v];
+        }
+        if (!(total > 0.0)) {  // uniform: every thread sees the same total
+            for (int j = k + tid; j < K; j += SEED_THREADS) idx[j] = -1;
+            return;
+        }
+        const double target = double(u[k - 1]) * total;
+        double run = before + (incl - mine);
+        int pick = 0x7fffffff, last = -1;
+#pragma unroll
+        for (int r = 0; r < SEED_RPT; ++r)
+            if (r < R && r0 + r < M) {
+                const float wd = wt[r] * dist[r];
+                run += double(wd);
+                if (wd > 0.f) {
+                    last = r0 + r;
+                    if (run > target && pick == 0x7fffffff) pick = r0 + r;
+                }
+            }
+        if (pick != 0x7fffffff) atomicMin(&s_pick, pick);
+        if (last >= 0) atomicMax(&s_last, last);
+        __syncthreads();
+        // rounding may leave the last prefix a hair below u * total: the last row with mass then
+        cur = s_pick != 0x7fffffff ? s_pick : s_last;
+        if (tid == 0) idx[k] = cur;
+        __syncthreads();  // s_pick / s_last are reset at the top of the next draw
+    }
+}
+
+int launch_seed_plus_plus(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
+                          const float* u, int32_t K, int32_t p, int64_t* idx, hipStream_t st) {
+    if (p == 1)
+        hipLaunchKernelGGL(seed_plus_plus_kernel<1>, dim3(1), dim3(SEED_THREADS), 0, st, X, M, D, ldx, w, first, u, K,
+                           reinterpret_cast<long long*>(idx));
+    else
+        hipLaunchKernelGGL(seed_plus_plus_kernel<2>, dim3(1), dim3(SEED_THREADS), 0, st, X, M, D, ldx, w, first, u, K,
+                           reinterpret_cast<long long*>(idx));
+    return check_launch("seed_plus_plus_kernel");
 }
 
 }  // namespace hkm

@@ -162,6 +162,23 @@ int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* c
                          void* hip_stream);
 
 /*
+ * k-means++ seeding of a small row set in one launch: the reclustering of the k-means|| candidates
+ * (heat/cluster/_kcluster.py:216-225 -> heat/cluster/batchparallelclustering.py:22-46).
+ *   idx[0] = first;  for k = 1 .. K-1:  dist_i = min over the chosen rows of the p-norm distance
+ *   (p = 2: sqrt(sum (x_i - c)^2), p = 1: sum |x_i - c|), mass_i = w_i * dist_i in fp32 (w = NULL: 1),
+ *   idx[k] = the first row whose inclusive prefix sum of the mass (fp64, row order) exceeds
+ *   u[k-1] * total, u[k-1] in [0, 1).
+ * The reference draws with torch.multinomial from torch's unseeded global generator, which cannot be
+ * reproduced; the inverse-CDF draw from caller-supplied uniform numbers is the same distribution.
+ * A row without mass (every chosen row) is never drawn.  If the total mass is not positive the
+ * remaining entries of idx are set to -1 (torch.multinomial raises there).
+ * 1 <= M <= HKM_SEED_MAX_ROWS, 0 <= first < M, K >= 1, p in {1, 2}; X, w, u, idx are device pointers.
+ */
+#define HKM_SEED_MAX_ROWS 16384
+int hkm_seed_plus_plus_f32(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
+                           const float* u, int32_t K, int32_t p, int64_t* idx, void* hip_stream);
+
+/*
  * Manhattan-metric siblings for k-medians / k-medoids (heat/cluster/kmedians.py:60-106,
  * heat/cluster/kmedoids.py:57-115, heat/cluster/batchparallelclustering.py:49-97 with p = 1).
  *

@@ -45,6 +45,9 @@ Pins (what each function is checked against, see tests/test_oracle_pins.py):
   rule and the allclose stop of ``_kmex``, and recovery of well-separated blobs.  **Parity unpinned**
   for the random draws themselves: the reference takes them from Heat's counter-based generator and
   from torch's unseeded global generator, and stores no seeded result anywhere.
+* InverseCdfSampler (categorical draw of the one-launch k-means++ seeding as the inverse CDF of a
+  given uniform number): a hand-made case (weights 1, 0, 2, 1 and u on both sides of every boundary),
+  zero-weight entries are never drawn, and the frequencies of 20 000 draws against the weights.
 * manhattan / assign_l1 / heat_median_axis0 / update_medians / kmedians_fit / kmedoids_fit: the
   known answers of ``tests/spatial/test_distances.py:20-23,42-48,67-73`` (ones vs zeros, D=4 -> 4.0;
   X vs X -> 0), scipy's cityblock distances, ``numpy.median`` and a python sort, hand-made cases for
@@ -506,6 +509,30 @@ def centroid_sampling_helper(x: torch.Tensor, centroids: torch.Tensor, oversampl
         idx = torch.where(sample <= prob)[0]
         centroids = torch.cat((centroids, x[idx].reshape(-1, x.shape[1])), dim=0)
     return centroids
+
+
+class InverseCdfSampler:
+    """Sampler for :func:`initialize_plus_plus` whose categorical draw is the inverse CDF of one given
+    uniform number per draw: the first index whose inclusive prefix sum (float64) of the weights
+    exceeds u * total.  ``picks`` records the drawn indices, ``prefixes`` (prefix sums, u * total) of
+    every draw so a test can tell a rounding tie from a wrong pick."""
+
+    def __init__(self, first: int, u: torch.Tensor):
+        self.first, self.u, self.k = int(first), u.double().cpu(), 0
+        self.picks, self.prefixes = [], []
+
+    def randint(self, high: int) -> int:
+        return self.first
+
+    def multinomial(self, weights: torch.Tensor) -> int:
+        cum = torch.cumsum(weights.double(), 0)
+        target = float(self.u[self.k]) * float(cum[-1])
+        self.k += 1
+        hit = torch.nonzero((cum > target) & (weights > 0))
+        i = int(hit[0]) if hit.numel() else int(torch.nonzero(weights > 0)[-1])
+        self.picks.append(i)
+        self.prefixes.append((cum, target))
+        return i
 
 
 def initialize_plus_plus(x: torch.Tensor, n_clusters: int, sampler, weights=1.0, p: int = 2) -> torch.Tensor:

@@ -13,6 +13,7 @@ import torch
 import heat_amd as ht
 from heat_amd import _native
 from heat_amd.cluster import batchparallelclustering as bpc
+from heat_amd.cluster._sampling import DeviceSampler
 from heat_amd.utils import synthetic
 from oracle import heat_oracle as orc
 
@@ -213,3 +214,54 @@ def test_batchparallel_matches_oracle_and_errors(cuda):
         bp.predict(ht.array(torch.randn(4, 10, device=cuda), split=1))
     with pytest.raises(ValueError):
         bp.predict(ht.array(torch.randn(10, 3, device=cuda), split=0))
+
+
+@pytest.mark.parametrize("m,d,k,p,weighted", [(440, 32, 256, 2, True), (7, 5, 6, 2, False), (5000, 6, 40, 1, True),
+                                              (16384, 3, 64, 2, False), (1025, 9, 30, 1, False)])
+def test_one_launch_plus_plus_seeding(cuda, m, d, k, p, weighted):
+    """hkm_seed_plus_plus_f32 against the reference's op sequence with the inverse-CDF draw, step by
+    step along the kernel's own picks: the drawn row is the first whose inclusive prefix of
+    weight * distance exceeds u * total (up to 1e-5 of the total around a boundary), it has mass, and
+    all but a handful of picks equal the oracle's exactly."""
+    g = torch.Generator().manual_seed(m + 3 * k + p)
+    x = torch.randn((m, d), generator=g) * 3
+    x[m // 2] = x[0]  # a duplicated row: no mass once its twin is chosen
+    w = torch.rand(m, generator=g) + 0.25 if weighted else None
+    u = torch.rand(k - 1, generator=g)
+    first = int(torch.randint(0, m, (1,), generator=g))
+    idx = torch.full((k,), -5, dtype=torch.int64, device=cuda)
+    _native.seed_plus_plus(x.to(cuda), None if w is None else w.to(cuda), first, u.to(cuda), k, p, idx)
+    got = idx.cpu()
+    assert int(got[0]) == first and int(got.min()) >= 0 and int(got.max()) < m
+    assert len(set(got.tolist())) == k, "a chosen row has no mass and cannot be drawn again"
+    ws = torch.ones(m) if w is None else w
+    exact = 0
+    for j in range(1, k):
+        dist = torch.cdist(x, x[got[:j]], p=float(p), compute_mode="donot_use_mm_for_euclid_dist").min(dim=1)[0]
+        mass = ws * dist
+        s = orc.InverseCdfSampler(first, u[j - 1 : j])
+        want = s.multinomial(mass)
+        cum, target = s.prefixes[0]
+        i = int(got[j])
+        tol = 1e-5 * float(cum[-1])
+        assert float(mass[i]) > 0
+        assert float(cum[i]) > target - tol and float(cum[i] - mass[i].double()) <= target + tol, (j, i, want)
+        exact += int(i == want)
+    assert exact >= (k - 1) - max(1, (k - 1) // 100)
+
+
+def test_one_launch_plus_plus_seeding_without_mass(cuda):
+    # three distinct rows, five centres wanted: after three draws no row has mass left
+    x = torch.tensor([[0.0, 0.0], [1.0, 0.0], [0.0, 2.0]]).repeat(4, 1).to(cuda)
+    u = torch.full((4,), 0.5, device=cuda)
+    idx = torch.full((5,), -5, dtype=torch.int64, device=cuda)
+    _native.seed_plus_plus(x, None, 1, u, 5, 2, idx)
+    got = idx.cpu().tolist()
+    assert got[0] == 1 and got[3:] == [-1, -1] and len({tuple(x[i].tolist()) for i in got[:3]}) == 3
+    with pytest.raises(RuntimeError, match="invalid multinomial distribution"):
+        bpc._initialize_plus_plus(x, 5, 2, DeviceSampler(cuda, 0))
+    # through the estimator-side helper: K distinct rows, reproducible for a seed
+    xb, _ = _blobs(3000, 4, 6, seed=2)
+    a = bpc._initialize_plus_plus(xb.to(cuda), 6, 2, DeviceSampler(cuda, 11))
+    b = bpc._initialize_plus_plus(xb.to(cuda), 6, 2, DeviceSampler(cuda, 11))
+    assert torch.equal(a, b) and a.shape == (6, 4) and len({tuple(r.tolist()) for r in a.cpu()}) == 6

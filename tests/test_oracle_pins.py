@@ -411,3 +411,18 @@ def test_kmedians_and_kmedoids_closed_forms():
     far = torch.cat([x2[[0, 301]], torch.full((1, 4), 1e4)])
     c, _ = orc.kmex(x2, 3, far.clone(), 20, 1e-4, p=1)
     assert torch.equal(c[2], far[2]) and torch.equal(c[0], torch.median(x, dim=0)[0])
+
+
+def test_inverse_cdf_sampler_draws_the_given_distribution():
+    w = torch.tensor([1.0, 0.0, 2.0, 1.0])
+    # boundaries of the inclusive prefix (1, 1, 3, 4) / 4: u < 0.25 -> 0, 0.25 <= u < 0.75 -> 2, above -> 3
+    for u, want in ((0.0, 0), (0.2499, 0), (0.25, 2), (0.5, 2), (0.7499, 2), (0.75, 3), (0.999999, 3)):
+        assert orc.InverseCdfSampler(0, torch.tensor([u])).multinomial(w) == want
+    g = torch.Generator().manual_seed(5)
+    us = torch.rand(20000, generator=g)
+    s = orc.InverseCdfSampler(0, us)
+    picks = torch.tensor([s.multinomial(w) for _ in range(20000)])
+    freq = torch.bincount(picks, minlength=4).double() / 20000
+    assert freq[1] == 0
+    assert torch.allclose(freq, (w / w.sum()).double(), atol=0.012)
+    assert s.randint(99) == 0
