@@ -11,7 +11,10 @@
 // arithmetic in the loop) and staged through double-buffered LDS (row stride 36 floats keeps the
 // 16-byte operand reads conflict-free).  The squared norms are accumulated by the staging threads
 // from the registers they stage.  The epilogue follows the reference's order: (|x|^2 + |y|^2) first,
-// then - 2 x.y, clamp at 0 (NaN passes through), then sqrt / exp.
+// then - 2 x.y, clamp at 0 (NaN passes through), then sqrt / exp.  Every vector instruction of the
+// epilogue takes issue time from the fp32 matrix pipe, so it is kept short: one compare + select for
+// the clamp, and the square root in its short correctly rounded form (sqrt_rn_short) unless a wave
+// holds a positive value below that form's range.
 #include "hkm_common.h"
 
 namespace hkm {

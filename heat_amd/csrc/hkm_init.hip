@@ -1,8 +1,9 @@
 // Device side of the k-means|| centroid initialisation (heat/cluster/_kcluster.py:146-247,283-350):
 // the distance work is the assign kernel with its min d^2 output; what is left are an ordered
-// Bernoulli selection of candidate rows and a histogram of labels.  Both are integer work and
-// reproducible: the selection is a count / scan / write compaction in row order, the histogram
-// uses integer atomics only.
+// Bernoulli selection of candidate rows, a histogram of labels and the k-means++ seeding of the
+// candidates.  The first two are integer work and reproducible: the selection is a count / scan /
+// write compaction in row order, the histogram uses integer atomics only; the seeding runs in one
+// workgroup with a fixed order of every sum.
 #include "hkm_common.h"
 
 namespace hkm {
