@@ -40,6 +40,7 @@ SIGNATURES = {
     "hkm_pairwise_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
                                         c_void_p, c_int64, c_int32, ctypes.c_float, c_void_p]),
     "hkm_min_dist_sum_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_min_merge_sum_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_sample_select_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int64, c_void_p, ctypes.c_float, c_void_p,
                                              c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_label_counts_i64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
@@ -284,6 +285,16 @@ def min_dist_sum(min_d2: torch.Tensor, out: torch.Tensor, ws: Workspace) -> None
     n = min_d2.numel()
     buf = ws.get(workspace_bytes(n, 1, 1, WS_ASSIGN))
     check(load().hkm_min_dist_sum_f32(_ptr(min_d2), n, _ptr(out), _ptr(buf), buf.numel(), _stream()))
+
+
+def min_merge_sum(min_d2: torch.Tensor, new_d2: torch.Tensor, out: torch.Tensor, ws: Workspace) -> None:
+    """min_d2 = min(min_d2, new_d2) in place and out = sum(sqrt(min_d2)) of the result, one pass."""
+    _require_gpu(min_d2, new_d2, out)
+    if min_d2.numel() != new_d2.numel() or min_d2.dtype != torch.float32 or new_d2.dtype != torch.float32:
+        raise ValueError("min_d2 and new_d2 must be float32 vectors of one length")
+    buf = ws.get(workspace_bytes(min_d2.numel(), 1, 1, WS_ASSIGN))
+    check(load().hkm_min_merge_sum_f32(_ptr(min_d2), _ptr(new_d2), min_d2.numel(), _ptr(out), _ptr(buf),
+                                       buf.numel(), _stream()))
 
 
 def sample_select(min_d2: torch.Tensor, u: torch.Tensor, cost: torch.Tensor, oversampling: float,

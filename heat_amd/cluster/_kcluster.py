@@ -185,8 +185,9 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         closest of the candidates passed in (it is overwritten).  The reference recomputes the distances to ALL
         candidates in every round; the minimum over a grown set is the minimum of the old minimum and
         the distances to the new members, so a round here costs one fused distance+argmin launch
-        against the handful of NEW candidates, one elementwise minimum, one reduction and one ordered
-        selection; only the number of new candidates comes back to the host.
+        against the handful of NEW candidates, one pass that merges the minimum and sums the next
+        round's cost, and one ordered selection; only the number of new candidates comes back to the
+        host.
         """
         n = xt.shape[0]
         dev = xt.device
@@ -198,9 +199,10 @@ class _KCluster(ClusteringMixin, BaseEstimator):
         cost = torch.empty((), dtype=torch.float32, device=dev)
         count = torch.zeros((), dtype=torch.int64, device=dev)
         idx = torch.empty((max(1024, int(16 * oversampling)),), dtype=torch.int64, device=dev)
+        f32 = dmin.dtype == torch.float32
+        _native.min_dist_sum(dmin if f32 else dmin.float(), cost, ws)
         for it in range(num_iters):
-            d2 = dmin if dmin.dtype == torch.float32 else dmin.float()  # the draw itself runs in float32
-            _native.min_dist_sum(d2, cost, ws)
+            d2 = dmin if f32 else dmin.float()  # the draw itself runs in float32
             u = sampler.uniform(n)
             _native.sample_select(d2, u, cost, oversampling, idx, count, ws)
             c = int(count.item())
@@ -213,7 +215,11 @@ class _KCluster(ClusteringMixin, BaseEstimator):
             centroids = torch.cat((centroids, fresh), dim=0)
             if it + 1 < num_iters:
                 _native.assign(xt, fresh, lab, dnew, ws)
-                torch.minimum(dmin, dnew, out=dmin)
+                if f32:
+                    _native.min_merge_sum(dmin, dnew, cost, ws)  # running minimum and the next round's cost
+                else:
+                    torch.minimum(dmin, dnew, out=dmin)
+                    _native.min_dist_sum(dmin.float(), cost, ws)
         return centroids
 
     def _kmeans_parallel(self, x: DNDarray, oversampling: float, iter_multiplier: float) -> torch.Tensor:

@@ -350,6 +350,18 @@ int hkm_min_dist_sum_f32(const float* min_d2, int64_t N, float* out, void* ws, s
     return launch_sum_min_d2(min_d2, N, out, w.red, 3, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_min_merge_sum_f32(float* min_d2, const float* new_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
+                          void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
+    if (((!min_d2 || !new_d2) && N > 0) || !out) return fail(HKM_EINVAL, "NULL pointer argument");
+    const size_t need = carve(nullptr, N, 1, 1, HKM_WS_ASSIGN).total;
+    int rc = check_ws(ws, ws_bytes, need);
+    if (rc) return rc;
+    const Workspace w = carve(ws, N, 1, 1, HKM_WS_ASSIGN);
+    return launch_min_merge_sum(min_d2, new_d2, N, out, w.red, static_cast<hipStream_t>(hip_stream));
+}
+
 int hkm_sample_select_f32(const float* min_d2, const float* u, int64_t N, const float* cost,
                           float oversampling, int64_t* idx, int64_t cap, int64_t* count, void* ws,
                           size_t ws_bytes, void* hip_stream) {

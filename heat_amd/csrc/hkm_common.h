@@ -184,6 +184,7 @@ int launch_shift(const float* C_old, const float* C_new, int32_t K, int32_t D, f
                  hipStream_t st);
 int launch_sum_min_d2(const float* min_d2, int64_t N, float* out, double* red, int mode,
                       hipStream_t st);
+int launch_min_merge_sum(float* dmin, const float* dnew, int64_t N, float* out, double* red, hipStream_t st);
 bool split_eligible(int32_t D, int32_t K, bool fused);
 int split_fused_grid(int64_t N);
 int launch_split_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,

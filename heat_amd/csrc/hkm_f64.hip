@@ -127,8 +127,82 @@ __global__ __launch_bounds__(256) void assign_f64_kernel(const double* __restric
     }
 }
 
+// Narrow rows and few centroids (D <= 8, K (D + 1) <= F64S_LDS): the 64 x 64 tile would be mostly
+// padding.  One point per lane, the centroids and their squared norms broadcast from LDS; every sum
+// in feature order with fma, so the values equal those of the tiled kernel bit for bit.
+static constexpr int F64S_THREADS = 256;
+static constexpr int F64S_LDS = 2048;  // doubles: K rows of D coordinates + the squared norm
+
+template <int D>
+__global__ __launch_bounds__(F64S_THREADS) void assign_f64_small_kernel(
+    const double* __restrict__ X, int64_t N, int64_t ldx, const double* __restrict__ C, int K, int64_t ldc,
+    int32_t* __restrict__ labels, double* __restrict__ min_d2, int64_t nbatches) {
+    __shared__ double sC[F64S_LDS];
+    const int tid = threadIdx.x;
+    for (int k = tid; k < K; k += F64S_THREADS) {
+        const double* row = C + int64_t(k) * ldc;
+        double s = 0.0;
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            sC[k * (D + 1) + d] = row[d];
+            s = fma(row[d], row[d], s);
+        }
+        sC[k * (D + 1) + D] = s;
+    }
+    __syncthreads();
+    for (int64_t b = blockIdx.x; b < nbatches; b += gridDim.x) {
+        const int64_t i = b * F64S_THREADS + tid;
+        const double* xp = X + (i < N ? i : N - 1) * ldx;
+        double x[D], xn = 0.0;
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            x[d] = xp[d];
+            xn = fma(x[d], x[d], xn);
+        }
+        double m = __builtin_inf();
+        int mi = 0x7fffffff;
+#pragma unroll 4
+        for (int k = 0; k < K; ++k) {
+            const double* c = sC + k * (D + 1);
+            double dot = 0.0;
+#pragma unroll
+            for (int d = 0; d < D; ++d) dot = fma(x[d], c[d], dot);
+            double v = fma(-2.0, dot, xn + c[D]);
+            v = v > 0.0 ? v : (v != v ? v : 0.0);
+            if (v < m) {  // ascending index, strict '<': first index wins ties
+                m = v;
+                mi = k;
+            }
+        }
+        if (i < N) {
+            labels[i] = mi == 0x7fffffff ? 0 : mi;
+            if (min_d2) min_d2[i] = m;
+        }
+    }
+}
+
+template <int D>
+static int launch_assign_f64_small_t(const double* X, int64_t N, int64_t ldx, const double* C, int32_t K,
+                                     int64_t ldc, int32_t* labels, double* min_d2, hipStream_t st) {
+    const int64_t nbatches = (N + F64S_THREADS - 1) / F64S_THREADS;
+    int64_t grid = int64_t(num_cus()) * 8;
+    if (grid > nbatches) grid = nbatches;
+    hipLaunchKernelGGL(assign_f64_small_kernel<D>, dim3((unsigned)grid), dim3(F64S_THREADS), 0, st, X, N, ldx, C, K,
+                       ldc, labels, min_d2, nbatches);
+    return check_launch("assign_f64_small_kernel");
+}
+
 int launch_assign_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, int32_t K,
                       int64_t ldc, int32_t* labels, double* min_d2, hipStream_t st) {
+    if (D <= 8 && int64_t(K) * (D + 1) <= F64S_LDS) {
+#define HKM_CASE(d) \
+    case d:         \
+        return launch_assign_f64_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, st);
+        switch (D) {
+            HKM_CASE(1) HKM_CASE(2) HKM_CASE(3) HKM_CASE(4) HKM_CASE(5) HKM_CASE(6) HKM_CASE(7) HKM_CASE(8)
+        }
+#undef HKM_CASE
+    }
     const int64_t tiles = (N + F64_T - 1) / F64_T;
     if (tiles > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "assign_f64: too many row tiles");
     hipLaunchKernelGGL(assign_f64_kernel, dim3((unsigned)tiles), dim3(256), 0, st, X, N, ldx, C, K, ldc, D,

@@ -444,6 +444,66 @@ static int launch_sum_t(const T* v, int64_t N, T* out, double* red, int mode, hi
     return check_launch("sum_final_kernel");
 }
 
+// dmin[i] = min(dmin[i], dnew[i]) and the partial sums of sqrt(dmin[i]) in one pass: the running minimum
+// of a k-means|| round merged with the cost of the next one.  Same blocking and order as
+// sum_partial_kernel, so the sum equals hkm_min_dist_sum_f32 of the merged array bit for bit.
+template <bool VEC>
+__global__ __launch_bounds__(256) void min_merge_partial_kernel(float* __restrict__ dmin, const float* __restrict__ dnew,
+                                                                int64_t n, int64_t per_block,
+                                                                double* __restrict__ red) {
+    __shared__ double sh[256];
+    const int64_t b0 = int64_t(blockIdx.x) * per_block;
+    const int64_t b1 = min(n, b0 + per_block);
+    double acc = 0.0;
+    int64_t i0 = b0;
+    if (VEC) {
+        double a[4] = {0.0, 0.0, 0.0, 0.0};
+        for (; i0 + 4096 <= b1; i0 += 4096) {
+            float4 q[4], r[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                q[t] = *reinterpret_cast<const float4*>(dmin + i0 + t * 1024 + threadIdx.x * 4);
+                r[t] = *reinterpret_cast<const float4*>(dnew + i0 + t * 1024 + threadIdx.x * 4);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                q[t].x = fminf(q[t].x, r[t].x);
+                q[t].y = fminf(q[t].y, r[t].y);
+                q[t].z = fminf(q[t].z, r[t].z);
+                q[t].w = fminf(q[t].w, r[t].w);
+                *reinterpret_cast<float4*>(dmin + i0 + t * 1024 + threadIdx.x * 4) = q[t];
+                a[t] += ((sum_term<float>(q[t].x, 3) + sum_term<float>(q[t].y, 3)) +
+                         (sum_term<float>(q[t].z, 3) + sum_term<float>(q[t].w, 3)));
+            }
+        }
+        acc = (a[0] + a[1]) + (a[2] + a[3]);
+    }
+    for (int64_t i = i0 + threadIdx.x; i < b1; i += 256) {
+        const float m = fminf(dmin[i], dnew[i]);
+        dmin[i] = m;
+        acc += sum_term<float>(m, 3);
+    }
+    const double t = block_sum_fixed(acc, sh);
+    if (threadIdx.x == 0) red[blockIdx.x] = t;
+}
+
+int launch_min_merge_sum(float* dmin, const float* dnew, int64_t N, float* out, double* red, hipStream_t st) {
+    int nb = int((N + 16383) / 16384);
+    if (nb < 1) nb = 1;
+    if (nb > RED_SLOTS) nb = RED_SLOTS;
+    const int64_t per_block = ((N + nb - 1) / nb + 4095) / 4096 * 4096;
+    nb = int((N + per_block - 1) / per_block);
+    if (nb < 1) nb = 1;
+    if (aligned16(dmin) && aligned16(dnew))
+        hipLaunchKernelGGL(min_merge_partial_kernel<true>, dim3(nb), dim3(256), 0, st, dmin, dnew, N, per_block, red);
+    else
+        hipLaunchKernelGGL(min_merge_partial_kernel<false>, dim3(nb), dim3(256), 0, st, dmin, dnew, N, per_block, red);
+    int rc = check_launch("min_merge_partial_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(sum_final_kernel<float>, dim3(1), dim3(256), 0, st, static_cast<const double*>(red), nb, 3, out);
+    return check_launch("sum_final_kernel");
+}
+
 int launch_sum_min_d2(const float* v, int64_t N, float* out, double* red, int mode, hipStream_t st) {
     return launch_sum_t<float>(v, N, out, red, mode, st);
 }

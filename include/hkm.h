@@ -145,6 +145,11 @@ int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int
  * hkm_min_dist_sum_f32: *out = sum_i sqrt(min_d2[i]) (fp64 accumulation, fixed order): the
  *   clustering cost `distance.min(axis=1).sum()` of _kcluster.py:163-170 and :312-316.
  *   ws as for hkm_functional_value_f32.
+ * hkm_min_merge_sum_f32: min_d2[i] = min(min_d2[i], new_d2[i]) in place and *out = sum_i
+ *   sqrt(min_d2[i]) of the merged array (the same sum hkm_min_dist_sum_f32 returns for it).  The
+ *   reference recomputes the distances to ALL candidates in every round (_kcluster.py:312-313); the
+ *   minimum over the grown candidate set is the minimum of the previous one and the distances to the
+ *   round's new candidates, which is what this merges.  ws as for hkm_functional_value_f32.
  * hkm_sample_select_f32: row i is a candidate iff u[i] <= (oversampling * sqrt(min_d2[i])) /
  *   max(*cost, 1e-12) in fp32 (_kcluster.py:314-322: `where(sample <= prob)`); the selected row
  *   indices are written to idx in ascending order (at most cap of them) and their number, which may
@@ -155,6 +160,8 @@ int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int
  */
 int hkm_min_dist_sum_f32(const float* min_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
                          void* hip_stream);
+int hkm_min_merge_sum_f32(float* min_d2, const float* new_d2, int64_t N, float* out, void* ws, size_t ws_bytes,
+                          void* hip_stream);
 int hkm_sample_select_f32(const float* min_d2, const float* u, int64_t N, const float* cost,
                           float oversampling, int64_t* idx, int64_t cap, int64_t* count, void* ws,
                           size_t ws_bytes, void* hip_stream);

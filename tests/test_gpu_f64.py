@@ -24,7 +24,7 @@ def _data(n, d, k, seed, spread=3.0):
 
 
 @pytest.mark.parametrize("n,d,k", [(1, 3, 8), (3000, 3, 8), (5000, 32, 256), (999, 17, 1), (1300, 50, 37),
-                                   (700, 130, 70), (2000, 64, 1030)])
+                                   (700, 130, 70), (2000, 64, 1030), (70000, 8, 200), (5000, 8, 300), (4097, 1, 5)])
 def test_assign_and_update_f64(cuda, n, d, k):
     print(f"f64 n={n} d={d} k={k}", flush=True)
     x, c = _data(n, d, k, seed=n + d + k)

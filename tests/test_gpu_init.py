@@ -265,3 +265,26 @@ def test_one_launch_plus_plus_seeding_without_mass(cuda):
     a = bpc._initialize_plus_plus(xb.to(cuda), 6, 2, DeviceSampler(cuda, 11))
     b = bpc._initialize_plus_plus(xb.to(cuda), 6, 2, DeviceSampler(cuda, 11))
     assert torch.equal(a, b) and a.shape == (6, 4) and len({tuple(r.tolist()) for r in a.cpu()}) == 6
+
+
+@pytest.mark.parametrize("n", [1, 255, 4096, 50_001, 3_000_017])
+def test_min_merge_sum(cuda, n):
+    """min_d2 = min(min_d2, new_d2) in place, and the cost of the merged array equal to what
+    hkm_min_dist_sum_f32 returns for it -- bit for bit -- and to the float64 sum of square roots."""
+    g = torch.Generator().manual_seed(n)
+    a = (torch.rand(n, generator=g) * 50.0)
+    b = (torch.rand(n, generator=g) * 50.0)
+    a[::7] = 0.0
+    ws = _native.Workspace(cuda)
+    for off in (0, 1):  # 16-byte aligned and not
+        ag = torch.empty((n + 1,), device=cuda)[off:off + n].copy_(a)
+        bg = torch.empty((n + 1,), device=cuda)[off:off + n].copy_(b)
+        cost = torch.empty((), device=cuda)
+        _native.min_merge_sum(ag, bg, cost, ws)
+        want = torch.minimum(a, b)
+        assert torch.equal(ag.cpu(), want)
+        again = torch.empty((), device=cuda)
+        _native.min_dist_sum(ag, again, ws)
+        assert float(cost) == float(again)
+        ref = float(want.double().sqrt().sum())
+        assert abs(float(cost) - ref) <= 2e-7 * ref + 1e-30
