@@ -330,7 +330,7 @@ int hkm_functional_value_f32(const float* min_d2, int64_t N, float* out, void* w
                              void* hip_stream) {
     g_err[0] = 0;
     if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
-    if (!min_d2 || !out) return fail(HKM_EINVAL, "NULL pointer argument");
+    if ((!min_d2 && N > 0) || !out) return fail(HKM_EINVAL, "NULL pointer argument");
     const size_t need = carve(nullptr, N, 1, 1, HKM_WS_ASSIGN).total;
     int rc = check_ws(ws, ws_bytes, need);
     if (rc) return rc;

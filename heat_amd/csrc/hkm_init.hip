@@ -118,7 +118,7 @@ int launch_select(const float* d2, const float* u, int64_t N, const float* cost,
     int nb = int((N + 2047) / 2048);
     if (nb < 1) nb = 1;
     if (nb > RED_SLOTS) nb = RED_SLOTS;
-    int64_t per_block = (N + nb - 1) / nb;
+    int64_t per_block = N > 0 ? (N + nb - 1) / nb : 1;
     per_block = (per_block + 1023) / 1024 * 1024;
     nb = int((N + per_block - 1) / per_block);
     if (nb < 1) nb = 1;

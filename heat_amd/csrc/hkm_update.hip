@@ -430,7 +430,7 @@ static int launch_sum_t(const T* v, int64_t N, T* out, double* red, int mode, hi
     int nb = int((N + 16383) / 16384);
     if (nb < 1) nb = 1;
     if (nb > RED_SLOTS) nb = RED_SLOTS;
-    const int64_t per_block = ((N + nb - 1) / nb + 4095) / 4096 * 4096;
+    const int64_t per_block = ((N > 0 ? (N + nb - 1) / nb : 1) + 4095) / 4096 * 4096;
     nb = int((N + per_block - 1) / per_block);
     if (nb < 1) nb = 1;
     if (sizeof(T) == 4 && aligned16(v))
@@ -491,7 +491,7 @@ int launch_min_merge_sum(float* dmin, const float* dnew, int64_t N, float* out, 
     int nb = int((N + 16383) / 16384);
     if (nb < 1) nb = 1;
     if (nb > RED_SLOTS) nb = RED_SLOTS;
-    const int64_t per_block = ((N + nb - 1) / nb + 4095) / 4096 * 4096;
+    const int64_t per_block = ((N > 0 ? (N + nb - 1) / nb : 1) + 4095) / 4096 * 4096;
     nb = int((N + per_block - 1) / per_block);
     if (nb < 1) nb = 1;
     if (aligned16(dmin) && aligned16(dnew))

@@ -392,3 +392,19 @@ def test_widen_and_empty_inputs(cuda):
     c_new = torch.full((4, 8), 9.0, device=cuda)
     _native.update(x, torch.empty((0,), dtype=torch.int32, device=cuda), c_new, None, _native.Workspace(cuda))
     assert torch.all(c_new == 0)
+    # the reductions and the selection of the initialiser on empty vectors: sums 0, nothing selected
+    ws = _native.Workspace(cuda)
+    e = torch.empty((0,), device=cuda)
+    s = torch.full((), 7.0, device=cuda)
+    _native.min_dist_sum(e, s, ws)
+    assert float(s) == 0.0
+    s.fill_(7.0)
+    _native.min_merge_sum(e, e.clone(), s, ws)
+    assert float(s) == 0.0
+    s.fill_(7.0)
+    _native.functional_value(e, s, ws)
+    assert float(s) == 0.0
+    cnt = torch.full((), 5, dtype=torch.int64, device=cuda)
+    idx = torch.empty((4,), dtype=torch.int64, device=cuda)
+    _native.sample_select(e, e.clone(), torch.ones((), device=cuda), 2.0, idx, cnt, ws)
+    assert int(cnt) == 0
