@@ -174,7 +174,8 @@ __global__ __launch_bounds__(256) void srt_segsum_kernel(const T* __restrict__ X
                                                          const int64_t* __restrict__ offsets,
                                                          const int32_t* __restrict__ chunk_start, int K,
                                                          T* __restrict__ part, int DPAD) {
-    __shared__ T red[8][33];
+    __shared__ double red[8][33];  // fp64 inside a chunk: the pass is bound by its loads, and 256 fp32
+                                    // additions per lane would cost two decimal digits of the mean
     const int chunk = blockIdx.x;
     if (chunk >= chunk_start[K]) return;
     const int k = srt_find_cluster(chunk_start, K, chunk);
@@ -185,23 +186,23 @@ __global__ __launch_bounds__(256) void srt_segsum_kernel(const T* __restrict__ X
     const bool ok = d < D;
     const T* xc = X + (ok ? d : 0);
     constexpr int U = 8;
-    T acc = T(0);
+    double acc = 0.0;
     int64_t r = r0 + rl;
     for (; r + 8 * (U - 1) < r1; r += 8 * U) {
         T v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = xc[int64_t(perm[r + 8 * u]) * ldx];
 #pragma unroll
-        for (int u = 0; u < U; ++u) acc += v[u];
+        for (int u = 0; u < U; ++u) acc += double(v[u]);
     }
-    for (; r < r1; r += 8) acc += xc[int64_t(perm[r]) * ldx];
-    red[rl][col] = ok ? acc : T(0);
+    for (; r < r1; r += 8) acc += double(xc[int64_t(perm[r]) * ldx]);
+    red[rl][col] = ok ? acc : 0.0;
     __syncthreads();
     if (rl == 0) {
-        T s = red[0][col];
+        double s = red[0][col];
 #pragma unroll
         for (int q = 1; q < 8; ++q) s += red[q][col];
-        part[int64_t(chunk) * DPAD + blockIdx.y * 32 + col] = s;
+        part[int64_t(chunk) * DPAD + blockIdx.y * 32 + col] = T(s);
     }
 }
 
