@@ -28,8 +28,14 @@ def _d2_f64(x, c):
     return ((xd * xd).sum(1, keepdim=True) + (cd * cd).sum(1)[None] - 2 * xd @ cd.T).clamp_min(0), xd, cd
 
 
+@pytest.mark.parametrize("products", ["fp32", "bf16x3"])
 @pytest.mark.parametrize("seed", [1, 2, 3])
-def test_kmeans_entry_points_on_random_shapes(cuda, seed):
+def test_kmeans_entry_points_on_random_shapes(cuda, seed, products, monkeypatch):
+    # bf16x3: the opt-in split-product kernels (read from the environment on every call), same bars
+    if products == "bf16x3":
+        monkeypatch.setenv("HKM_PRODUCTS", "bf16x3")
+    else:
+        monkeypatch.delenv("HKM_PRODUCTS", raising=False)
     rng = random.Random(seed)
     ws = _native.Workspace(cuda)
     for case in range(40):
