@@ -10,7 +10,9 @@
 //      does not depend on scheduling.
 //   2. segmented sums: a workgroup takes up to 2048 consecutive entries of one cluster's segment and a
 //      32-column slice; its 8 row-lanes add rows r, r+8, ... in order (several independent loads in
-//      flight, no LDS traffic, no atomics) and are combined in lane order.
+//      flight, no LDS traffic, no atomics) and are combined in lane order -- all in fp64, like the
+//      reference's float64 x * selection: the sum of a cluster is rounded once, when the mean is
+//      stored, so the means equal the reference's bit for bit except where its own fp64 sum rounds.
 //   3. finalize: the chunk partials of a cluster are added in chunk order in fp64, divided by the
 //      count (rounded through fp32 like the reference, heat/core/rounding.py:156-164), stored as fp32;
 //      an empty cluster gives a zero row (heat/cluster/kmeans.py:88-101).
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(256) void srt_segsum_kernel(const T* __restrict__ X
                                                          const int32_t* __restrict__ perm,
                                                          const int64_t* __restrict__ offsets,
                                                          const int32_t* __restrict__ chunk_start, int K,
-                                                         T* __restrict__ part, int DPAD) {
+                                                         double* __restrict__ part, int DPAD) {
     __shared__ double red[8][33];  // fp64 inside a chunk: the pass is bound by its loads, and 256 fp32
                                     // additions per lane would cost two decimal digits of the mean
     const int chunk = blockIdx.x;
@@ -202,12 +204,12 @@ __global__ __launch_bounds__(256) void srt_segsum_kernel(const T* __restrict__ X
         double s = red[0][col];
 #pragma unroll
         for (int q = 1; q < 8; ++q) s += red[q][col];
-        part[int64_t(chunk) * DPAD + blockIdx.y * 32 + col] = T(s);
+        part[int64_t(chunk) * DPAD + blockIdx.y * 32 + col] = s;
     }
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void srt_finalize_kernel(const T* __restrict__ part, int DPAD,
+__global__ __launch_bounds__(256) void srt_finalize_kernel(const double* __restrict__ part, int DPAD,
                                                            const int32_t* __restrict__ chunk_start,
                                                            const int64_t* __restrict__ cnts, int K, int D,
                                                            T* __restrict__ C_new, int64_t ldcn,
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(256) void srt_finalize_kernel(const T* __restrict__
     if (ok) {
         const int k = int(i / D), d = int(i - int64_t(k) * D);
         double sum = 0.0;
-        for (int c = chunk_start[k]; c < chunk_start[k + 1]; ++c) sum += double(part[int64_t(c) * DPAD + d]);
+        for (int c = chunk_start[k]; c < chunk_start[k + 1]; ++c) sum += part[int64_t(c) * DPAD + d];
         const int64_t n = cnts[k];
         const double cnt = double(float(n < 1 ? 1 : n));
         const T cnew = T(sum / cnt);
@@ -279,7 +281,7 @@ SortedWorkspace carve_sorted(void* base, int64_t N, int32_t D, int32_t K, int32_
     w.offsets = reinterpret_cast<int64_t*>(take((size_t(K) + 1) * sizeof(int64_t)));
     w.chunk_start = reinterpret_cast<int32_t*>(take((size_t(K) + 1) * sizeof(int32_t)));
     w.perm = reinterpret_cast<int32_t*>(take(size_t(N < 1 ? 1 : N) * sizeof(int32_t)));
-    w.part = take(size_t(max_chunks) * dpad * elem);
+    w.part = take(size_t(max_chunks) * dpad * sizeof(double));  // chunk sums stay in fp64 until the division
     w.shift_part = reinterpret_cast<double*>(take((size_t(K) * D / 256 + 1) * sizeof(double)));
     w.total = off;
     return w;
@@ -305,7 +307,7 @@ static int launch_update_sorted_t(const T* X, int64_t N, int32_t D, int64_t ldx,
                        w.chunk_start);
     if ((rc = check_launch("srt_scan_clusters_kernel"))) return rc;
     const int dpad = (D + 31) / 32 * 32;
-    T* part = reinterpret_cast<T*>(w.part);
+    double* part = reinterpret_cast<double*>(w.part);
     if (N > 0) {
         hipLaunchKernelGGL(srt_scatter_kernel, dim3(gblocks), dim3(256), glds, st, labels, N, K, nbits, blk_rows,
                            nblk, w.blk_cnt, w.offsets, w.perm);
@@ -316,7 +318,7 @@ static int launch_update_sorted_t(const T* X, int64_t N, int32_t D, int64_t ldx,
         if ((rc = check_launch("srt_segsum_kernel"))) return rc;
     }
     const int nb = int((int64_t(K) * D + 255) / 256);
-    hipLaunchKernelGGL(srt_finalize_kernel<T>, dim3(nb), dim3(256), 0, st, static_cast<const T*>(part), dpad,
+    hipLaunchKernelGGL(srt_finalize_kernel<T>, dim3(nb), dim3(256), 0, st, static_cast<const double*>(part), dpad,
                        w.chunk_start, w.counts, K, D, C_new, ldcn, counts, C_old, w.shift_part);
     if ((rc = check_launch("srt_finalize_kernel")) || !C_old) return rc;
     hipLaunchKernelGGL(srt_shift_final_kernel<T>, dim3(1), dim3(256), 0, st,
