@@ -33,6 +33,10 @@ class DeviceSampler:
         """One integer in [0, high)."""
         return int(torch.randint(0, int(high), (1,), generator=self._gen, device=self.device).item())
 
+    def randint_rows(self, high: int, count: int) -> torch.Tensor:
+        """``count`` integers in [0, high) as an int64 vector on the device, without a host round trip."""
+        return torch.randint(0, int(high), (int(count),), generator=self._gen, device=self.device)
+
     def uniform(self, n: int) -> torch.Tensor:
         """n float32 numbers in [0, 1) on the device."""
         return torch.rand((int(n),), generator=self._gen, device=self.device, dtype=torch.float32)
@@ -44,3 +48,12 @@ class DeviceSampler:
     def multinomial_on_device(self, weights: torch.Tensor) -> torch.Tensor:
         """The same draw as :meth:`multinomial`, left on the device as a 0-d int64 tensor."""
         return torch.multinomial(weights, 1, generator=self._gen).reshape(())
+
+
+def draw_rows(sampler, high: int, count: int, device) -> torch.Tensor:
+    """``count`` row indices in [0, high) on ``device``: one vector draw where the sampler offers it
+    (no host round trip), its scalar draws otherwise (test samplers that replay recorded numbers)."""
+    vec = getattr(sampler, "randint_rows", None)
+    if vec is not None:
+        return vec(high, count).to(device=device, dtype=torch.int64)
+    return torch.tensor([sampler.randint(high) for _ in range(count)], dtype=torch.int64, device=device)

@@ -19,7 +19,7 @@ from .. import _native
 from ..core import types
 from ..core.base import BaseEstimator, ClusteringMixin
 from ..core.dndarray import DNDarray
-from ._sampling import DeviceSampler
+from ._sampling import DeviceSampler, draw_rows
 
 
 def _dist_to_row(x: torch.Tensor, row: torch.Tensor, p: int) -> torch.Tensor:
@@ -44,8 +44,7 @@ def _initialize_plus_plus(x: torch.Tensor, n_clusters: int, p: int, sampler, wei
     the same number and needs one N x 1 distance column per step.
     """
     if x.shape[0] > max_samples:
-        sub = torch.tensor([sampler.randint(x.shape[0]) for _ in range(max_samples)], device=x.device)
-        x = x[sub].contiguous()
+        x = x[draw_rows(sampler, x.shape[0], max_samples, x.device)].contiguous()
     if (getattr(sampler, "fused_seeding", False) and x.dtype == torch.float32 and x.shape[0] <= _native.SEED_MAX_ROWS
             and p in (1, 2)):
         # a small row set (the candidates of k-means||): all draws in one launch, from one uniform number each
@@ -92,7 +91,7 @@ def _kmex(x: torch.Tensor, p: int, n_clusters: int, init: Union[str, torch.Tenso
     elif init == "++":
         centers = _initialize_plus_plus(x, n_clusters, p, sampler, weights, ws=ws)
     elif init == "random":
-        centers = x[torch.tensor([sampler.randint(x.shape[0]) for _ in range(n_clusters)], device=x.device)]
+        centers = x[draw_rows(sampler, x.shape[0], n_clusters, x.device)]
     else:
         raise ValueError("init must be a torch tensor with initial centers, string '++', or 'random'.")
     n = x.shape[0]

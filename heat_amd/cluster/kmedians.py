@@ -18,6 +18,7 @@ from ..core import types
 from ..core.dndarray import DNDarray
 from ..spatial import distance
 from ._kcluster import _KCluster
+from ._sampling import draw_rows
 
 
 class KMedians(_KCluster):
@@ -45,7 +46,7 @@ class KMedians(_KCluster):
         k, dev = self.n_clusters, xt.device
         # the reference draws a row only for clusters that turn out empty; drawing one per cluster up
         # front keeps the update free of a host round trip (its random stream is not reproducible anyway)
-        fallback = torch.tensor([sampler.randint(xt.shape[0]) for _ in range(k)], dtype=torch.int64, device=dev)
+        fallback = draw_rows(sampler, xt.shape[0], k, dev)
         c_new = torch.empty_like(centers)
         _native.update_median(xt, lab32, c_new, self._workspace(dev), fallback_rows=fallback, skip_zero_rows=True)
         return c_new

@@ -14,6 +14,7 @@ from ..core import types
 from ..core.dndarray import DNDarray
 from ..spatial import distance
 from ._kcluster import _KCluster
+from ._sampling import draw_rows
 
 
 class KMedoids(_KCluster):
@@ -40,7 +41,7 @@ class KMedoids(_KCluster):
         """
         k, dev = self.n_clusters, xt.device
         ws = self._workspace(dev)
-        fallback = torch.tensor([sampler.randint(xt.shape[0]) for _ in range(k)], dtype=torch.int64, device=dev)
+        fallback = draw_rows(sampler, xt.shape[0], k, dev)
         med = torch.empty_like(centers)
         counts = torch.empty((k,), dtype=torch.int64, device=dev)
         _native.update_median(xt, lab32, med, ws, fallback_rows=fallback, counts=counts, skip_zero_rows=True)
