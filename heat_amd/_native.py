@@ -46,6 +46,8 @@ SIGNATURES = {
     "hkm_label_counts_i64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
     "hkm_seed_plus_plus_f32": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                               c_int32, c_int32, c_void_p, c_void_p]),
+    "hkm_seed_plus_plus_rows_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int64, c_void_p,
+                                                   c_int32, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_assign_l1_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                          c_void_p, c_void_p, c_void_p]),
     "hkm_closest_rows_l1_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
@@ -333,6 +335,26 @@ def seed_plus_plus(x: torch.Tensor, weights: Optional[torch.Tensor], first: int,
         raise ValueError("weights must be a contiguous float32 vector with one entry per row")
     check(load().hkm_seed_plus_plus_f32(_ptr(x), m, d, x.stride(0) if m > 1 else d, _ptr(weights), int(first),
                                         _ptr(u), k, p, _ptr(idx), _stream()))
+
+
+SEED_ROWS_MAX = 1 << 24  # HKM_SEED_ROWS_MAX
+
+
+def seed_plus_plus_rows(x: torch.Tensor, weights: Optional[torch.Tensor], first: int, u: torch.Tensor, k: int, p: int,
+                        idx: torch.Tensor, ws: Workspace) -> None:
+    """The draws of :func:`seed_plus_plus` for up to SEED_ROWS_MAX rows: two launches per centre, none of
+    them waits for the host (see hkm_seed_plus_plus_rows_f32 in include/hkm.h)."""
+    _require_gpu(x, weights, u, idx)
+    m, d = x.shape
+    if idx.numel() != k or idx.dtype != torch.int64:
+        raise ValueError("idx must hold k int64 entries")
+    if u.numel() < k - 1 or u.dtype != torch.float32:
+        raise ValueError("u must hold k - 1 float32 numbers")
+    if weights is not None and (weights.numel() != m or weights.dtype != torch.float32 or not weights.is_contiguous()):
+        raise ValueError("weights must be a contiguous float32 vector with one entry per row")
+    buf = ws.get(workspace_bytes(m, 1, 1, WS_ASSIGN | WS_SSE))
+    check(load().hkm_seed_plus_plus_rows_f32(_ptr(x), m, d, x.stride(0) if m > 1 else d, _ptr(weights), int(first),
+                                             _ptr(u), k, p, _ptr(idx), _ptr(buf), buf.numel(), _stream()))
 
 
 def assign_l1(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_dist: Optional[torch.Tensor]) -> None:

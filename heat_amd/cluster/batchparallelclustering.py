@@ -45,9 +45,10 @@ def _initialize_plus_plus(x: torch.Tensor, n_clusters: int, p: int, sampler, wei
     """
     if x.shape[0] > max_samples:
         x = x[draw_rows(sampler, x.shape[0], max_samples, x.device)].contiguous()
-    if (getattr(sampler, "fused_seeding", False) and x.dtype == torch.float32 and x.shape[0] <= _native.SEED_MAX_ROWS
+    if (getattr(sampler, "fused_seeding", False) and x.dtype == torch.float32 and x.shape[0] <= _native.SEED_ROWS_MAX
             and p in (1, 2)):
-        # a small row set (the candidates of k-means||): all draws in one launch, from one uniform number each
+        # every draw by inverse CDF from one uniform number, none of them waiting for the host: a small
+        # row set (the candidates of k-means||) in ONE launch, a large one in two launches per centre
         w = None
         if isinstance(weights, torch.Tensor):
             w = weights.to(device=x.device, dtype=torch.float32).contiguous()
@@ -56,7 +57,11 @@ def _initialize_plus_plus(x: torch.Tensor, n_clusters: int, p: int, sampler, wei
         first = sampler.randint(x.shape[0])
         u = sampler.uniform(max(n_clusters - 1, 1))
         idx = torch.empty((n_clusters,), dtype=torch.int64, device=x.device)
-        _native.seed_plus_plus(x.contiguous() if x.stride(1) != 1 else x, w, first, u, n_clusters, p, idx)
+        xc = x.contiguous() if x.stride(1) != 1 else x
+        if x.shape[0] <= _native.SEED_MAX_ROWS:
+            _native.seed_plus_plus(xc, w, first, u, n_clusters, p, idx)
+        else:
+            _native.seed_plus_plus_rows(xc, w, first, u, n_clusters, p, idx, ws or _native.Workspace(x.device))
         if bool((idx < 0).any()):
             raise RuntimeError("invalid multinomial distribution (sum of probabilities <= 0)")
         return x[idx]

@@ -402,6 +402,27 @@ int hkm_seed_plus_plus_f32(const float* X, int32_t M, int32_t D, int64_t ldx, co
     return launch_seed_plus_plus(X, M, D, ldx, w, first, u, K, p, idx, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_seed_plus_plus_rows_f32(const float* X, int64_t M, int32_t D, int64_t ldx, const float* w, int64_t first,
+                                const float* u, int32_t K, int32_t p, int64_t* idx, void* ws, size_t ws_bytes,
+                                void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 1 || M > HKM_SEED_ROWS_MAX)
+        return fail(HKM_EINVAL, "M = %lld outside 1..%lld", (long long)M, (long long)HKM_SEED_ROWS_MAX);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
+    if (ldx < D) return fail(HKM_EINVAL, "leading dimension of X (%lld) < columns (%d)", (long long)ldx, D);
+    if (first < 0 || first >= M) return fail(HKM_EINVAL, "first = %lld outside 0..%lld", (long long)first, (long long)(M - 1));
+    if (p != 1 && p != 2) return fail(HKM_EINVAL, "p = %d must be 1 or 2", p);
+    if (!X || !idx || (K > 1 && !u)) return fail(HKM_EINVAL, "NULL pointer argument");
+    const int32_t flags = HKM_WS_ASSIGN | HKM_WS_SSE;
+    const size_t need = carve(nullptr, M, 1, 1, flags).total;
+    int rc = check_ws(ws, ws_bytes, need);
+    if (rc) return rc;
+    const Workspace wk = carve(ws, M, 1, 1, flags);
+    return launch_seed_plus_plus_rows(X, M, D, ldx, w, first, u, K, p, idx, wk.min_d2, wk.red,
+                                      static_cast<hipStream_t>(hip_stream));
+}
+
 // ---- float64 data -----------------------------------------------------------------------------
 static int check_matrix64(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
     if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);

@@ -39,6 +39,21 @@ __device__ __forceinline__ float sqrt_rn_short(float t) {
     r = eu > 0.f ? su : r;
     return r;
 }
+// Sum of one value per thread over the workgroup (power-of-two size, sh holds blockDim.x doubles) as a
+// fixed binary tree: the result depends on the values only, never on scheduling.
+__device__ __forceinline__ double block_sum_fixed(double v, double* sh) {
+    const int tid = threadIdx.x;
+    sh[tid] = v;
+    __syncthreads();
+    for (int w = blockDim.x / 2; w > 0; w >>= 1) {
+        if (tid < w) sh[tid] += sh[tid + w];
+        __syncthreads();
+    }
+    const double r = sh[0];
+    __syncthreads();
+    return r;
+}
+
 // Key that orders non-negative floats with zero moved to the top: a minimum over keys below
 // SQRT_SHORT_KEY_LIMIT means some value is positive and below 2^-96, outside sqrt_rn_short's range.
 __device__ __forceinline__ unsigned sqrt_short_key(float t) { return __float_as_uint(t) - 1u; }
@@ -202,6 +217,9 @@ int launch_label_counts(const int32_t* labels, int64_t N, int32_t K, int64_t* co
                         hipStream_t st);
 int launch_seed_plus_plus(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
                           const float* u, int32_t K, int32_t p, int64_t* idx, hipStream_t st);
+int launch_seed_plus_plus_rows(const float* X, int64_t M, int32_t D, int64_t ldx, const float* w, int64_t first,
+                               const float* u, int32_t K, int32_t p, int64_t* idx, float* dist, double* red,
+                               hipStream_t st);
 int launch_assign_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                      int64_t ldc, int32_t* labels, float* min_dist, hipStream_t st);
 int launch_closest_rows_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const float* Qm,

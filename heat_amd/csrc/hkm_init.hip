@@ -288,6 +288,241 @@ __global__ __launch_bounds__(SEED_THREADS) void seed_plus_plus_kernel(const floa
     }
 }
 
+// ---- k-means++ seeding of a large row set: two launches per draw, no host round trip --------------
+// The same draws as seed_plus_plus_kernel for up to 2^24 rows (BatchParallelKMeans seeds its local rows
+// this way, heat/cluster/batchparallelclustering.py:22-46,270-276).  Per draw:
+//   seed_rows_dist_kernel  one read of X: distance of every row to the newest centre (eight lanes per
+//                          row, 16-byte loads, four rows in flight per lane group), running minimum
+//                          in `dist`, and the fp64 sum of weight * distance of every block of rows;
+//   seed_rows_pick_kernel  one workgroup: scans the block sums in block order, finds the block that
+//                          holds u * total, then scans that block's rows in row order.
+// The newest centre is read from idx[k - 1] on the device, so the K - 1 draws are enqueued back to back.
+// A draw that finds no mass writes -1; every later launch sees it and passes it on.
+__global__ void seed_rows_first_kernel(long long* __restrict__ idx, long long first) { idx[0] = first; }
+
+static constexpr int SEEDR_THREADS = 256;
+static constexpr int SEEDR_LPR = 8;     // lanes per row
+static constexpr int SEEDR_PICK_T = 1024;
+static constexpr int SEEDR_MAX_PER_BLOCK = 8192;  // rows of one block: 8 per thread of the pick kernel
+
+template <int P, bool VEC>
+__global__ __launch_bounds__(SEEDR_THREADS) void seed_rows_dist_kernel(
+    const float* __restrict__ X, int64_t M, int D, int64_t ldx, const float* __restrict__ w,
+    const long long* __restrict__ idx, int k, int64_t per_block, float* __restrict__ dist,
+    double* __restrict__ block_sum) {
+    __shared__ double sh[SEEDR_THREADS];
+    const long long cur = idx[k - 1];
+    if (cur < 0) return;  // an earlier draw found no mass
+    const float* c = X + cur * ldx;
+    const int tid = threadIdx.x, sub = tid & (SEEDR_LPR - 1), grp = tid / SEEDR_LPR;
+    constexpr int GROUPS = SEEDR_THREADS / SEEDR_LPR;  // rows per pass of the workgroup
+    constexpr int UF = 4;
+    const int64_t b0 = int64_t(blockIdx.x) * per_block, b1 = min(M, b0 + per_block);
+    double mass = 0.0;
+    for (int64_t r0 = b0 + grp; r0 < b1; r0 += int64_t(GROUPS) * UF) {
+        float acc[UF];
+#pragma unroll
+        for (int t = 0; t < UF; ++t) acc[t] = 0.f;
+        if (VEC) {
+            for (int f = 4 * sub; f < D; f += 4 * SEEDR_LPR) {
+                const float4 cv = *reinterpret_cast<const float4*>(c + f);
+                float4 xv[UF];
+#pragma unroll
+                for (int t = 0; t < UF; ++t) {
+                    const int64_t r = r0 + int64_t(t) * GROUPS;
+                    xv[t] = *reinterpret_cast<const float4*>(X + (r < b1 ? r : b0) * ldx + f);
+                }
+#pragma unroll
+                for (int t = 0; t < UF; ++t) {
+                    const float d0 = xv[t].x - cv.x, d1 = xv[t].y - cv.y, d2 = xv[t].z - cv.z, d3 = xv[t].w - cv.w;
+                    if (P == 1) acc[t] += (fabsf(d0) + fabsf(d1)) + (fabsf(d2) + fabsf(d3));
+                    else acc[t] = fmaf(d3, d3, fmaf(d2, d2, fmaf(d1, d1, fmaf(d0, d0, acc[t]))));
+                }
+            }
+        } else {
+            for (int f = sub; f < D; f += SEEDR_LPR) {
+                const float cv = c[f];
+#pragma unroll
+                for (int t = 0; t < UF; ++t) {
+                    const int64_t r = r0 + int64_t(t) * GROUPS;
+                    const float df = X[(r < b1 ? r : b0) * ldx + f] - cv;
+                    acc[t] = P == 1 ? acc[t] + fabsf(df) : fmaf(df, df, acc[t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < UF; ++t) {
+            float a = acc[t];
+            a += __shfl_xor(a, 1);
+            a += __shfl_xor(a, 2);
+            a += __shfl_xor(a, 4);
+            const int64_t r = r0 + int64_t(t) * GROUPS;
+            if (sub == 0 && r < b1) {
+                float d = P == 1 ? a : sqrtf(a);
+                if (r == cur) d = 0.f;  // exactly zero for the row itself, whatever the summation order
+                if (k > 1) d = fminf(dist[r], d);
+                dist[r] = d;
+                mass += double((w ? w[r] : 1.0f) * d);
+            }
+        }
+    }
+    const double t = block_sum_fixed(mass, sh);
+    if (tid == 0) block_sum[blockIdx.x] = t;
+}
+
+// inclusive scan of one value per thread in thread order; *total receives the sum (all threads)
+__device__ __forceinline__ double seed_block_scan(double v, double* s_wave, double& total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    double incl = v;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+        const double o = __shfl_up(incl, s);
+        if (lane >= s) incl += o;
+    }
+    __syncthreads();  // s_wave may still be read from the previous scan
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    double before = 0.0;
+    total = 0.0;
+    for (int q = 0; q < SEEDR_PICK_T / 64; ++q) {
+        if (q < wave) before += s_wave[q];
+        total += s_wave[q];
+    }
+    return before + incl;
+}
+
+__global__ __launch_bounds__(SEEDR_PICK_T) void seed_rows_pick_kernel(
+    int64_t M, const float* __restrict__ w, const float* __restrict__ u, int k, int K, int64_t per_block,
+    int nb, const float* __restrict__ dist, const double* __restrict__ block_sum, long long* __restrict__ idx) {
+    __shared__ double s_wave[SEEDR_PICK_T / 64];
+    __shared__ int s_pick, s_last;
+    __shared__ double s_before;
+    const int tid = threadIdx.x;
+    if (idx[k - 1] < 0) {
+        if (tid == 0) idx[k] = -1;
+        return;
+    }
+    // 1. the block that holds u * total
+    const int bper = (nb + SEEDR_PICK_T - 1) / SEEDR_PICK_T;
+    double mine = 0.0;
+    for (int q = 0; q < bper; ++q) {
+        const int b = tid * bper + q;
+        if (b < nb) mine += block_sum[b];
+    }
+    if (tid == 0) {
+        s_pick = 0x7fffffff;
+        s_last = -1;
+    }
+    double total;
+    const double incl = seed_block_scan(mine, s_wave, total);
+    if (!(total > 0.0)) {
+        if (tid == 0) idx[k] = -1;
+        return;
+    }
+    const double target = double(u[k - 1]) * total;
+    {
+        double run = incl - mine;
+        int pick = 0x7fffffff, last = -1;
+        double before_pick = 0.0;
+        for (int q = 0; q < bper; ++q) {
+            const int b = tid * bper + q;
+            if (b < nb) {
+                const double v = block_sum[b];
+                if (v > 0.0) {
+                    last = b;
+                    if (run + v > target && pick == 0x7fffffff) {
+                        pick = b;
+                        before_pick = run;
+                    }
+                }
+                run += v;
+            }
+        }
+        if (pick != 0x7fffffff) atomicMin(&s_pick, pick);
+        if (last >= 0) atomicMax(&s_last, last);
+        __syncthreads();
+        const int chosen = s_pick != 0x7fffffff ? s_pick : s_last;
+        // the mass in front of the chosen block, from the thread that owns it
+        if (chosen >= tid * bper && chosen < (tid + 1) * bper) {
+            double r2 = incl - mine;
+            for (int b = tid * bper; b < chosen; ++b) r2 += block_sum[b];
+            s_before = r2;
+        }
+        __syncthreads();
+        (void)before_pick;
+    }
+    const int blk = s_pick != 0x7fffffff ? s_pick : s_last;
+    const double tin = target - s_before;  // target inside the block
+    __syncthreads();
+    if (tid == 0) {
+        s_pick = 0x7fffffff;
+        s_last = -1;
+    }
+    // 2. the row inside the block, rows in row order: thread t owns R consecutive rows
+    const int64_t b0 = int64_t(blk) * per_block, b1 = min(M, b0 + per_block);
+    const int R = int((per_block + SEEDR_PICK_T - 1) / SEEDR_PICK_T);
+    float wd[SEEDR_MAX_PER_BLOCK / SEEDR_PICK_T];
+    double rows = 0.0;
+#pragma unroll
+    for (int q = 0; q < SEEDR_MAX_PER_BLOCK / SEEDR_PICK_T; ++q) {
+        const int64_t r = b0 + int64_t(tid) * R + q;
+        wd[q] = (q < R && r < b1) ? (w ? w[r] : 1.0f) * dist[r] : 0.f;
+        rows += double(wd[q]);
+    }
+    double tot2;
+    const double incl2 = seed_block_scan(rows, s_wave, tot2);
+    double run = incl2 - rows;
+    int pick = 0x7fffffff, last = -1;
+#pragma unroll
+    for (int q = 0; q < SEEDR_MAX_PER_BLOCK / SEEDR_PICK_T; ++q) {
+        run += double(wd[q]);
+        if (wd[q] > 0.f) {
+            last = tid * R + q;
+            if (run > tin && pick == 0x7fffffff) pick = tid * R + q;
+        }
+    }
+    if (pick != 0x7fffffff) atomicMin(&s_pick, pick);
+    if (last >= 0) atomicMax(&s_last, last);
+    __syncthreads();
+    if (tid == 0) {
+        const int off = s_pick != 0x7fffffff ? s_pick : s_last;  // the chosen block has mass, so off >= 0
+        idx[k] = off >= 0 ? b0 + off : -1;
+    }
+}
+
+int launch_seed_plus_plus_rows(const float* X, int64_t M, int32_t D, int64_t ldx, const float* w, int64_t first,
+                               const float* u, int32_t K, int32_t p, int64_t* idx, float* dist, double* red,
+                               hipStream_t st) {
+    long long* idx_ll = reinterpret_cast<long long*>(idx);
+    hipLaunchKernelGGL(seed_rows_first_kernel, dim3(1), dim3(1), 0, st, idx_ll, (long long)first);
+    int rc = check_launch("seed_rows_first_kernel");
+    if (rc) return rc;
+    int nb = int((M + 4095) / 4096);
+    if (nb < 1) nb = 1;
+    if (nb > RED_SLOTS) nb = RED_SLOTS;
+    int64_t per_block = ((M + nb - 1) / nb + 31) / 32 * 32;
+    nb = int((M + per_block - 1) / per_block);
+    const bool vec = aligned16(X) && ldx % 4 == 0 && D % 4 == 0;
+    for (int k = 1; k < K; ++k) {
+#define HKM_GO(PP, V)                                                                                          \
+    hipLaunchKernelGGL((seed_rows_dist_kernel<PP, V>), dim3(nb), dim3(SEEDR_THREADS), 0, st, X, M, D, ldx, w, \
+                       idx_ll, k, per_block, dist, red)
+        if (p == 1) {
+            if (vec) HKM_GO(1, true);
+            else HKM_GO(1, false);
+        } else {
+            if (vec) HKM_GO(2, true);
+            else HKM_GO(2, false);
+        }
+#undef HKM_GO
+        if ((rc = check_launch("seed_rows_dist_kernel"))) return rc;
+        hipLaunchKernelGGL(seed_rows_pick_kernel, dim3(1), dim3(SEEDR_PICK_T), 0, st, M, w, u, k, K, per_block, nb,
+                           dist, red, idx_ll);
+        if ((rc = check_launch("seed_rows_pick_kernel"))) return rc;
+    }
+    return HKM_OK;
+}
+
 int launch_seed_plus_plus(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
                           const float* u, int32_t K, int32_t p, int64_t* idx, hipStream_t st) {
     if (p == 1)

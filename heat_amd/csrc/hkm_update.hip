@@ -322,18 +322,6 @@ int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const
 // mode 1: sum of v[i]                      (sum of clamped squared distances)
 // mode 2: sum of sqrtf(v[i])^2, then (sqrtf(total))^2   (heat/cluster/_kcluster.py:367-368)
 // mode 3: sum of sqrtf(v[i])               (clustering cost of k-means||, _kcluster.py:163-170,312-316)
-__device__ __forceinline__ double block_sum_fixed(double v, double* sh) {
-    const int tid = threadIdx.x;
-    sh[tid] = v;
-    __syncthreads();
-    for (int w = blockDim.x / 2; w > 0; w >>= 1) {
-        if (tid < w) sh[tid] += sh[tid + w];
-        __syncthreads();
-    }
-    const double r = sh[0];
-    __syncthreads();
-    return r;
-}
 
 __device__ __forceinline__ float hkm_sqrt(float v) { return sqrtf(v); }
 __device__ __forceinline__ double hkm_sqrt(double v) { return sqrt(v); }

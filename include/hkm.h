@@ -182,8 +182,19 @@ int hkm_label_counts_i64(const int32_t* labels, int64_t N, int32_t K, int64_t* c
  * 1 <= M <= HKM_SEED_MAX_ROWS, 0 <= first < M, K >= 1, p in {1, 2}; X, w, u, idx are device pointers.
  */
 #define HKM_SEED_MAX_ROWS 16384
+/* The same draws for up to HKM_SEED_ROWS_MAX rows (BatchParallelKMeans / BatchParallelKMedians seed their
+ * local rows this way, heat/cluster/batchparallelclustering.py:22-46,270-276; the reference subsamples
+ * larger sets to 2^24 - 1 rows first).  Two launches per centre, all enqueued without a host round
+ * trip: one read of X that updates the running distances and sums their mass per block of rows, and
+ * one workgroup that finds the block and then the row holding u[k-1] * total.  Prefix sums are taken
+ * over blocks in block order and inside the chosen block in row order.
+ * ws needs hkm_workspace_bytes(M, 1, 1, HKM_WS_ASSIGN | HKM_WS_SSE) bytes. */
+#define HKM_SEED_ROWS_MAX 16777216
 int hkm_seed_plus_plus_f32(const float* X, int32_t M, int32_t D, int64_t ldx, const float* w, int32_t first,
                            const float* u, int32_t K, int32_t p, int64_t* idx, void* hip_stream);
+int hkm_seed_plus_plus_rows_f32(const float* X, int64_t M, int32_t D, int64_t ldx, const float* w, int64_t first,
+                                const float* u, int32_t K, int32_t p, int64_t* idx, void* ws, size_t ws_bytes,
+                                void* hip_stream);
 
 /*
  * Manhattan-metric siblings for k-medians / k-medoids (heat/cluster/kmedians.py:60-106,

@@ -288,3 +288,53 @@ def test_min_merge_sum(cuda, n):
         assert float(cost) == float(again)
         ref = float(want.double().sqrt().sum())
         assert abs(float(cost) - ref) <= 2e-7 * ref + 1e-30
+
+
+@pytest.mark.parametrize("m,d,k,p,weighted", [(20000, 32, 24, 2, True), (70001, 6, 16, 1, False), (16385, 3, 12, 2, False),
+                                              (300000, 17, 10, 2, True), (50000, 64, 8, 1, True)])
+def test_plus_plus_seeding_of_many_rows(cuda, m, d, k, p, weighted):
+    """hkm_seed_plus_plus_rows_f32 (two launches per centre, no host round trip), checked like the
+    one-launch kernel: step by step along its own picks against the reference's op sequence with the
+    inverse-CDF draw.  The prefix sums run over blocks of rows and then over the rows of one block, so a
+    pick may differ from the oracle's only within 1e-5 of the total mass around a boundary."""
+    g = torch.Generator().manual_seed(m + 5 * k + p)
+    x = torch.randn((m, d), generator=g) * 3
+    x[m // 2] = x[0]
+    w = torch.rand(m, generator=g) + 0.25 if weighted else None
+    u = torch.rand(k - 1, generator=g)
+    u[0] = 0.0          # the very first row with mass
+    u[1] = 0.99999994   # the largest float32 below 1: the very last one
+    first = int(torch.randint(0, m, (1,), generator=g))
+    idx = torch.full((k,), -5, dtype=torch.int64, device=cuda)
+    ws = _native.Workspace(cuda)
+    _native.seed_plus_plus_rows(x.to(cuda), None if w is None else w.to(cuda), first, u.to(cuda), k, p, idx, ws)
+    got = idx.cpu()
+    assert int(got[0]) == first and int(got.min()) >= 0 and int(got.max()) < m
+    assert len(set(got.tolist())) == k
+    wts = torch.ones(m) if w is None else w
+    exact = 0
+    for j in range(1, k):
+        dist = torch.cdist(x, x[got[:j]], p=float(p), compute_mode="donot_use_mm_for_euclid_dist").min(dim=1)[0]
+        mass = wts * dist
+        s = orc.InverseCdfSampler(first, u[j - 1 : j])
+        want = s.multinomial(mass)
+        cum, target = s.prefixes[0]
+        i = int(got[j])
+        tol = 1e-5 * float(cum[-1])
+        assert float(mass[i]) > 0
+        assert float(cum[i]) > target - tol and float(cum[i] - mass[i].double()) <= target + tol, (j, i, want)
+        exact += int(i == want)
+    assert exact >= (k - 1) - 1
+    # the same function through the estimator-side helper: reproducible, K distinct rows
+    a = bpc._initialize_plus_plus(x.to(cuda), k, p, DeviceSampler(cuda, 3), 1.0 if w is None else w.to(cuda))
+    b = bpc._initialize_plus_plus(x.to(cuda), k, p, DeviceSampler(cuda, 3), 1.0 if w is None else w.to(cuda))
+    assert torch.equal(a, b) and a.shape == (k, d)
+
+
+def test_plus_plus_seeding_of_many_rows_without_mass(cuda):
+    x = torch.tensor([[0.0, 0.0], [1.0, 0.0], [0.0, 2.0]]).repeat(7000, 1).to(cuda)
+    u = torch.full((5,), 0.5, device=cuda)
+    idx = torch.full((6,), -5, dtype=torch.int64, device=cuda)
+    _native.seed_plus_plus_rows(x, None, 1, u, 6, 2, idx, _native.Workspace(cuda))
+    got = idx.cpu().tolist()
+    assert got[0] == 1 and got[3:] == [-1, -1, -1] and len({tuple(x[i].tolist()) for i in got[:3]}) == 3
