@@ -123,6 +123,25 @@ def _require_gpu(*tensors: torch.Tensor) -> None:
             )
 
 
+def _require_rows(*mats: Optional[torch.Tensor]) -> None:
+    """The library reads matrices row by row with unit stride inside a row: anything else (a transposed
+    view, a column slice with a step) would be read as different numbers, so it is refused here."""
+    for t in mats:
+        if t is None or t.dim() != 2:
+            continue
+        if t.shape[1] > 1 and t.stride(1) != 1:
+            raise ValueError("matrix rows must be contiguous (stride 1 along the last axis); call .contiguous()")
+        if t.shape[0] > 1 and t.stride(0) < t.shape[1]:
+            raise ValueError("matrix rows overlap (row stride below the row length)")
+
+
+def _require_dense(*mats: Optional[torch.Tensor]) -> None:
+    """For the arguments the C ABI takes without a leading dimension (centroid matrices of the step)."""
+    for t in mats:
+        if t is not None and not t.is_contiguous():
+            raise ValueError("this matrix must be dense (row stride equal to the row length); call .contiguous()")
+
+
 class Workspace:
     """A reusable device scratch buffer, grown on demand."""
 
@@ -159,6 +178,7 @@ def _is_f64(*tensors: Optional[torch.Tensor]) -> bool:
 def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optional[torch.Tensor],
            ws: Workspace) -> None:
     _require_gpu(x, c, labels, min_d2)
+    _require_rows(x, c)
     n, d = x.shape
     k = c.shape[0]
     if _is_f64(x, c, min_d2):
@@ -174,6 +194,7 @@ def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optio
 def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: Optional[torch.Tensor],
            ws: Workspace) -> None:
     _require_gpu(x, labels, c_new, counts)
+    _require_rows(x, c_new)
     n, d = x.shape
     k = c_new.shape[0]
     if _is_f64(x, c_new):
@@ -190,6 +211,8 @@ def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: O
 def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],
                shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace) -> None:
     _require_gpu(x, c, c_new, labels, sse)
+    _require_rows(x, c, c_new)
+    _require_dense(c, c_new)
     if not (shift.is_cuda or shift.is_pinned()):
         # a pinned host scalar is written by the kernel itself over the bus: no copy engine, no
         # extra stream operation between two steps
@@ -216,6 +239,8 @@ def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, la
     For loops that issue thousands of steps on small problems, where building the argument list costs
     as much as the step.  The tensors are kept alive by the returned function."""
     _require_gpu(x, c, c_new, labels, sse)
+    _require_rows(x, c, c_new)
+    _require_dense(c, c_new)
     if not (shift.is_cuda or shift.is_pinned()):
         raise RuntimeError("shift must live on the GPU or in pinned host memory")
     n, d = x.shape
@@ -238,6 +263,8 @@ def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, la
 
 def shift(c_old: torch.Tensor, c_new: torch.Tensor, out: torch.Tensor) -> None:
     _require_gpu(c_old, c_new, out)
+    _require_rows(c_old, c_new)
+    _require_dense(c_old, c_new)
     k, d = c_old.shape
     if _is_f64(c_old, c_new, out):
         check(load().hkm_shift_f64(_ptr(c_old), _ptr(c_new), k, d, _ptr(out), _stream()))
@@ -258,6 +285,7 @@ def functional_value(min_d2: torch.Tensor, out: torch.Tensor, ws: Workspace) -> 
 
 def cdist(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, sqrt: bool = True) -> None:
     _require_gpu(x, y, out)
+    _require_rows(x, y, out)
     m, d = x.shape
     nn = y.shape[0]
     check(load().hkm_cdist_f32(_ptr(x), m, x.stride(0) if m > 1 else d, _ptr(y), nn, y.stride(0) if nn > 1 else d,
@@ -269,6 +297,7 @@ METRIC_EUCLID_QE, METRIC_EUCLID, METRIC_GAUSS_QE, METRIC_GAUSS, METRIC_MANHATTAN
 
 def pairwise(x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, metric: int, sigma: float = 1.0) -> None:
     _require_gpu(x, y, out)
+    _require_rows(x, y, out)
     m, d = x.shape
     nn = y.shape[0]
     if _is_f64(x, y, out):
@@ -326,6 +355,7 @@ def seed_plus_plus(x: torch.Tensor, weights: Optional[torch.Tensor], first: int,
     """k-means++ seeding of at most SEED_MAX_ROWS rows in one launch (see hkm_seed_plus_plus_f32 in
     include/hkm.h): idx[0] = first, idx[j] drawn by inverse CDF from u[j - 1]; -1 where no row has mass."""
     _require_gpu(x, weights, u, idx)
+    _require_rows(x)
     m, d = x.shape
     if idx.numel() != k or idx.dtype != torch.int64:
         raise ValueError("idx must hold k int64 entries")
@@ -345,6 +375,7 @@ def seed_plus_plus_rows(x: torch.Tensor, weights: Optional[torch.Tensor], first:
     """The draws of :func:`seed_plus_plus` for up to SEED_ROWS_MAX rows: two launches per centre, none of
     them waits for the host (see hkm_seed_plus_plus_rows_f32 in include/hkm.h)."""
     _require_gpu(x, weights, u, idx)
+    _require_rows(x)
     m, d = x.shape
     if idx.numel() != k or idx.dtype != torch.int64:
         raise ValueError("idx must hold k int64 entries")
@@ -360,6 +391,7 @@ def seed_plus_plus_rows(x: torch.Tensor, weights: Optional[torch.Tensor], first:
 def assign_l1(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_dist: Optional[torch.Tensor]) -> None:
     """labels[i] = argmin_k sum|x_i - c_k| (Manhattan), optional minimum distance."""
     _require_gpu(x, c, labels, min_dist)
+    _require_rows(x, c)
     n, d = x.shape
     k = c.shape[0]
     check(load().hkm_assign_l1_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
@@ -370,6 +402,7 @@ def closest_rows_l1(x: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, dist: O
                     ws: Workspace) -> None:
     """idx[m] = row of x closest to q[m] in the Manhattan metric (first index on ties)."""
     _require_gpu(x, q, idx, dist)
+    _require_rows(x, q)
     n, d = x.shape
     m = q.shape[0]
     buf = ws.get(workspace_bytes(n, d, m, WS_MEDIAN))
@@ -383,6 +416,8 @@ def update_median(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, ws
                   counts: Optional[torch.Tensor] = None, lower: bool = False, skip_zero_rows: bool = False) -> None:
     """Per-cluster, per-coordinate median (see hkm_update_median_f32 in include/hkm.h)."""
     _require_gpu(x, labels, c_new, fallback_rows, c_old, counts)
+    _require_rows(x, c_new, c_old)
+    _require_dense(c_old)
     n, d = x.shape
     k = c_new.shape[0]
     buf = ws.get(workspace_bytes(n, d, k, WS_MEDIAN))

@@ -408,3 +408,25 @@ def test_widen_and_empty_inputs(cuda):
     idx = torch.empty((4,), dtype=torch.int64, device=cuda)
     _native.sample_select(e, e.clone(), torch.ones((), device=cuda), 2.0, idx, cnt, ws)
     assert int(cnt) == 0
+
+
+def test_binding_refuses_matrices_it_would_misread(cuda):
+    """Rows must have unit stride inside (a transposed view would be read as other numbers), and the
+    centroid matrices of the step, which the C ABI takes without a leading dimension, must be dense."""
+    ws = _native.Workspace(cuda)
+    xt = torch.randn((8, 100), device=cuda).T            # (100, 8) with stride (1, 100)
+    c = torch.randn((4, 8), device=cuda)
+    lab = torch.empty((100,), dtype=torch.int32, device=cuda)
+    with pytest.raises(ValueError, match="contiguous"):
+        _native.assign(xt, c, lab, None, ws)
+    with pytest.raises(ValueError, match="contiguous"):
+        _native.pairwise(xt, c, torch.empty((100, 4), device=cuda), _native.METRIC_EUCLID)
+    x = xt.contiguous()
+    wide = torch.randn((4, 12), device=cuda)
+    shift = torch.empty((), device=cuda)
+    with pytest.raises(ValueError, match="dense"):
+        _native.lloyd_step(x, wide[:, :8], torch.empty_like(c), lab, shift, None, ws)
+    # a padded X is fine: it has a leading dimension
+    xp = torch.randn((100, 12), device=cuda)[:, :8]
+    _native.lloyd_step(xp, c, torch.empty_like(c), lab, shift, None, ws)
+    _native.assign(xp, wide[:, :8], lab, None, ws)
