@@ -55,6 +55,11 @@ SIGNATURES = {
     "hkm_update_median_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                              c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p,
                                              c_size_t, c_void_p]),
+    "hkm_update_median_q64_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
+                                                 c_void_p, c_void_p, c_int64, c_void_p, c_int32, c_int32, c_void_p,
+                                                 c_void_p, c_size_t, c_void_p]),
+    "hkm_closest_rows_l1_q64_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
+                                                   c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_assign_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p]),
     "hkm_update_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
@@ -411,16 +416,45 @@ def closest_rows_l1(x: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, dist: O
                                          buf.numel(), _stream()))
 
 
+def closest_rows_l1_q64(x: torch.Tensor, q64: torch.Tensor, idx: torch.Tensor, dist64: Optional[torch.Tensor],
+                        ws: Workspace) -> None:
+    """idx[m] = row of the float32 x closest to the float64 q64[m] in the Manhattan metric, distances in
+    float64, first index on exact ties (see hkm_closest_rows_l1_q64_f32 in include/hkm.h)."""
+    _require_gpu(x, q64, idx, dist64)
+    _require_rows(x)
+    _require_dense(q64)
+    if q64.dtype != torch.float64 or x.dtype != torch.float32:
+        raise TypeError("x must be float32 and q64 float64")
+    n, d = x.shape
+    m = q64.shape[0]
+    buf = ws.get(workspace_bytes(n, d, m, WS_MEDIAN))
+    check(load().hkm_closest_rows_l1_q64_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(q64), m, _ptr(idx),
+                                             _ptr(dist64), _ptr(buf), buf.numel(), _stream()))
+
+
 def update_median(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, ws: Workspace,
                   fallback_rows: Optional[torch.Tensor] = None, c_old: Optional[torch.Tensor] = None,
-                  counts: Optional[torch.Tensor] = None, lower: bool = False, skip_zero_rows: bool = False) -> None:
-    """Per-cluster, per-coordinate median (see hkm_update_median_f32 in include/hkm.h)."""
-    _require_gpu(x, labels, c_new, fallback_rows, c_old, counts)
+                  counts: Optional[torch.Tensor] = None, lower: bool = False, skip_zero_rows: bool = False,
+                  median64: Optional[torch.Tensor] = None) -> None:
+    """Per-cluster, per-coordinate median (see hkm_update_median_f32 in include/hkm.h); ``median64``
+    (K x D float64) additionally receives every median before its rounding to float32."""
+    _require_gpu(x, labels, c_new, fallback_rows, c_old, counts, median64)
+    if median64 is not None:
+        _require_dense(median64)
+        if median64.dtype != torch.float64 or tuple(median64.shape) != tuple(c_new.shape):
+            raise ValueError("median64 must be a float64 matrix of the shape of c_new")
     _require_rows(x, c_new, c_old)
     _require_dense(c_old)
     n, d = x.shape
     k = c_new.shape[0]
     buf = ws.get(workspace_bytes(n, d, k, WS_MEDIAN))
+    if median64 is not None:
+        check(load().hkm_update_median_q64_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k,
+                                               _ptr(fallback_rows), _ptr(c_old), _ptr(c_new),
+                                               c_new.stride(0) if k > 1 else d, _ptr(counts), 1 if lower else 0,
+                                               1 if skip_zero_rows else 0, _ptr(median64), _ptr(buf), buf.numel(),
+                                               _stream()))
+        return
     check(load().hkm_update_median_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k,
                                        _ptr(fallback_rows), _ptr(c_old), _ptr(c_new),
                                        c_new.stride(0) if k > 1 else d, _ptr(counts), 1 if lower else 0,

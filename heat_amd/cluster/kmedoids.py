@@ -36,17 +36,21 @@ class KMedoids(_KCluster):
         """
         heat/cluster/kmedoids.py:57-115: median of the cluster's non-zero rows, then the row of the
         WHOLE data set closest to it (first index on ties); an empty cluster restarts at a random row.
-        The reference measures that distance in float64 against the float64 median; here the median
-        is rounded to float32 first, which can only matter for rows that tie to within an ulp.
+        The reference measures that distance in float64 against the float64 median, and so does the
+        snap here (``hkm_update_median_q64_f32`` hands over the medians before their rounding to float32,
+        ``hkm_closest_rows_l1_q64_f32`` sums in float64): two rows at exactly the same distance -- the two
+        members of a cluster on either side of their midpoint -- come out equal and the first one wins.
         """
         k, dev = self.n_clusters, xt.device
         ws = self._workspace(dev)
         fallback = draw_rows(sampler, xt.shape[0], k, dev)
         med = torch.empty_like(centers)
+        med64 = torch.empty(centers.shape, dtype=torch.float64, device=dev)
         counts = torch.empty((k,), dtype=torch.int64, device=dev)
-        _native.update_median(xt, lab32, med, ws, fallback_rows=fallback, counts=counts, skip_zero_rows=True)
+        _native.update_median(xt, lab32, med, ws, fallback_rows=fallback, counts=counts, skip_zero_rows=True,
+                              median64=med64)
         idx = torch.empty((k,), dtype=torch.int64, device=dev)
-        _native.closest_rows_l1(xt, med, idx, None, ws)
+        _native.closest_rows_l1_q64(xt, med64, idx, None, ws)
         # an empty cluster already holds its restart row, which is its own closest row
         return xt[idx]
 

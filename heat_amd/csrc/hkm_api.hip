@@ -119,6 +119,8 @@ MedianWorkspace carve_median(void* base, int64_t N, int32_t D, int32_t K) {
     w.next = reinterpret_cast<unsigned*>(take(kd * sizeof(unsigned)));
     w.hist = reinterpret_cast<unsigned*>(take(kd * 256 * sizeof(unsigned)));
     w.keys = reinterpret_cast<unsigned long long*>(take(size_t(K) * sizeof(unsigned long long)));
+    w.snap_d = reinterpret_cast<double*>(take(size_t(closest64_slots(K)) * sizeof(double)));
+    w.snap_i = reinterpret_cast<unsigned*>(take(size_t(closest64_slots(K)) * sizeof(unsigned)));
     w.total = off;
     return w;
 }
@@ -553,10 +555,52 @@ int hkm_closest_rows_l1_f32(const float* X, int64_t N, int32_t D, int64_t ldx, c
     return launch_closest_rows_l1(X, N, D, ldx, Q, M, ldq, idx, dist, w.keys, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const double* Q, int32_t M,
+                                int64_t* idx, double* dist, void* ws, size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, M);
+    if (rc) return rc;
+    if (N < 1) return fail(HKM_EINVAL, "N = %lld: there is no closest row in an empty matrix", (long long)N);
+    if (N > 0xfffffffeLL) return fail(HKM_EUNSUPPORTED, "N = %lld exceeds 32-bit row indices", (long long)N);
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix64("Q", Q, M, D, D))) return rc;
+    if (!idx) return fail(HKM_EINVAL, "idx is NULL");
+    const size_t need = carve_median(nullptr, N, D, M).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const MedianWorkspace w = carve_median(ws, N, D, M);
+    return launch_closest_rows_l1_q64(X, N, D, ldx, Q, M, idx, dist, w.snap_d, w.snap_i,
+                                      static_cast<hipStream_t>(hip_stream));
+}
+
+static int update_median_common(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                                const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
+                                int64_t* counts, int32_t mode, int32_t skip_zero_rows, double* medians_f64, void* ws,
+                                size_t ws_bytes, void* hip_stream);
+
+int hkm_update_median_q64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                              const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
+                              int64_t* counts, int32_t mode, int32_t skip_zero_rows, double* medians_f64, void* ws,
+                              size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    if (!medians_f64) return fail(HKM_EINVAL, "medians_f64 is NULL");
+    if (reinterpret_cast<uintptr_t>(medians_f64) & 7u) return fail(HKM_EINVAL, "medians_f64 is not 8-byte aligned");
+    return update_median_common(X, N, D, ldx, labels, K, fallback_rows, C_old, C_new, ldcn, counts, mode,
+                                skip_zero_rows, medians_f64, ws, ws_bytes, hip_stream);
+}
+
 int hkm_update_median_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
                           const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
                           int64_t* counts, int32_t mode, int32_t skip_zero_rows, void* ws, size_t ws_bytes,
                           void* hip_stream) {
+    g_err[0] = 0;
+    return update_median_common(X, N, D, ldx, labels, K, fallback_rows, C_old, C_new, ldcn, counts, mode,
+                                skip_zero_rows, nullptr, ws, ws_bytes, hip_stream);
+}
+
+static int update_median_common(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                                const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
+                                int64_t* counts, int32_t mode, int32_t skip_zero_rows, double* medians_f64, void* ws,
+                                size_t ws_bytes, void* hip_stream) {
     g_err[0] = 0;
     int rc = check_shape(N, D, K);
     if (rc) return rc;
@@ -570,7 +614,7 @@ int hkm_update_median_f32(const float* X, int64_t N, int32_t D, int64_t ldx, con
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const MedianWorkspace w = carve_median(ws, N, D, K);
     return launch_update_median(X, N, D, ldx, labels, K, fallback_rows, C_old, C_new, ldcn, counts, mode,
-                                skip_zero_rows, w, static_cast<hipStream_t>(hip_stream));
+                                skip_zero_rows, w, static_cast<hipStream_t>(hip_stream), medians_f64);
 }
 
 int hkm_cdist_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int64_t Nn, int64_t ldy,

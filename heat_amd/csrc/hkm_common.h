@@ -139,9 +139,14 @@ struct MedianWorkspace {
     unsigned* next;        // [K * D]
     unsigned* hist;        // [K * D * 256]
     unsigned long long* keys;  // [K] merge keys of the closest-row search
+    double* snap_d;        // [closest64_slots(K)] best distance of every (split, query) of the float64 snap
+    unsigned* snap_i;      // [closest64_slots(K)] and its row
     size_t total;
 };
 MedianWorkspace carve_median(void* base, int64_t N, int32_t D, int32_t K);
+int64_t closest64_slots(int32_t M);
+int launch_closest_rows_l1_q64(const float* X, int64_t N, int32_t D, int64_t ldx, const double* Qm, int32_t M,
+                               int64_t* idx, double* dist, double* part_d, unsigned* part_i, hipStream_t st);
 
 // ---- launchers (one per .hip file) ------------------------------------------------------------
 int launch_norms(const float* C, int32_t K, int32_t D, int64_t ldc, float* cn, int32_t kpad,
@@ -228,7 +233,7 @@ int launch_closest_rows_l1(const float* X, int64_t N, int32_t D, int64_t ldx, co
 int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                          int32_t K, const int64_t* fallback_rows, const float* C_old, float* C_new,
                          int64_t ldcn, int64_t* counts_out, int32_t mode, int32_t skip_zero_rows,
-                         const MedianWorkspace& w, hipStream_t st);
+                         const MedianWorkspace& w, hipStream_t st, double* med64 = nullptr);
 int launch_widen(const int32_t* in, int64_t N, int64_t* out, hipStream_t st);
 
 int num_cus();

@@ -23,20 +23,35 @@ namespace hkm {
 // ------------------------------------------------------------------------------------------------
 static constexpr int L1_T = 64;
 static constexpr int L1_KC = 16;
+static constexpr int CLOSEST64_ITEMS = 4096;  // (query tile, row split) workgroups of the float64 snap
 
-__device__ __forceinline__ void l1_better(float& bd, unsigned& bi, float d, unsigned i) {
+template <typename T>
+__device__ __forceinline__ void l1_better(T& bd, unsigned& bi, T d, unsigned i) {
     if (d < bd || (d == bd && i < bi)) {
         bd = d;
         bi = i;
     }
 }
+__device__ __forceinline__ float l1_abs(float v) { return fabsf(v); }
+__device__ __forceinline__ double l1_abs(double v) { return fabs(v); }
 
+// T = float: everything in fp32.  T = double: the rows of Q are float64 and every distance is summed in
+// float64 from the float32 rows of R widened on the way into LDS -- the medoid snap of the reference,
+// which measures float64 distances to the float64 median (heat/cluster/kmedoids.py:91-106): two rows at
+// exactly the same distance (the two members of a cluster on either side of their midpoint, the two
+// middle values of a one-dimensional cluster) must come out EQUAL so that the first one wins, and in
+// fp32 against a rounded median they come out one rounding error apart in either direction.  The
+// float64 variant writes the best (distance, row) of every split to part_d / part_i; the splits are
+// merged in row order by l1_merge_splits_kernel.
+template <typename T>
 __global__ __launch_bounds__(256) void l1_argmin_kernel(
-    const float* __restrict__ Q, int64_t M, int64_t ldq, const float* __restrict__ R, int64_t Nn,
+    const T* __restrict__ Q, int64_t M, int64_t ldq, const float* __restrict__ R, int64_t Nn,
     int64_t ldr, int D, int64_t rows_per_split, int32_t* __restrict__ labels,
-    float* __restrict__ min_dist, unsigned long long* __restrict__ keys) {
-    __shared__ float sQ[L1_KC][L1_T + 4];
-    __shared__ float sR[L1_KC][L1_T + 4];
+    float* __restrict__ min_dist, unsigned long long* __restrict__ keys, double* __restrict__ part_d,
+    unsigned* __restrict__ part_i) {
+    constexpr bool F64 = sizeof(T) == 8;
+    __shared__ T sQ[L1_KC][L1_T + 4];
+    __shared__ T sR[L1_KC][L1_T + 4];
     const int tid = threadIdx.x;
     const int tx = tid & 15, ty = tid >> 4;
     const int lk = tid & 15, lr = tid >> 4;
@@ -44,20 +59,20 @@ __global__ __launch_bounds__(256) void l1_argmin_kernel(
     const int64_t r_begin = int64_t(blockIdx.y) * rows_per_split;
     const int64_t r_end = min(Nn, r_begin + rows_per_split);
 
-    float bd[4];
+    T bd[4];
     unsigned bi[4];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-        bd[a] = HKM_INF;
+        bd[a] = T(HKM_INF);
         bi[a] = 0xffffffffu;
     }
 
     for (int64_t j0 = r_begin; j0 < r_end; j0 += L1_T) {
-        float acc[4][4];
+        T acc[4][4];
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) acc[a][b] = 0.f;
+            for (int b = 0; b < 4; ++b) acc[a][b] = T(0);
         for (int d0 = 0; d0 < D; d0 += L1_KC) {
             __syncthreads();
 #pragma unroll
@@ -65,13 +80,13 @@ __global__ __launch_bounds__(256) void l1_argmin_kernel(
                 const int r = lr + 16 * q;
                 const int d = d0 + lk;
                 const int64_t gi = i0 + r, gj = j0 + r;
-                sQ[lk][r] = (gi < M && d < D) ? Q[gi * ldq + d] : 0.f;
-                sR[lk][r] = (gj < r_end && d < D) ? R[gj * ldr + d] : 0.f;
+                sQ[lk][r] = (gi < M && d < D) ? Q[gi * ldq + d] : T(0);
+                sR[lk][r] = (gj < r_end && d < D) ? T(R[gj * ldr + d]) : T(0);
             }
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < L1_KC; ++k) {
-                float qa[4], rb[4];
+                T qa[4], rb[4];
 #pragma unroll
                 for (int a = 0; a < 4; ++a) qa[a] = sQ[k][ty * 4 + a];
 #pragma unroll
@@ -79,27 +94,27 @@ __global__ __launch_bounds__(256) void l1_argmin_kernel(
 #pragma unroll
                 for (int a = 0; a < 4; ++a)
 #pragma unroll
-                    for (int b = 0; b < 4; ++b) acc[a][b] += fabsf(qa[a] - rb[b]);
+                    for (int b = 0; b < 4; ++b) acc[a][b] += l1_abs(qa[a] - rb[b]);
             }
         }
         // this lane's four candidates per row in ascending index order, then the 16 lanes that hold
         // the other columns of the same rows
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            float d = HKM_INF;
+            T d = T(HKM_INF);
             unsigned i = 0xffffffffu;
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
                 const int64_t gj = j0 + tx * 4 + b;
-                if (gj < r_end) l1_better(d, i, acc[a][b], unsigned(gj));
+                if (gj < r_end) l1_better<T>(d, i, acc[a][b], unsigned(gj));
             }
 #pragma unroll
             for (int w = 1; w < 16; w <<= 1) {
-                const float od = __shfl_xor(d, w);
+                const T od = __shfl_xor(d, w);
                 const unsigned oi = unsigned(__shfl_xor(int(i), w));
-                l1_better(d, i, od, oi);
+                l1_better<T>(d, i, od, oi);
             }
-            l1_better(bd[a], bi[a], d, i);
+            l1_better<T>(bd[a], bi[a], d, i);
         }
     }
 
@@ -108,14 +123,17 @@ __global__ __launch_bounds__(256) void l1_argmin_kernel(
         for (int a = 0; a < 4; ++a) {
             const int64_t gi = i0 + ty * 4 + a;
             if (gi >= M) continue;
-            if (keys) {
+            if (F64) {
+                part_d[int64_t(blockIdx.y) * M + gi] = double(bd[a]);
+                part_i[int64_t(blockIdx.y) * M + gi] = bi[a];
+            } else if (keys) {
                 // distances are >= 0, so their bit patterns order like the values; a row whose
                 // distances were all NaN keeps the initial key
                 if (bi[a] != 0xffffffffu)
-                    atomicMin(&keys[gi], (unsigned long long)(__float_as_uint(bd[a])) << 32 | bi[a]);
+                    atomicMin(&keys[gi], (unsigned long long)(__float_as_uint(float(bd[a]))) << 32 | bi[a]);
             } else {
                 labels[gi] = bi[a] == 0xffffffffu ? 0 : int32_t(bi[a]);
-                if (min_dist) min_dist[gi] = bd[a];
+                if (min_dist) min_dist[gi] = float(bd[a]);
             }
         }
     }
@@ -220,9 +238,10 @@ int launch_assign_l1(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
     }
     const int64_t tiles = (N + L1_T - 1) / L1_T;
     if (tiles > 0x7fffffffLL) return fail(HKM_EUNSUPPORTED, "assign_l1: too many row tiles");
-    hipLaunchKernelGGL(l1_argmin_kernel, dim3((unsigned)tiles, 1), dim3(256), 0, st, X, N, ldx, C,
+    hipLaunchKernelGGL(l1_argmin_kernel<float>, dim3((unsigned)tiles, 1), dim3(256), 0, st, X, N, ldx, C,
                        int64_t(K), ldc, D, int64_t(K), labels, min_dist,
-                       static_cast<unsigned long long*>(nullptr));
+                       static_cast<unsigned long long*>(nullptr), static_cast<double*>(nullptr),
+                       static_cast<unsigned*>(nullptr));
     return check_launch("l1_argmin_kernel");
 }
 
@@ -241,13 +260,50 @@ int launch_closest_rows_l1(const float* X, int64_t N, int32_t D, int64_t ldx, co
     const int64_t nsplit = (N + rps - 1) / rps;
     if (nsplit > 65535) return fail(HKM_EUNSUPPORTED, "closest_rows_l1: too many splits");
     if (N > 0)
-        hipLaunchKernelGGL(l1_argmin_kernel, dim3((unsigned)qtiles, (unsigned)nsplit), dim3(256), 0, st, Qm,
+        hipLaunchKernelGGL(l1_argmin_kernel<float>, dim3((unsigned)qtiles, (unsigned)nsplit), dim3(256), 0, st, Qm,
                            int64_t(M), ldq, X, N, ldx, D, rps, static_cast<int32_t*>(nullptr),
-                           static_cast<float*>(nullptr), keys);
+                           static_cast<float*>(nullptr), keys, static_cast<double*>(nullptr),
+                           static_cast<unsigned*>(nullptr));
     if ((rc = check_launch("l1_argmin_kernel"))) return rc;
     hipLaunchKernelGGL(l1_unpack_rows_kernel, dim3((M + 255) / 256), dim3(256), 0, st, keys, int64_t(M), idx,
                        dist);
     return check_launch("l1_unpack_rows_kernel");
+}
+
+// best (distance, row) of every query over the splits, in split order = ascending row order: on equal
+// distances the first row wins
+__global__ void l1_merge_splits_kernel(const double* __restrict__ part_d, const unsigned* __restrict__ part_i,
+                                       int nsplit, int64_t M, int64_t* __restrict__ idx,
+                                       double* __restrict__ dist) {
+    const int64_t q = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (q >= M) return;
+    double bd = double(HKM_INF);
+    unsigned bi = 0xffffffffu;
+    for (int s = 0; s < nsplit; ++s) l1_better<double>(bd, bi, part_d[int64_t(s) * M + q], part_i[int64_t(s) * M + q]);
+    idx[q] = bi == 0xffffffffu ? 0 : int64_t(bi);
+    if (dist) dist[q] = bd;
+}
+
+// slots of part_d / part_i: the splits are chosen so that nsplit * qtiles <= CLOSEST64_ITEMS
+int64_t closest64_slots(int32_t M) { return int64_t(CLOSEST64_ITEMS) * L1_T + M; }
+
+int launch_closest_rows_l1_q64(const float* X, int64_t N, int32_t D, int64_t ldx, const double* Qm, int32_t M,
+                               int64_t* idx, double* dist, double* part_d, unsigned* part_i, hipStream_t st) {
+    const int64_t qtiles = (int64_t(M) + L1_T - 1) / L1_T;
+    int64_t want = CLOSEST64_ITEMS / qtiles;
+    if (want < 1) want = 1;
+    int64_t rps = (N + want - 1) / want;
+    rps = (rps + L1_T - 1) / L1_T * L1_T;
+    if (rps < 4 * L1_T) rps = 4 * L1_T;
+    const int64_t nsplit = (N + rps - 1) / rps;
+    hipLaunchKernelGGL(l1_argmin_kernel<double>, dim3((unsigned)qtiles, (unsigned)nsplit), dim3(256), 0, st, Qm,
+                       int64_t(M), int64_t(D), X, N, ldx, D, rps, static_cast<int32_t*>(nullptr),
+                       static_cast<float*>(nullptr), static_cast<unsigned long long*>(nullptr), part_d, part_i);
+    int rc = check_launch("l1_argmin_kernel<double>");
+    if (rc) return rc;
+    hipLaunchKernelGGL(l1_merge_splits_kernel, dim3((M + 255) / 256), dim3(256), 0, st, part_d, part_i, int(nsplit),
+                       int64_t(M), idx, dist);
+    return check_launch("l1_merge_splits_kernel");
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -576,12 +632,15 @@ __global__ __launch_bounds__(256) void med_final_kernel(const unsigned* __restri
                                                         int64_t N, const int64_t* __restrict__ fallback_rows,
                                                         const float* __restrict__ C_old,
                                                         float* __restrict__ C_new, int64_t ldcn,
-                                                        int64_t* __restrict__ counts_out) {
+                                                        int64_t* __restrict__ counts_out,
+                                                        double* __restrict__ med64) {
     const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (i >= int64_t(K) * D) return;
     const int k = int(i / D), d = int(i - int64_t(k) * D);
     const int64_t n = counts[k];
     float v = 0.f;
+    double v64 = 0.0;  // the value before it is rounded to fp32 (differs for an even count only)
+    bool have64 = false;
     if (n == 0) {
         if (fallback_rows) {
             int64_t r = fallback_rows[k];
@@ -597,17 +656,20 @@ __global__ __launch_bounds__(256) void med_final_kernel(const unsigned* __restri
             // rank of lo inside its run of equal values; the next order statistic is another copy
             // of lo unless lo is the last of the run
             const float hi = (rank[i] + 1 < int64_t(eqcnt[i])) ? lo : from_key(next_g[i]);
-            v = float(double(lo) + (double(hi) - double(lo)) * 0.5);
+            v64 = double(lo) + (double(hi) - double(lo)) * 0.5;
+            have64 = true;
+            v = float(v64);
         }
     }
     C_new[int64_t(k) * ldcn + d] = v;
+    if (med64) med64[i] = have64 ? v64 : double(v);
     if (d == 0 && counts_out) counts_out[k] = n;
 }
 
 int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                          int32_t K, const int64_t* fallback_rows, const float* C_old, float* C_new,
                          int64_t ldcn, int64_t* counts_out, int32_t mode, int32_t skip_zero_rows,
-                         const MedianWorkspace& w, hipStream_t st) {
+                         const MedianWorkspace& w, hipStream_t st, double* med64) {
     int rc;
     const int32_t* eff = labels;
     if (N > 0 && skip_zero_rows) {
@@ -673,7 +735,7 @@ int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, cons
         if ((rc = check_launch("med_pass_kernel<1>"))) return rc;
     }
     hipLaunchKernelGGL(med_final_kernel, dim3(kd_blocks), dim3(256), 0, st, w.prefix, w.rank, w.eqcnt, w.next,
-                       w.counts, K, D, mode, X, ldx, N, fallback_rows, C_old, C_new, ldcn, counts_out);
+                       w.counts, K, D, mode, X, ldx, N, fallback_rows, C_old, C_new, ldcn, counts_out, med64);
     return check_launch("med_final_kernel");
 }
 

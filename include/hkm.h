@@ -224,6 +224,24 @@ int hkm_update_median_f32(const float* X, int64_t N, int32_t D, int64_t ldx, con
                           const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
                           int64_t* counts, int32_t mode, int32_t skip_zero_rows, void* ws, size_t ws_bytes,
                           void* hip_stream);
+/*
+ * The medoid snap in the reference's precision (heat/cluster/kmedoids.py:91-106 measures float64
+ * distances from the float64 rows of `x` to the float64 median):
+ * hkm_update_median_q64_f32 is hkm_update_median_f32 that also returns every median BEFORE it is
+ *   rounded to float32 (medians_f64, K x D dense; it differs from C_new for even counts in mode 0);
+ * hkm_closest_rows_l1_q64_f32 is hkm_closest_rows_l1_f32 for float64 queries Q (M x D dense) with every
+ *   distance summed in float64 from the float32 rows widened on the way; the row splits are merged in
+ *   row order, so of two rows at EXACTLY the same distance -- the two members of a cluster on either
+ *   side of their midpoint, the two middle values of a one-dimensional cluster -- the first wins, as
+ *   with the reference's argmin.  In float32 against a rounded median such rows come out one rounding
+ *   error apart in either direction.  dist (M doubles) may be NULL.  Same workspace as the f32 forms.
+ */
+int hkm_update_median_q64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
+                              const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
+                              int64_t* counts, int32_t mode, int32_t skip_zero_rows, double* medians_f64, void* ws,
+                              size_t ws_bytes, void* hip_stream);
+int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const double* Q, int32_t M,
+                                int64_t* idx, double* dist, void* ws, size_t ws_bytes, void* hip_stream);
 
 /*
  * float64 data.  The reference keeps float64 inputs in float64 through the same op sequence

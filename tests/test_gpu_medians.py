@@ -225,3 +225,43 @@ def test_batchparallel_kmedians_matches_oracle(cuda):
     bp.fit(ht.array(x.to(cuda), split=0))
     assert bp.n_iter_ == n_it
     assert orc.rel_err_centers(bp.cluster_centers_.larray.cpu(), ref) <= 1e-6
+
+
+def test_closest_rows_in_float64_resolves_exact_ties_like_the_reference(cuda):
+    """hkm_update_median_q64_f32 + hkm_closest_rows_l1_q64_f32: the medians before their rounding to
+    float32, and the snap in float64.  Clusters of two rows have their median at the midpoint, where
+    both rows are at exactly the same float64 distance: the first row must win (the reference's argmin),
+    whichever way float32 rounding would have tipped it."""
+    g = torch.Generator().manual_seed(9)
+    n_pairs, d = 300, 7
+    a = torch.randn((n_pairs, d), generator=g) * 5
+    b = a + torch.randn((n_pairs, d), generator=g)
+    x = torch.empty((2 * n_pairs, d))
+    x[0::2], x[1::2] = a, b                       # rows 2k and 2k + 1 form cluster k
+    lab = torch.arange(n_pairs).repeat_interleave(2).to(torch.int32)
+    ws = _native.Workspace(cuda)
+    xg = x.to(cuda)
+    med = torch.empty((n_pairs, d), device=cuda)
+    med64 = torch.empty((n_pairs, d), dtype=torch.float64, device=cuda)
+    _native.update_median(xg, lab.to(cuda), med, ws, skip_zero_rows=True, median64=med64)
+    want64 = a.double() + (b.double() - a.double()) * 0.5
+    lo, hi = torch.minimum(a, b).double(), torch.maximum(a, b).double()
+    assert torch.equal(med64.cpu(), lo + (hi - lo) * 0.5) and torch.allclose(med64.cpu(), want64, rtol=0, atol=1e-12)
+    assert torch.equal(med.cpu(), med64.cpu().float())
+    idx = torch.empty((n_pairs,), dtype=torch.int64, device=cuda)
+    dist = torch.empty((n_pairs,), dtype=torch.float64, device=cuda)
+    _native.closest_rows_l1_q64(xg, med64, idx, dist, ws)
+    ref = (x.double()[None, :, :] - med64.cpu()[:, None, :]).abs().sum(-1)   # (pairs, rows) in float64
+    assert torch.equal(idx.cpu(), ref.argmin(dim=1))
+    # the two members are equidistant, so the argmin is the even row unless a third row is closer
+    own = ref[torch.arange(n_pairs), 2 * torch.arange(n_pairs)]
+    mine = idx.cpu() // 2 == torch.arange(n_pairs)
+    assert int(mine.sum()) > n_pairs // 2 and bool((idx.cpu()[mine] % 2 == 0).all())
+    assert torch.allclose(dist.cpu(), ref.min(dim=1).values, rtol=1e-14, atol=0) and bool((dist.cpu() <= own).all())
+    # general case against a float64 evaluation: many rows, several splits of the data
+    x2 = torch.randn((50_000, 19), generator=g)
+    q = torch.randn((70, 19), generator=g, dtype=torch.float64)
+    idx2 = torch.empty((70,), dtype=torch.int64, device=cuda)
+    _native.closest_rows_l1_q64(x2.to(cuda), q.to(cuda), idx2, None, ws)
+    ref2 = torch.cdist(q, x2.double(), p=1.0)
+    assert torch.equal(idx2.cpu(), ref2.argmin(dim=1))
