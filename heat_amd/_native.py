@@ -60,6 +60,11 @@ SIGNATURES = {
                                                  c_void_p, c_size_t, c_void_p]),
     "hkm_closest_rows_l1_q64_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                                    c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_knn_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "hkm_knn_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p,
+                                   c_int64, c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
+    "hkm_knn_vote_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int64,
+                                        c_void_p, c_void_p]),
     "hkm_assign_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p]),
     "hkm_update_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
@@ -464,3 +469,45 @@ def update_median(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, ws
 def widen_labels(labels32: torch.Tensor, out64: torch.Tensor) -> None:
     _require_gpu(labels32, out64)
     check(load().hkm_widen_labels_i64(_ptr(labels32), labels32.numel(), _ptr(out64), _stream()))
+
+
+KNN_MAX_K = 1024  # HKM_KNN_MAX_K
+
+
+def knn(q: torch.Tensor, x: torch.Tensor, k: int, idx: torch.Tensor, dist: Optional[torch.Tensor],
+        ws: Workspace) -> None:
+    """idx[m, :k] = the k rows of x closest (Euclidean) to q[m], ascending in (distance, row index);
+    dist[m, :k] their distances (see hkm_knn_f32 in include/hkm.h)."""
+    _require_gpu(q, x, idx, dist)
+    _require_rows(q, x, idx, dist)
+    if q.dtype != torch.float32 or x.dtype != torch.float32:
+        raise TypeError("q and x must be float32")
+    if idx.dtype != torch.int64 or (dist is not None and dist.dtype != torch.float32):
+        raise TypeError("idx must be int64 and dist float32")
+    m, d = q.shape
+    n = x.shape[0]
+    if x.shape[1] != d:
+        raise ValueError(f"feature counts differ: {d} != {x.shape[1]}")
+    if tuple(idx.shape) != (m, k) or (dist is not None and tuple(dist.shape) != (m, k)):
+        raise ValueError(f"idx and dist must have shape ({m}, {k})")
+    lib = load()
+    buf = ws.get(lib.hkm_knn_workspace_bytes(m, n))
+    check(lib.hkm_knn_f32(_ptr(q), m, q.stride(0) if m > 1 else d, _ptr(x), n, x.stride(0) if n > 1 else d, d, k,
+                          _ptr(idx), idx.stride(0) if m > 1 else k, _ptr(dist),
+                          (dist.stride(0) if m > 1 else k) if dist is not None else k, _ptr(buf), buf.numel(),
+                          _stream()))
+
+
+def knn_vote(idx: torch.Tensor, y: torch.Tensor, classes: torch.Tensor) -> None:
+    """classes[m] = first index of the largest entry of the sum of the label rows y[idx[m, j]]
+    (see hkm_knn_vote_f32 in include/hkm.h)."""
+    _require_gpu(idx, y, classes)
+    _require_rows(idx, y)
+    if idx.dtype != torch.int64 or classes.dtype != torch.int64 or y.dtype != torch.float32:
+        raise TypeError("idx and classes must be int64, y float32")
+    m, k = idx.shape
+    n, c = y.shape
+    if classes.numel() != m or not classes.is_contiguous():
+        raise ValueError(f"classes must hold {m} contiguous entries")
+    check(load().hkm_knn_vote_f32(_ptr(idx), m, k, idx.stride(0) if m > 1 else k, _ptr(y), n, c,
+                                  y.stride(0) if n > 1 else c, _ptr(classes), _stream()))

@@ -1,6 +1,6 @@
 """
-Estimator protocol, mirroring heat/core/base.py:13-93 (BaseEstimator), :184-212 (ClusteringMixin)
-and :284-306 (is_estimator / is_clusterer).
+Estimator protocol, mirroring heat/core/base.py:13-93 (BaseEstimator), :96-140 (ClassificationMixin),
+:184-212 (ClusteringMixin) and :260-306 (is_classifier / is_estimator / is_clusterer).
 """
 
 from __future__ import annotations
@@ -58,6 +58,22 @@ class ClusteringMixin:
         return self.predict(x)
 
 
+class ClassificationMixin:
+    def fit(self, x, y):
+        raise NotImplementedError()
+
+    def fit_predict(self, x, y):
+        self.fit(x, y)
+        return self.predict(x)
+
+    def predict(self, x):
+        raise NotImplementedError()
+
+
+def is_classifier(obj: object) -> bool:
+    return isinstance(obj, ClassificationMixin)
+
+
 def is_estimator(obj: object) -> bool:
     return isinstance(obj, BaseEstimator)
 
@@ -66,4 +82,4 @@ def is_clusterer(obj: object) -> bool:
     return isinstance(obj, ClusteringMixin)
 
 
-__all__ = ["BaseEstimator", "ClusteringMixin", "is_estimator", "is_clusterer"]
+__all__ = ["BaseEstimator", "ClassificationMixin", "ClusteringMixin", "is_classifier", "is_estimator", "is_clusterer"]

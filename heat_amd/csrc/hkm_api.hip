@@ -572,6 +572,78 @@ int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ld
                                       static_cast<hipStream_t>(hip_stream));
 }
 
+struct KnnWorkspace {
+    float* last_d2;
+    unsigned* last_i;
+    float* part_d;
+    unsigned* part_i;
+    size_t total;
+};
+
+static KnnWorkspace carve_knn(void* base, int64_t M, int64_t N) {
+    KnnWorkspace w;
+    char* p = static_cast<char*>(base);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* r = p ? p + off : nullptr;
+        off += align_up(bytes, 256);
+        return r;
+    };
+    const size_t m = size_t(M < 1 ? 1 : M);
+    const size_t slots = knn_plan(M, N).part_slots;
+    w.last_d2 = reinterpret_cast<float*>(take(m * sizeof(float)));
+    w.last_i = reinterpret_cast<unsigned*>(take(m * sizeof(unsigned)));
+    w.part_d = reinterpret_cast<float*>(take((slots ? slots : 1) * sizeof(float)));
+    w.part_i = reinterpret_cast<unsigned*>(take((slots ? slots : 1) * sizeof(unsigned)));
+    w.total = off;
+    return w;
+}
+
+size_t hkm_knn_workspace_bytes(int64_t M, int64_t N) {
+    if (M < 0 || N < 1) return 0;
+    return carve_knn(nullptr, M, N).total;
+}
+
+int hkm_knn_f32(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx, int32_t D, int32_t k,
+                int64_t* idx, int64_t ldi, float* dist, int64_t ldd, void* ws, size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 0) return fail(HKM_EINVAL, "M = %lld is negative", (long long)M);
+    if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
+    if (N < 1) return fail(HKM_EINVAL, "N = %lld: there are no neighbours in an empty matrix", (long long)N);
+    if (N > 0xfffffffeLL) return fail(HKM_EUNSUPPORTED, "N = %lld exceeds 32-bit row indices", (long long)N);
+    if (k < 1 || k > N) return fail(HKM_EINVAL, "k = %d must be in [1, N = %lld]", k, (long long)N);
+    if (k > HKM_KNN_MAX_K) return fail(HKM_EUNSUPPORTED, "k = %d exceeds HKM_KNN_MAX_K = %d", k, HKM_KNN_MAX_K);
+    int rc;
+    if ((rc = check_matrix("Q", Q, M, D, ldq))) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if (!idx && M > 0) return fail(HKM_EINVAL, "idx is NULL");
+    if (ldi < k) return fail(HKM_EINVAL, "leading dimension of idx (%lld) < k (%d)", (long long)ldi, k);
+    if (dist && ldd < k) return fail(HKM_EINVAL, "leading dimension of dist (%lld) < k (%d)", (long long)ldd, k);
+    if (reinterpret_cast<uintptr_t>(idx) & 7u) return fail(HKM_EINVAL, "idx is not 8-byte aligned");
+    if (reinterpret_cast<uintptr_t>(dist) & 3u) return fail(HKM_EINVAL, "dist is not 4-byte aligned");
+    const size_t need = carve_knn(nullptr, M, N).total;
+    if ((rc = check_ws(ws, ws_bytes, need))) return rc;
+    const KnnWorkspace w = carve_knn(ws, M, N);
+    return launch_knn(Q, M, ldq, X, N, ldx, D, k, idx, ldi, dist, ldd, w.last_d2, w.last_i, w.part_d, w.part_i,
+                      static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_knn_vote_f32(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
+                     int64_t ldy, int64_t* classes, void* hip_stream) {
+    g_err[0] = 0;
+    if (M < 0) return fail(HKM_EINVAL, "M = %lld is negative", (long long)M);
+    if (k < 1) return fail(HKM_EINVAL, "k = %d must be >= 1", k);
+    if (C < 1) return fail(HKM_EINVAL, "C = %d must be >= 1", C);
+    if (N < 1) return fail(HKM_EINVAL, "N = %lld must be >= 1", (long long)N);
+    if (ldi < k) return fail(HKM_EINVAL, "leading dimension of idx (%lld) < k (%d)", (long long)ldi, k);
+    int rc;
+    if ((rc = check_matrix("Y", Y, N, C, ldy))) return rc;
+    if (M > 0 && (!idx || !classes)) return fail(HKM_EINVAL, "idx or classes is NULL");
+    if ((reinterpret_cast<uintptr_t>(idx) | reinterpret_cast<uintptr_t>(classes)) & 7u)
+        return fail(HKM_EINVAL, "idx or classes is not 8-byte aligned");
+    return launch_knn_vote(idx, M, k, ldi, Y, N, C, ldy, classes, static_cast<hipStream_t>(hip_stream));
+}
+
 static int update_median_common(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels, int32_t K,
                                 const int64_t* fallback_rows, const float* C_old, float* C_new, int64_t ldcn,
                                 int64_t* counts, int32_t mode, int32_t skip_zero_rows, double* medians_f64, void* ws,

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stddef.h>
+#include <algorithm>
 #include <stdint.h>
 
 #include "hkm.h"
@@ -237,5 +238,19 @@ int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, cons
 int launch_widen(const int32_t* in, int64_t N, int64_t* out, hipStream_t st);
 
 int num_cus();
+
+// k nearest rows (hkm_knn.hip).  The split of the reference rows over workgroups and the scratch it needs
+// follow from the two row counts alone, so that the workspace can be sized before the call.
+struct KnnPlan {
+    int nsplit;
+    int64_t rows_per_split;
+    size_t part_slots;  // (distance, row) pairs of the per-split lists; 0 when one split covers all rows
+};
+KnnPlan knn_plan(int64_t M, int64_t N);
+int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx, int32_t D, int32_t k,
+               int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* last_d2, unsigned* last_i, float* part_d,
+               unsigned* part_i, hipStream_t st);
+int launch_knn_vote(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
+                    int64_t ldy, int64_t* classes, hipStream_t st);
 
 }  // namespace hkm

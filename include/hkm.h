@@ -244,6 +244,30 @@ int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ld
                                 int64_t* idx, double* dist, void* ws, size_t ws_bytes, void* hip_stream);
 
 /*
+ * k nearest rows and their label vote: the predict chain of the k-nearest-neighbours classifier,
+ *   distances = cdist(x, self.x); _, indices = topk(distances, k, largest=False);
+ *   classes = argmax(sum(self.y[indices], axis=1), axis=1)
+ * heat/classification/kneighborsclassifier.py:114-132 (heat/spatial/distance.py:17-29 for the metric,
+ * heat/core/manipulations.py `topk` for the selection), without the M x N distance matrix.
+ *
+ * hkm_knn_f32: for every row of Q (M x D) the k closest rows of X (N x D) in the Euclidean metric:
+ *   idx (M x k int64, leading dimension ldi) in ascending order of (distance, row index) -- of rows at
+ *   exactly the same squared distance the smaller index comes first -- and, if dist is not NULL, the
+ *   distances themselves (M x k float32, leading dimension ldd).  Squared distances are summed directly
+ *   as sum (q - x)^2 in fp32, the square root is correctly rounded.  A slot for which no finite distance
+ *   is left (NaN or overflowing rows) holds index -1 and distance inf.  1 <= k <= min(N, HKM_KNN_MAX_K).
+ *   ws needs hkm_knn_workspace_bytes(M, N) bytes.
+ * hkm_knn_vote_f32: classes[m] = the first index of the largest entry of sum_j Y[idx[m][j]] (Y: N x C
+ *   float32 label rows, one-hot or weights; the neighbours are added in their order; index -1 is skipped).
+ */
+#define HKM_KNN_MAX_K 1024
+size_t hkm_knn_workspace_bytes(int64_t M, int64_t N);
+int hkm_knn_f32(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx, int32_t D, int32_t k,
+                int64_t* idx, int64_t ldi, float* dist, int64_t ldd, void* ws, size_t ws_bytes, void* hip_stream);
+int hkm_knn_vote_f32(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
+                     int64_t ldy, int64_t* classes, void* hip_stream);
+
+/*
  * float64 data.  The reference keeps float64 inputs in float64 through the same op sequence
  * (promote(X, Y, float32), heat/spatial/distance.py:392-403; heat/cluster/kmeans.py:76-148), so these
  * mirror the *_f32 entry points of the same name with double operands: quadratic-expansion distance +

@@ -55,6 +55,11 @@ Pins (what each function is checked against, see tests/test_oracle_pins.py):
   minimal Manhattan distance from the median), K = 1 closed form (the coordinate-wise median after
   one iteration), and the reference's own assertion that every medoid is a data point
   (``tests/cluster/test_kmedoids.py:44-48``).  End-to-end numbers: parity unpinned, as for KMeans.
+* knn_one_hot / knn_predict (k-nearest-neighbours classifier): the one-hot known answer of
+  ``tests/classification/test_knn.py:69-76``; scikit-learn's brute-force ``KNeighborsClassifier`` and
+  ``NearestNeighbors`` (neighbour sets and classes on the iris data and on random blobs); a python
+  sort of float64 distances on a tiny input; k = 1 on the training rows returns every row itself.
+  The reference stores no predicted class anywhere (``test_knn.py`` asserts types and shapes).
 """
 
 from __future__ import annotations
@@ -715,3 +720,54 @@ def label_agreement_l1(x: torch.Tensor, centers: torch.Tensor, lab_a: torch.Tens
         da, db = d.gather(1, a[diff].view(-1, 1)).view(-1), d.gather(1, b[diff].view(-1, 1)).view(-1)
         out["n_unexcused"] = int(((da - best > tol) | (db - best > tol)).sum())
     return out
+
+
+# --------------------------------------------------------------------------------------------------
+# k-nearest-neighbours classifier
+# --------------------------------------------------------------------------------------------------
+def knn_one_hot(labels: torch.Tensor) -> torch.Tensor:
+    """heat/classification/kneighborsclassifier.py:44-61: float32 (n, max + 1), one 1 per row."""
+    lab = labels.reshape(-1).long()
+    n_features = int(lab.max().item()) + 1
+    one_hot = torch.zeros((lab.shape[0], n_features), dtype=torch.float32)
+    one_hot[range(lab.shape[0]), lab] = 1
+    return one_hot
+
+
+def knn_predict(x_train: torch.Tensor, y: torch.Tensor, x_test: torch.Tensor, n_neighbors: int):
+    """
+    heat/classification/kneighborsclassifier.py:114-132 at one rank: ``cdist`` with its default
+    ``quadratic_expansion=False`` is ``torch.cdist`` (heat/spatial/distance.py:17-29), ``ht.topk`` is
+    ``torch.topk(..., largest=False, sorted=True)`` on the local matrix, the label rows of the neighbours
+    are summed over the neighbour axis and the first largest entry is the class.
+    Returns (classes, indices, distances).
+    """
+    y2 = knn_one_hot(y) if y.dim() == 1 else y
+    distances = torch.cdist(x_test, x_train)
+    values, indices = torch.topk(distances, n_neighbors, dim=-1, largest=False, sorted=True)
+    predictions = y2[indices.flatten()]
+    predictions = predictions.reshape(tuple(indices.shape) + (y2.shape[1],))
+    predictions = torch.sum(predictions, dim=1)
+    return torch.argmax(predictions, dim=1), indices, values
+
+
+def knn_neighbours_f64(x_train: torch.Tensor, x_test: torch.Tensor, n_neighbors: int, chunk: int = 2048):
+    """The k + 1 smallest float64 distances of every test row and their rows, ascending in distance (rows
+    at exactly the same distance in no particular order): what a neighbour list is judged against.
+    Candidates are chosen with the float64 expansion |q|^2 + |x|^2 - 2 q.x (a plain matrix product, safe
+    at any size), their distances are then recomputed directly as sqrt(sum (q - x)^2).
+    Returns (distances (m, k + 1), rows)."""
+    xt, xq = x_train.double(), x_test.double()
+    kk = min(n_neighbors + 1, xt.shape[0])
+    wide = min(kk + 2, xt.shape[0])
+    xn = (xt * xt).sum(1)
+    out_d, out_i = [], []
+    for a in range(0, xq.shape[0], chunk):
+        qa = xq[a:a + chunk]
+        d2 = (qa * qa).sum(1, keepdim=True) + xn[None, :] - 2.0 * (qa @ xt.T)
+        _, cand = torch.topk(d2, wide, dim=1, largest=False, sorted=True)
+        direct = (qa[:, None, :] - xt[cand]).pow(2).sum(-1).sqrt()
+        vals, pos = torch.sort(direct, dim=1, stable=True)
+        out_d.append(vals[:, :kk])
+        out_i.append(torch.gather(cand, 1, pos)[:, :kk])
+    return torch.cat(out_d), torch.cat(out_i)

@@ -349,3 +349,27 @@ def test_load_csv():
         ht.load("data.txt")
     with pytest.raises(RuntimeError):
         ht.load("data.h5")
+
+
+def test_knn_classifier_surface():
+    """tests/classification/test_knn.py:50-76 of the reference: the exception matrix of fit and the one-hot
+    utility, plus the estimator protocol.  No kernel runs."""
+    knn_cls = ht.classification.KNeighborsClassifier
+    a, b, c = ht.zeros((3,)), ht.zeros((3, 2)), ht.zeros((2, 2, 2))
+    for x, y in ((a, b), (b, c), (c, a)):
+        with pytest.raises(ValueError):
+            knn_cls(n_neighbors=1).fit(x, y)
+    with pytest.raises(TypeError):
+        knn_cls().fit(torch.zeros((3, 2)), b)
+    one_hot = knn_cls.one_hot_encoding(ht.array([1, 2, 3, 4]))
+    want = torch.tensor([[0, 1, 0, 0, 0], [0, 0, 1, 0, 0], [0, 0, 0, 1, 0], [0, 0, 0, 0, 1]], dtype=torch.float32)
+    assert torch.equal(one_hot.larray, want)
+    knn = knn_cls(n_neighbors=3)
+    assert ht.is_estimator(knn) and ht.is_classifier(knn) and not ht.is_clusterer(knn)
+    assert knn.get_params()["n_neighbors"] == 3 and knn.get_params()["effective_metric_"] is ht.spatial.cdist
+    with pytest.raises(RuntimeError):
+        knn.predict(b)
+    with pytest.raises(NotImplementedError):
+        other = knn_cls(effective_metric_=ht.spatial.manhattan)
+        other.fit(b, ht.zeros((3,)))
+        other.predict(b)

@@ -4,6 +4,7 @@ NOT written from -- the known-answer vectors of the reference's own tests, close
 force in fp64, library routines (torch.cdist, torch.argmin, scikit-learn's Lloyd) -- chosen so
 that a dropped term, a wrong sign or a transposed operand fails.
 """
+import math
 import os
 
 import numpy as np
@@ -426,3 +427,46 @@ def test_inverse_cdf_sampler_draws_the_given_distribution():
     assert freq[1] == 0
     assert torch.allclose(freq, (w / w.sum()).double(), atol=0.012)
     assert s.randint(99) == 0
+
+
+def test_knn_oracle_against_scikit_learn_and_a_python_sort():
+    """knn_one_hot / knn_predict: the one-hot known answer of the reference's tests/classification/
+    test_knn.py:69-76, scikit-learn's brute-force neighbours and classes, a python sort, k = 1."""
+    from sklearn.neighbors import KNeighborsClassifier, NearestNeighbors
+
+    want = torch.tensor([[0, 1, 0, 0, 0], [0, 0, 1, 0, 0], [0, 0, 0, 1, 0], [0, 0, 0, 0, 1]], dtype=torch.float32)
+    assert torch.equal(orc.knn_one_hot(torch.tensor([1, 2, 3, 4])), want)
+
+    iris = torch.from_numpy(np.loadtxt(os.path.join(GOLD, "iris.csv"), delimiter=";", dtype=np.float32))
+    y = torch.zeros(150, dtype=torch.int64)
+    y[50:100], y[100:] = 1, 2
+    g = torch.Generator().manual_seed(5)
+    blobs_c = torch.randn((6, 9), generator=g) * 4
+    lab = torch.randint(0, 6, (700,), generator=g)
+    blobs = blobs_c[lab] + torch.randn((700, 9), generator=g)
+    queries = blobs_c[torch.randint(0, 6, (90,), generator=g)] + torch.randn((90, 9), generator=g)
+    for train, labels, test, k in ((iris, y, iris, 5), (blobs, lab, queries, 7), (blobs, lab, queries, 1)):
+        cls, idx, dist = orc.knn_predict(train, labels, test, k)
+        sk = KNeighborsClassifier(n_neighbors=k, algorithm="brute").fit(train.numpy(), labels.numpy())
+        nn_d, nn_i = NearestNeighbors(n_neighbors=k, algorithm="brute").fit(train.double().numpy()).kneighbors(
+            test.double().numpy())
+        # neighbours: the same distances (torch.cdist expands the square above 25 rows: compare squares at
+        # the fp32 resolution of the squared norms); the same rows wherever no two candidates come close
+        assert np.allclose(dist.double().numpy() ** 2, nn_d ** 2, rtol=1e-4, atol=2e-4)
+        d64, _ = orc.knn_neighbours_f64(train, test, k)
+        clear = (d64[:, 1:] - d64[:, :-1]).min(dim=1).values > 1e-3
+        assert int(clear.sum()) > 0.5 * test.shape[0] or train is iris
+        assert np.array_equal(np.sort(idx.numpy()[clear.numpy()], axis=1), np.sort(nn_i[clear.numpy()], axis=1))
+        # classes: scikit-learn's vote (mode, smallest label on ties) on rows whose neighbour set is unambiguous
+        assert np.array_equal(cls.numpy()[clear.numpy()], sk.predict(test.numpy())[clear.numpy()])
+    # python sort of float64 distances on a tiny input
+    tr = torch.tensor([[0.0, 0.0], [1.0, 0.0], [0.0, 2.0], [5.0, 5.0], [1.0, 1.0]])
+    te = torch.tensor([[0.1, 0.1], [4.0, 4.0]])
+    cls, idx, dist = orc.knn_predict(tr, torch.tensor([0, 0, 1, 1, 1]), te, 3)
+    for m in range(2):
+        order = sorted(range(5), key=lambda j: math.dist(te[m].tolist(), tr[j].tolist()))[:3]
+        assert idx[m].tolist() == order
+    assert cls.tolist() == [0, 1]
+    # k = 1 on the training rows: every row is its own neighbour (distinct rows)
+    cls, idx, dist = orc.knn_predict(blobs, lab, blobs, 1)
+    assert torch.equal(idx.view(-1), torch.arange(700)) and torch.equal(cls, lab)
