@@ -573,6 +573,7 @@ int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ld
 }
 
 struct KnnWorkspace {
+    float* xn;  // squared norms of the reference rows, padded to a whole tile
     float* last_d2;
     unsigned* last_i;
     float* part_d;
@@ -591,6 +592,7 @@ static KnnWorkspace carve_knn(void* base, int64_t M, int64_t N) {
     };
     const size_t m = size_t(M < 1 ? 1 : M);
     const size_t slots = knn_plan(M, N).part_slots;
+    w.xn = reinterpret_cast<float*>(take((size_t(N < 1 ? 1 : N) + 64) * sizeof(float)));
     w.last_d2 = reinterpret_cast<float*>(take(m * sizeof(float)));
     w.last_i = reinterpret_cast<unsigned*>(take(m * sizeof(unsigned)));
     w.part_d = reinterpret_cast<float*>(take((slots ? slots : 1) * sizeof(float)));
@@ -624,7 +626,7 @@ int hkm_knn_f32(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t 
     const size_t need = carve_knn(nullptr, M, N).total;
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const KnnWorkspace w = carve_knn(ws, M, N);
-    return launch_knn(Q, M, ldq, X, N, ldx, D, k, idx, ldi, dist, ldd, w.last_d2, w.last_i, w.part_d, w.part_i,
+    return launch_knn(Q, M, ldq, X, N, ldx, D, k, idx, ldi, dist, ldd, w.xn, w.last_d2, w.last_i, w.part_d, w.part_i,
                       static_cast<hipStream_t>(hip_stream));
 }
 

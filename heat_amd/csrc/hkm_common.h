@@ -248,8 +248,9 @@ struct KnnPlan {
 };
 KnnPlan knn_plan(int64_t M, int64_t N);
 int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx, int32_t D, int32_t k,
-               int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* last_d2, unsigned* last_i, float* part_d,
-               unsigned* part_i, hipStream_t st);
+               int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* xn, float* last_d2, unsigned* last_i,
+               float* part_d, unsigned* part_i, hipStream_t st);
+bool knn_uses_mfma(int32_t D);
 int launch_knn_vote(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
                     int64_t ldy, int64_t* classes, hipStream_t st);
 

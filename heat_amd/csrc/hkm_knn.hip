@@ -5,16 +5,25 @@
 //     tiles of 64 (4 x 4 register block per lane, both tiles staged through LDS in chunks of 16
 //     features, sum (q - r)^2 in fp32 -- the direct form, no cancellation).  Every lane keeps the KL
 //     best (distance, row) pairs of its four query rows, sorted, in registers; a candidate is only
-//     looked at when it beats the row's threshold, the smallest KL-th entry among the 16 lanes that
-//     share the row (that lane alone holds KL closer rows, so nothing above it can rank).  At the end
+//     looked at when it beats the row's threshold, the smallest k-th entry among the 16 lanes that
+//     share the row (that lane alone holds k closer rows, so nothing above it can rank).  At the end
 //     the 16 lists of a row are merged with shuffles.  Reference rows can be split over several
 //     workgroups (grid.y); their lists are merged by knn_merge_kernel.  More than KL neighbours are
 //     found in passes: a pass only admits pairs that rank after the last pair of the pass before.
 //   * order: ascending (squared distance, row index) -- the first row wins exact ties.
 //   * knn_vote_kernel: sum of the label rows of the k neighbours, argmax with the first class on ties.
 //
-// Bound: the vector ALU, 2 operations (subtract, fused multiply-add) per (query, row, feature).
-#include "hkm_common.h"
+//   * knn_mfma_kernel (16 <= D <= 128): the same walk with the products q.x on the matrix cores and the
+//     squared distance as (|q|^2 + |x|^2) - 2 q.x clamped at zero, the form torch.cdist itself takes above
+//     25 rows.  A wave owns 32 query rows, held in registers for the whole kernel; a tile of 32 reference
+//     rows goes from global memory straight into the A operand (lane = row, half of the features each:
+//     the order of the features inside the sum is free as long as both operands agree), 32x32x2 fp32
+//     MFMAs leave every lane with 16 candidates of ONE query row, so a lane keeps one list and the
+//     two lanes of a query row merge at the end.  |x|^2 comes from knn_norms_kernel.
+//
+// Bound: knn_tile_kernel the vector ALU, 2 operations (subtract, fused multiply-add) per (query, row,
+// feature); knn_mfma_kernel the fp32 matrix cores, 2 flops per (query, row, feature).
+#include "hkm_mfma_util.h"
 
 namespace hkm {
 
@@ -39,6 +48,14 @@ __device__ __forceinline__ void knn_insert(float (&ld)[KL], unsigned (&li)[KL], 
         ld[s] = nd;
         li[s] = ni;
     }
+}
+
+// The lists live in registers and must be updated in place: a branch per lane around the insertion makes
+// the compiler copy a whole list at every candidate, so the branch is taken by the wave as a whole (any
+// lane with a hit) and lanes without one insert +inf, which changes nothing.
+template <int KL>
+__device__ __forceinline__ void knn_offer(float (&ld)[KL], unsigned (&li)[KL], bool ok, float d, unsigned i) {
+    if (__builtin_amdgcn_ballot_w64(ok) != 0) knn_insert<KL>(ld, li, ok ? d : HKM_INF, i);
 }
 
 template <int KL>
@@ -115,6 +132,8 @@ __global__ __launch_bounds__(256) void knn_tile_kernel(
             // candidate of this one: a candidate at exactly the threshold ranks after KL entries
             float thr = ld[a][KL - 1];
 #pragma unroll
+            for (int s = 0; s < KL - 1; ++s) thr = s == kcount - 1 ? ld[a][s] : thr;  // only kcount entries are asked for
+#pragma unroll
             for (int w = 1; w < 16; w <<= 1) thr = fminf(thr, __shfl_xor(thr, w));
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
@@ -122,7 +141,7 @@ __global__ __launch_bounds__(256) void knn_tile_kernel(
                 const float d = acc[a][b];
                 bool ok = gj < r_end && d < thr;
                 if (has_bound) ok = ok && (d > bd[a] || (d == bd[a] && unsigned(gj) > bi[a]));
-                if (ok) knn_insert<KL>(ld[a], li[a], d, unsigned(gj));
+                knn_offer<KL>(ld[a], li[a], ok, d, unsigned(gj));
             }
         }
     }
@@ -170,6 +189,273 @@ __global__ __launch_bounds__(256) void knn_tile_kernel(
             }
         }
     }
+}
+
+// ---- shared by the two matrix-core kernels -------------------------------------------------------
+// candidates of one 32 x 32 block: accumulator element i is reference row j0 + 8 (i / 4) + 4 h + i % 4
+template <int KL>
+__device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (&li)[KL], const floatx16& acc,
+                                                     const floatx16& xnv, float qn, int64_t j0, int h, int64_t r_end,
+                                                     int kcount, int has_bound, float bd, unsigned bi) {
+    // pairs in the lists stem from earlier tiles, i.e. from smaller rows than any candidate here; a
+    // candidate at exactly the threshold ranks after kcount of them
+    float thr = ld[KL - 1];
+#pragma unroll
+    for (int s = 0; s < KL - 1; ++s) thr = s == kcount - 1 ? ld[s] : thr;  // only kcount entries are asked for
+    thr = fminf(thr, __shfl_xor(thr, 32));
+    const unsigned gj0 = unsigned(j0) + 4 * h;
+    if (j0 + 32 <= r_end && !has_bound) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float d = fmaxf(fmaf(-2.0f, acc[i], qn + xnv[i]), 0.0f);
+            knn_offer<KL>(ld, li, d < thr, d, gj0 + 8 * (i >> 2) + (i & 3));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const unsigned gj = gj0 + 8 * (i >> 2) + (i & 3);
+            const float d = fmaxf(fmaf(-2.0f, acc[i], qn + xnv[i]), 0.0f);
+            bool ok = gj < unsigned(r_end) && d < thr;
+            if (has_bound) ok = ok && (d > bd || (d == bd && gj > bi));
+            knn_offer<KL>(ld, li, ok, d, gj);
+        }
+    }
+}
+
+// The two lanes of a query row (h = 0, 1): KL times the smaller head, whose lane pops it; lane h = 0
+// writes -- the final output when one split covers all rows, else the split's list for knn_merge_kernel.
+template <int KL>
+__device__ __forceinline__ void knn_pair_merge_write(float (&ld)[KL], unsigned (&li)[KL], int kcount, int h, bool live,
+                                                     int64_t gi, int64_t M, bool final_out, float* last_d2,
+                                                     unsigned* last_i, float* part_d, unsigned* part_i, int64_t* out_i,
+                                                     int64_t ldi, float* out_d, int64_t ldd, int col0) {
+#pragma unroll
+    for (int r = 0; r < KL; ++r) {
+        const float od = __shfl_xor(ld[0], 32);
+        const unsigned oi = unsigned(__shfl_xor(int(li[0]), 32));
+        const bool other = knn_less(od, oi, ld[0], li[0]);
+        const float md = other ? od : ld[0];
+        const unsigned mi = other ? oi : li[0];
+        if (!other && mi != KNN_NONE) {
+#pragma unroll
+            for (int s = 0; s + 1 < KL; ++s) {
+                ld[s] = ld[s + 1];
+                li[s] = li[s + 1];
+            }
+            ld[KL - 1] = HKM_INF;
+            li[KL - 1] = KNN_NONE;
+        }
+        if (h == 0 && live) {
+            if (final_out) {
+                if (r < kcount) {
+                    out_i[gi * ldi + col0 + r] = mi == KNN_NONE ? int64_t(-1) : int64_t(mi);
+                    if (out_d) out_d[gi * ldd + col0 + r] = sqrtf(md);
+                    if (r == kcount - 1) {
+                        last_d2[gi] = md;
+                        last_i[gi] = mi;
+                    }
+                }
+            } else {
+                part_d[(int64_t(blockIdx.y) * M + gi) * KL + r] = md;
+                part_i[(int64_t(blockIdx.y) * M + gi) * KL + r] = mi;
+            }
+        }
+    }
+}
+
+// |x|^2 of every reference row: 16 lanes per row, features strided over the lanes, fixed-order tree.
+__global__ __launch_bounds__(256) void knn_norms_kernel(const float* __restrict__ R, int64_t Nn, int64_t ldr, int D,
+                                                        float* __restrict__ xn) {
+    const int t = threadIdx.x & 15;
+    const int64_t row = int64_t(blockIdx.x) * 16 + (threadIdx.x >> 4);
+    float s = 0.0f;
+    if (row < Nn)
+        for (int d = t; d < D; d += 16) {
+            const float v = R[row * ldr + d];
+            s = fmaf(v, v, s);
+        }
+#pragma unroll
+    for (int w = 1; w < 16; w <<= 1) s += __shfl_xor(s, w);
+    if (t == 0 && row < Nn) xn[row] = s;
+}
+
+// H features per lane: lanes 0..31 hold features [0, H) of their row, lanes 32..63 features [H, 2H).
+template <int KL, int H, bool VEC>
+__global__ __launch_bounds__(256) void knn_mfma_kernel(
+    const float* __restrict__ Q, int64_t M, int64_t ldq, const float* __restrict__ R, int64_t Nn, int64_t ldr,
+    int D, const float* __restrict__ xn, int64_t rows_per_split, int has_bound, float* __restrict__ last_d2,
+    unsigned* __restrict__ last_i, float* __restrict__ part_d, unsigned* __restrict__ part_i,
+    int64_t* __restrict__ out_i, int64_t ldi, float* __restrict__ out_d, int64_t ldd, int col0, int kcount) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int64_t gi = int64_t(blockIdx.x) * 128 + wave * 32 + col;
+    const bool live = gi < M;
+    const int64_t r_begin = int64_t(blockIdx.y) * rows_per_split;
+    const int64_t r_end = min(Nn, r_begin + rows_per_split);
+
+    float qv[H];
+    float qn = 0.0f;
+    {
+        const float* qrow = Q + (live ? gi : 0) * ldq;
+#pragma unroll
+        for (int g = 0; g < H / 4; ++g) {
+            const floatx4 t = load_row4<VEC>(qrow, h * H + 4 * g, D);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                qv[4 * g + e] = live ? t[e] : 0.0f;
+                qn = fmaf(qv[4 * g + e], qv[4 * g + e], qn);
+            }
+        }
+        qn += __shfl_xor(qn, 32);
+    }
+
+    float ld[KL];
+    unsigned li[KL];
+#pragma unroll
+    for (int s = 0; s < KL; ++s) {
+        ld[s] = HKM_INF;
+        li[s] = KNN_NONE;
+    }
+    float bd = -1.0f;
+    unsigned bi = 0;
+    if (has_bound && live) {
+        bd = last_d2[gi];
+        bi = last_i[gi];
+    }
+
+    auto load_tile = [&](int64_t j0, float (&av)[H]) {
+        const int64_t gj = min(j0 + col, Nn - 1);  // rows past the end are read as the last row and never admitted
+        const float* row = R + gj * ldr;
+#pragma unroll
+        for (int g = 0; g < H / 4; ++g) {
+            const floatx4 t = load_row4<VEC>(row, h * H + 4 * g, D);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) av[4 * g + e] = t[e];
+        }
+    };
+
+    float av[H];
+    load_tile(r_begin, av);
+    for (int64_t j0 = r_begin; j0 < r_end; j0 += 32) {
+        float an[H];
+        load_tile(min(j0 + 32, r_end - 1), an);  // the next tile while this one is multiplied
+        const floatx16 xnv = load_cn16(xn + j0 + 4 * h);
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < H; ++s) acc = MFMA32(av[s], qv[s], acc);
+        knn_block_candidates<KL>(ld, li, acc, xnv, qn, j0, h, r_end, kcount, has_bound, bd, bi);
+#pragma unroll
+        for (int s = 0; s < H; ++s) av[s] = an[s];
+    }
+
+    knn_pair_merge_write<KL>(ld, li, kcount, h, live, gi, M, gridDim.y == 1, last_d2, last_i, part_d, part_i, out_i, ldi,
+                             out_d, ldd, col0);
+}
+
+// The same kernel with the tile of reference rows staged through LDS: one coalesced read per workgroup
+// (D % 4 == 0, 16-byte aligned rows) instead of one strided read per wave, double-buffered, one barrier
+// per tile.  Columns from D on are zeroed once and never written.
+template <int KL, int H>
+__global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
+    const float* __restrict__ Q, int64_t M, int64_t ldq, const float* __restrict__ R, int64_t Nn, int64_t ldr,
+    int D, const float* __restrict__ xn, int64_t rows_per_split, int has_bound, float* __restrict__ last_d2,
+    unsigned* __restrict__ last_i, float* __restrict__ part_d, unsigned* __restrict__ part_i,
+    int64_t* __restrict__ out_i, int64_t ldi, float* __restrict__ out_d, int64_t ldd, int col0, int kcount) {
+    constexpr int RS = 2 * H + 4;            // floats per staged row; the pad spreads 16 rows over all banks
+    constexpr int NV = H >= 16 ? H / 16 : 1;  // float4 groups a thread moves per tile
+    __shared__ __attribute__((aligned(16))) float sA[2][32][RS];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, h = lane >> 5;
+    const int64_t gi = int64_t(blockIdx.x) * 128 + wave * 32 + col;
+    const bool live = gi < M;
+    const int64_t r_begin = int64_t(blockIdx.y) * rows_per_split;
+    const int64_t r_end = min(Nn, r_begin + rows_per_split);
+
+    for (int i = tid; i < 2 * 32 * RS; i += 256) (&sA[0][0][0])[i] = 0.0f;
+
+    float qv[H];
+    float qn = 0.0f;
+    {
+        const float* qrow = Q + (live ? gi : 0) * ldq;
+#pragma unroll
+        for (int g = 0; g < H / 4; ++g) {
+            const floatx4 t = load_row4<true>(qrow, h * H + 4 * g, D);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                qv[4 * g + e] = live ? t[e] : 0.0f;
+                qn = fmaf(qv[4 * g + e], qv[4 * g + e], qn);
+            }
+        }
+        qn += __shfl_xor(qn, 32);
+    }
+
+    float ld[KL];
+    unsigned li[KL];
+#pragma unroll
+    for (int s = 0; s < KL; ++s) {
+        ld[s] = HKM_INF;
+        li[s] = KNN_NONE;
+    }
+    float bd = -1.0f;
+    unsigned bi = 0;
+    if (has_bound && live) {
+        bd = last_d2[gi];
+        bi = last_i[gi];
+    }
+
+    // which float4 groups of a tile this thread moves: group t + 256 j of the 32 x D/4 groups, row-major
+    const int c4n = D >> 2;
+    int srow[NV], scol[NV];
+    bool sval[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int idx = tid + 256 * j;
+        srow[j] = idx / c4n;
+        scol[j] = 4 * (idx - srow[j] * c4n);
+        sval[j] = idx < 32 * c4n;
+    }
+    floatx4 st[NV];
+    auto fetch = [&](int64_t j0) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            if (sval[j]) st[j] = ld4(R + min(j0 + srow[j], Nn - 1) * ldr + scol[j]);  // rows past the end: never admitted
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            if (sval[j]) *reinterpret_cast<floatx4*>(&sA[buf][srow[j]][scol[j]]) = st[j];
+    };
+    __syncthreads();
+    fetch(r_begin);
+    stash(0);
+    __syncthreads();
+
+    int buf = 0;
+    for (int64_t j0 = r_begin; j0 < r_end; j0 += 32) {
+        const bool more = j0 + 32 < r_end;
+        if (more) fetch(j0 + 32);  // the next tile while this one is multiplied
+        const floatx16 xnv = load_cn16(xn + j0 + 4 * h);
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+        const float* arow = &sA[buf][col][h * H];
+#pragma unroll
+        for (int g = 0; g < H / 4; ++g) {
+            const floatx4 a = *reinterpret_cast<const floatx4*>(arow + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc = MFMA32(a[e], qv[4 * g + e], acc);
+        }
+        knn_block_candidates<KL>(ld, li, acc, xnv, qn, j0, h, r_end, kcount, has_bound, bd, bi);
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    knn_pair_merge_write<KL>(ld, li, kcount, h, live, gi, M, gridDim.y == 1, last_d2, last_i, part_d, part_i, out_i, ldi,
+                             out_d, ldd, col0);
 }
 
 // One wave per query row: kcount times the smallest (distance, row) pair after the one before among the
@@ -269,8 +555,10 @@ __global__ __launch_bounds__(256) void knn_vote_kernel(const int64_t* __restrict
 // ------------------------------------------------------------------------------------------------
 KnnPlan knn_plan(int64_t M, int64_t N) {
     KnnPlan p;
-    const int64_t qtiles = (M + KNN_T - 1) / KNN_T;
-    int64_t ns = qtiles > 0 ? (2048 + qtiles - 1) / qtiles : 1;
+    const int64_t qtiles = (M + 127) / 128;  // the larger of the two kernels' query tiles
+    // every workgroup pays for filling its lists before its threshold bites, so no more splits than it
+    // takes to give each CU three workgroups
+    int64_t ns = qtiles > 0 ? (768 + qtiles - 1) / qtiles : 1;
     ns = std::min<int64_t>(ns, std::max<int64_t>(1, N / 256));
     ns = std::max<int64_t>(1, std::min<int64_t>(ns, KNN_MAX_SPLITS));
     int64_t rps = ((N + ns - 1) / ns + KNN_T - 1) / KNN_T * KNN_T;
@@ -292,26 +580,71 @@ static void knn_launch_tiles(const float* Q, int64_t M, int64_t ldq, const float
                        col0, kcount);
 }
 
+template <int KL, int H>
+static void knn_launch_mfma(bool vec, const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx,
+                            int D, const float* xn, const KnnPlan& p, int has_bound, float* last_d2, unsigned* last_i,
+                            float* part_d, unsigned* part_i, int64_t* idx, int64_t ldi, float* dist, int64_t ldd,
+                            int col0, int kcount, hipStream_t st) {
+    const dim3 grid((unsigned)((M + 127) / 128), (unsigned)p.nsplit);
+    if (vec)
+        hipLaunchKernelGGL((knn_mfma_lds_kernel<KL, H>), grid, dim3(256), 0, st, Q, M, ldq, X, N, ldx, D, xn,
+                           p.rows_per_split, has_bound, last_d2, last_i, part_d, part_i, idx, ldi, dist, ldd, col0,
+                           kcount);
+    else
+        hipLaunchKernelGGL((knn_mfma_kernel<KL, H, false>), grid, dim3(256), 0, st, Q, M, ldq, X, N, ldx, D, xn,
+                           p.rows_per_split, has_bound, last_d2, last_i, part_d, part_i, idx, ldi, dist, ldd, col0,
+                           kcount);
+}
+
+bool knn_uses_mfma(int32_t D) { return D >= 16 && D <= 128; }
+
 int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx, int32_t D, int32_t k,
-               int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* last_d2, unsigned* last_i, float* part_d,
-               unsigned* part_i, hipStream_t st) {
+               int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* xn, float* last_d2, unsigned* last_i,
+               float* part_d, unsigned* part_i, hipStream_t st) {
     if (M == 0) return HKM_OK;
     const KnnPlan p = knn_plan(M, N);
-    const int KL = k <= 4 ? 4 : (k <= 8 ? 8 : 16);
+    const bool mfma = knn_uses_mfma(D);
+    const int KL = mfma ? (k <= 8 ? 8 : 16) : (k <= 4 ? 4 : (k <= 8 ? 8 : 16));
+    int rc;
+    if (mfma) {
+        hipLaunchKernelGGL(knn_norms_kernel, dim3((unsigned)((N + 15) / 16)), dim3(256), 0, st, X, N, ldx, D, xn);
+        if ((rc = check_launch("knn_norms_kernel"))) return rc;
+    }
+    const bool vec = D % 4 == 0 && ldq % 4 == 0 && ldx % 4 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(X)) & 15u) == 0;
     for (int col0 = 0; col0 < k; col0 += KL) {
         const int kcount = std::min(KL, k - col0);
         const int has_bound = col0 > 0;
-        if (KL == 4)
-            knn_launch_tiles<4>(Q, M, ldq, X, N, ldx, D, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi, dist,
-                                ldd, col0, kcount, st);
-        else if (KL == 8)
-            knn_launch_tiles<8>(Q, M, ldq, X, N, ldx, D, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi, dist,
-                                ldd, col0, kcount, st);
-        else
-            knn_launch_tiles<16>(Q, M, ldq, X, N, ldx, D, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi, dist,
-                                 ldd, col0, kcount, st);
-        int rc = check_launch("knn_tile_kernel");
-        if (rc) return rc;
+#define HKM_KNN_MFMA(KLV, HV)                                                                                        \
+    knn_launch_mfma<KLV, HV>(vec, Q, M, ldq, X, N, ldx, D, xn, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi, \
+                             dist, ldd, col0, kcount, st)
+        if (mfma) {
+            const int H = D <= 16 ? 8 : (D <= 32 ? 16 : (D <= 64 ? 32 : 64));
+            if (KL == 8) {
+                if (H == 8) HKM_KNN_MFMA(8, 8);
+                else if (H == 16) HKM_KNN_MFMA(8, 16);
+                else if (H == 32) HKM_KNN_MFMA(8, 32);
+                else HKM_KNN_MFMA(8, 64);
+            } else {
+                if (H == 8) HKM_KNN_MFMA(16, 8);
+                else if (H == 16) HKM_KNN_MFMA(16, 16);
+                else if (H == 32) HKM_KNN_MFMA(16, 32);
+                else HKM_KNN_MFMA(16, 64);
+            }
+            if ((rc = check_launch("knn_mfma_kernel"))) return rc;
+        } else {
+            if (KL == 4)
+                knn_launch_tiles<4>(Q, M, ldq, X, N, ldx, D, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi,
+                                    dist, ldd, col0, kcount, st);
+            else if (KL == 8)
+                knn_launch_tiles<8>(Q, M, ldq, X, N, ldx, D, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi,
+                                    dist, ldd, col0, kcount, st);
+            else
+                knn_launch_tiles<16>(Q, M, ldq, X, N, ldx, D, p, has_bound, last_d2, last_i, part_d, part_i, idx, ldi,
+                                     dist, ldd, col0, kcount, st);
+            if ((rc = check_launch("knn_tile_kernel"))) return rc;
+        }
+#undef HKM_KNN_MFMA
         if (p.nsplit > 1) {
             hipLaunchKernelGGL(knn_merge_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, st, part_d, part_i,
                                p.nsplit, KL, M, last_d2, last_i, idx, ldi, dist, ldd, col0, kcount);
