@@ -209,6 +209,68 @@ def bench_cdist(args, w, x, t_gen) -> int:
     return 0
 
 
+def bench_knn(args, w, x, t_gen) -> int:
+    """k nearest rows + label vote (KNeighborsClassifier.predict, k = 5) on rows of the c2 data: test rows =
+    the first 32768 rows, training rows = the next 32768 (D = 64), 10 classes.  flops = 2 M N D (the
+    products on the matrix cores); the 4.29 GB distance matrix is never formed."""
+    import torch
+
+    from heat_amd import _native
+
+    if args.config != "c2":
+        print("--estimator knn runs on the c2 data", file=sys.stderr)
+        return 2
+    m = nn = min(32768, x.shape[0] // 2)
+    d = x.shape[1]
+    k, ncls = 5, 10
+    q, train = x[:m], x[m:m + nn]
+    g = torch.Generator(device=x.device).manual_seed(w.seed)
+    y = torch.zeros((nn, ncls), dtype=torch.float32, device=x.device)
+    y.scatter_(1, torch.randint(0, ncls, (nn, 1), device=x.device, generator=g), 1.0)
+    idx = torch.empty((m, k), dtype=torch.int64, device=x.device)
+    cls = torch.empty((m,), dtype=torch.int64, device=x.device)
+    ws = _native.Workspace(x.device)
+
+    def step():
+        _native.knn(q, train, k, idx, None, ws)
+        _native.knn_vote(idx, y, cls)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ev = []
+    for _ in range(args.steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step()
+        e1.record()
+        torch.cuda.synchronize()
+        ev.append(e0.elapsed_time(e1))
+    kern_ms = sum(ev) / len(ev)
+    flops = 2.0 * m * nn * d
+    res = {
+        "metric": "kNN predict test rows/s", "value": round(m * args.steps / elapsed, 1), "unit": "rows/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32",
+        "data": f"synthetic (seed {w.seed}, generated on CPU in {t_gen:.1f} s, resident in HBM before timing)",
+        "config": {"workload": f"knn_predict_m{m}_n{nn}_d{d}_k{k}", "M": m, "N": nn, "D": d, "k": k,
+                   "classes": ncls, "scale": args.scale},
+        "roofline": {"bound": "mfma", "achieved": round(flops / (kern_ms * 1e-3) / 1e12, 3), "peak": 157.3,
+                     "unit": "TFLOP/s", "frac": round(flops / (kern_ms * 1e-3) / 1e12 / 157.3, 4),
+                     "kernel": "knn_mfma_lds + knn_merge + knn_vote (whole step)", "kernel_ms": round(kern_ms, 4),
+                     "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(res))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -217,9 +279,9 @@ def main() -> int:
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink N (testing only; invalidates the figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians", "cdist", "init"],
+    ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians", "cdist", "init", "knn"],
                     help="kmedians: the Manhattan-metric sibling on the same data; cdist: the full-matrix "
-                         "public cdist on rows of c2; init: the k-means|| initialiser (none is the headline metric)")
+                         "public cdist on rows of c2; init: the k-means|| initialiser; knn: k nearest rows + label vote on rows of c2 (none is the headline metric)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: this build has no multi-GPU path (run with --gpus 1).", file=sys.stderr)
@@ -255,6 +317,8 @@ def main() -> int:
         return bench_cdist(args, w, x, t_gen)
     if args.estimator == "init":
         return bench_init(args, w, x, t_gen)
+    if args.estimator == "knn":
+        return bench_knn(args, w, x, t_gen)
     if args.config == "c2":
         # assignment only: labels + min squared distance
         y = w.y.to(dev)
