@@ -53,9 +53,36 @@ __device__ __forceinline__ void knn_insert(float (&ld)[KL], unsigned (&li)[KL], 
 // The lists live in registers and must be updated in place: a branch per lane around the insertion makes
 // the compiler copy a whole list at every candidate, so the branch is taken by the wave as a whole (any
 // lane with a hit) and lanes without one insert +inf, which changes nothing.
+// x = take ? y : x, written so that x stays in its register (the compiler's own selects end up in fresh
+// registers and the list is copied back at every candidate)
+__device__ __forceinline__ void knn_keep_or(float& x, float y, unsigned long long take) {
+    asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(x) : "v"(y), "s"(take));
+}
+__device__ __forceinline__ void knn_keep_or(unsigned& x, unsigned y, unsigned long long take) {
+    asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(x) : "v"(y), "s"(take));
+}
+
+// the insertion of knn_insert slot by slot from the end: slot s takes the candidate if it is smaller, and
+// the pair in front of it instead if the candidate is smaller than that one too
+template <int KL>
+__device__ __forceinline__ void knn_insert_in_place(float (&ld)[KL], unsigned (&li)[KL], float d, unsigned i) {
+    unsigned long long lt[KL];
+#pragma unroll
+    for (int s = 0; s < KL; ++s) lt[s] = __builtin_amdgcn_ballot_w64(d < ld[s]);
+#pragma unroll
+    for (int s = KL - 1; s >= 0; --s) {
+        knn_keep_or(ld[s], d, lt[s]);
+        knn_keep_or(li[s], i, lt[s]);
+        if (s > 0) {
+            knn_keep_or(ld[s], ld[s - 1], lt[s - 1]);
+            knn_keep_or(li[s], li[s - 1], lt[s - 1]);
+        }
+    }
+}
+
 template <int KL>
 __device__ __forceinline__ void knn_offer(float (&ld)[KL], unsigned (&li)[KL], bool ok, float d, unsigned i) {
-    if (__builtin_amdgcn_ballot_w64(ok) != 0) knn_insert<KL>(ld, li, ok ? d : HKM_INF, i);
+    if (__builtin_amdgcn_ballot_w64(ok) != 0) knn_insert_in_place<KL>(ld, li, ok ? d : HKM_INF, i);
 }
 
 template <int KL>
