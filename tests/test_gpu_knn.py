@@ -56,6 +56,74 @@ def test_integer_data_gives_the_exact_sorted_lists(cuda, m, n, d, k):
     assert torch.equal(idx2, idx)
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_random_shapes_give_the_exact_sorted_lists(cuda, seed):
+    """Seeded sweep on both sides of every tile and dispatch boundary (feature counts around 16, 32, 64, 128,
+    rows around 32, 64, 128), dense and padded rows (the padded ones take the kernels without vector
+    loads), integer-valued data so that the expected lists are exact."""
+    import random
+
+    rng = random.Random(seed)
+    ws = _native.Workspace(cuda)
+    for case in range(40):
+        m = rng.choice([1, 2, 31, 32, 33, 127, 128, 129, 500])
+        n = rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 257, 1000, 5000])
+        d = rng.choice([1, 3, 4, 8, 15, 16, 17, 20, 31, 32, 33, 36, 48, 63, 64, 65, 100, 128, 129, 200])
+        k = min(n, rng.choice([1, 2, 5, 8, 9, 16, 17, 33]))
+        padq, padx = rng.choice([0, 0, 1, 4]), rng.choice([0, 0, 1, 4])
+        what = f"seed={seed} case={case} m={m} n={n} d={d} k={k} padq={padq} padx={padx}"
+        print(what, flush=True)
+        g = torch.Generator().manual_seed(seed * 7919 + case)
+        x = torch.randint(-5, 6, (n, d), generator=g).float()
+        q = torch.randint(-5, 6, (m, d), generator=g).float()
+        want_i, want_d2 = _exact_lists(q, x, k)
+        xg = torch.zeros((n, d + padx), device=cuda)[:, :d]
+        xg.copy_(x)
+        qg = torch.zeros((m, d + padq), device=cuda)[:, :d]
+        qg.copy_(q)
+        idx = torch.full((m, k), -7, dtype=torch.int64, device=cuda)
+        dist = torch.full((m, k), -7.0, device=cuda)
+        _native.knn(qg, xg, k, idx, dist, ws)
+        assert torch.equal(idx.cpu(), want_i), what
+        assert torch.equal(dist.cpu(), torch.from_numpy(np.sqrt(want_d2.numpy()).astype(np.float32))), what
+
+
+def test_training_rows_beyond_4gib(cuda):
+    """A training matrix whose byte offsets do not fit 32 bits: the neighbours of a few test rows placed next
+    to known training rows on both sides of the 4 GiB offset and at the very end."""
+    n, d, k = 40_000_000, 32, 5
+    g = torch.Generator(device=cuda).manual_seed(3)
+    x = torch.empty((n, d), device=cuda)
+    step = 1 << 23
+    for a in range(0, n, step):
+        b = min(n, a + step)
+        x[a:b] = torch.randn((b - a, d), device=cuda, generator=g) * 4
+    assert x.numel() * 4 > 1 << 32
+    r4 = (1 << 32) // (4 * d)
+    rows = torch.tensor([0, 77, r4 - 1, r4, r4 + 1, n // 2 + 5, n - 2, n - 1], device=cuda)
+    q = torch.cat([x[rows] + 1e-3, torch.randn((120, d), device=cuda, generator=g) * 4])
+    idx = torch.empty((q.shape[0], k), dtype=torch.int64, device=cuda)
+    dist = torch.empty((q.shape[0], k), device=cuda)
+    _native.knn(q, x, k, idx, dist, _native.Workspace(cuda))
+    assert torch.equal(idx[:8, 0], rows)
+    # all lists against a float64 evaluation in row chunks
+    best_d = torch.full((q.shape[0], k), float("inf"), dtype=torch.float64, device=cuda)
+    best_i = torch.zeros((q.shape[0], k), dtype=torch.int64, device=cuda)
+    qd = q.double()
+    for a in range(0, n, 1 << 22):
+        b = min(n, a + (1 << 22))
+        xd = x[a:b].double()
+        d2 = (qd * qd).sum(1, keepdim=True) + (xd * xd).sum(1)[None] - 2.0 * (qd @ xd.T)
+        v, i = torch.topk(d2, k, dim=1, largest=False)
+        cat_d, cat_i = torch.cat([best_d, v], 1), torch.cat([best_i, i + a], 1)
+        best_d, pos = torch.topk(cat_d, k, dim=1, largest=False)
+        best_i = torch.gather(cat_i, 1, pos)
+    got_d2 = (qd[:, None, :] - x[idx].double()).pow(2).sum(-1)
+    scale2 = (qd * qd).sum(1, keepdim=True) + float((x[:1 << 20].double() ** 2).sum(1).max())
+    assert int(((got_d2 - best_d.clamp_min(0)).abs() > 1e-5 * best_d.abs() + 1e-6 * scale2).sum()) == 0
+    assert float((idx == best_i).double().mean()) > 0.99
+
+
 @pytest.mark.parametrize("m,n,d,k,spread", [
     (300, 4000, 32, 5, 3.0), (64, 50000, 64, 10, 0.1), (5000, 700, 7, 8, 100.0), (1000, 1000, 130, 20, 1.0),
     (20000, 100000, 16, 5, 3.0),
