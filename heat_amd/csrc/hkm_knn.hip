@@ -231,22 +231,22 @@ __device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (
     for (int s = 0; s < KL - 1; ++s) thr = s == kcount - 1 ? ld[s] : thr;  // only kcount entries are asked for
     thr = fminf(thr, __shfl_xor(thr, 32));
     const unsigned gj0 = unsigned(j0) + 4 * h;
-    if (j0 + 32 <= r_end && !has_bound) {
+    float dv[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float d = fmaxf(fmaf(-2.0f, acc[i], qn + xnv[i]), 0.0f);
-            knn_offer<KL>(ld, li, d < thr, d, gj0 + 8 * (i >> 2) + (i & 3));
-        }
-    } else {
+    for (int i = 0; i < 16; ++i) dv[i] = fmaxf(fmaf(-2.0f, acc[i], qn + xnv[i]), 0.0f);
+    if (j0 + 32 > r_end || has_bound) {
+        // the last tile of a split and the later passes: rows past the end and pairs that do not rank
+        // after the bound become +inf here, so that one chain of offers serves every tile
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const unsigned gj = gj0 + 8 * (i >> 2) + (i & 3);
-            const float d = fmaxf(fmaf(-2.0f, acc[i], qn + xnv[i]), 0.0f);
-            bool ok = gj < unsigned(r_end) && d < thr;
-            if (has_bound) ok = ok && (d > bd || (d == bd && gj > bi));
-            knn_offer<KL>(ld, li, ok, d, gj);
+            bool ok = gj < unsigned(r_end);
+            if (has_bound) ok = ok && (dv[i] > bd || (dv[i] == bd && gj > bi));
+            dv[i] = ok ? dv[i] : HKM_INF;
         }
     }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) knn_offer<KL>(ld, li, dv[i] < thr, dv[i], gj0 + 8 * (i >> 2) + (i & 3));
 }
 
 // The two lanes of a query row (h = 0, 1): KL times the smaller head, whose lane pops it; lane h = 0
