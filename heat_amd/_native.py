@@ -65,6 +65,10 @@ SIGNATURES = {
                                    c_int64, c_void_p, c_int64, c_void_p, c_size_t, c_void_p]),
     "hkm_knn_vote_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int64, c_int32, c_int64,
                                         c_void_p, c_void_p]),
+    "hkm_cluster_distance_sums_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
+                                                     c_void_p, c_int64, c_void_p]),
+    "hkm_silhouette_finish_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_void_p,
+                                                 c_void_p]),
     "hkm_assign_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p]),
     "hkm_update_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
@@ -511,3 +515,46 @@ def knn_vote(idx: torch.Tensor, y: torch.Tensor, classes: torch.Tensor) -> None:
         raise ValueError(f"classes must hold {m} contiguous entries")
     check(load().hkm_knn_vote_f32(_ptr(idx), m, k, idx.stride(0) if m > 1 else k, _ptr(y), n, c,
                                   y.stride(0) if n > 1 else c, _ptr(classes), _stream()))
+
+
+def cluster_distance_sums(x: torch.Tensor, perm: torch.Tensor, offsets: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i, c] = sum of the Euclidean distances from row i to the rows perm[offsets[c]:offsets[c + 1]]
+    (see hkm_cluster_distance_sums_f32 in include/hkm.h).  perm and offsets are checked here, on the
+    device, because the kernel gathers rows through them."""
+    _require_gpu(x, perm, offsets, out)
+    _require_rows(x, out)
+    if x.dtype != torch.float32 or out.dtype != torch.float32:
+        raise TypeError("x and out must be float32")
+    if perm.dtype != torch.int64 or offsets.dtype != torch.int64 or not perm.is_contiguous() or not offsets.is_contiguous():
+        raise TypeError("perm and offsets must be contiguous int64 vectors")
+    n, d = x.shape
+    k = offsets.numel() - 1
+    if k < 1 or perm.numel() != n or tuple(out.shape) != (n, k):
+        raise ValueError(f"perm must hold {n} entries and out must be ({n}, {k})")
+    if n:
+        ok = (int(perm.min()) >= 0 and int(perm.max()) < n and int(offsets[0]) == 0 and int(offsets[-1]) == n
+              and bool((offsets[1:] >= offsets[:-1]).all()))
+        if not ok:
+            raise ValueError("perm must index rows of x and offsets must rise from 0 to the number of rows")
+    check(load().hkm_cluster_distance_sums_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(perm), _ptr(offsets), k,
+                                               _ptr(out), out.stride(0) if n > 1 else k, _stream()))
+
+
+def silhouette_finish(sums: torch.Tensor, labels: torch.Tensor, counts: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i] = silhouette coefficient of sample i from its per-cluster distance sums (see
+    hkm_silhouette_finish_f32 in include/hkm.h); labels are checked here against the number of clusters."""
+    _require_gpu(sums, labels, counts, out)
+    _require_rows(sums)
+    n, k = sums.shape
+    if sums.dtype != torch.float32 or out.dtype != torch.float32:
+        raise TypeError("sums and out must be float32")
+    if labels.dtype != torch.int64 or counts.dtype != torch.int64:
+        raise TypeError("labels and counts must be int64")
+    if labels.numel() != n or counts.numel() != k or out.numel() != n:
+        raise ValueError("labels and out need one entry per sample, counts one per cluster")
+    if not (labels.is_contiguous() and counts.is_contiguous() and out.is_contiguous()):
+        raise ValueError("labels, counts and out must be contiguous")
+    if n and (int(labels.min()) < 0 or int(labels.max()) >= k):
+        raise ValueError("labels must lie in [0, number of clusters)")
+    check(load().hkm_silhouette_finish_f32(_ptr(sums), n, k, sums.stride(0) if n > 1 else k, _ptr(labels), _ptr(counts),
+                                           _ptr(out), _stream()))

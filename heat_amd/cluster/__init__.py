@@ -4,3 +4,4 @@ from ._kcluster import _KCluster  # noqa: F401
 from .kmedians import KMedians  # noqa: F401
 from .kmedoids import KMedoids  # noqa: F401
 from .batchparallelclustering import BatchParallelKMeans, BatchParallelKMedians  # noqa: F401
+from .metrics import silhouette_samples, silhouette_score  # noqa: F401

@@ -630,6 +630,33 @@ int hkm_knn_f32(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t 
                       static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_cluster_distance_sums_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int64_t* perm,
+                                  const int64_t* offsets, int32_t K, float* S, int64_t lds, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if (K > 65535) return fail(HKM_EUNSUPPORTED, "K = %d exceeds 65535 clusters", K);
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("S", S, N, K, lds))) return rc;
+    if (!offsets || (N > 0 && !perm)) return fail(HKM_EINVAL, "perm or offsets is NULL");
+    if ((reinterpret_cast<uintptr_t>(perm) | reinterpret_cast<uintptr_t>(offsets)) & 7u)
+        return fail(HKM_EINVAL, "perm or offsets is not 8-byte aligned");
+    return launch_silhouette_sums(X, N, D, ldx, perm, offsets, K, S, lds, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds, const int64_t* labels,
+                              const int64_t* counts, float* out, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, 1, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("S", S, N, K, lds))) return rc;
+    if (!counts || (N > 0 && (!labels || !out))) return fail(HKM_EINVAL, "labels, counts or out is NULL");
+    if ((reinterpret_cast<uintptr_t>(labels) | reinterpret_cast<uintptr_t>(counts)) & 7u)
+        return fail(HKM_EINVAL, "labels or counts is not 8-byte aligned");
+    if (reinterpret_cast<uintptr_t>(out) & 3u) return fail(HKM_EINVAL, "out is not 4-byte aligned");
+    return launch_silhouette_finish(S, N, K, lds, labels, counts, out, static_cast<hipStream_t>(hip_stream));
+}
+
 int hkm_knn_vote_f32(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
                      int64_t ldy, int64_t* classes, void* hip_stream) {
     g_err[0] = 0;

@@ -254,4 +254,10 @@ bool knn_uses_mfma(int32_t D);
 int launch_knn_vote(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
                     int64_t ldy, int64_t* classes, hipStream_t st);
 
+// per-sample, per-cluster sums of Euclidean distances (hkm_silhouette.hip)
+int launch_silhouette_finish(const float* S, int64_t N, int32_t K, int64_t lds, const int64_t* enc,
+                             const int64_t* counts, float* out, hipStream_t st);
+int launch_silhouette_sums(const float* X, int64_t N, int32_t D, int64_t ldx, const int64_t* perm,
+                           const int64_t* offsets, int32_t K, float* S, int64_t lds, hipStream_t st);
+
 }  // namespace hkm

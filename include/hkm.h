@@ -268,6 +268,28 @@ int hkm_knn_vote_f32(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, cons
                      int64_t ldy, int64_t* classes, void* hip_stream);
 
 /*
+ * hkm_cluster_distance_sums_f32: S[i][c] = sum over the rows j of cluster c of the Euclidean distance
+ * |x_i - x_j| (direct form, correctly rounded square root, float64 accumulation rounded to float32 at the
+ * end) -- `clust_dists = matmul(cdist(X, X), labels == unique_labels)` of silhouette_samples,
+ * heat/cluster/metrics.py:135-151, without the N x N matrix.  The caller groups the rows by cluster:
+ * perm (int64[N]) lists the row indices cluster by cluster, offsets (int64[K + 1]) the start of every
+ * cluster in perm (offsets[0] = 0, offsets[K] = N; device arrays, whose contents are not checked: an
+ * index outside [0, N) reads outside X).  S is N x K float32 with leading dimension lds.
+ */
+int hkm_cluster_distance_sums_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int64_t* perm,
+                                  const int64_t* offsets, int32_t K, float* S, int64_t lds, void* hip_stream);
+/*
+ * hkm_silhouette_finish_f32: the silhouette coefficient of every sample from those sums
+ * (heat/cluster/metrics.py:153-176): a = S[i][own] / max(n_own - 1, 1), b = min over the other clusters
+ * of S[i][c] / n_c, out[i] = (b - a) / max(a, b); 0 for a sample alone in its cluster and where the
+ * quotient is not a number (one cluster only).  labels (int64[N]) are the cluster numbers 0 .. K-1 of the
+ * samples, counts (int64[K]) the cluster sizes (labels outside [0, K) read outside S: not checked here).
+ * Also serves metric="precomputed" with S = matmul(D, labels == unique_labels).
+ */
+int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds, const int64_t* labels,
+                              const int64_t* counts, float* out, void* hip_stream);
+
+/*
  * float64 data.  The reference keeps float64 inputs in float64 through the same op sequence
  * (promote(X, Y, float32), heat/spatial/distance.py:392-403; heat/cluster/kmeans.py:76-148), so these
  * mirror the *_f32 entry points of the same name with double operands: quadratic-expansion distance +

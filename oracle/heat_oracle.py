@@ -60,6 +60,11 @@ Pins (what each function is checked against, see tests/test_oracle_pins.py):
   ``NearestNeighbors`` (neighbour sets and classes on the iris data and on random blobs); a python
   sort of float64 distances on a tiny input; k = 1 on the training rows returns every row itself.
   The reference stores no predicted class anywhere (``test_knn.py`` asserts types and shapes).
+* silhouette_samples / silhouette_score: the known answers of ``tests/cluster/test_metrics.py:92-122``
+  (sample 0 of the four-point example = 0.9, score 0.76439) and of the docstring
+  (``heat/cluster/metrics.py:121-126``: 0.7452, 0.7836, 0.7452, 0.7836), the special cases of
+  ``test_metrics.py:45-88`` (all samples alone, one cluster, perfect and worst clustering), and
+  scikit-learn's ``silhouette_samples`` to 1e-6 as in the reference's own test (``:16-42``).
 """
 
 from __future__ import annotations
@@ -771,3 +776,32 @@ def knn_neighbours_f64(x_train: torch.Tensor, x_test: torch.Tensor, n_neighbors:
         out_d.append(vals[:, :kk])
         out_i.append(torch.gather(cand, 1, pos)[:, :kk])
     return torch.cat(out_d), torch.cat(out_i)
+
+
+# --------------------------------------------------------------------------------------------------
+# silhouette coefficient
+# --------------------------------------------------------------------------------------------------
+def silhouette_samples(x: torch.Tensor, labels: torch.Tensor, metric: str = "euclidean") -> torch.Tensor:
+    """heat/cluster/metrics.py:128-177 at one rank, op for op: the full distance matrix (``torch.cdist``,
+    heat/spatial/distance.py:17-29), its product with the label mask, a, b and the quotient."""
+    labels = labels.reshape(-1)
+    unique_labels, labels_encoded = torch.unique(labels, sorted=True, return_inverse=True)
+    labels_freqs = torch.bincount(labels_encoded)
+    dist = x if metric == "precomputed" else torch.cdist(x, x)
+    full_mask = labels.reshape(-1, 1) == unique_labels.reshape(1, -1)
+    clust_dists = torch.matmul(dist, full_mask.to(dist.dtype))
+    a_clust_dists = torch.sum(clust_dists * full_mask, dim=1)
+    denominator_a = labels_freqs[labels_encoded] - 1
+    denominator_a = torch.where(denominator_a > 0, denominator_a, torch.ones_like(denominator_a))
+    a = a_clust_dists / denominator_a
+    b_clust_means = clust_dists / labels_freqs
+    b_clust_means[full_mask] = float("inf")
+    b = torch.min(b_clust_means, dim=1).values
+    sil = (b - a) / torch.maximum(a, b)
+    sil = torch.where(labels_freqs[labels_encoded] > 1, sil, torch.zeros_like(sil))
+    return torch.nan_to_num(sil)
+
+
+def silhouette_score(x: torch.Tensor, labels: torch.Tensor, metric: str = "euclidean") -> float:
+    """heat/cluster/metrics.py:269: the mean of the per-sample coefficients."""
+    return float(torch.mean(silhouette_samples(x, labels, metric=metric)))

@@ -470,3 +470,41 @@ def test_knn_oracle_against_scikit_learn_and_a_python_sort():
     # k = 1 on the training rows: every row is its own neighbour (distinct rows)
     cls, idx, dist = orc.knn_predict(blobs, lab, blobs, 1)
     assert torch.equal(idx.view(-1), torch.arange(700)) and torch.equal(cls, lab)
+
+
+def test_silhouette_oracle_known_answers_special_cases_and_scikit_learn():
+    """silhouette_samples / silhouette_score against the values the reference's tests and docstring hold
+    (tests/cluster/test_metrics.py:45-122, heat/cluster/metrics.py:121-126) and against scikit-learn."""
+    from sklearn.metrics import silhouette_samples as sk_silhouette
+
+    x = torch.tensor([[0.0, 0.0], [10.0, 10.0], [20.0, 20.0], [1.0, 1.0]])
+    assert float(orc.silhouette_samples(x, torch.tensor([0, 2, 1, 0]))[0]) == pytest.approx(0.9, abs=1e-6)
+    x = torch.tensor([[1.0, 2.0], [1.0, 1.0], [4.0, 4.0], [4.0, 5.0]])
+    lab = torch.tensor([0, 0, 1, 1])
+    assert orc.silhouette_samples(x, lab).tolist() == pytest.approx([0.7452, 0.7836, 0.7452, 0.7836], abs=5e-5)
+    assert orc.silhouette_score(x.double(), lab) == pytest.approx(0.76439, abs=5e-6)
+    g = torch.Generator().manual_seed(4)
+    n = 16
+    data = torch.rand((n, 3), generator=g)
+    assert orc.silhouette_score(data, torch.arange(n)) == 0.0          # every sample alone
+    assert orc.silhouette_score(data, torch.zeros(n, dtype=torch.int64)) == 0.0   # one cluster
+    data = torch.zeros((n, 3))
+    data[n // 2:, 0] = 1.0
+    lab = torch.zeros(n, dtype=torch.int64)
+    lab[n // 2:] = 2                                                       # perfect, label values with a gap
+    assert orc.silhouette_score(data, lab) == pytest.approx(1.0)
+    worst = (n / 4) / (n / 2) / ((n / 4) / (n / 2 - 1)) - 1
+    assert orc.silhouette_score(data, torch.arange(n) % 2) == pytest.approx(worst)
+    for n_p, n_c, d in ((8, 3, 1), (17, 5, 2), (17, 3, 3), (300, 7, 5)):
+        data = torch.rand((n_p, d), generator=g)
+        lab = torch.randint(0, n_c, (n_p,), generator=g)
+        if len(torch.unique(lab)) < 2:
+            continue
+        want = sk_silhouette(data.numpy(), lab.numpy(), metric="euclidean")
+        # above 25 rows torch.cdist expands the square: self-distances of ~3e-4 instead of 0 and distance
+        # errors of that order move the coefficients by up to a few 1e-5 (the reference's test stops at 17)
+        assert np.allclose(orc.silhouette_samples(data, lab).numpy(), want, atol=2e-6 if n_p <= 25 else 1e-4)
+        dist = torch.cdist(data, data)
+        dist.fill_diagonal_(0.0)
+        want = sk_silhouette(dist.numpy(), lab.numpy(), metric="precomputed")
+        assert np.allclose(orc.silhouette_samples(dist, lab, metric="precomputed").numpy(), want, atol=2e-6)
