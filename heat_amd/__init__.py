@@ -13,7 +13,7 @@ Arithmetic runs in hand-written gfx950 kernels loaded through ctypes (``heat_amd
 """
 from .core import *  # noqa: F401,F403
 from .core import types, devices, communication, factories, base, dndarray  # noqa: F401
-from . import classification, cluster, spatial, utils  # noqa: F401
+from . import classification, cluster, graph, spatial, utils  # noqa: F401
 from . import _native  # noqa: F401
 
 __version__ = "0.1.0"

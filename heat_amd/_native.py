@@ -69,6 +69,8 @@ SIGNATURES = {
                                                      c_void_p, c_int64, c_void_p]),
     "hkm_silhouette_finish_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_void_p,
                                                  c_void_p]),
+    "hkm_laplacian_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, ctypes.c_float,
+                                         c_void_p, c_int64, c_void_p, c_void_p]),
     "hkm_assign_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p]),
     "hkm_update_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
@@ -558,3 +560,20 @@ def silhouette_finish(sums: torch.Tensor, labels: torch.Tensor, counts: torch.Te
         raise ValueError("labels must lie in [0, number of clusters)")
     check(load().hkm_silhouette_finish_f32(_ptr(sums), n, k, sums.stride(0) if n > 1 else k, _ptr(labels), _ptr(counts),
                                            _ptr(out), _stream()))
+
+
+def laplacian(sim: torch.Tensor, out: torch.Tensor, definition: int, mode: int, weighted: bool, eps: float,
+              degree: torch.Tensor) -> None:
+    """out = graph Laplacian of the similarity matrix sim (see hkm_laplacian_f32 in include/hkm.h):
+    definition 0 simple / 1 norm_sym, mode 0 fully connected / 1 keep below eps / 2 keep above eps."""
+    _require_gpu(sim, out, degree)
+    _require_rows(sim, out)
+    n = sim.shape[0]
+    if sim.dim() != 2 or sim.shape[1] != n or tuple(out.shape) != (n, n):
+        raise ValueError("sim and out must be square matrices of the same size")
+    if sim.dtype != torch.float32 or out.dtype != torch.float32 or degree.dtype != torch.float32:
+        raise TypeError("sim, out and degree must be float32")
+    if degree.numel() != n or not degree.is_contiguous():
+        raise ValueError(f"degree must hold {n} contiguous entries")
+    check(load().hkm_laplacian_f32(_ptr(sim), n, sim.stride(0) if n > 1 else n, definition, mode, 1 if weighted else 0,
+                                   float(eps), _ptr(out), out.stride(0) if n > 1 else n, _ptr(degree), _stream()))

@@ -657,6 +657,23 @@ int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds,
     return launch_silhouette_finish(S, N, K, lds, labels, counts, out, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_laplacian_f32(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                      float eps, float* L, int64_t ldl, float* degree, void* hip_stream) {
+    g_err[0] = 0;
+    if (N < 0 || N > 65535) return fail(HKM_EUNSUPPORTED, "N = %lld must be in [0, 65535]", (long long)N);
+    if (definition != HKM_LAPLACIAN_SIMPLE && definition != HKM_LAPLACIAN_NORM_SYM)
+        return fail(HKM_EINVAL, "definition = %d is neither simple (0) nor norm_sym (1)", definition);
+    if (mode < 0 || mode > 2) return fail(HKM_EINVAL, "mode = %d must be 0 (fully connected), 1 (upper) or 2 (lower)", mode);
+    if (N == 0) return HKM_OK;
+    int rc;
+    if ((rc = check_matrix("S", S, N, (int32_t)N, lds))) return rc;
+    if ((rc = check_matrix("L", L, N, (int32_t)N, ldl))) return rc;
+    if (!degree) return fail(HKM_EINVAL, "degree is NULL");
+    if (reinterpret_cast<uintptr_t>(degree) & 3u) return fail(HKM_EINVAL, "degree is not 4-byte aligned");
+    return launch_laplacian(S, N, lds, definition, mode, weighted ? 1 : 0, eps, L, ldl, degree,
+                            static_cast<hipStream_t>(hip_stream));
+}
+
 int hkm_knn_vote_f32(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,
                      int64_t ldy, int64_t* classes, void* hip_stream) {
     g_err[0] = 0;

@@ -260,4 +260,8 @@ int launch_silhouette_finish(const float* S, int64_t N, int32_t K, int64_t lds, 
 int launch_silhouette_sums(const float* X, int64_t N, int32_t D, int64_t ldx, const int64_t* perm,
                            const int64_t* offsets, int32_t K, float* S, int64_t lds, hipStream_t st);
 
+// graph Laplacian from a similarity matrix (hkm_laplacian.hip)
+int launch_laplacian(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                     float eps, float* L, int64_t ldl, float* degree, hipStream_t st);
+
 }  // namespace hkm

@@ -1,0 +1,53 @@
+"""
+Graph Laplacian with the interface of heat/graph/laplacian.py.
+
+``construct`` calls the similarity function (``ht.spatial.cdist`` / ``rbf`` ..., whose full-matrix kernels
+produce S) and hands S to ``hkm_laplacian_f32``: one read for the degrees, one read and one write for L,
+in place of the reference's chain of whole-matrix operations (:119-142).
+"""
+
+from __future__ import annotations
+
+from typing import Callable
+
+import torch
+
+from .. import _native
+from ..core import types
+from ..core.dndarray import DNDarray
+
+
+class Laplacian:
+    def __init__(self, similarity: Callable, weighted: bool = True, definition: str = "norm_sym",
+                 mode: str = "fully_connected", threshold_key: str = "upper", threshold_value: float = 1.0,
+                 neighbours: int = 10):  # noqa: D107
+        self.similarity_metric = similarity
+        self.weighted = weighted
+        if definition not in ["simple", "norm_sym"]:
+            raise NotImplementedError("Currently only simple and normalized symmetric graph laplacians are supported")
+        self.definition = definition
+        if mode not in ["eNeighbour", "fully_connected"]:
+            raise NotImplementedError("Only eNeighborhood and fully-connected graphs supported at the moment.")
+        self.mode = mode
+        if threshold_key not in ["upper", "lower"]:
+            raise ValueError("Only 'upper' and 'lower' threshold types supported for eNeighbouhood graph construction")
+        self.epsilon = (threshold_key, threshold_value)
+        self.neighbours = neighbours
+
+    def construct(self, X: DNDarray) -> DNDarray:
+        """heat/graph/laplacian.py:100-142.  The result is always float32 (the reference's unweighted graphs
+        go through an integer adjacency matrix, which changes the dtype of the simple Laplacian only)."""
+        S = self.similarity_metric(X)
+        if not isinstance(S, DNDarray) or len(S.shape) != 2 or S.shape[0] != S.shape[1]:
+            raise ValueError("the similarity function must return a square DNDarray")
+        if S.dtype is not types.float32:
+            raise NotImplementedError("the Laplacian kernel exists in float32 only")
+        s = S.larray
+        if s.stride(-1) != 1:
+            s = s.contiguous()
+        n = s.shape[0]
+        mode = 0 if self.mode == "fully_connected" else (1 if self.epsilon[0] == "upper" else 2)
+        degree = torch.empty((n,), dtype=torch.float32, device=s.device)
+        _native.laplacian(s, s, 0 if self.definition == "simple" else 1, mode, bool(self.weighted),
+                          float(self.epsilon[1]), degree)
+        return DNDarray(s, (n, n), types.float32, S.split, S.device, S.comm, True)

@@ -290,6 +290,24 @@ int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds,
                               const int64_t* counts, float* out, void* hip_stream);
 
 /*
+ * hkm_laplacian_f32: graph Laplacian L (N x N, leading dimension ldl; may be S itself) from a similarity
+ * matrix S (N x N, leading dimension lds) -- Laplacian.construct after the similarity call,
+ * heat/graph/laplacian.py:63-98,119-142: the diagonal of S is zeroed, then
+ *   mode 0 (fully_connected) A = S; mode 1 (eNeighbour, upper) keeps entries < eps; mode 2 (lower) keeps
+ *   entries > eps; weighted != 0 keeps their values, else a kept entry counts 1 (the zeroed diagonal goes
+ *   through the same test, so an unweighted upper graph has ones on its diagonal, as in the reference);
+ *   degree[i] (N floats, output) = sum_j A[i][j];
+ *   definition HKM_LAPLACIAN_SIMPLE: L = diag(degree) - A;
+ *   definition HKM_LAPLACIAN_NORM_SYM: L = -(A / sqrt(d_i)) / sqrt(d_j) with zero degrees taken as 1, and
+ *   ones on the diagonal.
+ * N <= 65535.  Always float32 (the reference's unweighted simple Laplacian is an integer matrix).
+ */
+#define HKM_LAPLACIAN_SIMPLE 0
+#define HKM_LAPLACIAN_NORM_SYM 1
+int hkm_laplacian_f32(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                      float eps, float* L, int64_t ldl, float* degree, void* hip_stream);
+
+/*
  * float64 data.  The reference keeps float64 inputs in float64 through the same op sequence
  * (promote(X, Y, float32), heat/spatial/distance.py:392-403; heat/cluster/kmeans.py:76-148), so these
  * mirror the *_f32 entry points of the same name with double operands: quadratic-expansion distance +

@@ -65,6 +65,12 @@ Pins (what each function is checked against, see tests/test_oracle_pins.py):
   (``heat/cluster/metrics.py:121-126``: 0.7452, 0.7836, 0.7452, 0.7836), the special cases of
   ``test_metrics.py:45-88`` (all samples alone, one cluster, perfect and worst clustering), and
   scikit-learn's ``silhouette_samples`` to 1e-6 as in the reference's own test (``:16-42``).
+* laplacian (graph Laplacian from a similarity matrix): ``scipy.sparse.csgraph.laplacian`` (plain and
+  normalised) on fully connected weighted graphs, closed forms (rows of D - A sum to zero, unit diagonal
+  and symmetry of the normalised form, an isolated vertex keeps degree 1 in the normalisation), a
+  hand-made 3-vertex case for both thresholds, and the ones on the diagonal of the unweighted "upper"
+  graph that follow from thresholding after the diagonal is zeroed.  The reference's test
+  (``tests/graph/test_laplacian.py``) asserts types and shapes only.
 """
 
 from __future__ import annotations
@@ -805,3 +811,27 @@ def silhouette_samples(x: torch.Tensor, labels: torch.Tensor, metric: str = "euc
 def silhouette_score(x: torch.Tensor, labels: torch.Tensor, metric: str = "euclidean") -> float:
     """heat/cluster/metrics.py:269: the mean of the per-sample coefficients."""
     return float(torch.mean(silhouette_samples(x, labels, metric=metric)))
+
+
+# --------------------------------------------------------------------------------------------------
+# graph Laplacian
+# --------------------------------------------------------------------------------------------------
+def laplacian(sim: torch.Tensor, definition: str = "norm_sym", mode: str = "fully_connected", weighted: bool = True,
+              threshold_key: str = "upper", threshold_value: float = 1.0) -> torch.Tensor:
+    """heat/graph/laplacian.py:63-98,119-142 on a given similarity matrix, op for op (the unweighted
+    adjacency is the reference's ``ht.int(S < eps)``, an int32 matrix)."""
+    s = sim.clone()
+    s.fill_diagonal_(0.0)
+    if mode == "eNeighbour":
+        keep = s < threshold_value if threshold_key == "upper" else s > threshold_value
+        s = torch.where(keep, s, torch.zeros_like(s)) if weighted else keep.to(torch.int32)
+    if definition == "simple":
+        degree = torch.sum(s, dim=1)
+        return torch.diag(degree) - s
+    degree = torch.sum(s, dim=1)
+    degree = torch.where(degree == 0, torch.ones_like(degree), degree)
+    lap = s / torch.sqrt(degree.unsqueeze(1))
+    lap = lap / torch.sqrt(degree.unsqueeze(0))
+    lap = lap * (-1.0)
+    lap.fill_diagonal_(1.0)
+    return lap

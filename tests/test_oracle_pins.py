@@ -508,3 +508,31 @@ def test_silhouette_oracle_known_answers_special_cases_and_scikit_learn():
         dist.fill_diagonal_(0.0)
         want = sk_silhouette(dist.numpy(), lab.numpy(), metric="precomputed")
         assert np.allclose(orc.silhouette_samples(dist, lab, metric="precomputed").numpy(), want, atol=2e-6)
+
+
+def test_laplacian_oracle_against_scipy_and_closed_forms():
+    from scipy.sparse.csgraph import laplacian as sp_laplacian
+
+    g = torch.Generator().manual_seed(8)
+    x = torch.rand((40, 3), generator=g)
+    sim = torch.exp(-torch.cdist(x, x) ** 2 / 0.5)
+    a = sim.clone()
+    a.fill_diagonal_(0.0)
+    assert np.allclose(orc.laplacian(sim, "simple").numpy(), sp_laplacian(a.numpy(), normed=False), atol=1e-5)
+    assert np.allclose(orc.laplacian(sim, "norm_sym").numpy(), sp_laplacian(a.numpy(), normed=True), atol=1e-6)
+    simple = orc.laplacian(sim, "simple")
+    assert float(simple.sum(1).abs().max()) < 1e-4
+    norm = orc.laplacian(sim, "norm_sym", mode="eNeighbour", threshold_key="lower", threshold_value=0.5)
+    assert torch.equal(norm.diagonal(), torch.ones(40)) and torch.allclose(norm, norm.T)
+    # hand-made: similarities 0.2, 0.6, 0.9 between three vertices
+    s3 = torch.tensor([[9.0, 0.2, 0.6], [0.2, 9.0, 0.9], [0.6, 0.9, 9.0]])
+    up = orc.laplacian(s3, "simple", "eNeighbour", True, "upper", 0.7)       # keeps 0.2 and 0.6
+    assert torch.allclose(up, torch.tensor([[0.8, -0.2, -0.6], [-0.2, 0.2, 0.0], [-0.6, 0.0, 0.6]]))
+    lo = orc.laplacian(s3, "simple", "eNeighbour", True, "lower", 0.7)       # keeps 0.9
+    assert torch.allclose(lo, torch.tensor([[0.0, 0.0, 0.0], [0.0, 0.9, -0.9], [0.0, -0.9, 0.9]]))
+    # vertex 0 is isolated there: its degree counts as 1 in the normalised form
+    lo_n = orc.laplacian(s3, "norm_sym", "eNeighbour", True, "lower", 0.7)
+    assert torch.allclose(lo_n, torch.tensor([[1.0, 0.0, 0.0], [0.0, 1.0, -1.0], [0.0, -1.0, 1.0]]))
+    # unweighted upper: the zeroed diagonal passes "< eps", so every vertex has a self-loop
+    un = orc.laplacian(s3, "simple", "eNeighbour", False, "upper", 0.7)
+    assert un.tolist() == [[2, -1, -1], [-1, 1, 0], [-1, 0, 1]]
