@@ -373,3 +373,52 @@ def test_knn_classifier_surface():
         other = knn_cls(effective_metric_=ht.spatial.manhattan)
         other.fit(b, ht.zeros((3,)))
         other.predict(b)
+
+
+def test_argument_validation_of_the_neighbour_silhouette_and_laplacian_entry_points():
+    """Every call fails validation on the host, before anything touches a device."""
+    lib = _native.load()
+    P = ctypes.c_void_p
+    good, other, ws = P(4096), P(8192), P(1 << 20)
+    big = 1 << 30
+
+    def err():
+        return lib.hkm_last_error().decode()
+
+    einval, eunsup, ews = _native.HKM_EINVAL, _native.HKM_EUNSUPPORTED, _native.HKM_EWORKSPACE
+    # hkm_knn_f32(Q, M, ldq, X, N, ldx, D, k, idx, ldi, dist, ldd, ws, ws_bytes, stream)
+    assert lib.hkm_knn_f32(good, 4, 3, other, 10, 3, 3, 11, good, 11, None, 11, ws, big, None) == einval
+    assert "k = 11" in err()
+    assert lib.hkm_knn_f32(good, 4, 3, other, 10, 3, 3, 0, good, 1, None, 1, ws, big, None) == einval
+    assert lib.hkm_knn_f32(good, 4, 3, other, 0, 3, 3, 1, good, 1, None, 1, ws, big, None) == einval
+    assert "empty" in err()
+    assert lib.hkm_knn_f32(good, 4, 2, other, 10, 3, 3, 2, good, 2, None, 2, ws, big, None) == einval
+    assert "leading dimension of Q" in err()
+    assert lib.hkm_knn_f32(good, 4, 3, other, 10, 3, 3, 2, good, 1, None, 2, ws, big, None) == einval
+    assert "leading dimension of idx" in err()
+    assert lib.hkm_knn_f32(good, 4, 3, other, 10, 3, 3, 2, None, 2, None, 2, ws, big, None) == einval
+    assert lib.hkm_knn_f32(good, 4, 3, other, 3000, 3, 3, 2000, good, 2000, None, 2000, ws, big, None) == eunsup
+    assert lib.hkm_knn_f32(good, 4, 3, other, 10, 3, 3, 2, good, 2, None, 2, ws, 16, None) == ews
+    assert lib.hkm_knn_f32(good, 4, 3, other, 10, 3, 3, 2, good, 2, None, 2, None, 0, None) == ews
+    assert lib.hkm_knn_workspace_bytes(4, 0) == 0 and lib.hkm_knn_workspace_bytes(4, 10) >= 4 * 8
+    # a few query rows against many reference rows: room for the per-split lists
+    assert lib.hkm_knn_workspace_bytes(64, 1 << 20) > lib.hkm_knn_workspace_bytes(64, 100)
+    # hkm_knn_vote_f32(idx, M, k, ldi, Y, N, C, ldy, classes, stream)
+    assert lib.hkm_knn_vote_f32(good, 4, 2, 1, other, 10, 3, 3, good, None) == einval
+    assert lib.hkm_knn_vote_f32(good, 4, 2, 2, other, 10, 3, 2, good, None) == einval
+    assert lib.hkm_knn_vote_f32(good, 4, 2, 2, other, 10, 0, 3, good, None) == einval
+    assert lib.hkm_knn_vote_f32(good, 4, 2, 2, other, 10, 3, 3, None, None) == einval
+    # hkm_cluster_distance_sums_f32(X, N, D, ldx, perm, offsets, K, S, lds, stream)
+    assert lib.hkm_cluster_distance_sums_f32(good, 10, 3, 3, None, other, 2, good, 2, None) == einval
+    assert lib.hkm_cluster_distance_sums_f32(good, 10, 3, 3, other, other, 2, good, 1, None) == einval
+    assert lib.hkm_cluster_distance_sums_f32(good, 10, 3, 3, other, other, 70000, good, 70000, None) == eunsup
+    # hkm_silhouette_finish_f32(S, N, K, lds, labels, counts, out, stream)
+    assert lib.hkm_silhouette_finish_f32(good, 10, 3, 2, other, other, good, None) == einval
+    assert lib.hkm_silhouette_finish_f32(good, 10, 3, 3, other, None, good, None) == einval
+    # hkm_laplacian_f32(S, N, lds, definition, mode, weighted, eps, L, ldl, degree, stream)
+    assert lib.hkm_laplacian_f32(good, 10, 10, 2, 0, 1, 1.0, good, 10, other, None) == einval
+    assert "definition" in err()
+    assert lib.hkm_laplacian_f32(good, 10, 10, 0, 3, 1, 1.0, good, 10, other, None) == einval
+    assert lib.hkm_laplacian_f32(good, 10, 9, 0, 0, 1, 1.0, good, 10, other, None) == einval
+    assert lib.hkm_laplacian_f32(good, 10, 10, 0, 0, 1, 1.0, good, 10, None, None) == einval
+    assert lib.hkm_laplacian_f32(good, 70000, 70000, 0, 0, 1, 1.0, good, 70000, other, None) == eunsup
