@@ -591,7 +591,8 @@ static KnnWorkspace carve_knn(void* base, int64_t M, int64_t N) {
         return r;
     };
     const size_t m = size_t(M < 1 ? 1 : M);
-    const size_t slots = knn_plan(M, N).part_slots;
+    // sized for the largest number of splits any feature count asks for
+    const size_t slots = knn_plan(M, N, knn_max_target_workgroups()).part_slots;
     w.xn = reinterpret_cast<float*>(take((size_t(N < 1 ? 1 : N) + 64) * sizeof(float)));
     w.last_d2 = reinterpret_cast<float*>(take(m * sizeof(float)));
     w.last_i = reinterpret_cast<unsigned*>(take(m * sizeof(unsigned)));

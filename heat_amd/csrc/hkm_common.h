@@ -246,7 +246,8 @@ struct KnnPlan {
     int64_t rows_per_split;
     size_t part_slots;  // (distance, row) pairs of the per-split lists; 0 when one split covers all rows
 };
-KnnPlan knn_plan(int64_t M, int64_t N);
+KnnPlan knn_plan(int64_t M, int64_t N, int target);
+int knn_max_target_workgroups();
 int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N, int64_t ldx, int32_t D, int32_t k,
                int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* xn, float* last_d2, unsigned* last_i,
                float* part_d, unsigned* part_i, hipStream_t st);

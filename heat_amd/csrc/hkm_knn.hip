@@ -30,6 +30,7 @@ namespace hkm {
 static constexpr int KNN_T = 64;
 static constexpr int KNN_KC = 16;
 static constexpr int KNN_MAX_SPLITS = 64;
+static constexpr int KNN_MAX_TARGET = 1536;
 static constexpr unsigned KNN_NONE = 0xffffffffu;
 
 __device__ __forceinline__ bool knn_less(float d, unsigned i, float e, unsigned j) {
@@ -580,12 +581,22 @@ __global__ __launch_bounds__(256) void knn_vote_kernel(const int64_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------
-KnnPlan knn_plan(int64_t M, int64_t N) {
+bool knn_uses_mfma(int32_t D);
+
+// Workgroups to aim for when the reference rows are split: every workgroup pays for filling its lists
+// before its threshold bites, so no more splits than it takes to fill the CUs at the kernel's occupancy
+// (4 workgroups per CU up to 32 features, 3 up to 64, fewer above; measured best 1536 / 768).
+int knn_target_workgroups(int32_t D) {
+    if (!knn_uses_mfma(D)) return 768;
+    return D <= 32 ? KNN_MAX_TARGET : (D <= 64 ? 768 : 512);
+}
+
+int knn_max_target_workgroups() { return KNN_MAX_TARGET; }
+
+KnnPlan knn_plan(int64_t M, int64_t N, int target) {
     KnnPlan p;
     const int64_t qtiles = (M + 127) / 128;  // the larger of the two kernels' query tiles
-    // every workgroup pays for filling its lists before its threshold bites, so no more splits than it
-    // takes to give each CU three workgroups
-    int64_t ns = qtiles > 0 ? (768 + qtiles - 1) / qtiles : 1;
+    int64_t ns = qtiles > 0 ? (target + qtiles - 1) / qtiles : 1;
     ns = std::min<int64_t>(ns, std::max<int64_t>(1, N / 256));
     ns = std::max<int64_t>(1, std::min<int64_t>(ns, KNN_MAX_SPLITS));
     int64_t rps = ((N + ns - 1) / ns + KNN_T - 1) / KNN_T * KNN_T;
@@ -629,7 +640,7 @@ int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N
                int64_t* idx, int64_t ldi, float* dist, int64_t ldd, float* xn, float* last_d2, unsigned* last_i,
                float* part_d, unsigned* part_i, hipStream_t st) {
     if (M == 0) return HKM_OK;
-    const KnnPlan p = knn_plan(M, N);
+    const KnnPlan p = knn_plan(M, N, knn_target_workgroups(D));
     const bool mfma = knn_uses_mfma(D);
     const int KL = mfma ? (k <= 8 ? 8 : 16) : (k <= 4 ? 4 : (k <= 8 ? 8 : 16));
     int rc;
