@@ -29,6 +29,9 @@ SIGNATURES = {
     "hkm_lloyd_kernel_name": (c_char_p, [c_int64, c_int32, c_int32]),
     "hkm_assign_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_static_scratch_bytes": (c_size_t, []),
+    "hkm_assign_static_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                             c_void_p, c_void_p, c_void_p]),
     "hkm_update_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
@@ -205,6 +208,16 @@ def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optio
     buf = ws.get(need)
     check(load().hkm_assign_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k, c.stride(0) if k > 1 else d,
                                 _ptr(labels), _ptr(min_d2), _ptr(buf), buf.numel(), _stream()))
+
+
+def assign_static(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optional[torch.Tensor]) -> None:
+    """:func:`assign` (float32) on the library's built-in scratch array: no workspace, no allocation."""
+    _require_gpu(x, c, labels, min_d2)
+    _require_rows(x, c)
+    n, d = x.shape
+    k = c.shape[0]
+    check(load().hkm_assign_static_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
+                                       c.stride(0) if k > 1 else d, _ptr(labels), _ptr(min_d2), _stream()))
 
 
 def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: Optional[torch.Tensor],

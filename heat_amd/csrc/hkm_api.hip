@@ -1,5 +1,6 @@
 // C ABI of libhkm: host-side validation, workspace carving and kernel dispatch.
 // Nothing here allocates device memory or synchronises; every entry point only enqueues kernels.
+#include <pthread.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -257,6 +258,62 @@ int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const floa
     const size_t need = carve(nullptr, N, D, K, HKM_WS_ASSIGN).total;
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const Workspace w = carve(ws, N, D, K, HKM_WS_ASSIGN);
+    return do_assign(X, N, D, ldx, C, K, ldc, labels, min_d2, w, static_cast<hipStream_t>(hip_stream));
+}
+
+// ---- hkm_assign_static_f32: the assignment without a caller-supplied workspace -----------------
+// The scratch of the assignment kernels (reduction slots, squared centroid norms, merge keys of the
+// streaming kernel) lives in this file-scope device array.  Its name is a host-side handle only: the
+// device address is looked up once per device with hipGetSymbolAddress and that pointer is what the
+// launchers receive.
+static __device__ __align__(256) unsigned char scratch[HKM_STATIC_SCRATCH_BYTES];
+
+static const int STATIC_MAX_DEVICES = 64;
+static void* g_scratch_ptr[STATIC_MAX_DEVICES];  // device address of `scratch` on every device, once known
+static pthread_mutex_t g_scratch_lock = PTHREAD_MUTEX_INITIALIZER;
+
+// Address of the current device's copy of `scratch` (every device holds its own).
+static int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(HKM_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES)
+        return fail(HKM_EUNSUPPORTED, "device ordinal %d outside 0..%d", dev, STATIC_MAX_DEVICES - 1);
+    pthread_mutex_lock(&g_scratch_lock);
+    void* p = g_scratch_ptr[dev];
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e == hipSuccess && !p) e = hipErrorInvalidSymbol;
+        if (e == hipSuccess) g_scratch_ptr[dev] = p;
+    }
+    pthread_mutex_unlock(&g_scratch_lock);
+    if (e != hipSuccess) return fail(HKM_EHIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    *out = p;
+    return HKM_OK;
+}
+
+size_t hkm_static_scratch_bytes(void) { return HKM_STATIC_SCRATCH_BYTES; }
+
+int hkm_assign_static_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                          int64_t ldc, int32_t* labels, float* min_d2, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C", C, K, D, ldc))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    const size_t need = carve(nullptr, N, D, K, HKM_WS_ASSIGN).total;
+    if (need > HKM_STATIC_SCRATCH_BYTES)
+        return fail(HKM_EUNSUPPORTED,
+                    "N = %lld, D = %d, K = %d needs %zu bytes of scratch, the built-in array holds %zu: "
+                    "use hkm_assign_f32 with a workspace",
+                    (long long)N, D, K, need, size_t(HKM_STATIC_SCRATCH_BYTES));
+    if (N == 0) return HKM_OK;
+    void* base = nullptr;
+    if ((rc = static_scratch(&base))) return rc;
+    // every kernel that reads the scratch is preceded on the stream by the one that fills it (norms,
+    // key fill), so nothing of an earlier call's contents is read
+    const Workspace w = carve(base, N, D, K, HKM_WS_ASSIGN);
     return do_assign(X, N, D, ldx, C, K, ldc, labels, min_d2, w, static_cast<hipStream_t>(hip_stream));
 }
 

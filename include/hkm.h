@@ -76,6 +76,23 @@ int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const floa
                    void* hip_stream);
 
 /*
+ * hkm_assign_f32 for callers that cannot allocate device memory or carry a workspace: code under HIP
+ * graph capture, tight serving loops (predict), harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  Same arguments, results and kernels as hkm_assign_f32, but the scratch (reduction slots,
+ * squared centroid norms, the merge keys of the D > 64 kernel) is a device array of
+ * HKM_STATIC_SCRATCH_BYTES built into the library, which every GPU the library runs on holds from the
+ * first call on it until the process ends.  The call allocates and frees nothing.  Shapes whose
+ * hkm_workspace_bytes(N, D, K, HKM_WS_ASSIGN) exceeds HKM_STATIC_SCRATCH_BYTES return HKM_EUNSUPPORTED
+ * (D <= 64: every K up to about four million; D > 64: up to about two million rows, 8 bytes each).
+ * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
+ * calls on one stream are ordered and each refills what it reads.
+ */
+#define HKM_STATIC_SCRATCH_BYTES (16u << 20)
+size_t hkm_static_scratch_bytes(void);
+int hkm_assign_static_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                          int64_t ldc, int32_t* labels, float* min_d2, void* hip_stream);
+
+/*
  * Deterministic per-cluster mean: C_new[k] = (sum over {i: labels[i]==k} of x_i) / count_k, sums
  * in fp64, count rounded through fp32 like the reference does; an empty cluster gives a zero row.
  * counts (int64[K]) may be NULL.  labels outside [0, K) are ignored.
