@@ -234,7 +234,12 @@ __device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (
     const unsigned gj0 = unsigned(j0) + 4 * h;
     float dv[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) dv[i] = fmaxf(fmaf(-2.0f, acc[i], qn + xnv[i]), 0.0f);
+    for (int i = 0; i < 16; ++i) {
+        // compare + select, not fmaxf: a NaN (a NaN row, inf - inf of overflowing norms) must stay a NaN,
+        // which fails every `< thr` below and is never admitted; fmaxf would turn it into distance 0
+        const float t = fmaf(-2.0f, acc[i], qn + xnv[i]);
+        dv[i] = t < 0.0f ? 0.0f : t;
+    }
     if (j0 + 32 > r_end || has_bound) {
         // the last tile of a split and the later passes: rows past the end and pairs that do not rank
         // after the bound become +inf here, so that one chain of offers serves every tile

@@ -422,13 +422,29 @@ def label_agreement(
     that magnitude, so its value is a multiple of their ulp and carries the rounding of a D-term dot
     product; squared distances closer than that are not ordered reliably by the reference either.
 
-    Returns dict(n, n_diff, n_unexcused, agreement).
+    Next to that, the rule is also evaluated WITHOUT the second term, exactly as it is stated: a
+    differing row is *strict* when its fp64 best and second-best squared distances (over all centroids)
+    are further apart than ``rel_gap`` relative, ``(d2_second - d2_best) / d2_best > rel_gap`` -- such a
+    row has one clear nearest centroid and the two labelings should not differ on it.  ``n_strict`` counts
+    them, ``max_strict_gap`` is the largest such relative gap over all differing rows (0 if none differ)
+    and ``max_strict_abs`` the largest absolute gap in units of eps32 * (|x|^2 + |c|^2), i.e. in units of
+    the resolution of the fp32 expansion at that row.  On a strict row one of the two labelings is not the
+    fp64 nearest centroid: ``n_strict_a_wrong`` counts the strict rows where that is ``labels_a``,
+    ``n_strict_b_wrong`` those where it is ``labels_b`` (with ``labels_b`` the reference's labels these are
+    the rows its own fp32 rounding misorders: an evaluation in exact arithmetic differs from it there too).
+
+    Returns dict(n, n_diff, n_unexcused, agreement, n_strict, n_strict_a_wrong, n_strict_b_wrong,
+    max_strict_gap, max_strict_abs).
     """
     a = labels_a.view(-1).to(torch.int64).cpu()
     b = labels_b.view(-1).to(torch.int64).cpu()
     n = a.numel()
     diff = torch.nonzero(a != b).view(-1)
     n_unexcused = 0
+    n_strict = n_strict_a = n_strict_b = 0
+    max_strict_gap = 0.0
+    max_strict_abs = 0.0
+    eps32 = float(torch.finfo(torch.float32).eps)
     c64 = centers.to(torch.float64).cpu()
     cn = (c64**2).sum(1)
     dfac = max(2.0, math.sqrt(x.shape[1]) / 4.0) * float(torch.finfo(torch.float32).eps)
@@ -443,11 +459,27 @@ def label_agreement(
         lim = best * (1.0 + rel_gap) + dfac * mag + 1e-300
         ok = (da <= lim) & (db <= lim)
         n_unexcused += int((~ok).sum())
+        if d2.shape[1] > 1:
+            two = torch.topk(d2, 2, dim=1, largest=False).values
+            gap_abs = two[:, 1] - two[:, 0]
+            gap = gap_abs / two[:, 0].clamp_min(1e-300)
+            strict = gap > rel_gap
+            n_strict += int(strict.sum())
+            true_lab = d2.argmin(dim=1)
+            n_strict_a += int((strict & (a[rows] != true_lab)).sum())
+            n_strict_b += int((strict & (b[rows] != true_lab)).sum())
+            max_strict_gap = max(max_strict_gap, float(gap.max()))
+            max_strict_abs = max(max_strict_abs, float((gap_abs / (eps32 * mag).clamp_min(1e-300)).max()))
     return {
         "n": n,
         "n_diff": int(diff.numel()),
         "n_unexcused": n_unexcused,
         "agreement": 1.0 - diff.numel() / max(n, 1),
+        "n_strict": n_strict,
+        "n_strict_a_wrong": n_strict_a,
+        "n_strict_b_wrong": n_strict_b,
+        "max_strict_gap": max_strict_gap,
+        "max_strict_abs": max_strict_abs,
     }
 
 

@@ -7,6 +7,19 @@ Bar (fp32): labels equal wherever the fp64 best/second-best squared distances di
 1e-5 relative and >= 99.99 % overall; centroids, inertia_ (the last centroid shift) and
 functional_value_ within 1e-4 relative (shift with an absolute floor of 1e-6 * mean|c|^2);
 n_iter_ equal; repeated runs bit-identical.
+
+Labels, in detail.  Every comparison reports (and the session prints, after the test summary) the number
+of differing rows and, of those, the *strict* ones: rows whose fp64 best and second-best squared
+distances are more than 1e-5 relative apart.  The reference computes (|x|^2 + |c|^2) - 2 x.c in fp32, whose
+own rounding (an ulp of |x|^2 + |c|^2 is 1e-5 of a typical squared distance on the D = 32 workload and up
+to 1e-4 on the D = 3 one) misorders such rows now and then: an evaluation of its formula in EXACT
+arithmetic differs from it on the same rows (tests/test_oracle_pins.py).  What is asserted:
+  * no difference outside the resolution of the expansion (n_unexcused == 0, see oracle.label_agreement);
+  * on the D >= 8 workloads (c1 - c4) at most 4 strict rows per million comparisons, none with an fp64 gap
+    above 5e-5 relative (on such a row either side may be the one that missed the
+    fp64 nearest centroid: both evaluate in fp32; the report says which);
+  * on the D = 3 workload (c5; coordinates up to 100, squared distances from 3) every differing row within
+    2 ulp of |x|^2 + |c|^2 (max_strict_abs <= 2) and at most 2 strict rows per million.
 """
 import os
 
@@ -20,6 +33,18 @@ from oracle import heat_oracle as orc
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _label_bar(rep, name, report, narrow=False):
+    """The label bar of this file's header on one comparison; ``narrow`` selects the D = 3 form."""
+    report(f"{name}: n={rep['n']} differing={rep['n_diff']} strict(>1e-5 fp64 gap)={rep['n_strict']} "
+           f"[product misses fp64 nearest: {rep['n_strict_a_wrong']}, reference misses it: {rep['n_strict_b_wrong']}] "
+           f"max_strict_gap={rep['max_strict_gap']:.3e} max_gap_in_ulp_of_expansion={rep['max_strict_abs']:.2f}")
+    assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, (name, rep)
+    if narrow:
+        assert rep["max_strict_abs"] <= 2.0 and rep["n_strict"] <= max(2, 2e-6 * rep["n"]), (name, rep)
+    else:
+        assert rep["n_strict"] <= max(2, 4e-6 * rep["n"]) and rep["max_strict_gap"] <= 5e-5, (name, rep)
 
 
 def _fit(x_cpu, init_cpu, k, iters, tol, dev):
@@ -55,7 +80,7 @@ def _check_fit(km, x_cpu, ref_centers, ref_labels, ref_inertia, ref_n_iter, tie_
         assert agree >= 0.99, agree
 
 
-def _stepwise_parity(w, dev, iters, literal):
+def _stepwise_parity(w, dev, iters, literal, report=print):
     """Walk the ORACLE's trajectory; at every iteration run one GPU Lloyd step from the oracle's current
     centroids and compare: labels (gap rule, no unexcused difference), centroids against the oracle's
     update of the GPU's own labels (1e-5) and against the oracle's new centroids when the labels are
@@ -70,6 +95,8 @@ def _stepwise_parity(w, dev, iters, literal):
     c_ref = w.init.clone()
     flips = 0
     n_iter = 0
+    tot = dict(n=0, n_diff=0, n_strict=0, n_strict_a_wrong=0, n_strict_b_wrong=0, max_strict_gap=0.0,
+               max_strict_abs=0.0, n_unexcused=0)
     for _ in range(iters):
         n_iter += 1
         c_in = c_ref.to(dev)
@@ -84,6 +111,10 @@ def _stepwise_parity(w, dev, iters, literal):
         rep = orc.label_agreement(w.x, c_ref, lab.cpu(), ref_lab)
         assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, (n_iter, rep)
         flips += rep["n_diff"]
+        for key in ("n", "n_diff", "n_strict", "n_strict_a_wrong", "n_strict_b_wrong"):
+            tot[key] += rep[key]
+        for key in ("max_strict_gap", "max_strict_abs"):
+            tot[key] = max(tot[key], rep[key])
         own, _ = orc.update_centroids_fast(w.x, lab.cpu().long().view(-1, 1), w.k)
         assert orc.rel_err_centers(c_out.cpu(), own) <= 1e-5, n_iter
         if rep["n_diff"] == 0:
@@ -95,6 +126,9 @@ def _stepwise_parity(w, dev, iters, literal):
         c_ref = ref_new.clone()
         if bool(inertia <= 0.0):
             break
+    tot["agreement"] = 1.0 - tot["n_diff"] / max(tot["n"], 1)
+    _label_bar(tot, f"{w.name} {tuple(w.x.shape)}, {n_iter} steps along the oracle's trajectory", report,
+               narrow=w.x.shape[1] < 8)
     return flips, dict(cluster_centers=c_ref, labels=ref_lab, inertia=inertia, n_iter=n_iter)
 
 
@@ -126,9 +160,9 @@ def test_fit_restarts_from_cluster_centers(cuda):
     assert np.allclose(full.cluster_centers_.numpy(), z["centers"], rtol=1e-5)
 
 
-def test_config1_full_size_against_literal_oracle(cuda):
+def test_config1_full_size_against_literal_oracle(cuda, parity_report):
     w = synthetic.config1()
-    flips, ref = _stepwise_parity(w, cuda, w.max_iter, literal=True)
+    flips, ref = _stepwise_parity(w, cuda, w.max_iter, literal=True, report=parity_report)
     print(f"config1: {flips} excused tie flips over {ref['n_iter']} iterations", flush=True)
     km, xd = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
     _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
@@ -148,17 +182,17 @@ def test_config1_full_size_against_literal_oracle(cuda):
 
 
 @pytest.mark.parametrize("cfg,scale", [("c3", 0.01), ("c4", 0.004), ("c5", 0.005)])
-def test_scaled_configs_against_oracle(cuda, cfg, scale):
+def test_scaled_configs_against_oracle(cuda, cfg, scale, parity_report):
     w = synthetic.CONFIGS[cfg](scale)
     print(f"{w.name} scaled to {tuple(w.x.shape)}", flush=True)
-    flips, ref = _stepwise_parity(w, cuda, w.max_iter, literal=False)
+    flips, ref = _stepwise_parity(w, cuda, w.max_iter, literal=False, report=parity_report)
     print(f"{w.name}: {flips} excused tie flips over {ref['n_iter']} iterations", flush=True)
     km, _ = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
     _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
 
 
 @pytest.mark.parametrize("scale", [1.0 / 16, 1.0])
-def test_config2_cdist_argmin(cuda, scale):
+def test_config2_cdist_argmin(cuda, scale, parity_report):
     from heat_amd import _native
 
     w = synthetic.config2(scale)
@@ -168,15 +202,15 @@ def test_config2_cdist_argmin(cuda, scale):
     _native.assign(w.x.to(cuda), w.y.to(cuda), lab, md, _native.Workspace(cuda))
     ref_lab, ref_md = orc.assign_to_cluster_fast(w.x, w.y, want_min=True)
     rep = orc.label_agreement(w.x, w.y, lab.cpu(), ref_lab)
-    assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, rep
+    _label_bar(rep, f"{w.name} {tuple(w.x.shape)} vs {tuple(w.y.shape)}", parity_report)
     same = lab.cpu().long() == ref_lab.view(-1)
     assert torch.allclose(md.cpu()[same], ref_md[same], rtol=1e-4, atol=1e-3)
 
 
-def _full_size_properties(w, dev, iters):
+def _full_size_properties(w, dev, report, iters):
     """Properties that hold at any size: counts sum to N, sum_k n_k C_k = sum_i x_i, the shift
-    sequence is what the centroids say, SSE does not increase, predict == re-assignment, a random row
-    sample agrees with the oracle, and two runs are bit-identical."""
+    sequence is what the centroids say, SSE does not increase, predict == re-assignment, and two runs are
+    bit-identical; the labels of the first step are compared with the oracle's on EVERY row."""
     from heat_amd import _native
 
     n, d = w.x.shape
@@ -200,11 +234,10 @@ def _full_size_properties(w, dev, iters):
         assert orc.rel_err_scalar(float(shift), float(ref_shift), floor=1e-12) <= 1e-4
         sse_hist.append(float(sse))
         if it == 0:
-            # a seeded row sample against the oracle, same centroids
-            idx = torch.randperm(n, generator=torch.Generator().manual_seed(1))[:200_000]
-            ref_lab, _ = orc.assign_to_cluster_fast(w.x[idx], w.init)
-            rep = orc.label_agreement(w.x[idx], w.init, lab[idx.to(dev)].cpu(), ref_lab)
-            assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, rep
+            # every row against the oracle, same centroids
+            ref_lab, _ = orc.assign_to_cluster_fast(w.x, w.init)
+            rep = orc.label_agreement(w.x, w.init, lab.cpu(), ref_lab)
+            _label_bar(rep, f"{w.name} full size, first step", report, narrow=d < 8)
         c_cur, c_nxt = c_nxt, c_cur
     assert all(b <= a * (1 + 1e-5) for a, b in zip(sse_hist, sse_hist[1:])), sse_hist
     km = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(dev)), max_iter=iters, tol=0.0).fit(xd)
@@ -216,16 +249,16 @@ def _full_size_properties(w, dev, iters):
     assert torch.equal(pred.larray.view(-1), lab2.long())
 
 
-def test_config3_full_size_properties(cuda):
-    _full_size_properties(synthetic.config3(), cuda, iters=3)
+def test_config3_full_size_properties(cuda, parity_report):
+    _full_size_properties(synthetic.config3(), cuda, parity_report, iters=3)
 
 
-def test_config5_full_size_properties(cuda):
-    _full_size_properties(synthetic.config5(), cuda, iters=2)
+def test_config5_full_size_properties(cuda, parity_report):
+    _full_size_properties(synthetic.config5(), cuda, parity_report, iters=2)
 
 
-def test_config4_full_size_properties(cuda):
-    _full_size_properties(synthetic.config4(), cuda, iters=2)
+def test_config4_full_size_properties(cuda, parity_report):
+    _full_size_properties(synthetic.config4(), cuda, parity_report, iters=2)
 
 
 def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):

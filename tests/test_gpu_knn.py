@@ -236,3 +236,38 @@ def test_argument_checks(cuda):
         knn.predict(ht.array(x))
     empty = torch.empty((0, 2), dtype=torch.int64, device=cuda)
     _native.knn(x[:0], x, 2, empty, None, ws)             # no test rows: nothing to do
+
+
+@pytest.mark.parametrize("m,n,d,k", [
+    (40, 300, 8, 5),       # vector-ALU kernel
+    (500, 300, 32, 5),     # matrix-core kernel, one split of the training rows
+    (7, 20000, 32, 6),     # matrix-core kernel, many splits
+    (130, 400, 64, 16),    # matrix-core kernel, wide rows, full lists
+    (9, 30000, 64, 20),    # many splits and a second pass (k > 16)
+    (33, 200, 100, 3),     # unaligned feature count on the matrix cores
+])
+def test_non_finite_rows_are_never_neighbours(cuda, m, n, d, k):
+    """A NaN training row, a training row whose squared norm overflows, and a NaN query row: the bad training
+    rows must never be returned (torch.topk(largest=False) ranks NaN last), every other list must equal the
+    exact one over the remaining rows, and the NaN query's slots hold index -1 and distance inf."""
+    g = torch.Generator().manual_seed(m + n + d + k)
+    x = torch.randint(-6, 7, (n, d), generator=g).float()
+    q = torch.randint(-6, 7, (m, d), generator=g).float()
+    nan_row, big_row, nan_query = 3, n - 2, m - 1
+    x[nan_row, d // 2] = float("nan")
+    x[big_row] = 3e19           # |x|^2 = inf in float32
+    q[nan_query, 0] = float("nan")
+    good = torch.ones(n, dtype=torch.bool)
+    good[nan_row] = good[big_row] = False
+    rows = torch.nonzero(good).view(-1)
+    want_i, want_d2 = _exact_lists(q[:nan_query], x[good], k)
+    want_i = rows[want_i]
+    idx = torch.full((m, k), -7, dtype=torch.int64, device=cuda)
+    dist = torch.full((m, k), -7.0, device=cuda)
+    print(f"knn non-finite m={m} n={n} d={d} k={k}", flush=True)
+    _native.knn(q.to(cuda), x.to(cuda), k, idx, dist, _native.Workspace(cuda))
+    idx, dist = idx.cpu(), dist.cpu()
+    assert not bool(((idx == nan_row) | (idx == big_row)).any())
+    assert torch.equal(idx[:nan_query], want_i)
+    assert torch.equal(dist[:nan_query], torch.from_numpy(np.sqrt(want_d2.numpy()).astype(np.float32)))
+    assert bool((idx[nan_query] == -1).all()) and bool(torch.isinf(dist[nan_query]).all())

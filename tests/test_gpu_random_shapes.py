@@ -59,7 +59,9 @@ def test_kmeans_entry_points_on_random_shapes(cuda, seed, products, monkeypatch)
         assert int(((lab < 0) | (lab >= k)).sum()) == 0, what
         got = d2.gather(1, lab.long().view(-1, 1)).view(-1)
         scale = (xd * xd).sum(1) + (c.double() ** 2).sum(1).max()
-        tol = 1e-5 * best + 4e-7 * max(2.0, d ** 0.5 / 4) * scale
+        # accuracy against the exact distances (no reference labels here): the centroid chosen is the
+        # nearest up to 1e-5 relative plus two roundings of the fp32 expansion (eps32 = 1.19e-7)
+        tol = 1e-5 * best + 2.4e-7 * max(2.0, d ** 0.5 / 4) * scale
         assert int((got - best > tol).sum()) == 0, what
         assert int(((md.double() - best).abs() > tol + 1e-6 * scale).sum()) == 0, what
         if dup and k // 2 != 0:
