@@ -12,6 +12,17 @@ vector kernel (D <= 8), writing N labels is a quarter of the step's memory traff
 without storing labels and those of the last iteration are computed once, on demand, against the
 centroids that iteration started from -- the same kernel code, hence the same bits.  The values
 returned are exactly those of the sequential loop.
+
+The stop decision.  The two one-sweep kernels form their per-cluster sums on the way (rows pre-rounded
+to 28 bits below their largest coordinate on the matrix cores, fp32 partial sums per lane in the narrow
+kernel), so their means can differ from the fp64 divide-then-sum of heat/cluster/kmeans.py:76-103 in the
+last bit.  That is far inside the 1e-4 bar on the centroids but it decides ``shift <= tol`` when the shift
+is (nearly) zero: a fit sitting on a fixed point of the reference's arithmetic would run one iteration
+longer.  So whenever a one-sweep step reports a shift within its own rounding error of the tolerance --
+in particular before EVERY stop -- the means of that iteration are recomputed from its labels with the
+two-pass update (fp64 from the first addition to the division, fixed order: bit-identical to the
+reference's means in all but about one coordinate in a thousand), and the decision is taken on that
+shift.  If the loop goes on, the step enqueued ahead is re-issued from the recomputed centroids.
 """
 
 from __future__ import annotations
@@ -31,7 +42,13 @@ class LloydLoop:
         self.ws = ws
         self.c = [c0.clone(), torch.empty_like(c0), torch.empty_like(c0)]
         n, d = xt.shape
-        self.lazy_labels = xt.dtype == torch.float32 and _native.lloyd_kernel_name(n, d, c0.shape[0]) == "lloyd_small"
+        kernel = _native.lloyd_kernel_name(n, d, c0.shape[0]) if xt.dtype == torch.float32 else ""
+        self.lazy_labels = kernel == "lloyd_small"
+        # relative size (against sum |c|^2) of the squared centroid movement below which a one-sweep step's
+        # shift is within the rounding error of its own sums; 0 for the shapes that run the two-pass update
+        self._fuzz = {"lloyd_small": 1e-11 * d, "lloyd_mfma_resident": 1e-13 * d}.get(kernel, 0.0)
+        self._cscale: Optional[float] = None
+        self.rechecks = 0  # iterations whose means were recomputed by the two-pass update
         nbuf = 1 if self.lazy_labels else 2
         self.lab = [torch.empty((n,), dtype=torch.int32, device=dev) for _ in range(nbuf)]
         self._lab_of = -1  # iteration whose labels self.lab[0] holds (lazy mode)
@@ -72,9 +89,38 @@ class LloydLoop:
             self.ev[i % 2].synchronize()
             self.done = i + 1
             ran += 1
-            if float(self.shift_host[i % 2]) <= tol:
+            shift = float(self.shift_host[i % 2])
+            if self._fuzz and shift <= tol + self._margin(tol):
+                shift = self._recompute(i)
+            if shift <= tol:
                 break
         return ran
+
+    def _margin(self, tol: float) -> float:
+        """How far above ``tol`` a one-sweep step's shift may sit while the exact one is <= tol: with
+        e = the rounding error of the step's centroids, |shift - exact| <= 2 sqrt(exact) |e| + |e|^2."""
+        if self._cscale is None:
+            self._cscale = float((self.c[0].double() ** 2).sum())
+        e2 = self._fuzz * self._cscale
+        return 2.0 * (max(tol, 0.0) * e2) ** 0.5 + e2
+
+    def _recompute(self, i: int) -> float:
+        """Replace the centroids step i produced by the two-pass means of its labels; returns the shift."""
+        if self.lazy_labels:
+            if self._lab_of != i:
+                _native.assign(self.x, self.c[i % 3], self.lab[0], None, self.ws)
+                self._lab_of = i
+            lab = self.lab[0]
+        else:
+            lab = self.lab[i % 2]
+        _native.update(self.x, lab, self.c[(i + 1) % 3], None, self.ws)
+        out = torch.empty((), dtype=self.x.dtype, device=self.x.device)
+        _native.shift(self.c[i % 3], self.c[(i + 1) % 3], out)
+        self.shift_host[i % 2] = out.cpu()  # synchronises
+        self.ev[i % 2].record()
+        self.enqueued = i + 1  # a step enqueued ahead started from the centroids just replaced
+        self.rechecks += 1
+        return float(self.shift_host[i % 2])
 
     # results of the last iteration that counts
     @property

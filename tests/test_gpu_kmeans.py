@@ -270,6 +270,7 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
 
     w = synthetic.config1(0.5)
     x = w.x.to(cuda)
+    probe = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
     for tol in (1e-1, 1e-3, 0.0, None):
         ws = _native.Workspace(cuda)
         c_cur = w.init.to(cuda).clone()
@@ -280,6 +281,10 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
         for _ in range(40):
             n_seq += 1
             _native.lloyd_step(x, c_cur, c_nxt, lab, shift, None, ws)
+            if tol is not None and float(shift) <= tol + probe._margin(tol):
+                # the loop's rule: a one-sweep step near the stop decision is settled by the two-pass means
+                _native.update(x, lab, c_nxt, None, ws)
+                _native.shift(c_cur, c_nxt, shift)
             c_cur, c_nxt = c_nxt, c_cur
             if tol is not None and float(shift) <= tol:
                 break
@@ -298,6 +303,59 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
     assert torch.equal(a.centers, b.centers) and torch.equal(a.labels, b.labels)
     with pytest.raises(ValueError):
         ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(cuda)), max_iter=0).fit(ht.array(x, split=0))
+
+
+# ---- closed forms of the loop (heat/cluster/kmeans.py:131-146) through the public estimator --------
+# shapes: the one-sweep matrix-core step (D = 32), the narrow one-sweep step (D = 3 and D = 8), and a
+# shape that runs assignment + two-pass update (D = 100)
+@pytest.mark.parametrize("n,d", [(64, 32), (200, 32), (8, 3), (16, 8), (30, 5), (50, 100)])
+def test_every_row_its_own_centroid_is_a_fixed_point(cuda, n, d, parity_report):
+    """K = N distinct rows as init: every cluster holds exactly its own row, the means are the rows, the
+    shift is exactly 0 and the loop stops after ONE iteration (kmeans.py:141-143), as the oracle does."""
+    g = torch.Generator().manual_seed(n + d)
+    x = torch.randn((n, d), generator=g) * 3.0
+    x[:, 0] *= 1e-4  # coordinates far below the row's largest: the bits a pre-rounded sum would lose
+    ref = orc.kmeans_fit(x, x.clone(), 10, 0.0, literal=True)
+    assert ref["n_iter"] == 1 and float(ref["inertia"]) == 0.0
+    km, _ = _fit(x, x.clone(), n, 10, 0.0, cuda)
+    parity_report(f"fixed point K=N={n} D={d}: n_iter_ {km.n_iter_} (oracle {ref['n_iter']}), inertia_ {float(km.inertia_):.3g}")
+    assert km.n_iter_ == 1 and float(km.inertia_) == 0.0
+    assert torch.equal(km.cluster_centers_.larray.cpu(), x)
+    assert torch.equal(km.labels_.larray.cpu().view(-1), torch.arange(n))
+
+
+@pytest.mark.parametrize("n,d", [(20000, 32), (30000, 3), (20000, 8), (5000, 100)])
+def test_init_at_the_means_of_two_far_blobs_stops_like_the_oracle(cuda, n, d, parity_report):
+    """Two blobs far apart, init = their means (fp64 means rounded to fp32): the first iteration assigns
+    every point to its blob and reproduces the means, so the reference stops at once with shift 0."""
+    g = torch.Generator().manual_seed(d)
+    a = torch.randn((n // 2, d), generator=g) + 20.0
+    b = torch.randn((n - n // 2, d), generator=g) * 0.5 - 20.0
+    x = torch.cat([a, b])[torch.randperm(n, generator=g)].contiguous()
+    far = x[:, 0] > 0
+    init = torch.stack([x[far].double().mean(0), x[~far].double().mean(0)]).float()
+    ref = orc.kmeans_fit(x, init, 10, 0.0, literal=True)
+    km, _ = _fit(x, init, 2, 10, 0.0, cuda)
+    parity_report(f"two blobs N={n} D={d}: n_iter_ {km.n_iter_} (oracle {ref['n_iter']}), inertia_ {float(km.inertia_):.3g} "
+                  f"(oracle {float(ref['inertia']):.3g})")
+    assert km.n_iter_ == ref["n_iter"]
+    assert float(km.inertia_) == float(ref["inertia"])
+    assert torch.equal(km.labels_.larray.cpu().view(-1), ref["labels"].view(-1))
+    assert orc.rel_err_centers(km.cluster_centers_.larray.cpu(), ref["cluster_centers"]) <= 1e-6
+
+
+@pytest.mark.parametrize("n,d", [(5000, 32), (5000, 3), (3000, 100)])
+def test_one_cluster_is_the_global_mean(cuda, n, d, parity_report):
+    g = torch.Generator().manual_seed(n + d)
+    x = torch.randn((n, d), generator=g) * 2.0 + 1.0
+    init = x[:1].clone()
+    ref = orc.kmeans_fit(x, init, 10, 0.0, literal=True)
+    km, _ = _fit(x, init, 1, 10, 0.0, cuda)
+    parity_report(f"K=1 N={n} D={d}: n_iter_ {km.n_iter_} (oracle {ref['n_iter']})")
+    assert km.n_iter_ == ref["n_iter"] == 2
+    assert float(km.inertia_) == 0.0
+    assert torch.allclose(km.cluster_centers_.larray.cpu().double(), x.double().mean(0, keepdim=True), rtol=1e-6, atol=1e-7)
+    assert int(km.labels_.larray.abs().max()) == 0
 
 
 def test_random_init_and_fit_predict(cuda):
