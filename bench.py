@@ -11,11 +11,18 @@ already enqueued while it does.  Inputs are resident in HBM before the timed reg
 JSON line.  The default warm-up is 30 steps because a kernel launched on an idle device runs up to
 30 % longer during the first ~25 ms of load than afterwards (measured per launch with rocprofv3).
 
-value      points*iterations / s over the timed region (wall clock, synchronised both sides)
-roofline   the dominant kernel (fused distance+argmin; for the one-sweep shapes the whole step, whose
-           other launches take some 15 us) timed with events on the launch stream:
-           algorithmic flops 2*N*K*D (MFMA-bound shapes) or bytes N*(4D+4) (HBM-bound shapes) per
-           launch divided by its mean duration
+value      points*iterations / s over the timed region (wall clock, synchronised both sides).  The region
+           of --steps steps is run five times back to back; ms_per_step (and value) is the MEDIAN region,
+           ms_per_step_min / ms_per_step_max the fastest and slowest
+roofline   the dominant kernel -- the fused distance+argmin kernel, or the one-sweep kernel that also forms
+           the per-cluster sums -- timed ALONE: the library records an event pair on the launch stream
+           right around that kernel's launch (hkm_profile_enable) during one more pass of the same --steps
+           steps; kernel_ms is the mean over those launches, achieved = algorithmic flops 2*N*K*D
+           (MFMA-bound shapes) or bytes N*(4D+4) (HBM-bound shapes) per launch / kernel_ms.
+           step_ms_events is the whole step (all its launches, no host read) between two events.
+           traffic (HBM bytes per launch, rocprofv3 FETCH_SIZE / WRITE_SIZE) is read from
+           profiles/traffic.json and only reported while the library sources still hash to what they
+           were when it was measured (traffic_source says which)
 cpu_baseline  the CPU restatement of the reference's op sequence (oracle/, torch CPU, all host
            threads) on a bounded row sample of the same workload
 """
@@ -27,6 +34,20 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+
+def library_sources_sha1() -> str:
+    """Hash of the HIP sources the kernels are built from: ties a committed counter reading to the code."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha1()
+    files = sorted(glob.glob(os.path.join(ROOT, "heat_amd", "csrc", "*.hip")) +
+                   glob.glob(os.path.join(ROOT, "heat_amd", "csrc", "*.h")))
+    for f in files:
+        with open(f, "rb") as fh:
+            h.update(os.path.basename(f).encode() + b"\0" + fh.read())
+    return h.hexdigest()[:12]
+
 
 PEAK_HBM_GBS = 8000.0
 PEAK_FP32_MFMA_TFLOPS = 157.3
@@ -411,13 +432,28 @@ def main() -> int:
     if prewarm:
         steps(prewarm)
     steps(args.warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    steps(args.steps)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    regions = []
+    for _ in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps(args.steps)
+        torch.cuda.synchronize()
+        regions.append(time.perf_counter() - t0)
+    elapsed = sorted(regions)[len(regions) // 2]
 
-    # dominant kernel alone, event-timed on the stream it is launched on (torch's current stream)
+    # the dominant kernel alone: one more pass of the same steps with the library recording an event pair
+    # on the launch stream right around that kernel (and nothing else)
+    _native.profile_enable(True)
+    if args.config == "c2":
+        steps(min(args.steps, 512))
+    else:
+        assert loop.run(min(args.steps, 512), -1.0) == min(args.steps, 512)
+    torch.cuda.synchronize()
+    kern = _native.profile_collect()
+    _native.profile_enable(False)
+    kern_ms = sum(kern) / len(kern)
+
+    # the whole step (every launch of it, no host read) between two events on the same stream
     for _ in range(args.steps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -425,7 +461,7 @@ def main() -> int:
         e1.record()
         torch.cuda.synchronize()
         ev_ms.append(e0.elapsed_time(e1))
-    kern_ms = sum(ev_ms) / len(ev_ms)
+    step_ms = sum(ev_ms) / len(ev_ms)
 
     # both fractions for every workload; the binding one fills the standard fields
     flops = 2.0 * n * k * d
@@ -442,11 +478,21 @@ def main() -> int:
     roof["hbm_frac"] = round(gbs / PEAK_HBM_GBS, 4)
     roof["kernel"] = kernel
     roof["kernel_ms"] = round(kern_ms, 4)
+    roof["kernel_launches_timed"] = len(kern)
+    roof["step_ms_events"] = round(step_ms, 4)
     roof["traffic"] = None
+    roof["traffic_source"] = "none: profiles/traffic.json is missing"
     tfile = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tfile):
         with open(tfile) as f:
-            roof["traffic"] = json.load(f).get(w.name)
+            tj = json.load(f)
+        sha = library_sources_sha1()
+        if tj.get("sources_sha1") == sha and args.scale == 1.0:
+            roof["traffic"] = tj.get(w.name)
+            roof["traffic_source"] = f"profiles/traffic.json, measured on library sources sha1 {sha} (= this build)"
+        else:
+            roof["traffic_source"] = (f"dropped: profiles/traffic.json was measured on library sources sha1 "
+                                      f"{tj.get('sources_sha1')}, this build is {sha}")
 
     # Not the headline: the same timed loop with the opt-in split-bf16 products (HKM_PRODUCTS=bf16x3;
     # every product still accurate to fp32, evaluated as six bf16 partial products on the bf16 matrix
@@ -496,6 +542,9 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "ms_per_step_min": round(min(regions) / args.steps * 1e3, 4),
+        "ms_per_step_max": round(max(regions) / args.steps * 1e3, 4),
+        "timed_regions": len(regions),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -32,6 +32,8 @@ SIGNATURES = {
     "hkm_static_scratch_bytes": (c_size_t, []),
     "hkm_assign_static_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                              c_void_p, c_void_p, c_void_p]),
+    "hkm_profile_enable": (ctypes.c_int, [c_int32]),
+    "hkm_profile_collect": (ctypes.c_int, [c_void_p, c_int32, c_void_p]),
     "hkm_update_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
@@ -218,6 +220,19 @@ def assign_static(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2
     k = c.shape[0]
     check(load().hkm_assign_static_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
                                        c.stride(0) if k > 1 else d, _ptr(labels), _ptr(min_d2), _stream()))
+
+
+def profile_enable(on: bool) -> None:
+    """Benchmarks: record an event pair around the distance kernel of every assign / lloyd_step call."""
+    check(load().hkm_profile_enable(1 if on else 0))
+
+
+def profile_collect() -> list:
+    """Durations (ms) of the distance kernels launched since the last collect, in call order."""
+    buf = (ctypes.c_float * 512)()
+    cnt = c_int32(0)
+    check(load().hkm_profile_collect(ctypes.cast(buf, c_void_p), 512, ctypes.cast(ctypes.pointer(cnt), c_void_p)))
+    return [float(buf[i]) for i in range(min(cnt.value, 512))]
 
 
 def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: Optional[torch.Tensor],

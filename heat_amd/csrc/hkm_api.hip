@@ -26,6 +26,37 @@ int check_launch(const char* what) {
     return HKM_OK;
 }
 
+// ---- timing of the dominant kernel (benchmarks only; off unless hkm_profile_enable(1) was called) ----
+// Per calling thread: a ring of event pairs recorded on the launch stream right before and right after
+// the launch of the distance kernel of hkm_assign_f32 / hkm_lloyd_step_f32, read back (and waited for) by
+// hkm_profile_collect.  Nothing is recorded, created or kept while profiling is off.
+static const int PROF_RING = 512;
+struct ProfState {
+    int on = 0;
+    int count = 0;  // pairs recorded since the last collect
+    hipEvent_t ev[PROF_RING][2] = {};
+    bool made[PROF_RING] = {};
+};
+static thread_local ProfState g_prof;
+
+void prof_begin(hipStream_t st) {
+    ProfState& p = g_prof;
+    if (!p.on || p.count >= PROF_RING) return;
+    const int i = p.count;
+    if (!p.made[i]) {
+        if (hipEventCreate(&p.ev[i][0]) != hipSuccess || hipEventCreate(&p.ev[i][1]) != hipSuccess) return;
+        p.made[i] = true;
+    }
+    (void)hipEventRecord(p.ev[i][0], st);
+}
+
+void prof_end(hipStream_t st) {
+    ProfState& p = g_prof;
+    if (!p.on || p.count >= PROF_RING || !p.made[p.count]) return;
+    (void)hipEventRecord(p.ev[p.count][1], st);
+    p.count++;
+}
+
 int num_cus() {
     static thread_local int cached_dev = -1;
     static thread_local int cached_cus = 256;
@@ -215,6 +246,33 @@ extern "C" {
 int hkm_version(void) { return 200; }
 
 const char* hkm_last_error(void) { return g_err; }
+
+int hkm_profile_enable(int32_t on) {
+    g_err[0] = 0;
+    g_prof.on = on ? 1 : 0;
+    g_prof.count = 0;
+    return HKM_OK;
+}
+
+int hkm_profile_collect(float* ms, int32_t cap, int32_t* count) {
+    g_err[0] = 0;
+    if (!count || (cap > 0 && !ms) || cap < 0) return fail(HKM_EINVAL, "NULL pointer argument or negative capacity");
+    ProfState& p = g_prof;
+    int n = 0;
+    for (int i = 0; i < p.count; ++i) {
+        hipError_t e = hipEventSynchronize(p.ev[i][1]);
+        float t = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&t, p.ev[i][0], p.ev[i][1]);
+        if (e != hipSuccess) {
+            p.count = 0;
+            return fail(HKM_EHIP, "hkm_profile_collect: %s", hipGetErrorString(e));
+        }
+        if (n < cap) ms[n++] = t;
+    }
+    *count = p.count;
+    p.count = 0;
+    return HKM_OK;
+}
 
 size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags) {
     if (N < 0 || D < 1 || K < 1) return 0;

@@ -600,8 +600,10 @@ static int launch_split_tiled_t(const float* X, int64_t N, int32_t D, int64_t ld
     auto kern = assign_split_tiled_kernel<DP, VEC>;
     int64_t grid = int64_t(num_cus()) * 2;
     if (grid > ntiles) grid = ntiles;
+    prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc, cn, labels,
                        min_d2, ntiles);
+    prof_end(st);
     return check_launch("assign_split_tiled_kernel");
 }
 
@@ -620,8 +622,10 @@ static int launch_tiled_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return fail(HKM_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     }
+    prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc, cn,
                        labels, min_d2, ntiles);
+    prof_end(st);
     return check_launch("assign_mfma_tiled_kernel");
 }
 
@@ -661,8 +665,10 @@ static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, 
     auto kern = assign_mfma_resident_kernel<DP, PB, VEC>;
     int64_t grid = int64_t(num_cus()) * 3;
     if (grid > ntiles) grid = ntiles;
+    prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc,
                        labels, min_d2, ntiles);
+    prof_end(st);
     return check_launch("assign_mfma_resident_kernel");
 }
 
@@ -702,8 +708,10 @@ static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
     int lg = 0;
     while ((int64_t(1) << lg) < per_wg) ++lg;
     const int range_bits = 53 - FUSED_QBITS - lg;
+    prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(FUSED_THREADS), lds, st, X, N, D, ldx, C, K, ldc,
                        labels, min_d2, ntiles, fsum, fcnt, flags, range_bits);
+    prof_end(st);
     return check_launch("lloyd_mfma_resident_kernel");
 }
 
@@ -1258,6 +1266,7 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
     hipLaunchKernelGGL(fill_keys_kernel, dim3((unsigned)fgrid), dim3(256), 0, st, keys, N);
     int rc = check_launch("fill_keys_kernel");
     if (rc) return rc;
+    prof_begin(st);
     if (split && vec)
         hipLaunchKernelGGL(assign_split_stream_kernel<true>, dim3(pl.grid), dim3(256), 0, st, X, N, D, ldx,
                            C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
@@ -1270,6 +1279,7 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
     else
         hipLaunchKernelGGL(assign_mfma_stream_kernel<false>, dim3(pl.grid), dim3(256), 0, st, X, N, D,
                            ldx, C, K, ldc, cn, keys, ntiles, pl.nct, pl.ndc, pl.W, pl.PG);
+    prof_end(st);
     if ((rc = check_launch("assign_mfma_stream_kernel"))) return rc;
     hipLaunchKernelGGL(unpack_keys_kernel, dim3((unsigned)fgrid), dim3(256), 0, st, keys, N, labels, min_d2);
     return check_launch("unpack_keys_kernel");

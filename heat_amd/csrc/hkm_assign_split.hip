@@ -342,8 +342,10 @@ static int launch_split_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
     int lg = 0;
     while ((int64_t(1) << lg) < per_wg) ++lg;
     const int range_bits = 53 - SPLIT_QBITS - lg;
+    prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds, st, X, N, D, ldx, C, K, ldc, labels,
                        min_d2, ntiles, fsum, fcnt, flags, range_bits);
+    prof_end(st);
     return check_launch("split_resident_kernel");
 }
 

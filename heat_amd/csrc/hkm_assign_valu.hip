@@ -114,8 +114,10 @@ static int launch_valu_t(const float* X, int64_t N, int64_t ldx, const float* C,
     const int64_t nbatches = (N + VALU_THREADS - 1) / VALU_THREADS;
     int64_t grid = int64_t(num_cus()) * 8;
     if (grid > nbatches) grid = nbatches;
+    prof_begin(st);
     hipLaunchKernelGGL(assign_valu_kernel<D>, dim3((unsigned)grid), dim3(VALU_THREADS), 0, st, X, N,
                        ldx, C, K, ldc, labels, min_d2, ktile, nbatches);
+    prof_end(st);
     return check_launch("assign_valu_kernel");
 }
 

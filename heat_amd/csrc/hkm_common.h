@@ -238,6 +238,9 @@ int launch_update_median(const float* X, int64_t N, int32_t D, int64_t ldx, cons
 int launch_widen(const int32_t* in, int64_t N, int64_t* out, hipStream_t st);
 
 int num_cus();
+// benchmark timing of the dominant kernel: no-ops unless hkm_profile_enable(1) was called on this thread
+void prof_begin(hipStream_t st);
+void prof_end(hipStream_t st);
 
 // k nearest rows (hkm_knn.hip).  The split of the reference rows over workgroups and the scratch it needs
 // follow from the two row counts alone, so that the workspace can be sized before the call.

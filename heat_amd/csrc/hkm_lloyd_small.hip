@@ -609,6 +609,7 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
             hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, 0>), dim3(grid), dim3(SMALL_T), lds, st, X, \
                                N, ldx, C, K, ldc, labels, min_d2, part, vec);                            \
     } while (0)
+    prof_begin(st);
     if (acc_mode == 1) {
         if (want_sse) HKM_GO(1, false, true);
         else HKM_GO(1, false, false);
@@ -622,6 +623,7 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
         if (want_min) HKM_GO(0, true, false);
         else HKM_GO(0, false, false);
     }
+    prof_end(st);
 #undef HKM_GO
     return check_launch("lloyd_small_kernel");
 }

@@ -353,6 +353,20 @@ int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, i
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 
+/*
+ * Timing of the dominant kernel, for benchmarks (no counterpart in the reference).  After
+ * hkm_profile_enable(1) on the calling thread, every hkm_assign_f32 / hkm_assign_static_f32 /
+ * hkm_lloyd_step_f32 call of that thread records one pair of events on its stream, right before and right
+ * after the launch of its distance kernel (the one hkm_assign_kernel_name / hkm_lloyd_kernel_name names:
+ * the fused distance + argmin kernel, or the one-sweep kernel that also forms the per-cluster sums) and of
+ * nothing else.  hkm_profile_collect waits for the recorded pairs, writes their durations in milliseconds
+ * to ms (HOST pointer, at most cap of them, in call order), the number recorded to *count, and starts
+ * over.  At most 512 pairs are kept between two collects.  hkm_profile_enable(0) switches it off.  While
+ * off -- the default -- nothing is recorded and no event exists.
+ */
+int hkm_profile_enable(int32_t on);
+int hkm_profile_collect(float* ms, int32_t cap, int32_t* count);
+
 /* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "mfma_resident",
  * "mfma_tiled", "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
 const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K);
