@@ -14,9 +14,12 @@ from typing import Optional
 
 import torch
 
+from . import _f64_paths
+
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
+LIB_VERSION = 300  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
 WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64 = 1, 2, 3, 4, 8, 16
 
@@ -76,6 +79,8 @@ SIGNATURES = {
                                                  c_void_p]),
     "hkm_laplacian_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, ctypes.c_float,
                                          c_void_p, c_int64, c_void_p, c_void_p]),
+    "hkm_laplacian_f64": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_int32, c_int32, c_int32, ctypes.c_double,
+                                         c_void_p, c_int64, c_void_p, c_void_p]),
     "hkm_assign_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p]),
     "hkm_update_f64": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
@@ -110,6 +115,15 @@ def load() -> ctypes.CDLL:
                 "(or __graft_entry__.build()). heat_amd has no CPU fallback."
             )
         lib = ctypes.CDLL(_LIB_PATH)
+        lib.hkm_version.restype = ctypes.c_int
+        have = int(lib.hkm_version())
+        missing = [name for name in SIGNATURES if not hasattr(lib, name)]
+        if have != LIB_VERSION or missing:
+            raise ImportError(
+                f"{_LIB_PATH} is version {have} but this binding needs {LIB_VERSION}"
+                + (f" (missing: {', '.join(missing[:5])})" if missing else "")
+                + ": rebuild it with `make -C heat_amd/csrc`."
+            )
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = res
@@ -438,6 +452,9 @@ def assign_l1(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_dist: 
     _require_rows(x, c)
     n, d = x.shape
     k = c.shape[0]
+    if _is_f64(x, c, min_dist):
+        _f64_paths.assign_l1(x, c, labels, min_dist)
+        return
     check(load().hkm_assign_l1_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
                                    c.stride(0) if k > 1 else d, _ptr(labels), _ptr(min_dist), _stream()))
 
@@ -449,6 +466,9 @@ def closest_rows_l1(x: torch.Tensor, q: torch.Tensor, idx: torch.Tensor, dist: O
     _require_rows(x, q)
     n, d = x.shape
     m = q.shape[0]
+    if _is_f64(x, q, dist):
+        _f64_paths.closest_rows_l1(x, q, idx, dist)
+        return
     buf = ws.get(workspace_bytes(n, d, m, WS_MEDIAN))
     check(load().hkm_closest_rows_l1_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(q), m,
                                          q.stride(0) if m > 1 else d, _ptr(idx), _ptr(dist), _ptr(buf),
@@ -462,8 +482,11 @@ def closest_rows_l1_q64(x: torch.Tensor, q64: torch.Tensor, idx: torch.Tensor, d
     _require_gpu(x, q64, idx, dist64)
     _require_rows(x)
     _require_dense(q64)
+    if q64.dtype == torch.float64 and x.dtype == torch.float64:
+        _f64_paths.closest_rows_l1(x, q64, idx, dist64)
+        return
     if q64.dtype != torch.float64 or x.dtype != torch.float32:
-        raise TypeError("x must be float32 and q64 float64")
+        raise TypeError("x must be float32 (or float64) and q64 float64")
     n, d = x.shape
     m = q64.shape[0]
     buf = ws.get(workspace_bytes(n, d, m, WS_MEDIAN))
@@ -486,6 +509,9 @@ def update_median(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, ws
     _require_dense(c_old)
     n, d = x.shape
     k = c_new.shape[0]
+    if _is_f64(x, c_new, c_old):
+        _f64_paths.update_median(x, labels, c_new, fallback_rows, c_old, counts, lower, skip_zero_rows, median64)
+        return
     buf = ws.get(workspace_bytes(n, d, k, WS_MEDIAN))
     if median64 is not None:
         check(load().hkm_update_median_q64_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(labels), k,
@@ -514,8 +540,13 @@ def knn(q: torch.Tensor, x: torch.Tensor, k: int, idx: torch.Tensor, dist: Optio
     dist[m, :k] their distances (see hkm_knn_f32 in include/hkm.h)."""
     _require_gpu(q, x, idx, dist)
     _require_rows(q, x, idx, dist)
+    if q.dtype == torch.float64 and x.dtype == torch.float64 and idx.dtype == torch.int64:
+        if q.shape[1] != x.shape[1] or tuple(idx.shape) != (q.shape[0], k) or not 1 <= k <= x.shape[0]:
+            raise ValueError("shapes of q, x and idx do not fit together")
+        _f64_paths.knn(q, x, k, idx, dist)
+        return
     if q.dtype != torch.float32 or x.dtype != torch.float32:
-        raise TypeError("q and x must be float32")
+        raise TypeError("q and x must both be float32 or both be float64")
     if idx.dtype != torch.int64 or (dist is not None and dist.dtype != torch.float32):
         raise TypeError("idx must be int64 and dist float32")
     m, d = q.shape
@@ -599,9 +630,10 @@ def laplacian(sim: torch.Tensor, out: torch.Tensor, definition: int, mode: int, 
     n = sim.shape[0]
     if sim.dim() != 2 or sim.shape[1] != n or tuple(out.shape) != (n, n):
         raise ValueError("sim and out must be square matrices of the same size")
-    if sim.dtype != torch.float32 or out.dtype != torch.float32 or degree.dtype != torch.float32:
-        raise TypeError("sim, out and degree must be float32")
+    if sim.dtype not in (torch.float32, torch.float64) or out.dtype != sim.dtype or degree.dtype != sim.dtype:
+        raise TypeError("sim, out and degree must all be float32 or all be float64")
     if degree.numel() != n or not degree.is_contiguous():
         raise ValueError(f"degree must hold {n} contiguous entries")
-    check(load().hkm_laplacian_f32(_ptr(sim), n, sim.stride(0) if n > 1 else n, definition, mode, 1 if weighted else 0,
+    fn = load().hkm_laplacian_f64 if sim.dtype == torch.float64 else load().hkm_laplacian_f32
+    check(fn(_ptr(sim), n, sim.stride(0) if n > 1 else n, definition, mode, 1 if weighted else 0,
                                    float(eps), _ptr(out), out.stride(0) if n > 1 else n, _ptr(degree), _stream()))

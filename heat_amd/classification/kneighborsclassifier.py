@@ -64,16 +64,20 @@ class KNeighborsClassifier(BaseEstimator, ClassificationMixin):
 
     def predict(self, x: DNDarray) -> DNDarray:
         """
-        heat/classification/kneighborsclassifier.py:114-132.  Differences in arithmetic: squared distances are
-        summed directly as sum (a - b)^2 (the reference's ``torch.cdist`` switches to the quadratic expansion
-        above 25 rows), ties between training rows at exactly the same distance go to the smaller row index
-        (``torch.topk`` leaves their order open), and the label rows are added in float32 (exact for one-hot
-        labels and integer weights below 2^24).  The neighbours found are kept in ``kneighbors_``.
+        heat/classification/kneighborsclassifier.py:114-132.  With the default metric ``ht.spatial.cdist`` on
+        float32 data the distance matrix is never formed.  Arithmetic of that path: below 16 and above 128
+        features squared distances are summed directly as sum (a - b)^2, in between they are the clamped
+        expansion (|a|^2 + |b|^2) - 2 a.b with the products on the matrix cores -- the form the reference's
+        ``torch.cdist`` itself takes above 25 rows; it carries an absolute error of up to about
+        4e-7 (|a|^2 + |b|^2), so training rows closer together than that may swap places.  Ties between
+        training rows at exactly the same distance go to the smaller row index (``torch.topk`` leaves their
+        order open), and the label rows are added in float32 (exact for one-hot labels and integer weights
+        below 2^24).  Any other metric callable, and float64 / int64 data, take the reference's own route:
+        the full matrix from the callable, ``topk(largest=False)``, the label rows summed, ``argmax``.
+        The neighbours found are kept in ``kneighbors_``.
         """
         if self.x is None or self.y is None:
             raise RuntimeError("fit needs to be called before predict")
-        if self.effective_metric_ is not distance.cdist:
-            raise NotImplementedError("only the Euclidean metric ht.spatial.cdist has a fused k-nearest-rows kernel")
         if not isinstance(x, DNDarray):
             raise TypeError(f"x must be a DNDarray but was {type(x)}")
         if len(x.shape) != 2 or x.shape[1] != self.x.shape[1]:
@@ -82,8 +86,8 @@ class KNeighborsClassifier(BaseEstimator, ClassificationMixin):
         if k < 1 or k > self.n_samples_fit_:
             raise ValueError(f"n_neighbors = {k} must be in [1, {self.n_samples_fit_}]")
         promoted = types.promote_types(types.promote_types(x.dtype, self.x.dtype), types.float32)
-        if promoted is not types.float32:
-            raise NotImplementedError("the k-nearest-rows kernel exists in float32 only")
+        if self.effective_metric_ is not distance.cdist or promoted is not types.float32:
+            return self._predict_full_matrix(x, k)
         q = distance._as_f32_matrix(x, promoted)
         train = distance._as_f32_matrix(self.x, promoted)
         dev = q.device
@@ -97,6 +101,22 @@ class KNeighborsClassifier(BaseEstimator, ClassificationMixin):
         _native.knn(q, train, k, idx, None, self._ws)
         classes = torch.empty((m,), dtype=torch.int64, device=dev)
         _native.knn_vote(idx, yt, classes)
+        self.kneighbors_ = DNDarray(idx, (m, k), types.int64, x.split, x.device, x.comm, True)
+        self.classes_ = DNDarray(classes, (m,), types.int64, x.split, x.device, x.comm, True)
+        return self.classes_
+
+    def _predict_full_matrix(self, x: DNDarray, k: int) -> DNDarray:
+        """The reference's op sequence on the device: distances from the metric callable (the library's
+        full-matrix kernels when it is one of ht.spatial's), then torch's selection and reductions."""
+        distances = self.effective_metric_(x, self.x)
+        if not isinstance(distances, DNDarray) or tuple(distances.shape) != (x.shape[0], self.x.shape[0]):
+            raise ValueError("the metric must return a (test rows x training rows) DNDarray")
+        d = distances.larray
+        _, idx = torch.topk(d, k, dim=1, largest=False)
+        yt = self.y.larray.to(device=d.device)
+        votes = yt[idx.reshape(-1)].reshape(idx.shape[0], k, yt.shape[1]).sum(dim=1)
+        classes = torch.argmax(votes, dim=1)
+        m = idx.shape[0]
         self.kneighbors_ = DNDarray(idx, (m, k), types.int64, x.split, x.device, x.comm, True)
         self.classes_ = DNDarray(classes, (m,), types.int64, x.split, x.device, x.comm, True)
         return self.classes_

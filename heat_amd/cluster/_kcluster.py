@@ -85,14 +85,10 @@ class _KCluster(ClusteringMixin, BaseEstimator):
             t = t.contiguous()
         return t
 
-    def _local_f32_only(self, x: DNDarray) -> torch.Tensor:
-        """The local matrix for the kernels that exist in float32 only (Manhattan metric, medians)."""
-        t = self._local_f32(x)
-        if t.dtype != torch.float32:
-            raise NotImplementedError(
-                f"{type(self).__name__} is built for float32 data; {x.dtype.__name__} input promotes to float64"
-            )
-        return t
+    def _local_l1(self, x: DNDarray) -> torch.Tensor:
+        """The local matrix for the Manhattan-metric estimators: float32 runs on the fused kernels, float64
+        (float64 and int64 data, which the reference keeps in float64) on the composed float64 steps."""
+        return self._local_f32(x)
 
     def _manhattan_metric(self) -> bool:
         """True for the estimators constructed with the Manhattan metric (KMedians, KMedoids set it)."""

@@ -178,11 +178,9 @@ class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
         return DeviceSampler(device, seed)
 
     def _local_f32(self, x: DNDarray) -> torch.Tensor:
-        """Local rows in the compute dtype: float64 stays float64 for k-means, everything else float32."""
+        """Local rows in the compute dtype: float64 stays float64, everything else becomes float32."""
         t = x.larray
         if t.dtype == torch.float64:
-            if self._p == 1:
-                raise NotImplementedError("the Manhattan-metric kernels cover float32 data only")
             return t.contiguous()
         if t.dtype != torch.float32:
             t = t.to(torch.float32)
@@ -231,7 +229,10 @@ class _BatchParallelKCluster(ClusteringMixin, BaseEstimator):
             # sum of the Manhattan distances to the closest centre: min_dist_sum adds sqrt(v), so it is
             # fed the squared distances
             _native.assign_l1(xt, self._cluster_centers.larray.to(xt.dtype), lab.view(-1), d2)
-            _native.min_dist_sum(d2.mul_(d2), fv, self._ws)
+            if xt.dtype == torch.float64:
+                fv = d2.sum()
+            else:
+                _native.min_dist_sum(d2.mul_(d2), fv, self._ws)
         else:
             # ||x - C[labels]||_F ** 2 = sum of the squared distances to the closest centre
             _native.assign(xt, self._cluster_centers.larray.to(xt.dtype), lab.view(-1), d2, self._ws)

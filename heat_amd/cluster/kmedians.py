@@ -52,10 +52,10 @@ class KMedians(_KCluster):
         return c_new
 
     def _update_centroids(self, x: DNDarray, matching_centroids: DNDarray) -> DNDarray:
-        xt = self._local_f32_only(x)
+        xt = self._local_l1(x)
         lab = matching_centroids.larray.reshape(-1).to(torch.int32)
         c_new = self._median_step(xt, lab, self._local_f32(self._cluster_centers, like=xt), self._make_sampler(xt.device))
-        return DNDarray(c_new, tuple(c_new.shape), types.float32, None, x.device, x.comm, True)
+        return DNDarray(c_new, tuple(c_new.shape), types.canonical_heat_type(c_new.dtype), None, x.device, x.comm, True)
 
     def fit(self, x: DNDarray, oversampling: float = 2, iter_multiplier: float = 1) -> "KMedians":
         """Loop of heat/cluster/kmedians.py:120-147: assign, medians, squared centre movement <= tol."""
@@ -64,13 +64,13 @@ class KMedians(_KCluster):
         self._initialize_cluster_centers(x, oversampling, iter_multiplier)
         self._n_iter = 0
         self._check_split(x)
-        xt = self._local_f32_only(x)
+        xt = self._local_l1(x)
         dev = xt.device
         n, d = xt.shape
         sampler = self._make_sampler(dev)
         centers = self._local_f32(self._cluster_centers, like=xt).clone()
         lab32 = torch.empty((n,), dtype=torch.int32, device=dev)
-        shift = torch.zeros((), dtype=torch.float32, device=dev)
+        shift = torch.zeros((), dtype=xt.dtype, device=dev)
         if self.max_iter <= 0:
             raise ValueError(f"max_iter must be positive, but was {self.max_iter}")
         for _ in range(self.max_iter):
@@ -83,7 +83,7 @@ class KMedians(_KCluster):
                 break
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         _native.widen_labels(lab32, lab64)
-        self._cluster_centers = DNDarray(centers, (self.n_clusters, d), types.float32, None, x.device, x.comm, True)
-        self._inertia = DNDarray(shift.clone(), (), types.float32, None, x.device, x.comm, True)
+        self._cluster_centers = DNDarray(centers, (self.n_clusters, d), types.canonical_heat_type(centers.dtype), None, x.device, x.comm, True)
+        self._inertia = DNDarray(shift.clone(), (), types.canonical_heat_type(shift.dtype), None, x.device, x.comm, True)
         self._labels = DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
         return self

@@ -55,10 +55,10 @@ class KMedoids(_KCluster):
         return xt[idx]
 
     def _update_centroids(self, x: DNDarray, matching_centroids: DNDarray) -> DNDarray:
-        xt = self._local_f32_only(x)
+        xt = self._local_l1(x)
         lab = matching_centroids.larray.reshape(-1).to(torch.int32)
         c_new = self._medoid_step(xt, lab, self._local_f32(self._cluster_centers, like=xt), self._make_sampler(xt.device))
-        return DNDarray(c_new, tuple(c_new.shape), types.float32, None, x.device, x.comm, True)
+        return DNDarray(c_new, tuple(c_new.shape), types.canonical_heat_type(c_new.dtype), None, x.device, x.comm, True)
 
     def fit(self, x: DNDarray, oversampling: float = 2, iter_multiplier: float = 1) -> "KMedoids":
         """Loop of heat/cluster/kmedoids.py:117-156: stops when no centre changes."""
@@ -67,7 +67,7 @@ class KMedoids(_KCluster):
         self._initialize_cluster_centers(x, oversampling, iter_multiplier)
         self._n_iter = 0
         self._check_split(x)
-        xt = self._local_f32_only(x)
+        xt = self._local_l1(x)
         dev = xt.device
         n, d = xt.shape
         sampler = self._make_sampler(dev)
@@ -84,6 +84,6 @@ class KMedoids(_KCluster):
             centers = c_new
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         _native.widen_labels(lab32, lab64)
-        self._cluster_centers = DNDarray(centers, (self.n_clusters, d), types.float32, None, x.device, x.comm, True)
+        self._cluster_centers = DNDarray(centers, (self.n_clusters, d), types.canonical_heat_type(centers.dtype), None, x.device, x.comm, True)
         self._labels = DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
         return self

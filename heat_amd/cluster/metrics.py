@@ -55,8 +55,8 @@ def silhouette_samples(X: DNDarray, labels: DNDarray, *, metric: str = "euclidea
     if metric not in ("precomputed", "euclidean"):
         raise NotImplementedError(f"{metric=} not implemented, choose from 'precomputed' and 'euclidean'.")
     promoted = types.promote_types(X.dtype, types.float32)
-    if promoted is not types.float32:
-        raise NotImplementedError("the silhouette kernels exist in float32 only")
+    if promoted is types.float64:
+        return _silhouette_samples_f64(X, lab, metric)
     xt = distance._as_f32_matrix(X, promoted)
     dev = xt.device
     n = xt.shape[0]
@@ -78,6 +78,38 @@ def silhouette_samples(X: DNDarray, labels: DNDarray, *, metric: str = "euclidea
     out = torch.empty((n,), dtype=torch.float32, device=dev)
     _native.silhouette_finish(sums, enc, counts, out)
     return DNDarray(out, (n,), types.float32, X.split, X.device, X.comm, True)
+
+
+def _silhouette_samples_f64(X: DNDarray, lab: torch.Tensor, metric: str) -> DNDarray:
+    """float64 and int64 data, which the reference keeps in float64: the per-cluster sums come from the
+    library's float64 pairwise kernel in row chunks times the one-hot labels (metrics.py:135-151), the
+    coefficients (:153-176) from a few torch operations on the (samples x clusters) sums."""
+    from .. import _f64_paths
+
+    xt = X.larray.to(torch.float64)
+    if xt.stride(-1) != 1:
+        xt = xt.contiguous()
+    dev = xt.device
+    n = xt.shape[0]
+    _, enc = torch.unique(lab.to(dev), sorted=True, return_inverse=True)
+    enc = enc.to(torch.int64).contiguous()
+    k = int(enc.max().item()) + 1 if n else 1
+    counts = torch.bincount(enc, minlength=k)
+    if metric == "precomputed":
+        mask = torch.zeros((n, k), dtype=torch.float64, device=dev)
+        mask.scatter_(1, enc.view(-1, 1), 1.0)
+        sums = xt @ mask
+    else:
+        sums = _f64_paths.cluster_distance_sums(xt, enc, k)
+    own = counts[enc]
+    a = sums.gather(1, enc.view(-1, 1)).view(-1) / (own - 1).clamp_min(1).to(torch.float64)
+    mean_other = sums / counts.to(torch.float64).view(1, -1)
+    mean_other.scatter_(1, enc.view(-1, 1), float("inf"))
+    b = mean_other.min(dim=1).values
+    out = (b - a) / torch.maximum(a, b)
+    out = torch.where(own == 1, torch.zeros_like(out), out)
+    out = torch.nan_to_num(out, nan=0.0)
+    return DNDarray(out, (n,), types.float64, X.split, X.device, X.comm, True)
 
 
 def silhouette_score(X: DNDarray, labels: DNDarray, *, metric: str = "euclidean", sample_size: Optional[int] = None,

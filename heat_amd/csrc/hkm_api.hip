@@ -189,6 +189,13 @@ static int check_matrix(const char* name, const void* p, int64_t rows, int32_t c
     return HKM_OK;
 }
 
+static int check_matrix64(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
+    if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);
+    if (reinterpret_cast<uintptr_t>(p) & 7u) return fail(HKM_EINVAL, "%s is not 8-byte aligned", name);
+    if (ld < cols) return fail(HKM_EINVAL, "leading dimension of %s (%lld) < columns (%d)", name, (long long)ld, cols);
+    return HKM_OK;
+}
+
 static int check_shape(int64_t N, int32_t D, int32_t K) {
     if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
     if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
@@ -243,7 +250,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 200; }
+int hkm_version(void) { return 300; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -541,13 +548,6 @@ int hkm_seed_plus_plus_rows_f32(const float* X, int64_t M, int32_t D, int64_t ld
 }
 
 // ---- float64 data -----------------------------------------------------------------------------
-static int check_matrix64(const char* name, const void* p, int64_t rows, int32_t cols, int64_t ld) {
-    if (!p && rows > 0) return fail(HKM_EINVAL, "%s is NULL", name);
-    if (reinterpret_cast<uintptr_t>(p) & 7u) return fail(HKM_EINVAL, "%s is not 8-byte aligned", name);
-    if (ld < cols) return fail(HKM_EINVAL, "leading dimension of %s (%lld) < columns (%d)", name, (long long)ld, cols);
-    return HKM_OK;
-}
-
 int hkm_assign_f64(const double* X, int64_t N, int32_t D, int64_t ldx, const double* C, int32_t K,
                    int64_t ldc, int32_t* labels, double* min_d2, void* hip_stream) {
     g_err[0] = 0;
@@ -773,21 +773,46 @@ int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds,
     return launch_silhouette_finish(S, N, K, lds, labels, counts, out, static_cast<hipStream_t>(hip_stream));
 }
 
-int hkm_laplacian_f32(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
-                      float eps, float* L, int64_t ldl, float* degree, void* hip_stream) {
+// rows run along grid.x; 2^24 rows would already be a 1 PB matrix
+static const int64_t LAPLACIAN_MAX_N = int64_t(1) << 24;
+
+// 0: nothing to do, 1: arguments fine, launch; negative: error
+static int laplacian_check(size_t elem, const void* S, int64_t N, int64_t lds, int32_t definition, int32_t mode,
+                           const void* L, int64_t ldl, const void* degree) {
     g_err[0] = 0;
-    if (N < 0 || N > 65535) return fail(HKM_EUNSUPPORTED, "N = %lld must be in [0, 65535]", (long long)N);
+    if (N < 0 || N > LAPLACIAN_MAX_N)
+        return fail(HKM_EUNSUPPORTED, "N = %lld must be in [0, %lld]", (long long)N, (long long)LAPLACIAN_MAX_N);
     if (definition != HKM_LAPLACIAN_SIMPLE && definition != HKM_LAPLACIAN_NORM_SYM)
         return fail(HKM_EINVAL, "definition = %d is neither simple (0) nor norm_sym (1)", definition);
     if (mode < 0 || mode > 2) return fail(HKM_EINVAL, "mode = %d must be 0 (fully connected), 1 (upper) or 2 (lower)", mode);
-    if (N == 0) return HKM_OK;
+    if (N == 0) return 0;
     int rc;
-    if ((rc = check_matrix("S", S, N, (int32_t)N, lds))) return rc;
-    if ((rc = check_matrix("L", L, N, (int32_t)N, ldl))) return rc;
+    if (elem == 8) {
+        if ((rc = check_matrix64("S", S, N, (int32_t)N, lds))) return rc;
+        if ((rc = check_matrix64("L", L, N, (int32_t)N, ldl))) return rc;
+    } else {
+        if ((rc = check_matrix("S", S, N, (int32_t)N, lds))) return rc;
+        if ((rc = check_matrix("L", L, N, (int32_t)N, ldl))) return rc;
+    }
     if (!degree) return fail(HKM_EINVAL, "degree is NULL");
-    if (reinterpret_cast<uintptr_t>(degree) & 3u) return fail(HKM_EINVAL, "degree is not 4-byte aligned");
+    if (reinterpret_cast<uintptr_t>(degree) & (elem - 1)) return fail(HKM_EINVAL, "degree is misaligned");
+    return 1;
+}
+
+int hkm_laplacian_f32(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                      float eps, float* L, int64_t ldl, float* degree, void* hip_stream) {
+    const int rc = laplacian_check(4, S, N, lds, definition, mode, L, ldl, degree);
+    if (rc != 1) return rc;
     return launch_laplacian(S, N, lds, definition, mode, weighted ? 1 : 0, eps, L, ldl, degree,
                             static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_laplacian_f64(const double* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                      double eps, double* L, int64_t ldl, double* degree, void* hip_stream) {
+    const int rc = laplacian_check(8, S, N, lds, definition, mode, L, ldl, degree);
+    if (rc != 1) return rc;
+    return launch_laplacian_f64(S, N, lds, definition, mode, weighted ? 1 : 0, eps, L, ldl, degree,
+                                static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_knn_vote_f32(const int64_t* idx, int64_t M, int32_t k, int64_t ldi, const float* Y, int64_t N, int32_t C,

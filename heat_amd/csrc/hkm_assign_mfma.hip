@@ -190,8 +190,9 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 // partial sum is below n_wg * 2^Emax, so as long as Emax - Emin <= 53 - 28 - ceil(log2 n_wg) every
 // addition is exact in fp64 and the result does not depend on the order.  The rounding keeps 28 bits
 // below the row's largest coordinate (error <= 2^-29 of it per addend).  A workgroup whose rows
-// violate the range condition (or hold inf / NaN) raises its flag; the step then falls back to the
-// two-pass update, whose kernels start by looking at the flags.
+// violate the range condition, or hold a row whose |x|^2 is inf or NaN (coordinates above 1.8e19 or
+// non-finite ones: the bound 2^E is then meaningless), raises its flag; the step then falls back to
+// the two-pass update, whose kernels start by looking at the flags.
 // ------------------------------------------------------------------------------------------------
 static constexpr int FUSED_QBITS = 28;
 static constexpr int FUSED_THREADS = 768;
@@ -231,6 +232,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
     if (tid == 0) {
         sN[K] = 0x7fffffff;
         sN[K + 1] = -0x7fffffff;
+        sN[K + 2] = 0;
     }
     __syncthreads();
 
@@ -239,6 +241,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
     const int ncb = KP >> 5;
     const int64_t tile_rows = int64_t(nw) * PB * 32;
     int emin = 0x7fffffff, emax = -0x7fffffff;
+    int nonfinite = 0;  // a row whose |x|^2 is inf or NaN: its bound 2^E says nothing about its coordinates
 
     floatx4 bn[PB][NJ];
     auto fetch = [&](int64_t tile) {
@@ -292,6 +295,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
             if (valid && xnr[pb] != 0.f) {  // an all-zero row adds nothing
                 // |x_d| < 2^E: |x|^2 < 2^(e2+1) up to rounding, one more bit of slack
                 const int e2 = (__float_as_int(xnr[pb]) >> 23) - 127;
+                nonfinite |= int((e2 & 0xff) == 128);  // exponent field 255 (the sign bit of |x|^2 is clear or NaN)
                 const int E = (e2 >> 1) + 2;
                 emin = min(emin, E);
                 emax = max(emax, E);
@@ -311,6 +315,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
 
     atomicMin(&sN[K], emin);
     atomicMax(&sN[K + 1], emax);
+    if (nonfinite) atomicOr(&sN[K + 2], 1);
     __syncthreads();
     double* gs = fsum + size_t(blockIdx.x) * K * D;
     for (int i = tid; i < K * D; i += nthr) {
@@ -320,7 +325,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
     for (int i = tid; i < K; i += nthr) fcnt[size_t(blockIdx.x) * K + i] = sN[i];
     if (tid == 0) {
         const int lo = sN[K], hi = sN[K + 1];
-        flags[blockIdx.x] = (hi >= lo && hi - lo > range_bits) ? 1 : 0;
+        flags[blockIdx.x] = ((hi >= lo && hi - lo > range_bits) || sN[K + 2]) ? 1 : 0;
     }
 }
 

@@ -267,5 +267,7 @@ int launch_silhouette_sums(const float* X, int64_t N, int32_t D, int64_t ldx, co
 // graph Laplacian from a similarity matrix (hkm_laplacian.hip)
 int launch_laplacian(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
                      float eps, float* L, int64_t ldl, float* degree, hipStream_t st);
+int launch_laplacian_f64(const double* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                         double eps, double* L, int64_t ldl, double* degree, hipStream_t st);
 
 }  // namespace hkm

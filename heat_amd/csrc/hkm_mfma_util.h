@@ -50,26 +50,81 @@ __device__ __forceinline__ floatx16 load_cn16(const float* cn16) {
 // Minimum and first argmin over the 16 distances a lane holds of one centroid block, merged into the
 // running (m, mi).  The minimum is a tree of three-input minima (8 instructions, no dependence on
 // compare results); only lanes whose block minimum improves the running one look for its position,
-// by equality from the last register down so that the first one wins -- independent compares, then a
-// chain of selects with literal indices.  Strict '<' keeps the earlier block on ties.  NaNs never win.
+// by equality from the last register down so that the first one wins.  Strict '<' keeps the earlier
+// block on ties.  NaNs never win.
+//
+// Both halves are written out as instructions: the compiler's own form of the tree spends two more
+// instructions on canonicalising operands that are matrix-core results, and it places every compare of
+// the lookup directly in front of the select that consumes it, which on this chip costs two idle cycles
+// per pair (a vector instruction must not read a scalar register pair written by the instruction before
+// it).  Here the compares run two ahead of the selects through three scalar register pairs, so no pair
+// is read within two instructions of being written and nothing idles.
+__device__ __forceinline__ float block_min16(const floatx16& d) {
+    // The first step is left to the compiler (a median of three with -inf is the minimum of the other
+    // two): it knows how many idle cycles a read of fresh matrix-core results needs, which an instruction
+    // it cannot see into would not get.
+    const float t01 = __builtin_amdgcn_fmed3f(d[0], d[1], -HKM_INF);
+    float a, b, c, e;
+    asm("v_min3_f32 %[a], %[t01], %[d2], %[d3]\n\t"
+        "v_min3_f32 %[b], %[d4], %[d5], %[d6]\n\t"
+        "v_min3_f32 %[c], %[d7], %[d8], %[d9]\n\t"
+        "v_min3_f32 %[e], %[d10], %[d11], %[d12]\n\t"
+        "v_min3_f32 %[a], %[a], %[b], %[c]\n\t"
+        "v_min3_f32 %[b], %[d13], %[d14], %[d15]\n\t"
+        "v_min3_f32 %[a], %[a], %[e], %[b]"
+        : [a] "=&v"(a), [b] "=&v"(b), [c] "=&v"(c), [e] "=&v"(e)
+        : [t01] "v"(t01), [d2] "v"(d[2]), [d3] "v"(d[3]), [d4] "v"(d[4]), [d5] "v"(d[5]), [d6] "v"(d[6]),
+          [d7] "v"(d[7]), [d8] "v"(d[8]), [d9] "v"(d[9]), [d10] "v"(d[10]), [d11] "v"(d[11]), [d12] "v"(d[12]),
+          [d13] "v"(d[13]), [d14] "v"(d[14]), [d15] "v"(d[15]));
+    return a;
+}
+
+// position (8 * (v / 4) + v % 4 for register v: the centroid row inside the block, without the
+// lane-half term) of the first of the 16 distances that equals bm
+__device__ __forceinline__ int block_pos16(const floatx16& d, float bm) {
+    int bi;
+    unsigned long long s0, s1, s2;
+    asm("v_cmp_eq_f32_e64 %[s0], %[d14], %[bm]\n\t"
+        "v_cmp_eq_f32_e64 %[s1], %[d13], %[bm]\n\t"
+        "v_cmp_eq_f32_e64 %[s2], %[d12], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], 27, 26, %[s0]\n\t"
+        "v_cmp_eq_f32_e64 %[s0], %[d11], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 25, %[s1]\n\t"
+        "v_cmp_eq_f32_e64 %[s1], %[d10], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 24, %[s2]\n\t"
+        "v_cmp_eq_f32_e64 %[s2], %[d9], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 19, %[s0]\n\t"
+        "v_cmp_eq_f32_e64 %[s0], %[d8], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 18, %[s1]\n\t"
+        "v_cmp_eq_f32_e64 %[s1], %[d7], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 17, %[s2]\n\t"
+        "v_cmp_eq_f32_e64 %[s2], %[d6], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 16, %[s0]\n\t"
+        "v_cmp_eq_f32_e64 %[s0], %[d5], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 11, %[s1]\n\t"
+        "v_cmp_eq_f32_e64 %[s1], %[d4], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 10, %[s2]\n\t"
+        "v_cmp_eq_f32_e64 %[s2], %[d3], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 9, %[s0]\n\t"
+        "v_cmp_eq_f32_e64 %[s0], %[d2], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 8, %[s1]\n\t"
+        "v_cmp_eq_f32_e64 %[s1], %[d1], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 3, %[s2]\n\t"
+        "v_cmp_eq_f32_e64 %[s2], %[d0], %[bm]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 2, %[s0]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 1, %[s1]\n\t"
+        "v_cndmask_b32_e64 %[bi], %[bi], 0, %[s2]"
+        : [bi] "=&v"(bi), [s0] "=&s"(s0), [s1] "=&s"(s1), [s2] "=&s"(s2)
+        : [d0] "v"(d[0]), [d1] "v"(d[1]), [d2] "v"(d[2]), [d3] "v"(d[3]), [d4] "v"(d[4]), [d5] "v"(d[5]),
+          [d6] "v"(d[6]), [d7] "v"(d[7]), [d8] "v"(d[8]), [d9] "v"(d[9]), [d10] "v"(d[10]), [d11] "v"(d[11]),
+          [d12] "v"(d[12]), [d13] "v"(d[13]), [d14] "v"(d[14]), [bm] "v"(bm));
+    return bi;
+}
+
 __device__ __forceinline__ void block_argmin(const floatx16& d, int kb, float& m, int& mi) {
-    const float t0 = fminf(fminf(d[0], d[1]), d[2]);
-    const float t1 = fminf(fminf(d[3], d[4]), d[5]);
-    const float t2 = fminf(fminf(d[6], d[7]), d[8]);
-    const float t3 = fminf(fminf(d[9], d[10]), d[11]);
-    const float t4 = fminf(fminf(d[12], d[13]), d[14]);
-    const float bm = fminf(fminf(fminf(t0, t1), t2), fminf(fminf(t3, t4), d[15]));
+    const float bm = block_min16(d);
     if (bm < m) {
-        // all compares first (each into its own scalar register pair), then the selects: a select
-        // right behind the compare it consumes would wait for it
-        bool e[15];
-#pragma unroll
-        for (int v = 0; v < 15; ++v) e[v] = d[v] == bm;
-        __builtin_amdgcn_sched_barrier(0);
-        int bi = 8 * (15 >> 2) + (15 & 3);
-#pragma unroll
-        for (int v = 14; v >= 0; --v) bi = e[v] ? 8 * (v >> 2) + (v & 3) : bi;
-        mi = kb + bi;
+        mi = kb + block_pos16(d, bm);
         m = bm;
     }
 }

@@ -35,19 +35,28 @@ class Laplacian:
         self.neighbours = neighbours
 
     def construct(self, X: DNDarray) -> DNDarray:
-        """heat/graph/laplacian.py:100-142.  The result is always float32 (the reference's unweighted graphs
-        go through an integer adjacency matrix, which changes the dtype of the simple Laplacian only)."""
+        """heat/graph/laplacian.py:100-142.  float32 and float64 similarities keep their type; of an unweighted
+        eNeighbour graph the simple Laplacian is an int64 matrix and the normalised one float32, as in the
+        reference (an int32 adjacency matrix, :129-133, minus the int64 diagonal of its row sums, :110-112,
+        resp. divided by the float32 square roots of those sums, :96-97)."""
         S = self.similarity_metric(X)
         if not isinstance(S, DNDarray) or len(S.shape) != 2 or S.shape[0] != S.shape[1]:
             raise ValueError("the similarity function must return a square DNDarray")
-        if S.dtype is not types.float32:
-            raise NotImplementedError("the Laplacian kernel exists in float32 only")
         s = S.larray
+        if s.dtype not in (torch.float32, torch.float64):
+            s = s.to(torch.float32)
         if s.stride(-1) != 1:
             s = s.contiguous()
         n = s.shape[0]
         mode = 0 if self.mode == "fully_connected" else (1 if self.epsilon[0] == "upper" else 2)
-        degree = torch.empty((n,), dtype=torch.float32, device=s.device)
-        _native.laplacian(s, s, 0 if self.definition == "simple" else 1, mode, bool(self.weighted),
+        degree = torch.empty((n,), dtype=s.dtype, device=s.device)
+        # L gets storage of its own: the similarity callable may have returned a matrix it keeps (a cached
+        # or precomputed one), which the reference leaves intact apart from its zeroed diagonal
+        out = torch.empty((n, n), dtype=s.dtype, device=s.device)
+        _native.laplacian(s, out, 0 if self.definition == "simple" else 1, mode, bool(self.weighted),
                           float(self.epsilon[1]), degree)
-        return DNDarray(s, (n, n), types.float32, S.split, S.device, S.comm, True)
+        if self.mode == "eNeighbour" and not self.weighted:
+            # the reference's unweighted adjacency is an int32 matrix: D - A comes out as int64, and the
+            # normalised form divides it by float32 square roots of the integer degrees
+            out = out.to(torch.int64 if self.definition == "simple" else torch.float32)
+        return DNDarray(out, (n, n), types.canonical_heat_type(out.dtype), S.split, S.device, S.comm, True)

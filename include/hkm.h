@@ -270,8 +270,12 @@ int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ld
  * hkm_knn_f32: for every row of Q (M x D) the k closest rows of X (N x D) in the Euclidean metric:
  *   idx (M x k int64, leading dimension ldi) in ascending order of (distance, row index) -- of rows at
  *   exactly the same squared distance the smaller index comes first -- and, if dist is not NULL, the
- *   distances themselves (M x k float32, leading dimension ldd).  Squared distances are summed directly
- *   as sum (q - x)^2 in fp32, the square root is correctly rounded.  A slot for which no finite distance
+ *   distances themselves (M x k float32, leading dimension ldd).  For D < 16 and D > 128 the squared
+ *   distance is summed directly as sum (q - x)^2 in fp32; for 16 <= D <= 128 it is the clamped expansion
+ *   max(0, (|q|^2 + |x|^2) - 2 q.x) with the products on the matrix cores (the form torch.cdist itself takes
+ *   above 25 rows): it carries an absolute error of up to about 4e-7 (|q|^2 + |x|^2), so a row identical to
+ *   the query may come back at a small non-zero distance and rows whose squared distances are closer than
+ *   that may swap places.  The square root is correctly rounded.  A slot for which no finite distance
  *   is left (NaN or overflowing rows) holds index -1 and distance inf.  1 <= k <= min(N, HKM_KNN_MAX_K).
  *   ws needs hkm_knn_workspace_bytes(M, N) bytes.
  * hkm_knn_vote_f32: classes[m] = the first index of the largest entry of sum_j Y[idx[m][j]] (Y: N x C
@@ -317,12 +321,16 @@ int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds,
  *   definition HKM_LAPLACIAN_SIMPLE: L = diag(degree) - A;
  *   definition HKM_LAPLACIAN_NORM_SYM: L = -(A / sqrt(d_i)) / sqrt(d_j) with zero degrees taken as 1, and
  *   ones on the diagonal.
- * N <= 65535.  Always float32 (the reference's unweighted simple Laplacian is an integer matrix).
+ * N <= 2^24.  hkm_laplacian_f64 is the same on float64 matrices (the reference keeps float64 similarities in
+ * float64).  The reference's unweighted simple Laplacian is an integer matrix: its entries are small whole
+ * numbers here, which the caller may cast.
  */
 #define HKM_LAPLACIAN_SIMPLE 0
 #define HKM_LAPLACIAN_NORM_SYM 1
 int hkm_laplacian_f32(const float* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
                       float eps, float* L, int64_t ldl, float* degree, void* hip_stream);
+int hkm_laplacian_f64(const double* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
+                      double eps, double* L, int64_t ldl, double* degree, void* hip_stream);
 
 /*
  * float64 data.  The reference keeps float64 inputs in float64 through the same op sequence

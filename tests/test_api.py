@@ -369,9 +369,11 @@ def test_knn_classifier_surface():
     assert knn.get_params()["n_neighbors"] == 3 and knn.get_params()["effective_metric_"] is ht.spatial.cdist
     with pytest.raises(RuntimeError):
         knn.predict(b)
-    with pytest.raises(NotImplementedError):
-        other = knn_cls(effective_metric_=ht.spatial.manhattan)
-        other.fit(b, ht.zeros((3,)))
+    # any metric callable is accepted (the full-matrix route of the reference); on host tensors it ends where
+    # every compute call ends: there is no CPU path
+    other = knn_cls(n_neighbors=1, effective_metric_=ht.spatial.manhattan)
+    other.fit(b, ht.zeros((3,)))
+    with pytest.raises(RuntimeError):
         other.predict(b)
 
 
@@ -421,4 +423,7 @@ def test_argument_validation_of_the_neighbour_silhouette_and_laplacian_entry_poi
     assert lib.hkm_laplacian_f32(good, 10, 10, 0, 3, 1, 1.0, good, 10, other, None) == einval
     assert lib.hkm_laplacian_f32(good, 10, 9, 0, 0, 1, 1.0, good, 10, other, None) == einval
     assert lib.hkm_laplacian_f32(good, 10, 10, 0, 0, 1, 1.0, good, 10, None, None) == einval
-    assert lib.hkm_laplacian_f32(good, 70000, 70000, 0, 0, 1, 1.0, good, 70000, other, None) == eunsup
+    big = (1 << 24) + 1
+    assert lib.hkm_laplacian_f32(good, big, big, 0, 0, 1, 1.0, good, big, other, None) == eunsup
+    assert lib.hkm_laplacian_f64(good, big, big, 0, 0, 1, 1.0, good, big, other, None) == eunsup
+    assert lib.hkm_laplacian_f64(good, 10, 10, 0, 0, 1, 1.0, good, 10, None, None) == einval

@@ -236,11 +236,15 @@ def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
     x, _ = _data(n, d, k, seed=77)
     g = torch.Generator().manual_seed(2)
     scale = torch.pow(2.0, torch.randint(-30, 31, (n, 1), generator=g).float())
-    for variant in ("wide", "nonfinite"):
+    for variant in ("wide", "nonfinite", "allhuge", "allnan"):
         xv = x * scale if variant == "wide" else x.clone()
         if variant == "nonfinite":
             xv[5, 3] = float("inf")
             xv[4000, 0] = float("nan")
+        if variant == "allhuge":   # every |x|^2 overflows: no row has a usable magnitude bound, none differs from another
+            xv = xv * 3e19
+        if variant == "allnan":
+            xv[:, 1] = float("nan")
         c0 = xv[torch.randperm(n, generator=g)[:k]].contiguous()
         c0 = torch.nan_to_num(c0, nan=0.0, posinf=1.0, neginf=-1.0)
         xs, cs = xv.to(cuda), c0.to(cuda)

@@ -81,8 +81,9 @@ def test_known_answers_and_special_cases_of_the_reference_tests(cuda):
     sil = ht.cluster.silhouette_samples(arr(x), arr(torch.tensor([0, 2, 1, 0], dtype=torch.int32)))
     assert float(sil.larray[0]) == pytest.approx(0.9, abs=1e-6)
     lab = torch.tensor([0, 0, 1, 1])
-    with pytest.raises(NotImplementedError):     # int64 rows promote to float64 in the reference: not built
-        ht.cluster.silhouette_samples(arr(torch.tensor([[1, 2], [1, 1], [4, 4], [4, 5]])), arr(lab))
+    # int64 rows are float64 rows in the reference (the docstring example of heat/cluster/metrics.py:121-126)
+    s64 = ht.cluster.silhouette_samples(arr(torch.tensor([[1, 2], [1, 1], [4, 4], [4, 5]])), arr(lab))
+    assert s64.dtype is ht.float64 and s64.larray.tolist() == pytest.approx([0.7452, 0.7836, 0.7452, 0.7836], abs=5e-5)
     x = torch.tensor([[1.0, 2.0], [1.0, 1.0], [4.0, 4.0], [4.0, 5.0]])
     assert ht.cluster.silhouette_samples(arr(x), arr(lab)).larray.tolist() == pytest.approx(
         [0.7452, 0.7836, 0.7452, 0.7836], abs=5e-5)
