@@ -56,6 +56,61 @@ MFMA_BOUND = {"c2", "c3", "c4"}
 CPU_SAMPLE_DIV = {"c1": 1, "c2": 16, "c3": 16, "c4": 256, "c5": 128}
 
 
+def run_probe() -> int:
+    """bench.py --probe: the hardware figures the kernels are designed around, measured with the library's
+    microbenchmark kernels (hkm_probe_mfma_f32, hkm_probe_stream) and device events.  One JSON line."""
+    import ctypes
+
+    import torch
+
+    from heat_amd import _native
+
+    lib = _native.load()
+    dev = torch.device("cuda:0")
+    P = ctypes.c_void_p
+
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    stream = P(torch.cuda.current_stream().cuda_stream)
+    grid, iters = 1024, 2000
+    out = torch.empty((grid * 256,), dtype=torch.float32, device=dev)
+    flops = grid * 4 * iters * 16 * 4096.0
+    res = {"probe": "mfma+stream", "mfma_f32_32x32x2": {}, "stream": {}}
+    # warm the clocks
+    timed(lambda: _native.check(lib.hkm_probe_mfma_f32(0, 0, iters, grid, P(out.data_ptr()), stream)), 20)
+    base_ms = timed(lambda: _native.check(lib.hkm_probe_mfma_f32(0, 0, iters, grid, P(out.data_ptr()), stream)), 10)
+    base_tf = flops / (base_ms * 1e-3) / 1e12
+    res["mfma_f32_32x32x2"]["alone_tflops"] = round(base_tf, 1)
+    res["mfma_f32_32x32x2"]["alone_frac_of_157.3"] = round(base_tf / 157.3, 3)
+    names = {1: "v_fma_f32", 2: "v_cndmask_b32", 3: "v_min3_f32", 4: "s_add_u32", 5: "v_cmp_lt_f32"}
+    for op, name in names.items():
+        ms = timed(lambda: _native.check(lib.hkm_probe_mfma_f32(op, 8, iters, grid, P(out.data_ptr()), stream)), 10)
+        # cycles one matrix instruction's slot grows by per interleaved instruction (64 cycles = the matrix instruction alone)
+        res["mfma_f32_32x32x2"][f"cycles_per_{name}"] = round(64.0 * (ms / base_ms - 1.0) / 8.0, 2)
+    nbytes = 2_400_000_000
+    a = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    b = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    a.zero_()
+    sink = torch.zeros((1,), dtype=torch.float32, device=dev)
+    for mode, name, moved in ((0, "copy", 2 * nbytes), (1, "read", nbytes), (2, "read_nontemporal", nbytes), (3, "fill", nbytes)):
+        ms = timed(lambda: _native.check(lib.hkm_probe_stream(P(a.data_ptr()), P(b.data_ptr()), nbytes, mode,
+                                                              P(sink.data_ptr()), stream)), 20)
+        res["stream"][f"{name}_TBps"] = round(moved / (ms * 1e-3) / 1e12, 2)
+    res["stream"]["bytes"] = nbytes
+    print(json.dumps(res))
+    return 0
+
+
 def bench_kmedians(args, w, x, t_gen) -> int:
     """One KMedians iteration = fused Manhattan distance+argmin, per-cluster medians, centroid shift
     and its 4-byte read, as KMedians.fit issues them.  The dominant kernel is the assignment; it is
@@ -351,6 +406,9 @@ def main() -> int:
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink N (testing only; invalidates the figure)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--probe", action="store_true",
+                    help="run the hardware microbenchmarks (matrix-pipe throughput alone and with interleaved "
+                         "vector / scalar instructions; copy, read and fill bandwidth) instead of a workload")
     ap.add_argument("--estimator", default="kmeans", choices=["kmeans", "kmedians", "cdist", "init", "knn", "silhouette"],
                     help="kmedians: the Manhattan-metric sibling on the same data; cdist: the full-matrix "
                          "public cdist on rows of c2; init: the k-means|| initialiser; knn: k nearest rows + label vote on rows of c2; silhouette: silhouette_samples on 100 000 rows of c3 (none is the headline metric)")
@@ -369,6 +427,8 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
     _native.load()
+    if args.probe:
+        return run_probe()
     dev = torch.device("cuda:0")
 
     t_gen = time.perf_counter()

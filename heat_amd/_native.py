@@ -37,6 +37,8 @@ SIGNATURES = {
                                              c_void_p, c_void_p, c_void_p]),
     "hkm_profile_enable": (ctypes.c_int, [c_int32]),
     "hkm_profile_collect": (ctypes.c_int, [c_void_p, c_int32, c_void_p]),
+    "hkm_probe_mfma_f32": (ctypes.c_int, [c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "hkm_probe_stream": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_int32, c_void_p, c_void_p]),
     "hkm_update_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,

@@ -911,6 +911,21 @@ int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int
     return launch_cdist(X, M, ldx, Y, Nn, ldy, D, out, ldo, form, 1, gauss, static_cast<hipStream_t>(hip_stream));
 }
 
+int hkm_probe_mfma_f32(int32_t op, int32_t nops, int32_t iters, int32_t grid, float* out, void* hip_stream) {
+    g_err[0] = 0;
+    if (iters < 1 || grid < 1 || !out) return fail(HKM_EINVAL, "hkm_probe_mfma_f32: iters and grid must be >= 1 and out not NULL");
+    return launch_probe_mfma(op, nops, iters, grid, out, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_probe_stream(const void* src, void* dst, size_t bytes, int32_t mode, float* sink, void* hip_stream) {
+    g_err[0] = 0;
+    if (bytes < 16 || !sink || (mode != 3 && !src) || ((mode == 0 || mode == 3) && !dst))
+        return fail(HKM_EINVAL, "hkm_probe_stream: NULL buffer or fewer than 16 bytes");
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u)
+        return fail(HKM_EINVAL, "hkm_probe_stream: buffers must be 16-byte aligned");
+    return launch_probe_stream(src, dst, bytes, mode, sink, static_cast<hipStream_t>(hip_stream));
+}
+
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream) {
     g_err[0] = 0;
     if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);

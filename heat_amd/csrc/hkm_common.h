@@ -270,4 +270,8 @@ int launch_laplacian(const float* S, int64_t N, int64_t lds, int32_t definition,
 int launch_laplacian_f64(const double* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
                          double eps, double* L, int64_t ldl, double* degree, hipStream_t st);
 
+// microbenchmarks (hkm_probe.hip)
+int launch_probe_mfma(int32_t op, int32_t nops, int32_t iters, int32_t grid, float* out, hipStream_t st);
+int launch_probe_stream(const void* src, void* dst, size_t bytes, int32_t mode, float* sink, hipStream_t st);
+
 }  // namespace hkm

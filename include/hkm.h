@@ -375,6 +375,19 @@ int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_s
 int hkm_profile_enable(int32_t on);
 int hkm_profile_collect(float* ms, int32_t cap, int32_t* count);
 
+/*
+ * Microbenchmarks behind the hardware figures the kernels are designed around (no counterpart in the
+ * reference; bench.py --probe times them).  Each call enqueues ONE kernel.
+ * hkm_probe_mfma_f32: every wave issues iters * 16 fp32 matrix instructions (v_mfma_f32_32x32x2_f32, two
+ *   independent accumulators), each followed by `nops` instructions of kind `op`: 0 none (nops = 0),
+ *   1 v_fma_f32, 2 v_cndmask_b32, 3 v_min3_f32, 4 s_add_u32 (scalar unit), 5 v_cmp_lt_f32; nops 4 or 8.
+ *   grid workgroups of 256 threads; out receives grid * 256 floats.  flops = grid * 4 * iters * 16 * 4096.
+ * hkm_probe_stream: mode 0 copies bytes from src to dst, 1 reads src, 2 reads src with non-temporal loads,
+ *   3 fills dst; 16-byte vectors, four in flight per thread; sink is one device float.
+ */
+int hkm_probe_mfma_f32(int32_t op, int32_t nops, int32_t iters, int32_t grid, float* out, void* hip_stream);
+int hkm_probe_stream(const void* src, void* dst, size_t bytes, int32_t mode, float* sink, void* hip_stream);
+
 /* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "mfma_resident",
  * "mfma_tiled", "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
 const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K);
