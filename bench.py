@@ -93,7 +93,7 @@ def run_probe() -> int:
     base_tf = flops / (base_ms * 1e-3) / 1e12
     res["mfma_f32_32x32x2"]["alone_tflops"] = round(base_tf, 1)
     res["mfma_f32_32x32x2"]["alone_frac_of_157.3"] = round(base_tf / 157.3, 3)
-    names = {1: "v_fma_f32", 2: "v_cndmask_b32", 3: "v_min3_f32", 4: "s_add_u32", 5: "v_cmp_lt_f32"}
+    names = {1: "v_fma_f32", 2: "v_cndmask_b32", 3: "v_min3_f32", 4: "s_add_u32", 5: "v_cmp_lt_f32", 6: "v_mov_b64"}
     for op, name in names.items():
         ms = timed(lambda: _native.check(lib.hkm_probe_mfma_f32(op, 8, iters, grid, P(out.data_ptr()), stream)), 10)
         # cycles one matrix instruction's slot grows by per interleaved instruction (64 cycles = the matrix instruction alone)

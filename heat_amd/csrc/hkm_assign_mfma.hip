@@ -29,9 +29,11 @@ namespace hkm {
 //     as |c|^2 - 2 x.c.  |x|^2 is the same for every centroid: it is added to the minimum only;
 //   * the clamp at 0 is applied lazily: only if some running minimum went negative (a point that
 //     coincides with a centroid up to rounding) the tile is rescanned with the clamp on every value;
-//   * per block of 16 values a tree of three-input minima; only if that improves the running minimum
-//     the position is looked up by equality (see block_argmin).  The lane-half term of the index is
-//     added once per tile.
+//   * per block of 16 values a tree of three-input minima; if that improves the running minimum the
+//     block is only remembered (its number and a copy of the 16 values: ten instructions), and the
+//     position of the minimum is looked up by equality once per point, in the copy that survived the
+//     last block (block_min_keep / kept_argmin).  The lane-half term of the index is added once per
+//     tile.
 // ------------------------------------------------------------------------------------------------
 // One centroid block (32 rows) against the wave's PB point blocks: DP/2 MFMAs per point block.  The
 // accumulators start at the squared norms of the lane's 16 centroid rows (cn16 points at the norm of
@@ -53,18 +55,22 @@ __device__ __forceinline__ void resident_block(const float* arow, const floatx16
 }
 
 // Scan of all centroid blocks.  CLAMP applies max(. + |x|^2, 0) to every value (the rescan of a tile
-// whose lazy minimum came out negative).  Two blocks per trip: the squared norms of a block are
-// requested one block ahead into registers that then serve, in place, as an accumulator.
+// whose lazy minimum came out negative).  Two blocks per trip: the squared norms of both are requested
+// at the top of the trip into the registers that then serve, in place, as their accumulators (norms
+// carried over the loop's back edge instead were copied into place, eight moves per block).
 template <int DP, int PB, bool CLAMP>
 __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn, int ncb, int p, int h,
                                               const floatx4 (&b)[PB][DP / 8],
                                               const float (&xn)[PB], float (&m)[PB],
                                               int (&mi)[PB]) {
     constexpr int LDC = DP + 4;
+    int blk[PB];
+    floatx16 keep[PB];
 #pragma unroll
     for (int pb = 0; pb < PB; ++pb) {
         m[pb] = HKM_INF;
-        mi[pb] = 0;
+        blk[pb] = 0;
+        keep_undefined(keep[pb]);
     }
     auto one_block = [&](int cb, const floatx16& c0) {
         floatx16 acc[PB];
@@ -76,22 +82,49 @@ __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn,
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[pb][v] = fmaxf(acc[pb][v] + xn[pb], 0.0f);
             }
-            block_argmin(acc[pb], cb * 32, m[pb], mi[pb]);
+            block_min_keep(acc[pb], cb, m[pb], blk[pb], keep[pb]);
         }
     };
-    floatx16 ca = load_cn16(sCn + 4 * h);
     for (int cb = 0; cb < ncb; cb += 2) {
+        const floatx16 ca = load_cn16(sCn + cb * 32 + 4 * h);
         const floatx16 cb1 = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
         one_block(cb, ca);
-        if (cb + 1 < ncb) {
-            ca = load_cn16(sCn + (cb + 2 < ncb ? cb + 2 : cb + 1) * 32 + 4 * h);
-            one_block(cb + 1, cb1);
-        }
+        if (cb + 1 < ncb) one_block(cb + 1, cb1);
     }
-    // without CLAMP the minimum still lacks |x|^2
-    if (!CLAMP) {
 #pragma unroll
-        for (int pb = 0; pb < PB; ++pb) m[pb] += xn[pb];
+    for (int pb = 0; pb < PB; ++pb) {
+        mi[pb] = kept_argmin(keep[pb], m[pb], blk[pb]);
+        // without CLAMP the minimum still lacks |x|^2
+        if (!CLAMP) m[pb] += xn[pb];
+    }
+}
+
+// The rows of one tile for a wave: PB blocks of 32 rows starting at row0 (wave-uniform), a lane takes the
+// DP/2 columns of its half of row p of each block.  Whole tiles of whole, aligned rows (`fast`, decided
+// once per kernel) are addressed as a wave-uniform base plus a 32-bit lane offset, so a tile costs no
+// vector address arithmetic; the ragged last tile and narrow or unaligned rows take the general path
+// (row index clamped to N - 1, columns beyond D read as zero).
+template <int DP, int PB, bool VEC>
+__device__ __forceinline__ void fetch_rows(const float* __restrict__ X, int64_t N, int D, int64_t ldx, int64_t row0,
+                                           int p, int h, bool fast, unsigned lane_off,
+                                           floatx4 (&dst)[PB][DP / 8]) {
+    constexpr int NJ = DP / 8;
+    if (fast && row0 + PB * 32 <= N) {
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            const char* base = reinterpret_cast<const char*>(X + (row0 + pb * 32) * ldx);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) dst[pb][j] = *reinterpret_cast<const floatx4*>(base + lane_off + 16 * j);
+        }
+    } else {
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) {
+            int64_t r = row0 + pb * 32 + p;
+            r = r < N ? r : N - 1;
+            const float* xr = X + r * ldx;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) dst[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
+        }
     }
 }
 
@@ -122,42 +155,29 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
     }
     __syncthreads();
 
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
     const int ncb = KP >> 5;
+    const bool fast = VEC && D == DP && ldx < (int64_t(1) << 24);
+    const unsigned lane_off = unsigned((int64_t(p) * ldx + h * (DP / 2)) * 4);
 
-    // the rows of the next tile are requested before the current tile is scanned
-    floatx4 bn[PB][NJ];
-    auto fetch = [&](int64_t tile) {
+    // One tile: the rows of the next one are requested (into the other of two register sets, which swap
+    // roles from tile to tile) before this one is scanned.
+    auto step = [&](int64_t tile, const floatx4 (&b)[PB][NJ], floatx4 (&bnext)[PB][NJ]) {
         const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
-#pragma unroll
-        for (int pb = 0; pb < PB; ++pb) {
-            int64_t r = row0 + pb * 32 + p;
-            r = r < N ? r : N - 1;
-            const float* xr = X + r * ldx;
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) bn[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
-        }
-    };
-    if (int64_t(blockIdx.x) < ntiles) fetch(blockIdx.x);
-
-    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int64_t row0 = tile * (4 * PB * 32) + wave * (PB * 32);
-        floatx4 b[PB][NJ];
         float xn[PB], m[PB];
         int mi[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
             float s = 0.f;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                b[pb][j] = bn[pb][j];
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
-            }
             xn[pb] = s + __shfl_xor(s, 32);
         }
-        if (tile + gridDim.x < ntiles) fetch(tile + gridDim.x);
+        if (tile + gridDim.x < ntiles)
+            fetch_rows<DP, PB, VEC>(X, N, D, ldx, row0 + int64_t(gridDim.x) * (4 * PB * 32), p, h, fast, lane_off, bnext);
 
         resident_scan<DP, PB, false>(sC, sCn, ncb, p, h, b, xn, m, mi);
         bool neg = false;
@@ -169,12 +189,21 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
         for (int pb = 0; pb < PB; ++pb) {
             mi[pb] += 4 * h;
             merge_halves(m[pb], mi[pb]);
-            const int64_t r = row0 + pb * 32 + p;
-            if (h == 0 && r < N) {
-                labels[r] = mi[pb];
-                if (min_d2) min_d2[r] = m[pb];
+            const int64_t rb = row0 + pb * 32;  // wave-uniform: the stores take it as their scalar base
+            if (h == 0 && rb + p < N) {
+                labels[rb + p] = mi[pb];
+                if (min_d2) min_d2[rb + p] = m[pb];
             }
         }
+    };
+
+    floatx4 b0[PB][NJ], b1[PB][NJ];
+    if (int64_t(blockIdx.x) < ntiles)
+        fetch_rows<DP, PB, VEC>(X, N, D, ldx, int64_t(blockIdx.x) * (4 * PB * 32) + wave * (PB * 32), p, h, fast,
+                                lane_off, b0);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += 2 * int64_t(gridDim.x)) {
+        step(tile, b0, b1);
+        if (tile + gridDim.x < ntiles) step(tile + gridDim.x, b1, b0);
     }
 }
 
@@ -196,6 +225,7 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 // ------------------------------------------------------------------------------------------------
 static constexpr int FUSED_QBITS = 28;
 static constexpr int FUSED_THREADS = 768;
+static constexpr int FUSED_PB = 1;
 
 template <int DP, int PB, bool VEC>
 __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
@@ -236,44 +266,32 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
     }
     __syncthreads();
 
-    const int lane = tid & 63, wave = tid >> 6, nw = nthr >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), nw = nthr >> 6;
     const int p = lane & 31, h = lane >> 5;
     const int ncb = KP >> 5;
     const int64_t tile_rows = int64_t(nw) * PB * 32;
+    const bool fast = VEC && D == DP && ldx < (int64_t(1) << 24);
+    const unsigned lane_off = unsigned((int64_t(p) * ldx + h * (DP / 2)) * 4);
     int emin = 0x7fffffff, emax = -0x7fffffff;
     int nonfinite = 0;  // a row whose |x|^2 is inf or NaN: its bound 2^E says nothing about its coordinates
 
-    floatx4 bn[PB][NJ];
-    auto fetch = [&](int64_t tile) {
+    // One tile: the rows of the next one are requested (into the other of two register sets, which swap
+    // roles from tile to tile) before this one is scanned.
+    auto step = [&](int64_t tile, const floatx4 (&b)[PB][NJ], floatx4 (&bnext)[PB][NJ]) {
         const int64_t row0 = tile * tile_rows + wave * (PB * 32);
-#pragma unroll
-        for (int pb = 0; pb < PB; ++pb) {
-            int64_t r = row0 + pb * 32 + p;
-            r = r < N ? r : N - 1;
-            const float* xr = X + r * ldx;
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) bn[pb][j] = load_row4<VEC>(xr, h * (DP / 2) + 4 * j, D);
-        }
-    };
-    if (int64_t(blockIdx.x) < ntiles) fetch(blockIdx.x);
-
-    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int64_t row0 = tile * tile_rows + wave * (PB * 32);
-        floatx4 b[PB][NJ];
         float xnr[PB], m[PB];
         int mi[PB];
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
             float s = 0.f;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                b[pb][j] = bn[pb][j];
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) s = fmaf(b[pb][j][t], b[pb][j][t], s);
-            }
             xnr[pb] = s + __shfl_xor(s, 32);
         }
-        if (tile + gridDim.x < ntiles) fetch(tile + gridDim.x);
+        if (tile + gridDim.x < ntiles)
+            fetch_rows<DP, PB, VEC>(X, N, D, ldx, row0 + int64_t(gridDim.x) * tile_rows, p, h, fast, lane_off, bnext);
 
         resident_scan<DP, PB, false>(sC, sCn, ncb, p, h, b, xnr, m, mi);
         bool neg = false;
@@ -285,11 +303,11 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
         for (int pb = 0; pb < PB; ++pb) {
             mi[pb] += 4 * h;
             merge_halves(m[pb], mi[pb]);
-            const int64_t r = row0 + pb * 32 + p;
-            const bool valid = r < N;
+            const int64_t rb = row0 + pb * 32;  // wave-uniform: the stores take it as their scalar base
+            const bool valid = rb + p < N;
             if (h == 0 && valid) {
-                labels[r] = mi[pb];
-                if (min_d2) min_d2[r] = m[pb];
+                labels[rb + p] = mi[pb];
+                if (min_d2) min_d2[rb + p] = m[pb];
                 atomicAdd(&sN[mi[pb]], 1);
             }
             if (valid && xnr[pb] != 0.f) {  // an all-zero row adds nothing
@@ -311,6 +329,15 @@ __global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
                     }
             }
         }
+    };
+
+    floatx4 b0[PB][NJ], b1[PB][NJ];
+    if (int64_t(blockIdx.x) < ntiles)
+        fetch_rows<DP, PB, VEC>(X, N, D, ldx, int64_t(blockIdx.x) * tile_rows + wave * (PB * 32), p, h, fast, lane_off,
+                                b0);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += 2 * int64_t(gridDim.x)) {
+        step(tile, b0, b1);
+        if (tile + gridDim.x < ntiles) step(tile + gridDim.x, b1, b0);
     }
 
     atomicMin(&sN[K], emin);
@@ -377,7 +404,8 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
 
     floatx4 b[PB][NJ];
     float xn[PB], m[PB];
-    int mi[PB];
+    int blk[PB];
+    floatx16 keep[PB];
 
     for (int64_t it = 0; it < nsteps; ++it) {
         float* sC = lds + (it & 1) * (TC * LDC + TC);
@@ -414,7 +442,8 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
                 }
                 xn[pb] = s + __shfl_xor(s, 32);
                 m[pb] = HKM_INF;
-                mi[pb] = 0;
+                blk[pb] = 0;
+                keep_undefined(keep[pb]);
             }
         }
 
@@ -423,9 +452,9 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
             floatx16 acc[PB];
             const floatx16 c0 = load_cn16(sCn + cb * 32 + 4 * h);
             resident_block<DP, PB>(sC + (cb * 32 + p) * LDC, c0, h, b, acc);
-            const int kb = cur_ct * TC + cb * 32;
 #pragma unroll
-            for (int pb = 0; pb < PB; ++pb) block_argmin(acc[pb], kb, m[pb], mi[pb]);
+            for (int pb = 0; pb < PB; ++pb)
+                block_min_keep(acc[pb], cur_ct * (TC / 32) + cb, m[pb], blk[pb], keep[pb]);
         }
 
         if (cur_ct == nct - 1) {
@@ -433,7 +462,7 @@ __global__ __launch_bounds__(256) void assign_mfma_tiled_kernel(
             for (int pb = 0; pb < PB; ++pb) {
                 // the distance gets its |x|^2 and the clamp at 0 here, once per point
                 float mm = fmaxf(m[pb] + xn[pb], 0.0f);
-                int ii = mi[pb] + 4 * h;
+                int ii = kept_argmin(keep[pb], m[pb], blk[pb]) + 4 * h;
                 merge_halves(mm, ii);
                 const int64_t r = row0 + pb * 32 + p;
                 if (h == 0 && r < N) {
@@ -664,11 +693,17 @@ template <int DP, bool VEC>
 static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                              int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
                              hipStream_t st) {
-    constexpr int PB = 2;
+    constexpr int PB = 1;
     const int64_t ntiles = (N + 4 * PB * 32 - 1) / (4 * PB * 32);
     const size_t lds = resident_lds_bytes(D, K);
     auto kern = assign_mfma_resident_kernel<DP, PB, VEC>;
-    int64_t grid = int64_t(num_cus()) * 3;
+    // persistent grid: as many workgroups as are resident at once (registers allow four per CU up to
+    // 48 padded features, the centroids' LDS footprint decides the rest)
+    int per_cu = 0;
+    hipError_t oe = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), 256, lds);
+    if (oe != hipSuccess) return fail(HKM_EHIP, "hipOccupancyMaxActiveBlocksPerMultiprocessor: %s", hipGetErrorString(oe));
+    per_cu = per_cu < 1 ? 1 : per_cu > 4 ? 4 : per_cu;
+    int64_t grid = int64_t(num_cus()) * per_cu;
     if (grid > ntiles) grid = ntiles;
     prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, X, N, D, ldx, C, K, ldc,
@@ -684,7 +719,7 @@ size_t fused_lds_bytes(int32_t D, int32_t K) {
 }
 
 int fused_grid(int64_t N) {
-    constexpr int PB = 2;
+    constexpr int PB = FUSED_PB;
     const int64_t tile_rows = int64_t(FUSED_THREADS / 64) * PB * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
     int64_t grid = num_cus();
@@ -697,7 +732,7 @@ template <int DP, bool VEC>
 static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                           int64_t ldc, int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt,
                           int32_t* flags, hipStream_t st) {
-    constexpr int PB = 2;
+    constexpr int PB = FUSED_PB;
     const int64_t tile_rows = int64_t(FUSED_THREADS / 64) * PB * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
     const int grid = fused_grid(N);

@@ -53,27 +53,28 @@ __device__ __forceinline__ floatx16 load_cn16(const float* cn16) {
 // by equality from the last register down so that the first one wins.  Strict '<' keeps the earlier
 // block on ties.  NaNs never win.
 //
-// Both halves are written out as instructions: the compiler's own form of the tree spends two more
+// Both halves are written out as instructions: the compiler's own form of the tree spends more
 // instructions on canonicalising operands that are matrix-core results, and it places every compare of
 // the lookup directly in front of the select that consumes it, which on this chip costs two idle cycles
 // per pair (a vector instruction must not read a scalar register pair written by the instruction before
 // it).  Here the compares run two ahead of the selects through three scalar register pairs, so no pair
 // is read within two instructions of being written and nothing idles.
 __device__ __forceinline__ float block_min16(const floatx16& d) {
-    // The first step is left to the compiler (a median of three with -inf is the minimum of the other
-    // two): it knows how many idle cycles a read of fresh matrix-core results needs, which an instruction
-    // it cannot see into would not get.
-    const float t01 = __builtin_amdgcn_fmed3f(d[0], d[1], -HKM_INF);
+    // The first read of the block is left to the compiler (a canonicalisation: one instruction that
+    // returns its operand): it knows how many idle cycles a read of fresh matrix-core results needs,
+    // which an instruction sequence it cannot see into would not get.
+    const float t0 = __builtin_canonicalizef(d[0]);
     float a, b, c, e;
-    asm("v_min3_f32 %[a], %[t01], %[d2], %[d3]\n\t"
-        "v_min3_f32 %[b], %[d4], %[d5], %[d6]\n\t"
-        "v_min3_f32 %[c], %[d7], %[d8], %[d9]\n\t"
-        "v_min3_f32 %[e], %[d10], %[d11], %[d12]\n\t"
+    asm("v_min3_f32 %[a], %[t0], %[d1], %[d2]\n\t"
+        "v_min3_f32 %[b], %[d3], %[d4], %[d5]\n\t"
+        "v_min3_f32 %[c], %[d6], %[d7], %[d8]\n\t"
+        "v_min3_f32 %[e], %[d9], %[d10], %[d11]\n\t"
         "v_min3_f32 %[a], %[a], %[b], %[c]\n\t"
-        "v_min3_f32 %[b], %[d13], %[d14], %[d15]\n\t"
-        "v_min3_f32 %[a], %[a], %[e], %[b]"
+        "v_min3_f32 %[b], %[d12], %[d13], %[d14]\n\t"
+        "v_min3_f32 %[a], %[a], %[e], %[b]\n\t"
+        "v_min_f32 %[a], %[a], %[d15]"
         : [a] "=&v"(a), [b] "=&v"(b), [c] "=&v"(c), [e] "=&v"(e)
-        : [t01] "v"(t01), [d2] "v"(d[2]), [d3] "v"(d[3]), [d4] "v"(d[4]), [d5] "v"(d[5]), [d6] "v"(d[6]),
+        : [t0] "v"(t0), [d1] "v"(d[1]), [d2] "v"(d[2]), [d3] "v"(d[3]), [d4] "v"(d[4]), [d5] "v"(d[5]), [d6] "v"(d[6]),
           [d7] "v"(d[7]), [d8] "v"(d[8]), [d9] "v"(d[9]), [d10] "v"(d[10]), [d11] "v"(d[11]), [d12] "v"(d[12]),
           [d13] "v"(d[13]), [d14] "v"(d[14]), [d15] "v"(d[15]));
     return a;
@@ -127,6 +128,33 @@ __device__ __forceinline__ void block_argmin(const floatx16& d, int kb, float& m
         mi = kb + block_pos16(d, bm);
         m = bm;
     }
+}
+
+// The same running argmin with the lookup deferred: a block whose minimum improves the running one is
+// only remembered -- its number and a copy of its 16 distances (eight 64-bit moves) -- and the position
+// is looked up once, after the last block, in the copy that survived (kept_argmin).  Same result as
+// block_argmin bit for bit: strict '<' keeps the earliest block that reaches the final minimum, the
+// lookup its first position.  15 instead of 33 vector instructions per improving block.
+__device__ __forceinline__ void block_min_keep(const floatx16& d, int cb, float& m, int& blk, floatx16& keep) {
+    const float bm = block_min16(d);
+    if (bm < m) {
+        // written out so that the two values are updated where they live (the compiler's own form pairs the
+        // minima of two point blocks into 64-bit moves and shuffles them into place first)
+        asm("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "+v"(m), "+v"(blk) : "v"(bm), "s"(cb));
+        keep = d;
+    }
+}
+
+// The copy starts out without a value: it is only read after a block improved on +inf (kept_argmin
+// ignores it otherwise).  Declaring it written by an empty instruction sequence costs nothing, where
+// sixteen zeros would cost sixteen moves per point block.
+__device__ __forceinline__ void keep_undefined(floatx16& keep) { asm volatile("" : "=v"(keep)); }
+
+// index (without the lane-half term) of the minimum that block_min_keep tracked; 0 if no block ever
+// improved on +inf (all distances +inf or NaN), as block_argmin leaves it
+__device__ __forceinline__ int kept_argmin(const floatx16& keep, float m, int blk) {
+    const int pos = block_pos16(keep, m);
+    return m < HKM_INF ? blk * 32 + pos : 0;
 }
 
 // ---- split-bf16 products: an fp32 value as the sum of three bf16 parts ----

@@ -7,7 +7,7 @@
 
 namespace hkm {
 
-enum { PROBE_NONE = 0, PROBE_FMA = 1, PROBE_CNDMASK = 2, PROBE_MIN3 = 3, PROBE_SALU = 4, PROBE_CMP = 5 };
+enum { PROBE_NONE = 0, PROBE_FMA = 1, PROBE_CNDMASK = 2, PROBE_MIN3 = 3, PROBE_SALU = 4, PROBE_CMP = 5, PROBE_MOV64 = 6 };
 
 template <int OP, int NOPS>
 __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters, float a0, float b0) {
@@ -17,6 +17,7 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters, 
     float a = a0 + threadIdx.x, b = b0;
     float r0 = a0, r1 = b0, r2 = 3.f;
     int s0 = iters;
+    double q0 = a0, q1 = b0;
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -30,11 +31,12 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* out, int iters, 
                     if (OP == PROBE_MIN3) asm volatile("v_min3_f32 %0, %0, %1, %2" : "+v"(r0) : "v"(r1), "v"(r2));
                     if (OP == PROBE_SALU) asm volatile("s_add_u32 %0, %0, 1" : "+s"(s0) : : "scc");
                     if (OP == PROBE_CMP) asm volatile("v_cmp_lt_f32 vcc, %0, %1" : : "v"(r0), "v"(r1) : "vcc");
+                    if (OP == PROBE_MOV64) asm volatile("v_mov_b64 %0, %1" : "=v"(q0) : "v"(q1));
                 }
             }
         }
     }
-    float s = r0 + r1 + r2 + float(s0);
+    float s = r0 + r1 + r2 + float(s0) + float(q0);
     for (int i = 0; i < 2; ++i)
         for (int v = 0; v < 16; ++v) s += acc[i][v];
     out[size_t(blockIdx.x) * blockDim.x + threadIdx.x] = s;
@@ -73,7 +75,7 @@ int launch_probe_mfma(int32_t op, int32_t nops, int32_t iters, int32_t grid, flo
     HKM_P(PROBE_NONE, 0)
     HKM_P(PROBE_FMA, 4) HKM_P(PROBE_FMA, 8) HKM_P(PROBE_CNDMASK, 4) HKM_P(PROBE_CNDMASK, 8)
     HKM_P(PROBE_MIN3, 4) HKM_P(PROBE_MIN3, 8) HKM_P(PROBE_SALU, 4) HKM_P(PROBE_SALU, 8)
-    HKM_P(PROBE_CMP, 4) HKM_P(PROBE_CMP, 8)
+    HKM_P(PROBE_CMP, 4) HKM_P(PROBE_CMP, 8) HKM_P(PROBE_MOV64, 4) HKM_P(PROBE_MOV64, 8)
 #undef HKM_P
     return fail(HKM_EUNSUPPORTED, "hkm_probe_mfma_f32: no kernel for op = %d with %d instructions per matrix instruction", op, nops);
 }

@@ -380,7 +380,8 @@ int hkm_profile_collect(float* ms, int32_t cap, int32_t* count);
  * reference; bench.py --probe times them).  Each call enqueues ONE kernel.
  * hkm_probe_mfma_f32: every wave issues iters * 16 fp32 matrix instructions (v_mfma_f32_32x32x2_f32, two
  *   independent accumulators), each followed by `nops` instructions of kind `op`: 0 none (nops = 0),
- *   1 v_fma_f32, 2 v_cndmask_b32, 3 v_min3_f32, 4 s_add_u32 (scalar unit), 5 v_cmp_lt_f32; nops 4 or 8.
+ *   1 v_fma_f32, 2 v_cndmask_b32, 3 v_min3_f32, 4 s_add_u32 (scalar unit), 5 v_cmp_lt_f32, 6 v_mov_b64;
+ *   nops 4 or 8.
  *   grid workgroups of 256 threads; out receives grid * 256 floats.  flops = grid * 4 * iters * 16 * 4096.
  * hkm_probe_stream: mode 0 copies bytes from src to dst, 1 reads src, 2 reads src with non-temporal loads,
  *   3 fills dst; 16-byte vectors, four in flight per thread; sink is one device float.
