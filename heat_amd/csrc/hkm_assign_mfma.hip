@@ -54,6 +54,26 @@ __device__ __forceinline__ void resident_block(const float* arow, const floatx16
     }
 }
 
+// Two centroid blocks at once against one point block: two independent accumulator chains share the
+// point registers, so a wave always has a matrix instruction that does not wait for the one before it,
+// and the first block's minimum tree finds its results complete while the second chain ends.
+template <int DP>
+__device__ __forceinline__ void resident_block_pair(const float* arow0, const float* arow1, const floatx16& c0,
+                                                    const floatx16& c1, int h, const floatx4 (&b)[DP / 8],
+                                                    floatx16& acc0, floatx16& acc1) {
+    constexpr int NJ = DP / 8;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const floatx4 a0 = ld4(arow0 + h * (DP / 2) + 4 * j);
+        const floatx4 a1 = ld4(arow1 + h * (DP / 2) + 4 * j);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            acc0 = (j == 0 && t == 0) ? MFMA32(a0[t], b[j][t], c0) : MFMA32(a0[t], b[j][t], acc0);
+            acc1 = (j == 0 && t == 0) ? MFMA32(a1[t], b[j][t], c1) : MFMA32(a1[t], b[j][t], acc1);
+        }
+    }
+}
+
 // Scan of all centroid blocks.  CLAMP applies max(. + |x|^2, 0) to every value (the rescan of a tile
 // whose lazy minimum came out negative).  Two blocks per trip: the squared norms of both are requested
 // at the top of the trip into the registers that then serve, in place, as their accumulators (norms
@@ -85,11 +105,31 @@ __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn,
             block_min_keep(acc[pb], cb, m[pb], blk[pb], keep[pb]);
         }
     };
-    for (int cb = 0; cb < ncb; cb += 2) {
-        const floatx16 ca = load_cn16(sCn + cb * 32 + 4 * h);
-        const floatx16 cb1 = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
-        one_block(cb, ca);
-        if (cb + 1 < ncb) one_block(cb + 1, cb1);
+    if (PB == 1) {
+        int cb = 0;
+        for (; cb + 1 < ncb; cb += 2) {
+            const floatx16 c0 = load_cn16(sCn + cb * 32 + 4 * h);
+            const floatx16 c1 = load_cn16(sCn + (cb + 1) * 32 + 4 * h);
+            floatx16 acc0, acc1;
+            resident_block_pair<DP>(sC + (cb * 32 + p) * LDC, sC + ((cb + 1) * 32 + p) * LDC, c0, c1, h, b[0], acc0, acc1);
+            if (CLAMP) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    acc0[v] = fmaxf(acc0[v] + xn[0], 0.0f);
+                    acc1[v] = fmaxf(acc1[v] + xn[0], 0.0f);
+                }
+            }
+            block_min_keep(acc0, cb, m[0], blk[0], keep[0]);
+            block_min_keep(acc1, cb + 1, m[0], blk[0], keep[0]);
+        }
+        if (cb < ncb) one_block(cb, load_cn16(sCn + cb * 32 + 4 * h));
+    } else {
+        for (int cb = 0; cb < ncb; cb += 2) {
+            const floatx16 ca = load_cn16(sCn + cb * 32 + 4 * h);
+            const floatx16 cb1 = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
+            one_block(cb, ca);
+            if (cb + 1 < ncb) one_block(cb + 1, cb1);
+        }
     }
 #pragma unroll
     for (int pb = 0; pb < PB; ++pb) {
