@@ -20,6 +20,8 @@ roofline   the dominant kernel -- the fused distance+argmin kernel, or the one-s
            steps; kernel_ms is the mean over those launches, achieved = algorithmic flops 2*N*K*D
            (MFMA-bound shapes) or bytes N*(4D+4) (HBM-bound shapes) per launch / kernel_ms.
            step_ms_events is the whole step (all its launches, no host read) between two events.
+           sclk_mhz_under_load is the shader clock the driver reports while that step runs back to
+           back (peak assumes 2400 MHz; chips differ in what they hold under the matrix-core kernels)
            traffic (HBM bytes per launch, rocprofv3 FETCH_SIZE / WRITE_SIZE) is read from
            profiles/traffic.json and only reported while the library sources still hash to what they
            were when it was measured (traffic_source says which)
@@ -399,6 +401,35 @@ def bench_silhouette(args, w, x, t_gen) -> int:
     return 0
 
 
+def sclk_under_load(enqueue, seconds: float = 0.6):
+    """Median of the current shader clock (MHz) as /sys/class/drm/card*/device/pp_dpm_sclk reports it while
+    `enqueue` keeps the device busy; the first 0.2 s are left out (the clock ramps up)."""
+    import glob
+
+    import torch
+
+    files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    if not files:
+        return None
+    vals = []
+    t0 = time.perf_counter()
+    try:
+        while time.perf_counter() - t0 < seconds:
+            enqueue()
+            if time.perf_counter() - t0 < 0.2:
+                continue
+            with open(files[0]) as f:
+                for line in f:
+                    if "*" in line:
+                        vals.append(int(line.split(":")[1].strip().split("Mhz")[0]))
+    except (OSError, ValueError, IndexError):
+        vals = []
+    torch.cuda.synchronize()
+    if not vals:
+        return None
+    return sorted(vals)[len(vals) // 2]
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -524,6 +555,12 @@ def main() -> int:
         ev_ms.append(e0.elapsed_time(e1))
     step_ms = sum(ev_ms) / len(ev_ms)
 
+    # The shader clock while the dominant kernel runs back to back (best effort: the driver's own
+    # figure, read from sysfs between batches of launches; None where the file is not there).  `peak`
+    # assumes 2400 MHz; some chips hold less under the matrix-core kernels, and then `frac` is lower
+    # by that ratio although the kernel does the same work per clock.
+    sclk = sclk_under_load(lambda: [kernel_only() for _ in range(20)])
+
     # both fractions for every workload; the binding one fills the standard fields
     flops = 2.0 * n * k * d
     nbytes = float(n) * (4 * d + 4) if args.config != "c2" else float(n) * (4 * d + 8) + 4.0 * k * d
@@ -541,6 +578,7 @@ def main() -> int:
     roof["kernel_ms"] = round(kern_ms, 4)
     roof["kernel_launches_timed"] = len(kern)
     roof["step_ms_events"] = round(step_ms, 4)
+    roof["sclk_mhz_under_load"] = sclk
     roof["traffic"] = None
     roof["traffic_source"] = "none: profiles/traffic.json is missing"
     tfile = os.path.join(ROOT, "profiles", "traffic.json")
