@@ -21,7 +21,9 @@ roofline   the dominant kernel -- the fused distance+argmin kernel, or the one-s
            (MFMA-bound shapes) or bytes N*(4D+4) (HBM-bound shapes) per launch / kernel_ms.
            step_ms_events is the whole step (all its launches, no host read) between two events.
            sclk_mhz_under_load is the shader clock the driver reports while that step runs back to
-           back (peak assumes 2400 MHz; chips differ in what they hold under the matrix-core kernels)
+           back (peak assumes 2400 MHz; chips differ in what they hold under the matrix-core kernels),
+           mfma_alone_tflops_this_chip what a chain of nothing but fp32 matrix instructions reaches on
+           this chip right after (the probe of --probe)
            traffic (HBM bytes per launch, rocprofv3 FETCH_SIZE / WRITE_SIZE) is read from
            profiles/traffic.json and only reported while the library sources still hash to what they
            were when it was measured (traffic_source says which)
@@ -401,6 +403,35 @@ def bench_silhouette(args, w, x, t_gen) -> int:
     return 0
 
 
+def mfma_alone_tflops() -> float:
+    """What this chip sustains on fp32 matrix instructions and nothing else (the chain of bench.py --probe,
+    about 0.4 s of it, clocks already warm): the ceiling `frac` could reach here if the kernel issued
+    nothing but matrix instructions.  Chips differ: some hold 2.4 GHz under it, some do not."""
+    import ctypes
+
+    import torch
+
+    from heat_amd import _native
+
+    lib = _native.load()
+    grid, iters = 1024, 2000
+    out = torch.empty((grid * 256,), dtype=torch.float32, device="cuda:0")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    flops = grid * 4 * iters * 16 * 4096.0
+
+    def run(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            _native.check(lib.hkm_probe_mfma_f32(0, 0, iters, grid, ctypes.c_void_p(out.data_ptr()), stream))
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    run(40)
+    return flops / (run(40) * 1e-3) / 1e12
+
+
 def sclk_under_load(enqueue, seconds: float = 0.6):
     """Median of the current shader clock (MHz) as /sys/class/drm/card*/device/pp_dpm_sclk reports it while
     `enqueue` keeps the device busy; the first 0.2 s are left out (the clock ramps up)."""
@@ -579,6 +610,8 @@ def main() -> int:
     roof["kernel_launches_timed"] = len(kern)
     roof["step_ms_events"] = round(step_ms, 4)
     roof["sclk_mhz_under_load"] = sclk
+    if args.config in MFMA_BOUND:
+        roof["mfma_alone_tflops_this_chip"] = round(mfma_alone_tflops(), 1)
     roof["traffic"] = None
     roof["traffic_source"] = "none: profiles/traffic.json is missing"
     tfile = os.path.join(ROOT, "profiles", "traffic.json")

@@ -432,7 +432,7 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
                                             w.fcnt, w.fflags, st);
         if (rc) return rc;
         if ((rc = launch_update_fused(X, N, D, ldx, labels, K, C_new, D, nullptr, w,
-                                      split ? split_fused_grid(N) : fused_grid(N), C, shift, st)))
+                                      split ? split_fused_grid(N) : fused_grid(N, D), C, shift, st)))
             return rc;
     } else {
         if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;

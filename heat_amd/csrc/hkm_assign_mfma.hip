@@ -264,11 +264,24 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 // the two-pass update, whose kernels start by looking at the flags.
 // ------------------------------------------------------------------------------------------------
 static constexpr int FUSED_QBITS = 28;
-static constexpr int FUSED_THREADS = 768;
-static constexpr int FUSED_PB = 1;
+// Point blocks per wave of the resident kernels.  Up to 32 padded features there is a choice: TWO point
+// blocks against every centroid row a wave reads from LDS (eight waves per CU), or ONE with twelve waves.
+// Two halve the LDS reads per matrix instruction, and that decides on chips that lower their clock under
+// these kernels.  Measured on the 10M x 32 x 256 workload over a dozen chips of the same model: on those
+// that hold 2.39 GHz one point block is 2 % faster (one-sweep step 1.347 against 1.375 ms); on those that
+// do not it runs at 2.1-2.2 GHz and two point blocks at 2.3 GHz (1.430 against 1.391 ms).  Two is the
+// default -- never far from the better one; HKM_POINT_BLOCKS=1 selects the other.  Wider rows leave
+// registers for one point block only.
+__host__ __device__ constexpr int fused_threads(int pb) { return pb == 2 ? 512 : 768; }
+
+static int resident_point_blocks(int dp) {
+    if (dp > 32) return 1;
+    const char* e = getenv("HKM_POINT_BLOCKS");
+    return (e && e[0] == '1' && e[1] == 0) ? 1 : 2;
+}
 
 template <int DP, int PB, bool VEC>
-__global__ __launch_bounds__(FUSED_THREADS) void lloyd_mfma_resident_kernel(
+__global__ __launch_bounds__(fused_threads(PB)) void lloyd_mfma_resident_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles,
     double* __restrict__ fsum, int32_t* __restrict__ fcnt, int32_t* __restrict__ flags,
@@ -729,16 +742,15 @@ int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, 
 #undef HKM_CASE
 }
 
-template <int DP, bool VEC>
+template <int DP, int PB, bool VEC>
 static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                              int32_t K, int64_t ldc, int32_t* labels, float* min_d2,
                              hipStream_t st) {
-    constexpr int PB = 1;
     const int64_t ntiles = (N + 4 * PB * 32 - 1) / (4 * PB * 32);
     const size_t lds = resident_lds_bytes(D, K);
     auto kern = assign_mfma_resident_kernel<DP, PB, VEC>;
-    // persistent grid: as many workgroups as are resident at once (registers allow four per CU up to
-    // 48 padded features, the centroids' LDS footprint decides the rest)
+    // persistent grid: as many workgroups as are resident at once (registers and the centroids' LDS
+    // footprint decide: two per CU with two point blocks per wave, up to four with one)
     int per_cu = 0;
     hipError_t oe = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), 256, lds);
     if (oe != hipSuccess) return fail(HKM_EHIP, "hipOccupancyMaxActiveBlocksPerMultiprocessor: %s", hipGetErrorString(oe));
@@ -758,9 +770,9 @@ size_t fused_lds_bytes(int32_t D, int32_t K) {
     return kp * (dp + 5) * sizeof(float) + size_t(K) * (dp + 1) * sizeof(double) + (size_t(K) + 4) * sizeof(int);
 }
 
-int fused_grid(int64_t N) {
-    constexpr int PB = FUSED_PB;
-    const int64_t tile_rows = int64_t(FUSED_THREADS / 64) * PB * 32;
+int fused_grid(int64_t N, int32_t D) {
+    const int pb = resident_point_blocks(resident_dp(D));
+    const int64_t tile_rows = int64_t(fused_threads(pb) / 64) * pb * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
     int64_t grid = num_cus();
     if (grid > FUSED_MAX_GRID) grid = FUSED_MAX_GRID;
@@ -768,14 +780,14 @@ int fused_grid(int64_t N) {
     return int(grid < 1 ? 1 : grid);
 }
 
-template <int DP, bool VEC>
+template <int DP, int PB, bool VEC>
 static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                           int64_t ldc, int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt,
                           int32_t* flags, hipStream_t st) {
-    constexpr int PB = FUSED_PB;
-    const int64_t tile_rows = int64_t(FUSED_THREADS / 64) * PB * 32;
+    constexpr int THREADS = fused_threads(PB);
+    const int64_t tile_rows = int64_t(THREADS / 64) * PB * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
-    const int grid = fused_grid(N);
+    const int grid = fused_grid(N, D);
     const size_t lds = fused_lds_bytes(D, K);
     auto kern = lloyd_mfma_resident_kernel<DP, PB, VEC>;
     if (lds > 64 * 1024) {
@@ -789,7 +801,7 @@ static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
     while ((int64_t(1) << lg) < per_wg) ++lg;
     const int range_bits = 53 - FUSED_QBITS - lg;
     prof_begin(st);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(FUSED_THREADS), lds, st, X, N, D, ldx, C, K, ldc,
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), lds, st, X, N, D, ldx, C, K, ldc,
                        labels, min_d2, ntiles, fsum, fcnt, flags, range_bits);
     prof_end(st);
     return check_launch("lloyd_mfma_resident_kernel");
@@ -800,16 +812,14 @@ int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx
                                int32_t* fcnt, int32_t* flags, hipStream_t st) {
     const bool vec = aligned16(X) && (ldx % 4 == 0) && (D % 4 == 0);
     const int dp = resident_dp(D);
-#define HKM_CASE(d)                                                                                         \
-    case d:                                                                                                 \
-        return vec ? launch_fused_t<d, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st) \
-                   : launch_fused_t<d, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);
-    switch (dp) {
-        HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
-        default:
-            return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
-    }
+    const int pb = resident_point_blocks(dp);
+#define HKM_CASE(d, b)                                                                                         \
+    if (dp == d && pb == b)                                                                                    \
+        return vec ? launch_fused_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st) \
+                   : launch_fused_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);
+    HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2) HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
 #undef HKM_CASE
+    return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
 }
 
 int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
@@ -817,16 +827,14 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
                                 hipStream_t st) {
     const bool vec = aligned16(X) && (ldx % 4 == 0) && (D % 4 == 0);
     const int dp = resident_dp(D);
-#define HKM_CASE(d)                                                                         \
-    case d:                                                                                 \
-        return vec ? launch_resident_t<d, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, st) \
-                   : launch_resident_t<d, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
-    switch (dp) {
-        HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
-        default:
-            return fail(HKM_EUNSUPPORTED, "assign_mfma_resident: D=%d", D);
-    }
+    const int pb = resident_point_blocks(dp);
+#define HKM_CASE(d, b)                                                                         \
+    if (dp == d && pb == b)                                                                    \
+        return vec ? launch_resident_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, st) \
+                   : launch_resident_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
+    HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2) HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
 #undef HKM_CASE
+    return fail(HKM_EUNSUPPORTED, "assign_mfma_resident: D=%d", D);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -165,7 +165,7 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
                               int32_t* labels, float* min_d2, bool split, hipStream_t st);
 bool fused_eligible(int32_t D, int32_t K);
 size_t fused_lds_bytes(int32_t D, int32_t K);
-int fused_grid(int64_t N);
+int fused_grid(int64_t N, int32_t D);
 int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                                int32_t K, int64_t ldc, int32_t* labels, float* min_d2, double* fsum,
                                int32_t* fcnt, int32_t* flags, hipStream_t st);
