@@ -220,29 +220,48 @@ __global__ __launch_bounds__(256) void knn_tile_kernel(
 }
 
 // ---- shared by the two matrix-core kernels -------------------------------------------------------
-// candidates of one 32 x 32 block: accumulator element i is reference row j0 + 8 (i / 4) + 4 h + i % 4
+// The distance a list must beat: the kcount-th entry, the smaller one of the two lanes that share a query
+// row.  Pairs in the lists stem from earlier tiles, i.e. from smaller rows than any later candidate, so a
+// candidate at exactly the threshold ranks after kcount of them.
 template <int KL>
-__device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (&li)[KL], const floatx16& acc,
-                                                     const floatx16& xnv, float qn, int64_t j0, int h, int64_t r_end,
-                                                     int kcount, int has_bound, float bd, unsigned bi) {
-    // pairs in the lists stem from earlier tiles, i.e. from smaller rows than any candidate here; a
-    // candidate at exactly the threshold ranks after kcount of them
+__device__ __forceinline__ float knn_threshold(const float (&ld)[KL], int kcount) {
     float thr = ld[KL - 1];
 #pragma unroll
     for (int s = 0; s < KL - 1; ++s) thr = s == kcount - 1 ? ld[s] : thr;  // only kcount entries are asked for
-    thr = fminf(thr, __shfl_xor(thr, 32));
+    return fminf(thr, __shfl_xor(thr, 32));
+}
+
+// Candidates of one 32 x 32 block.  t holds |x|^2 - 2 q.x (the accumulators start at the squared norms of
+// their reference rows and the query operand carries the factor -2): element i is reference row
+// j0 + 8 (i / 4) + 4 h + i % 4, its squared distance max(t + |q|^2, 0).  The smallest of the 16 is found
+// first (a tree of three-input minima, nine instructions); only if it beats the threshold in some lane of
+// the wave are the 16 looked at one by one -- adding |q|^2 and clamping are monotone, so the test on the
+// minimum decides exactly as the tests on the elements would.  thr is carried from tile to tile and
+// recomputed only after the lists may have changed.
+template <int KL>
+__device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (&li)[KL], float& thr,
+                                                     const floatx16& t, float qn, int64_t j0, int h, int64_t r_end,
+                                                     int kcount, int has_bound, float bd, unsigned bi) {
+    // the last tile of a split (rows past the end) and the later passes of k > 16 (pairs ranked before the
+    // bound) need every element looked at
+    const bool edge = j0 + 32 > r_end || has_bound;
+    if (!edge) {
+        const float s = block_min16(t) + qn;
+        const float dmin = s < 0.0f ? 0.0f : s;
+        if (__builtin_amdgcn_ballot_w64(dmin < thr) == 0) return;
+    }
     const unsigned gj0 = unsigned(j0) + 4 * h;
     float dv[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         // compare + select, not fmaxf: a NaN (a NaN row, inf - inf of overflowing norms) must stay a NaN,
         // which fails every `< thr` below and is never admitted; fmaxf would turn it into distance 0
-        const float t = fmaf(-2.0f, acc[i], qn + xnv[i]);
-        dv[i] = t < 0.0f ? 0.0f : t;
+        const float s = t[i] + qn;
+        dv[i] = s < 0.0f ? 0.0f : s;
     }
-    if (j0 + 32 > r_end || has_bound) {
-        // the last tile of a split and the later passes: rows past the end and pairs that do not rank
-        // after the bound become +inf here, so that one chain of offers serves every tile
+    if (edge) {
+        // rows past the end and pairs that do not rank after the bound become +inf here, so that one chain
+        // of offers serves every tile
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const unsigned gj = gj0 + 8 * (i >> 2) + (i & 3);
@@ -253,6 +272,7 @@ __device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) knn_offer<KL>(ld, li, dv[i] < thr, dv[i], gj0 + 8 * (i >> 2) + (i & 3));
+    thr = knn_threshold<KL>(ld, kcount);
 }
 
 // The two lanes of a query row (h = 0, 1): KL times the smaller head, whose lane pops it; lane h = 0
@@ -335,8 +355,9 @@ __global__ __launch_bounds__(256) void knn_mfma_kernel(
             const floatx4 t = load_row4<VEC>(qrow, h * H + 4 * g, D);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                qv[4 * g + e] = live ? t[e] : 0.0f;
-                qn = fmaf(qv[4 * g + e], qv[4 * g + e], qn);
+                const float q = live ? t[e] : 0.0f;
+                qv[4 * g + e] = -2.0f * q;  // exact; the accumulators then hold |x|^2 - 2 q.x
+                qn = fmaf(q, q, qn);
             }
         }
         qn += __shfl_xor(qn, 32);
@@ -349,6 +370,7 @@ __global__ __launch_bounds__(256) void knn_mfma_kernel(
         ld[s] = HKM_INF;
         li[s] = KNN_NONE;
     }
+    float thr = HKM_INF;  // what a candidate must beat: the lists are empty
     float bd = -1.0f;
     unsigned bi = 0;
     if (has_bound && live) {
@@ -373,12 +395,10 @@ __global__ __launch_bounds__(256) void knn_mfma_kernel(
         float an[H];
         load_tile(min(j0 + 32, r_end - 1), an);  // the next tile while this one is multiplied
         const floatx16 xnv = load_cn16(xn + j0 + 4 * h);
-        floatx16 acc;
+        floatx16 acc = MFMA32(av[0], qv[0], xnv);  // starts at the squared norms of its reference rows
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-#pragma unroll
-        for (int s = 0; s < H; ++s) acc = MFMA32(av[s], qv[s], acc);
-        knn_block_candidates<KL>(ld, li, acc, xnv, qn, j0, h, r_end, kcount, has_bound, bd, bi);
+        for (int s = 1; s < H; ++s) acc = MFMA32(av[s], qv[s], acc);
+        knn_block_candidates<KL>(ld, li, thr, acc, qn, j0, h, r_end, kcount, has_bound, bd, bi);
 #pragma unroll
         for (int s = 0; s < H; ++s) av[s] = an[s];
     }
@@ -399,6 +419,7 @@ __global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
     constexpr int RS = 2 * H + 4;            // floats per staged row; the pad spreads 16 rows over all banks
     constexpr int NV = H >= 16 ? H / 16 : 1;  // float4 groups a thread moves per tile
     __shared__ __attribute__((aligned(16))) float sA[2][32][RS];
+    __shared__ __attribute__((aligned(16))) float sXn[2][32];  // squared norms of the staged rows
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, h = lane >> 5;
@@ -418,8 +439,9 @@ __global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
             const floatx4 t = load_row4<true>(qrow, h * H + 4 * g, D);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                qv[4 * g + e] = live ? t[e] : 0.0f;
-                qn = fmaf(qv[4 * g + e], qv[4 * g + e], qn);
+                const float q = live ? t[e] : 0.0f;
+                qv[4 * g + e] = -2.0f * q;  // exact; the accumulators then hold |x|^2 - 2 q.x
+                qn = fmaf(q, q, qn);
             }
         }
         qn += __shfl_xor(qn, 32);
@@ -432,6 +454,7 @@ __global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
         ld[s] = HKM_INF;
         li[s] = KNN_NONE;
     }
+    float thr = HKM_INF;  // what a candidate must beat: the lists are empty
     float bd = -1.0f;
     unsigned bi = 0;
     if (has_bound && live) {
@@ -451,15 +474,20 @@ __global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
         sval[j] = idx < 32 * c4n;
     }
     floatx4 st[NV];
+    floatx4 stn = {0.f, 0.f, 0.f, 0.f};
     auto fetch = [&](int64_t j0) {
 #pragma unroll
         for (int j = 0; j < NV; ++j)
             if (sval[j]) st[j] = ld4(R + min(j0 + srow[j], Nn - 1) * ldr + scol[j]);  // rows past the end: never admitted
+        // the norms ride along (eight threads): the first matrix instruction of a tile needs them, and
+        // a read from global memory at that point would be waited for (the buffer is padded by 64 floats)
+        if (tid < 8) stn = ld4(xn + j0 + 4 * tid);
     };
     auto stash = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < NV; ++j)
             if (sval[j]) *reinterpret_cast<floatx4*>(&sA[buf][srow[j]][scol[j]]) = st[j];
+        if (tid < 8) *reinterpret_cast<floatx4*>(&sXn[buf][4 * tid]) = stn;
     };
     __syncthreads();
     fetch(r_begin);
@@ -470,18 +498,17 @@ __global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
     for (int64_t j0 = r_begin; j0 < r_end; j0 += 32) {
         const bool more = j0 + 32 < r_end;
         if (more) fetch(j0 + 32);  // the next tile while this one is multiplied
-        const floatx16 xnv = load_cn16(xn + j0 + 4 * h);
+        const floatx16 xnv = load_cn16(&sXn[buf][4 * h]);
         floatx16 acc;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
         const float* arow = &sA[buf][col][h * H];
 #pragma unroll
         for (int g = 0; g < H / 4; ++g) {
             const floatx4 a = *reinterpret_cast<const floatx4*>(arow + 4 * g);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc = MFMA32(a[e], qv[4 * g + e], acc);
+            for (int e = 0; e < 4; ++e)  // the accumulators start at the squared norms of their reference rows
+                acc = (g == 0 && e == 0) ? MFMA32(a[e], qv[0], xnv) : MFMA32(a[e], qv[4 * g + e], acc);
         }
-        knn_block_candidates<KL>(ld, li, acc, xnv, qn, j0, h, r_end, kcount, has_bound, bd, bi);
+        knn_block_candidates<KL>(ld, li, thr, acc, qn, j0, h, r_end, kcount, has_bound, bd, bi);
         if (more) stash(buf ^ 1);
         __syncthreads();
         buf ^= 1;

@@ -272,8 +272,9 @@ int hkm_closest_rows_l1_q64_f32(const float* X, int64_t N, int32_t D, int64_t ld
  *   exactly the same squared distance the smaller index comes first -- and, if dist is not NULL, the
  *   distances themselves (M x k float32, leading dimension ldd).  For D < 16 and D > 128 the squared
  *   distance is summed directly as sum (q - x)^2 in fp32; for 16 <= D <= 128 it is the clamped expansion
- *   max(0, (|q|^2 + |x|^2) - 2 q.x) with the products on the matrix cores (the form torch.cdist itself takes
- *   above 25 rows): it carries an absolute error of up to about 4e-7 (|q|^2 + |x|^2), so a row identical to
+ *   max(0, (|x|^2 - 2 q.x) + |q|^2) with the products on the matrix cores, accumulated onto |x|^2 (the form
+ *   torch.cdist itself takes above 25 rows, in another order of additions): it carries an absolute error of up
+ *   to about 4e-7 (|q|^2 + |x|^2), so a row identical to
  *   the query may come back at a small non-zero distance and rows whose squared distances are closer than
  *   that may swap places.  The square root is correctly rounded.  A slot for which no finite distance
  *   is left (NaN or overflowing rows) holds index -1 and distance inf.  1 <= k <= min(N, HKM_KNN_MAX_K).
