@@ -228,6 +228,35 @@ def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
     assert torch.equal(again[0], c_step) and torch.equal(again[2], shift)
 
 
+@pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (768, 17, 5)])
+def test_one_point_block_per_wave_gives_the_same_labels(cuda, n, d, k, monkeypatch):
+    # HKM_POINT_BLOCKS=1 (16 < D <= 32): another launch geometry of the same kernels -- labels and minima
+    # bit for bit, centroids up to the grouping of the exact per-workgroup partial sums
+    print(f"point blocks n={n} d={d} k={k}", flush=True)
+    x, _ = _data(n, d, k, seed=3 * n + d)
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(9))[:k]].contiguous()
+    xs, cs = x.to(cuda), c0.to(cuda)
+    ws = _native.Workspace(cuda)
+
+    def run():
+        lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+        md = torch.empty((n,), device=cuda)
+        _native.assign(xs, cs, lab, md, ws)
+        cn = torch.empty_like(cs)
+        lab2 = torch.empty_like(lab)
+        shift = torch.empty((), device=cuda)
+        _native.lloyd_step(xs, cs, cn, lab2, shift, None, ws)
+        torch.cuda.synchronize()
+        return lab.cpu(), md.cpu(), lab2.cpu(), cn.cpu(), float(shift)
+
+    two = run()
+    monkeypatch.setenv("HKM_POINT_BLOCKS", "1")
+    one = run()
+    assert torch.equal(one[0], two[0]) and torch.equal(one[1], two[1]) and torch.equal(one[2], two[2])
+    assert orc.rel_err_centers(one[3], two[3]) <= 2e-7
+    assert abs(one[4] - two[4]) <= 1e-6 * max(abs(two[4]), 1e-30)
+
+
 def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
     # Row magnitudes spread over 2^60 (or rows holding inf / NaN) break the condition under which the
     # fp64 LDS sums are independent of the order of additions: the step must then produce exactly
