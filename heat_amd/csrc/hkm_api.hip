@@ -200,6 +200,10 @@ static int check_shape(int64_t N, int32_t D, int32_t K) {
     if (N < 0) return fail(HKM_EINVAL, "N = %lld is negative", (long long)N);
     if (D < 1) return fail(HKM_EINVAL, "D = %d must be >= 1", D);
     if (K < 1) return fail(HKM_EINVAL, "K = %d must be >= 1", K);
+    // sizes no device holds: refused here so that the byte counts computed from them cannot wrap around
+    if (N > (int64_t(1) << 40)) return fail(HKM_EUNSUPPORTED, "N = %lld exceeds 2^40 rows", (long long)N);
+    if (int64_t(K) * D > (int64_t(1) << 40))
+        return fail(HKM_EUNSUPPORTED, "K x D = %lld exceeds 2^40 centroid coordinates", (long long)(int64_t(K) * D));
     return HKM_OK;
 }
 
@@ -283,6 +287,7 @@ int hkm_profile_collect(float* ms, int32_t cap, int32_t* count) {
 
 size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags) {
     if (N < 0 || D < 1 || K < 1) return 0;
+    if (N > (int64_t(1) << 40) || int64_t(K) * D > (int64_t(1) << 40)) return 0;  // refused by every entry point
     if (flags == HKM_WS_MEDIAN) return carve_median(nullptr, N, D, K).total;
     return carve(nullptr, N, D, K, flags).total;
 }

@@ -60,7 +60,9 @@ int hkm_version(void);
 /* Message of the last error raised on the calling thread ("" if none). Host pointer, static storage. */
 const char* hkm_last_error(void);
 
-/* Bytes of device workspace needed by the entry points below for this problem size. */
+/* Bytes of device workspace needed by the entry points below for this problem size; 0 for sizes they
+ * refuse (N < 0, D < 1, K < 1, and N > 2^40 rows or K * D > 2^40 centroid coordinates, which return
+ * HKM_EUNSUPPORTED: no device holds them, and the byte counts derived from them could wrap around). */
 size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags);
 
 /*

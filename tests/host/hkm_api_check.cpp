@@ -1,0 +1,143 @@
+// Host-side driver for the argument-validation layer of libhkm (include/hkm.h), meant to run under the host
+// compiler's AddressSanitizer (heat_amd/csrc/Makefile, target asan-host): every call below is refused -- or
+// returns at once for an empty problem -- before anything reaches the device, so it runs without a GPU.  What
+// the sanitizer watches is the host code on those paths: the checks themselves, the formatting of the
+// thread-local message, the workspace carving arithmetic.  Pointers handed in are made-up non-null addresses
+// that are never dereferenced.
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "hkm.h"
+
+static int failures = 0;
+
+#define EXPECT(call, want)                                                                     \
+    do {                                                                                       \
+        const int rc_ = (call);                                                                \
+        if (rc_ != (want)) {                                                                   \
+            std::printf("FAIL %s:%d  %s  returned %d, expected %d (%s)\n", __FILE__, __LINE__, \
+                        #call, rc_, (want), hkm_last_error());                                 \
+            ++failures;                                                                        \
+        }                                                                                      \
+    } while (0)
+
+#define EXPECT_MSG(sub)                                                                                   \
+    do {                                                                                                  \
+        if (!std::strstr(hkm_last_error(), (sub))) {                                                      \
+            std::printf("FAIL %s:%d  message '%s' lacks '%s'\n", __FILE__, __LINE__, hkm_last_error(), (sub)); \
+            ++failures;                                                                                   \
+        }                                                                                                 \
+    } while (0)
+
+int main() {
+    float* const f = reinterpret_cast<float*>(uintptr_t(4096));
+    double* const d = reinterpret_cast<double*>(uintptr_t(4096));
+    int32_t* const i32 = reinterpret_cast<int32_t*>(uintptr_t(4096));
+    int64_t* const i64 = reinterpret_cast<int64_t*>(uintptr_t(4096));
+    void* const ws = reinterpret_cast<void*>(uintptr_t(1) << 20);
+    const size_t big = size_t(1) << 30;
+
+    if (hkm_version() < 300) {
+        std::printf("FAIL version %d\n", hkm_version());
+        ++failures;
+    }
+
+    // ---- hkm_assign_f32
+    EXPECT(hkm_assign_f32(nullptr, 10, 3, 3, f, 8, 3, i32, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT_MSG("X is NULL");
+    EXPECT(hkm_assign_f32(f, -1, 3, 3, f, 8, 3, i32, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_f32(f, 10, 0, 3, f, 8, 3, i32, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_f32(f, 10, 3, 3, f, 0, 3, i32, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_f32(f, 10, 3, 2, f, 8, 3, i32, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_f32(reinterpret_cast<float*>(uintptr_t(4098)), 10, 3, 3, f, 8, 3, i32, nullptr, ws, big, nullptr),
+           HKM_EINVAL);
+    EXPECT(hkm_assign_f32(f, 10, 3, 3, f, 8, 3, nullptr, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_f32(f, 10, 3, 3, f, 8, 3, i32, nullptr, nullptr, 0, nullptr), HKM_EWORKSPACE);
+    EXPECT(hkm_assign_f32(f, 10, 3, 3, f, 8, 3, i32, nullptr, ws, 16, nullptr), HKM_EWORKSPACE);
+    EXPECT(hkm_assign_f32(f, 10, 3, 3, f, 8, 3, i32, nullptr, reinterpret_cast<void*>((uintptr_t(1) << 20) + 8), big, nullptr),
+           HKM_EWORKSPACE);
+    // every kernel family's shape goes through the same checks and its own workspace arithmetic
+    const int32_t shapes[][2] = {{3, 8}, {8, 16}, {32, 256}, {64, 1024}, {512, 1024}, {100, 5000}, {17, 3}};
+    for (const auto& s : shapes) {
+        EXPECT(hkm_assign_f32(f, 1000, s[0], s[0], f, s[1], s[0], i32, nullptr, ws, 16, nullptr), HKM_EWORKSPACE);
+        EXPECT(hkm_lloyd_step_f32(f, 1000, s[0], s[0], f, f + 1024, s[1], i32, f, nullptr, ws, 16, nullptr), HKM_EWORKSPACE);
+        if (hkm_workspace_bytes(1000, s[0], s[1], HKM_WS_ASSIGN) > hkm_workspace_bytes(1000, s[0], s[1], HKM_WS_LLOYD)) {
+            std::printf("FAIL workspace sizes D=%d K=%d\n", s[0], s[1]);
+            ++failures;
+        }
+    }
+    // a message longer than most: formatted into the thread-local buffer
+    EXPECT(hkm_assign_f32(f, INT64_MAX / 2, INT32_MAX, INT64_MAX / 4, f, INT32_MAX, INT64_MAX / 8, i32, nullptr, ws, big, nullptr),
+           HKM_EUNSUPPORTED);
+
+    // ---- update / step / shift
+    EXPECT(hkm_update_f32(f, 10, 3, 3, nullptr, 8, f, 3, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_update_f32(f, 10, 3, 3, i32, 8, f, 2, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_update_f32(f, 10, 3, 3, i32, 8, f, 3, nullptr, ws, 8, nullptr), HKM_EWORKSPACE);
+    EXPECT(hkm_lloyd_step_f32(f, 10, 3, 3, f, f, 8, i32, f, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_shift_f32(nullptr, f, 8, 3, f, nullptr), HKM_EINVAL);
+    EXPECT(hkm_shift_f32(f, f, 0, 3, f, nullptr), HKM_EINVAL);
+    EXPECT(hkm_functional_value_f32(f, -1, f, ws, big, nullptr), HKM_EINVAL);
+
+    // ---- the allocation-free assignment: its built-in scratch has a stated size
+    EXPECT(hkm_assign_static_f32(nullptr, 10, 3, 3, f, 8, 3, i32, nullptr, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_static_f32(f, int64_t(1) << 26, 512, 512, f, 1024, 512, i32, nullptr, nullptr), HKM_EUNSUPPORTED);
+    if (hkm_static_scratch_bytes() != size_t(HKM_STATIC_SCRATCH_BYTES)) {
+        std::printf("FAIL static scratch size\n");
+        ++failures;
+    }
+
+    // ---- distances
+    EXPECT(hkm_cdist_f32(f, 4, 3, f, 4, 3, 3, f, 3, 1, nullptr), HKM_EINVAL);
+    EXPECT(hkm_cdist_f32(f, -4, 3, f, 4, 3, 3, f, 4, 1, nullptr), HKM_EINVAL);
+    EXPECT(hkm_pairwise_f32(f, 4, 3, f, 4, 3, 3, f, 4, 9, 1.0f, nullptr), HKM_EINVAL);
+    EXPECT(hkm_pairwise_f32(f, 4, 3, f, 4, 3, 3, f, 4, HKM_METRIC_GAUSS, 0.0f, nullptr), HKM_EINVAL);
+    EXPECT(hkm_pairwise_f64(d, 4, 3, d, 4, 3, 3, d, 4, 9, 1.0, nullptr), HKM_EINVAL);
+    EXPECT(hkm_widen_labels_i64(nullptr, 4, i64, nullptr), HKM_EINVAL);
+
+    // ---- float64 entry points
+    EXPECT(hkm_assign_f64(reinterpret_cast<double*>(uintptr_t(4100)), 10, 3, 3, d, 8, 3, i32, nullptr, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_f64(d, 10, 3, 2, d, 8, 3, i32, nullptr, nullptr), HKM_EINVAL);
+    EXPECT(hkm_update_f64(d, 10, 3, 3, i32, 8, d, 3, nullptr, ws, 8, nullptr), HKM_EWORKSPACE);
+    EXPECT(hkm_shift_f64(nullptr, d, 8, 3, d, nullptr), HKM_EINVAL);
+
+    // ---- k nearest neighbours
+    EXPECT(hkm_knn_f32(f, 4, 3, f, 0, 3, 3, 1, i64, 1, nullptr, 0, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_knn_f32(f, 4, 3, f, 10, 3, 3, 11, i64, 11, nullptr, 0, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_knn_f32(f, 4, 3, f, 10, 3, 3, 2, i64, 1, nullptr, 0, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_knn_f32(f, 4, 3, f, 10, 3, 3, 2, i64, 2, nullptr, 0, ws, 8, nullptr), HKM_EWORKSPACE);
+    if (hkm_knn_workspace_bytes(1000, 100000) == 0 || hkm_knn_workspace_bytes(-1, 10) != 0) {
+        std::printf("FAIL knn workspace size\n");
+        ++failures;
+    }
+
+    // ---- Laplacian (S, N, lds, definition, mode, weighted, eps, L, ldl, degree)
+    EXPECT(hkm_laplacian_f32(nullptr, 4, 4, 0, 0, 0, 0.0f, f, 4, f, nullptr), HKM_EINVAL);
+    EXPECT(hkm_laplacian_f32(f, 4, 3, 0, 0, 0, 0.0f, f, 4, f, nullptr), HKM_EINVAL);
+    EXPECT(hkm_laplacian_f32(f, (int64_t(1) << 24) + 1, int64_t(1) << 25, 0, 0, 0, 0.0f, f, int64_t(1) << 25, f, nullptr),
+           HKM_EUNSUPPORTED);
+    EXPECT(hkm_laplacian_f64(d, 4, 3, 0, 0, 0, 0.0, d, 4, d, nullptr), HKM_EINVAL);
+
+    // ---- empty problems succeed without touching the device, and clear the message
+    EXPECT(hkm_widen_labels_i64(i32, 0, i64, nullptr), HKM_OK);
+    EXPECT(hkm_cdist_f32(nullptr, 0, 3, f, 4, 3, 3, f, 4, 1, nullptr), HKM_OK);
+    if (hkm_last_error()[0] != 0) {
+        std::printf("FAIL message not cleared: %s\n", hkm_last_error());
+        ++failures;
+    }
+
+    // ---- the measurement hooks with nothing recorded
+    float ms[4];
+    int32_t count = -1;
+    EXPECT(hkm_profile_enable(1), HKM_OK);
+    EXPECT(hkm_profile_collect(ms, 4, &count), HKM_OK);
+    EXPECT(hkm_profile_enable(0), HKM_OK);
+    if (count != 0) {
+        std::printf("FAIL profile count %d\n", count);
+        ++failures;
+    }
+
+    std::printf(failures ? "%d check(s) failed\n" : "all checks passed\n", failures);
+    return failures ? 1 : 0;
+}

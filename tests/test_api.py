@@ -259,6 +259,36 @@ def test_argument_validation_happens_on_the_host():
     assert err() == ""
 
 
+def test_validation_layer_under_address_sanitizer():
+    # heat_amd/csrc/Makefile, target asan-host: hkm_api.hip with its host code instrumented, linked with the
+    # objects of the ordinary build and driven by tests/host/hkm_api_check.cpp, which only makes calls the
+    # library refuses (or finishes) before anything reaches the device
+    import shutil
+    import subprocess
+
+    csrc = os.path.join(os.path.dirname(_native.lib_path()))
+    if not shutil.which("make") or not os.path.exists("/opt/rocm/bin/hipcc"):
+        pytest.skip("no toolchain to build the instrumented library with")
+    if not os.path.exists(os.path.join(csrc, "hkm_knn.o")):
+        pytest.skip("the objects of the ordinary build are not there (make -C heat_amd/csrc)")
+    run = subprocess.run(["make", "-C", csrc, "asan-host"], capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stdout[-2000:] + run.stderr[-2000:]
+    assert "all checks passed" in run.stdout
+    assert "AddressSanitizer" not in run.stdout + run.stderr
+
+
+def test_sizes_no_device_holds_are_refused():
+    lib = _native.load()
+    P = ctypes.c_void_p
+    good, ws = P(4096), P(1 << 20)
+    assert lib.hkm_assign_f32(good, (1 << 40) + 1, 3, 3, good, 8, 3, good, None, ws, 1 << 30, None) == _native.HKM_EUNSUPPORTED
+    assert "2^40" in lib.hkm_last_error().decode()
+    assert lib.hkm_assign_f32(good, 10, 1 << 21, 1 << 21, good, 1 << 20, 1 << 21, good, None, ws, 1 << 30, None) == _native.HKM_EUNSUPPORTED
+    assert lib.hkm_workspace_bytes((1 << 40) + 1, 3, 8, 1) == 0
+    assert lib.hkm_workspace_bytes(1 << 62, (1 << 31) - 1, (1 << 31) - 1, 3) == 0
+    assert lib.hkm_workspace_bytes(1 << 40, 3, 8, 3) > (1 << 40)
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_native, "_lib", None)
     monkeypatch.setattr(_native, "_LIB_PATH", "/nonexistent/libhkm.so")
