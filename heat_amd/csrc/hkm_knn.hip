@@ -240,12 +240,15 @@ __device__ __forceinline__ float knn_threshold(const float (&ld)[KL], int kcount
 // recomputed only after the lists may have changed.
 template <int KL>
 __device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (&li)[KL], float& thr,
-                                                     const floatx16& t, float qn, int64_t j0, int h, int64_t r_end,
-                                                     int kcount, int has_bound, float bd, unsigned bi) {
+                                                     const floatx16& t, float qn, int64_t j0, int64_t seen, int h,
+                                                     int64_t r_end, int kcount, int has_bound, float bd, unsigned bi) {
     // the last tile of a split (rows past the end) and the later passes of k > 16 (pairs ranked before the
     // bound) need every element looked at
     const bool edge = j0 + 32 > r_end || has_bound;
-    if (!edge) {
+    // While the lists are young nearly every tile holds a candidate for some lane of the wave and the test
+    // on the minimum is thirteen instructions for nothing: after `seen` rows a wave of 32 queries expects
+    // 32 * 32 * kcount / seen admissions per tile, and the test pays once that is below about 1.7.
+    if (!edge && seen >= int64_t(608) * kcount) {
         const float s = block_min16(t) + qn;
         const float dmin = s < 0.0f ? 0.0f : s;
         if (__builtin_amdgcn_ballot_w64(dmin < thr) == 0) return;
@@ -398,7 +401,7 @@ __global__ __launch_bounds__(256) void knn_mfma_kernel(
         floatx16 acc = MFMA32(av[0], qv[0], xnv);  // starts at the squared norms of its reference rows
 #pragma unroll
         for (int s = 1; s < H; ++s) acc = MFMA32(av[s], qv[s], acc);
-        knn_block_candidates<KL>(ld, li, thr, acc, qn, j0, h, r_end, kcount, has_bound, bd, bi);
+        knn_block_candidates<KL>(ld, li, thr, acc, qn, j0, j0 - r_begin, h, r_end, kcount, has_bound, bd, bi);
 #pragma unroll
         for (int s = 0; s < H; ++s) av[s] = an[s];
     }
@@ -508,7 +511,7 @@ __global__ __launch_bounds__(256) void knn_mfma_lds_kernel(
             for (int e = 0; e < 4; ++e)  // the accumulators start at the squared norms of their reference rows
                 acc = (g == 0 && e == 0) ? MFMA32(a[e], qv[0], xnv) : MFMA32(a[e], qv[4 * g + e], acc);
         }
-        knn_block_candidates<KL>(ld, li, thr, acc, qn, j0, h, r_end, kcount, has_bound, bd, bi);
+        knn_block_candidates<KL>(ld, li, thr, acc, qn, j0, j0 - r_begin, h, r_end, kcount, has_bound, bd, bi);
         if (more) stash(buf ^ 1);
         __syncthreads();
         buf ^= 1;
