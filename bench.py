@@ -613,6 +613,12 @@ def main() -> int:
     roof["kernel_launches_timed"] = len(kern)
     roof["step_ms_events"] = round(step_ms, 4)
     roof["sclk_mhz_under_load"] = sclk
+    if kernel in ("lloyd_mfma_resident", "mfma_resident"):
+        # which of the two launch geometries of the resident kernels ran, and whether the library measured
+        # that on this device (the fit loop asks it to, once per device) or took the default / HKM_POINT_BLOCKS
+        pb, tuned = _native.point_blocks(d)
+        roof["point_blocks_per_wave"] = pb
+        roof["point_blocks_measured_here"] = tuned
     if args.config in MFMA_BOUND:
         roof["mfma_alone_tflops_this_chip"] = round(mfma_alone_tflops(), 1)
     roof["traffic"] = None

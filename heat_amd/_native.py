@@ -19,7 +19,7 @@ from . import _f64_paths
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
-LIB_VERSION = 300  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
+LIB_VERSION = 301  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
 WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64 = 1, 2, 3, 4, 8, 16
 
@@ -43,6 +43,9 @@ SIGNATURES = {
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_tune_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
+                                          c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_point_blocks": (ctypes.c_int, [c_int32, c_void_p]),
     "hkm_shift_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "hkm_functional_value_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_cdist_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
@@ -290,6 +293,35 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Op
     buf = ws.get(need)
     check(load().hkm_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
                                     _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
+
+
+def tune_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: torch.Tensor,
+                    shift: torch.Tensor, ws: Workspace) -> int:
+    """One Lloyd step as ``lloyd_step`` runs it (same results), after which the library times the step in
+    both launch geometries of the resident matrix-core kernels and keeps the faster one for this device
+    (hkm_tune_lloyd_step_f32 in include/hkm.h).  WAITS for the device.  Returns the point blocks per wave
+    chosen, 0 where the shape has no such choice."""
+    _require_gpu(x, c, c_new, labels)
+    _require_rows(x, c, c_new)
+    _require_dense(c, c_new)
+    if x.dtype != torch.float32:
+        return 0
+    n, d = x.shape
+    k = c.shape[0]
+    buf = ws.get(workspace_bytes(n, d, k, WS_LLOYD))
+    rc = load().hkm_tune_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
+                                        _ptr(labels), _ptr(shift), None, _ptr(buf), buf.numel(), _stream())
+    if rc < 0:
+        check(rc)
+    return rc
+
+
+def point_blocks(d: int):
+    """(point blocks per wave a resident matrix-core kernel would use for d features now -- 0 if d has no
+    such kernel --, whether that was measured on the current device)."""
+    tuned = ctypes.c_int32(0)
+    pb = load().hkm_point_blocks(d, ctypes.cast(ctypes.pointer(tuned), c_void_p))
+    return int(pb), bool(tuned.value)
 
 
 def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],

@@ -27,6 +27,7 @@ shift.  If the loop goes on, the step enqueued ahead is re-issued from the recom
 
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -57,6 +58,13 @@ class LloydLoop:
         self.enqueued = 0  # steps handed to the stream
         self.done = 0      # steps whose results count
         self._plans = {}   # prepared calls, one per rotation of the buffers (and stream)
+        # Large fits on the resident matrix-core kernels: let the library measure once per device which of
+        # its two launch geometries this chip runs faster (the results do not depend on it).  The call is a
+        # step from c[0] into c[1] that the loop's own first step then repeats.
+        if kernel == "lloyd_mfma_resident" and n >= (1 << 20):
+            pb, tuned = _native.point_blocks(d)
+            if pb and d <= 32 and not tuned and not os.environ.get("HKM_POINT_BLOCKS"):
+                _native.tune_lloyd_step(self.x, self.c[0], self.c[1], self.lab[0], self.shift_host[0], self.ws)
 
     def _enqueue(self) -> None:
         j = self.enqueued

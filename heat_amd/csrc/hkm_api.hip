@@ -254,7 +254,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 300; }
+int hkm_version(void) { return 301; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -445,6 +445,59 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     }
     if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
     return rc;
+}
+
+int hkm_point_blocks(int32_t D, int32_t* tuned) {
+    if (tuned) *tuned = (env_point_blocks() == 0 && tuned_point_blocks() != 0) ? 1 : 0;
+    if (D <= 16 || D > 64) return 0;
+    return resident_point_blocks(resident_dp(D));
+}
+
+// The step itself, then -- where there is a choice -- the same step a few more times in either geometry
+// between events; the faster one is remembered for the device.  Every run writes the same bits into the
+// same outputs, so the caller's buffers hold the step's results whatever was measured.
+int hkm_tune_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new,
+                            int32_t K, int32_t* labels, float* shift, float* sse, void* ws, size_t ws_bytes,
+                            void* hip_stream) {
+    int rc = hkm_lloyd_step_f32(X, N, D, ldx, C, C_new, K, labels, shift, sse, ws, ws_bytes, hip_stream);
+    if (rc) return rc;
+    const bool choice = N > 0 && !small_eligible(D, K) && fused_eligible(D, K) && resident_dp(D) <= 32 &&
+                        env_point_blocks() == 0 && !(use_split_products() && split_eligible(D, K, true));
+    if (!choice) return 0;
+    hipStream_t st = static_cast<hipStream_t>(hip_stream);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+        return fail(HKM_EUNSUPPORTED, "hkm_tune_lloyd_step_f32 waits for the device and cannot run under stream capture");
+    hipEvent_t ev[2][2];
+    for (auto& pair : ev)
+        for (auto& e : pair)
+            if (hipEventCreate(&e) != hipSuccess) return fail(HKM_EHIP, "hipEventCreate failed");
+    const int WARM = 10, TIMED = 10;  // a chip that lowers its clock under a kernel does so within milliseconds
+    float ms[3] = {0.f, 0.f, 0.f};
+    for (int pb = 2; pb >= 1 && !rc; --pb) {
+        force_point_blocks(pb);
+        for (int i = 0; i < WARM + TIMED && !rc; ++i) {
+            if (i == WARM) (void)hipEventRecord(ev[pb - 1][0], st);
+            rc = hkm_lloyd_step_f32(X, N, D, ldx, C, C_new, K, labels, shift, sse, ws, ws_bytes, hip_stream);
+        }
+        (void)hipEventRecord(ev[pb - 1][1], st);
+    }
+    force_point_blocks(0);
+    if (!rc) {
+        for (int pb = 1; pb <= 2 && !rc; ++pb) {
+            if (hipEventSynchronize(ev[pb - 1][1]) != hipSuccess ||
+                hipEventElapsedTime(&ms[pb], ev[pb - 1][0], ev[pb - 1][1]) != hipSuccess)
+                rc = fail(HKM_EHIP, "timing the trial steps failed");
+        }
+    }
+    for (auto& pair : ev)
+        for (auto& e : pair) (void)hipEventDestroy(e);
+    if (rc) return rc;
+    // two point blocks unless one is clearly faster here (repeated timings differ by up to half a percent,
+    // and chips on which the two are within one percent of each other exist)
+    const int best = ms[1] < 0.99f * ms[2] ? 1 : 2;
+    set_tuned_point_blocks(best);
+    return best;
 }
 
 int hkm_shift_f32(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,

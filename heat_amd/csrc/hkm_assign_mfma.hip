@@ -11,6 +11,8 @@
 //
 // Arithmetic mirrors heat/spatial/distance.py:59-64: d2 = (|x|^2 + |c|^2) - 2*(x.c), clamped at 0;
 // first index wins ties (torch.min, heat/core/statistics.py:177).
+#include <atomic>
+
 #include "hkm_common.h"
 #include "hkm_mfma_util.h"
 
@@ -265,23 +267,50 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 // ------------------------------------------------------------------------------------------------
 static constexpr int FUSED_QBITS = 28;
 // Point blocks per wave of the resident kernels.  Up to 32 padded features there is a choice: TWO point
-// blocks against every centroid row a wave reads from LDS (eight waves per CU), or ONE with twelve waves.
-// Two halve the LDS reads per matrix instruction, and that decides on chips that lower their clock under
-// these kernels.  Measured on the 10M x 32 x 256 workload over a dozen chips of the same model: on those
-// that hold 2.39 GHz one point block is 2 % faster (one-sweep step 1.347 against 1.375 ms); on those that
-// do not it runs at 2.1-2.2 GHz and two point blocks at 2.3 GHz (1.430 against 1.391 ms).  Two is the
-// default -- never far from the better one; HKM_POINT_BLOCKS=1 selects the other.  Wider rows leave
-// registers for one point block only.
-__host__ __device__ constexpr int fused_threads(int pb) { return pb == 2 ? 512 : 768; }
+// blocks against every centroid row a wave reads from LDS (eight waves per CU in the one-sweep kernel), or ONE
+// with sixteen waves.  Two halve the LDS reads per matrix instruction, and that decides on chips that lower
+// their clock under these kernels.  Measured on the 10M x 32 x 256 workload over a dozen chips of the same
+// model: on those that hold 2.39 GHz one point block is 3 % faster (one-sweep kernel 1.326 against 1.366 ms);
+// on those that do not it runs at 2.1-2.2 GHz and two point blocks at 2.3 GHz (1.45 against 1.39 ms).  Both
+// geometries cut the rows into the same tiles of 512 and hand them to the same workgroups, so every output
+// of a step is bit for bit the same whichever runs.  Which one: HKM_POINT_BLOCKS (1 or 2) if set; else what
+// hkm_tune_lloyd_step_f32 measured on this device; else two.  Wider rows leave registers for one point
+// block only (twelve waves).
+__host__ __device__ constexpr int fused_threads(int pb, int dp) { return pb == 2 ? 512 : (dp <= 32 ? 1024 : 768); }
 
-static int resident_point_blocks(int dp) {
-    if (dp > 32) return 1;
+static const int TUNE_MAX_DEVICES = 64;
+static std::atomic<int> g_tuned_pb[TUNE_MAX_DEVICES];  // per device: 0 not measured, else 1 or 2
+static thread_local int t_forced_pb = 0;                // set by the tuning call around its trial launches
+
+void force_point_blocks(int pb) { t_forced_pb = pb; }
+
+void set_tuned_point_blocks(int pb) {
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < TUNE_MAX_DEVICES) g_tuned_pb[dev].store(pb);
+}
+
+int env_point_blocks() {
     const char* e = getenv("HKM_POINT_BLOCKS");
-    return (e && e[0] == '1' && e[1] == 0) ? 1 : 2;
+    if (e && (e[0] == '1' || e[0] == '2') && e[1] == 0) return e[0] - '0';
+    return 0;
+}
+
+int tuned_point_blocks() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TUNE_MAX_DEVICES) return 0;
+    return g_tuned_pb[dev].load();
+}
+
+int resident_point_blocks(int dp) {
+    if (dp > 32) return 1;
+    if (t_forced_pb) return t_forced_pb;
+    if (const int e = env_point_blocks()) return e;
+    if (const int t = tuned_point_blocks()) return t;
+    return 2;
 }
 
 template <int DP, int PB, bool VEC>
-__global__ __launch_bounds__(fused_threads(PB)) void lloyd_mfma_resident_kernel(
+__global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles,
     double* __restrict__ fsum, int32_t* __restrict__ fcnt, int32_t* __restrict__ flags,
@@ -771,8 +800,9 @@ size_t fused_lds_bytes(int32_t D, int32_t K) {
 }
 
 int fused_grid(int64_t N, int32_t D) {
-    const int pb = resident_point_blocks(resident_dp(D));
-    const int64_t tile_rows = int64_t(fused_threads(pb) / 64) * pb * 32;
+    const int dp = resident_dp(D);
+    const int pb = resident_point_blocks(dp);
+    const int64_t tile_rows = int64_t(fused_threads(pb, dp) / 64) * pb * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
     int64_t grid = num_cus();
     if (grid > FUSED_MAX_GRID) grid = FUSED_MAX_GRID;
@@ -784,7 +814,7 @@ template <int DP, int PB, bool VEC>
 static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                           int64_t ldc, int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt,
                           int32_t* flags, hipStream_t st) {
-    constexpr int THREADS = fused_threads(PB);
+    constexpr int THREADS = fused_threads(PB, DP);
     const int64_t tile_rows = int64_t(THREADS / 64) * PB * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
     const int grid = fused_grid(N, D);

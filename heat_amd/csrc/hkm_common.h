@@ -166,6 +166,14 @@ int launch_assign_mfma_stream(const float* X, int64_t N, int32_t D, int64_t ldx,
 bool fused_eligible(int32_t D, int32_t K);
 size_t fused_lds_bytes(int32_t D, int32_t K);
 int fused_grid(int64_t N, int32_t D);
+// point blocks per wave of the resident matrix-core kernels (hkm_assign_mfma.hip): the choice for a padded
+// width, its sources (environment, what the tuning call measured on the current device), and the tuning
+// call's handles
+int resident_point_blocks(int dp);
+int env_point_blocks();
+int tuned_point_blocks();
+void force_point_blocks(int pb);
+void set_tuned_point_blocks(int pb);
 int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                                int32_t K, int64_t ldc, int32_t* labels, float* min_d2, double* fsum,
                                int32_t* fcnt, int32_t* flags, hipStream_t st);

@@ -365,6 +365,23 @@ int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, i
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 
 /*
+ * The resident matrix-core kernels (16 < D <= 32) come in two launch geometries -- two point blocks per wave,
+ * or one with twice the waves -- that produce the same bits and differ in speed by a few percent either way,
+ * depending on the clock the individual chip holds under them.  No counterpart in the reference.
+ * hkm_tune_lloyd_step_f32: hkm_lloyd_step_f32 with the same arguments and the same results, which -- where the
+ *   shape has the choice and HKM_POINT_BLOCKS is not set -- then runs the same step twenty more times in
+ *   either geometry, WAITS for the device, and remembers the faster geometry for the current device until the
+ *   process ends.  Returns the point blocks chosen (1 or 2), 0 if the shape has no choice, or a negative
+ *   error; refused under stream capture.  Not calling it leaves the default (two).
+ * hkm_point_blocks: the point blocks per wave a call with D features would use now (0: D has no resident
+ *   kernel); *tuned (if not NULL) tells whether that came from a measurement on the current device.
+ */
+int hkm_tune_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new,
+                            int32_t K, int32_t* labels, float* shift, float* sse, void* ws, size_t ws_bytes,
+                            void* hip_stream);
+int hkm_point_blocks(int32_t D, int32_t* tuned);
+
+/*
  * Timing of the dominant kernel, for benchmarks (no counterpart in the reference).  After
  * hkm_profile_enable(1) on the calling thread, every hkm_assign_f32 / hkm_assign_static_f32 /
  * hkm_lloyd_step_f32 call of that thread records one pair of events on its stream, right before and right

@@ -38,7 +38,7 @@ int main() {
     void* const ws = reinterpret_cast<void*>(uintptr_t(1) << 20);
     const size_t big = size_t(1) << 30;
 
-    if (hkm_version() < 300) {
+    if (hkm_version() < 301) {
         std::printf("FAIL version %d\n", hkm_version());
         ++failures;
     }
@@ -126,6 +126,16 @@ int main() {
         std::printf("FAIL message not cleared: %s\n", hkm_last_error());
         ++failures;
     }
+
+    // ---- the launch-geometry choice of the resident kernels: queries and refusals only
+    int32_t tuned = -1;
+    if (hkm_point_blocks(8, &tuned) != 0 || hkm_point_blocks(100, nullptr) != 0 || hkm_point_blocks(48, &tuned) != 1 ||
+        tuned != 0) {
+        std::printf("FAIL hkm_point_blocks\n");
+        ++failures;
+    }
+    EXPECT(hkm_tune_lloyd_step_f32(nullptr, 10, 32, 32, f, f + 4096, 8, i32, f, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_tune_lloyd_step_f32(f, 10, 32, 32, f, f + 4096, 8, i32, f, nullptr, ws, 16, nullptr), HKM_EWORKSPACE);
 
     // ---- the measurement hooks with nothing recorded
     float ms[4];

@@ -230,8 +230,7 @@ def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
 
 @pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (768, 17, 5)])
 def test_one_point_block_per_wave_gives_the_same_labels(cuda, n, d, k, monkeypatch):
-    # HKM_POINT_BLOCKS=1 (16 < D <= 32): another launch geometry of the same kernels -- labels and minima
-    # bit for bit, centroids up to the grouping of the exact per-workgroup partial sums
+    # HKM_POINT_BLOCKS=1 (16 < D <= 32): another launch geometry of the same kernels
     print(f"point blocks n={n} d={d} k={k}", flush=True)
     x, _ = _data(n, d, k, seed=3 * n + d)
     c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(9))[:k]].contiguous()
@@ -252,9 +251,41 @@ def test_one_point_block_per_wave_gives_the_same_labels(cuda, n, d, k, monkeypat
     two = run()
     monkeypatch.setenv("HKM_POINT_BLOCKS", "1")
     one = run()
+    # both geometries cut the rows into the same tiles for the same workgroups: every output bit for bit
     assert torch.equal(one[0], two[0]) and torch.equal(one[1], two[1]) and torch.equal(one[2], two[2])
-    assert orc.rel_err_centers(one[3], two[3]) <= 2e-7
-    assert abs(one[4] - two[4]) <= 1e-6 * max(abs(two[4]), 1e-30)
+    assert torch.equal(one[3], two[3]) and one[4] == two[4]
+
+
+def test_tuning_call_is_a_step_and_settles_on_a_geometry(cuda, monkeypatch):
+    monkeypatch.delenv("HKM_POINT_BLOCKS", raising=False)
+    n, d, k = 300000, 32, 64
+    x, _ = _data(n, d, k, seed=77)
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(2))[:k]].contiguous()
+    xs, cs = x.to(cuda), c0.to(cuda)
+    ws = _native.Workspace(cuda)
+    lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+    cn = torch.empty_like(cs)
+    shift = torch.empty((), device=cuda)
+    _native.lloyd_step(xs, cs, cn, lab, shift, None, ws)
+    torch.cuda.synchronize()
+    want = (lab.clone(), cn.clone(), float(shift))
+    lab.zero_(), cn.zero_()
+    chosen = _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws)
+    torch.cuda.synchronize()
+    assert chosen in (1, 2)
+    assert _native.point_blocks(d) == (chosen, True)
+    assert torch.equal(lab, want[0]) and torch.equal(cn, want[1]) and float(shift) == want[2]
+    # shapes without the choice: wider rows, the narrow kernels
+    assert _native.point_blocks(48) == (1, True) or _native.point_blocks(48) == (1, False)
+    assert _native.point_blocks(8)[0] == 0
+    x8 = torch.rand(5000, 8).to(cuda)
+    c8 = x8[:16].contiguous()
+    assert _native.tune_lloyd_step(x8, c8, torch.empty_like(c8), torch.empty((5000,), dtype=torch.int32, device=cuda),
+                                   shift, ws) == 0
+    # the environment decides where it is set
+    monkeypatch.setenv("HKM_POINT_BLOCKS", "1")
+    assert _native.point_blocks(d) == (1, False)
+    assert _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws) == 0
 
 
 def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
