@@ -521,7 +521,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 }
 
 // One workgroup of 1024 threads finishes the step.  Thread (j, s) adds the partial rows g = j, j+J,
-// ... of slot s in ascending order (8 independent loads in flight, additions still in row order);
+// ... of slot s in ascending order (up to 32 independent loads in flight, additions still in row order);
 // thread (0, s) then adds the J strided sums in ascending j.  The order depends only on (G, slots).
 __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
     const double* __restrict__ part, int G, int K, int D, const float* __restrict__ C_old,
@@ -529,23 +529,29 @@ __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
     float* __restrict__ shift, float* __restrict__ sse_out, int have_sse, int spad) {
     __shared__ double strided[1024];
     __shared__ double tot[256];
-    __shared__ double red[1024];
+    __shared__ double red[256];
     const int tid = threadIdx.x;
     const int slots = K * (D + 1);
     const int nslot = slots + 1;  // last = sum of min d2
     const int J = 1024 / spad;  // spad = nslot: as many row groups as fit the workgroup
     const int s = tid % spad, j = tid / spad;
+    // the old coordinate this thread will compare its mean with (K * D <= 240 < 1024: one per thread), asked
+    // for before the partial rows so that its latency hides behind theirs
+    float c_old = 0.0f;
+    if (C_old && tid < K * D) c_old = C_old[tid];
     double v = 0.0;
     if (j < J && s < nslot && (s < slots || have_sse)) {
-        int g = j;
-        for (; g + 7 * J < G; g += 8 * J) {
-            double t[8];
+        // a thread's rows are requested 32 at a time, the last batch with the rows beyond G left out: the
+        // kernel is nothing but the latency of these reads, and a few hundred rows should cost one round
+        // trip, not one per eight rows and one per row of the remainder
+        for (int g = j; g < G; g += 32 * J) {
+            double t[32];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) t[u] = part[int64_t(g + u * J) * nslot + s];
+            for (int u = 0; u < 32; ++u) t[u] = g + u * J < G ? part[int64_t(g + u * J) * nslot + s] : 0.0;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v += t[u];
+            for (int u = 0; u < 32; ++u)
+                if (g + u * J < G) v += t[u];
         }
-        for (; g < G; g += J) v += part[int64_t(g) * nslot + s];
     }
     strided[tid] = v;
     __syncthreads();
@@ -563,20 +569,26 @@ __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
         const float c = float(tot[k * (D + 1) + d] / cnt);
         C_new[int64_t(k) * ldcn + d] = c;
         if (C_old) {
-            const float df = C_old[int64_t(k) * D + d] - c;
+            const float df = c_old - c;  // i == tid here
             sq += double(df * df);
         }
         if (d == 0 && counts) counts[k] = n;
     }
-    red[tid] = sq;
+    // The pairwise tree over 1024 slots (t += t + w for w = 512 ... 1), of which only the first K * D <= 240
+    // are not zero: the two widest levels add zeros and are left out, two levels go through LDS, the last
+    // six stay inside the first wave.  Same association, same bits.
+    if (tid < 256) red[tid] = sq;
     __syncthreads();
-    for (int w = 512; w > 0; w >>= 1) {
-        if (tid < w) red[tid] += red[tid + w];
-        __syncthreads();
-    }
-    if (tid == 0) {
-        if (shift) *shift = float(red[0]);
-        if (sse_out && have_sse) *sse_out = float(tot[slots]);
+    if (tid < 128) red[tid] += red[tid + 128];
+    __syncthreads();
+    if (tid < 64) {
+        double r = red[tid] + red[tid + 64];
+#pragma unroll
+        for (int w = 32; w > 0; w >>= 1) r += __shfl_down(r, w);
+        if (tid == 0) {
+            if (shift) *shift = float(r);
+            if (sse_out && have_sse) *sse_out = float(tot[slots]);
+        }
     }
 }
 
