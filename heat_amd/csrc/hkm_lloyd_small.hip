@@ -169,6 +169,28 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     int* wlab = reinterpret_cast<int*>(wacc_all + NW * slots) + wave * (64 * PPT);  // ACC==3: [4][16*PPT]
     float* wstage = stage + wave * NV * 256;
 
+    const int64_t groups = (N + PPT - 1) / PPT;
+    const int64_t full = (vec & 1) ? N / PPT : 0;  // groups served by the 16-byte vector path
+    const int64_t stride = int64_t(gridDim.x) * T;
+    const int64_t wg0 = int64_t(blockIdx.x) * T;
+    int64_t base = wg0;
+    // A wave's 64 groups are NV*1024 contiguous bytes: fetched as NV fully coalesced 16-byte
+    // loads per lane, then redistributed through a wave-private LDS buffer so that every lane
+    // ends up with its own PPT consecutive points.  The first rounds are requested here, before the
+    // centroids are staged: for a matrix of a few megabytes the kernel is two memory latencies long,
+    // and this way they overlap.
+    constexpr int PF = 3;  // rounds in flight: enough bytes per CU to cover the HBM latency
+    floatx4 nxt[PF][NV];
+    const float* wsrc = X + (base + wave * 64) * (PPT * D) + lane * 4;
+    const int64_t rstride = stride * (PPT * D);
+#pragma unroll
+    for (int f = 0; f < PF; ++f) {
+        if (base + f * stride + T <= full) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + f * rstride + v * 256, stream);
+        }
+    }
+
     for (int i = tid; i < K * SC; i += T) {
         const int r = i / SC, c = i - r * SC;
         sC[i] = c < D ? C[int64_t(r) * ldc + c] : 0.f;  // scaled by -2 once the norms are taken
@@ -205,9 +227,6 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     }
 
     double sse = 0.0;
-    const int64_t groups = (N + PPT - 1) / PPT;
-    const int64_t full = (vec & 1) ? N / PPT : 0;  // groups served by the 16-byte vector path
-    const int64_t stride = int64_t(gridDim.x) * T;
 
     // ACC == 1: the additions of a round are deferred to the NEXT round and interleaved with its
     // arithmetic, so that the LDS read -> add -> write round trips of the PPT points (which must stay
@@ -399,23 +418,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     // Main loop, identical trip count for every lane of the workgroup.  Rounds in which the whole
     // workgroup lies inside the vector-loadable range take the fast path; the next round's rows are
     // requested before the current round is processed.
-    const int64_t wg0 = int64_t(blockIdx.x) * T;
-    int64_t base = wg0;
     {
-        // A wave's 64 groups are NV*1024 contiguous bytes: fetched as NV fully coalesced 16-byte
-        // loads per lane, then redistributed through a wave-private LDS buffer so that every lane
-        // ends up with its own PPT consecutive points.
-        constexpr int PF = 3;  // rounds in flight: enough bytes per CU to cover the HBM latency
-        floatx4 nxt[PF][NV];
-        const float* wsrc = X + (base + wave * 64) * (PPT * D) + lane * 4;
-        const int64_t rstride = stride * (PPT * D);
-#pragma unroll
-        for (int f = 0; f < PF; ++f) {
-            if (base + f * stride + T <= full) {
-#pragma unroll
-                for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + f * rstride + v * 256, stream);
-            }
-        }
         // The loop is unrolled PF times so that each round's buffer is a fixed set of registers: a
         // register rotation would make every round wait for ALL outstanding loads.
         bool more = base + T <= full;
