@@ -24,7 +24,7 @@ namespace hkm {
 // B-operand registers.  No barrier inside the tile loop.
 //
 // On this hardware every VALU instruction takes issue time away from the fp32 MFMA pipe (there is no
-// co-execution), so the epilogue is kept to fewer than three VALU instructions per distance:
+// co-execution), so the epilogue is kept short (about 1.3 VALU instructions per distance):
 //   * LDS row k holds -2*c_k (zero-padded to DP; scaling by -2 is exact) and a separate LDS array the
 //     squared norms |c_k|^2; the accumulators of a block START at the norms of their centroid rows
 //     (the C operand of the first MFMA, four 16-byte LDS reads, no vector instruction), so they end

@@ -48,7 +48,7 @@ __device__ __forceinline__ floatx16 load_cn16(const float* cn16) {
 }
 
 // Minimum and first argmin over the 16 distances a lane holds of one centroid block, merged into the
-// running (m, mi).  The minimum is a tree of three-input minima (8 instructions, no dependence on
+// running (m, mi).  The minimum is a tree of three-input minima (9 instructions, no dependence on
 // compare results); only lanes whose block minimum improves the running one look for its position,
 // by equality from the last register down so that the first one wins.  Strict '<' keeps the earlier
 // block on ties.  NaNs never win.
