@@ -101,8 +101,10 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         if (assign_kind(D, K) == ASSIGN_MFMA_STREAM)
             w.keys = reinterpret_cast<unsigned long long*>(take(size_t(N < 1 ? 1 : N) * sizeof(unsigned long long)));
     }
-    if ((flags & HKM_WS_UPDATE) && !(flags & HKM_WS_F64) && small_eligible(D, K))
+    if ((flags & HKM_WS_UPDATE) && !(flags & HKM_WS_F64) && small_eligible(D, K)) {
         w.small_part = reinterpret_cast<double*>(take(size_t(SMALL_MAX_GRID) * (size_t(K) * (D + 1) + 1) * sizeof(double)));
+        w.small_flags = reinterpret_cast<int32_t*>(take(size_t(SMALL_MAX_GRID) * sizeof(int32_t)));
+    }
     if (flags & HKM_WS_UPDATE) {
         const size_t elem = (flags & HKM_WS_F64) ? sizeof(double) : sizeof(float);
         const UpdateGeom g = update_geom(N, D, K, int32_t(elem));
@@ -229,7 +231,7 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
     switch (assign_kind(D, K)) {
         case ASSIGN_VALU:
             if (small_eligible(D, K))
-                return launch_small(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, 0, st);
+                return launch_small(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, 0, nullptr, st);
             return launch_assign_valu(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_RESIDENT:
             if (use_split_products() && split_eligible(D, K, false))
@@ -423,7 +425,8 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
     if (small_eligible(D, K) && N > 0) {
         // one sweep over X: labels + private per-lane sums, then a single-workgroup finish
-        if ((rc = launch_small(X, N, D, ldx, C, K, D, labels, nullptr, w.small_part, sse ? 3 : 1, st))) return rc;
+        if ((rc = launch_small(X, N, D, ldx, C, K, D, labels, nullptr, w.small_part, sse ? 3 : 1, w.small_flags, st)))
+            return rc;
         return launch_small_finalize(w.small_part, small_grid(N, D, K), K, D, C, C_new, D, nullptr, shift, sse, st);
     }
     if (fused_eligible(D, K) && N > 0) {

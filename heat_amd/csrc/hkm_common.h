@@ -115,6 +115,7 @@ struct Workspace {
     float* min_d2;      // [N] (only with the SSE flag)
     double* shift_part; // [ceil(K*D/64)] per-block shares of the squared centroid shift
     double* small_part; // [SMALL_MAX_GRID][K*(D+1)+1] partial rows of the one-sweep small-D step
+    int32_t* small_flags;  // [SMALL_MAX_GRID] 1 = this workgroup's integer sums cannot be trusted
     double* fsum;       // [FUSED_MAX_GRID][K][D] fp64 partial sums of the one-sweep MFMA step
     int32_t* fcnt;      // [FUSED_MAX_GRID][K]
     int32_t* fflags;    // [FUSED_MAX_GRID] 1 = this workgroup's sums may depend on the addition order
@@ -183,7 +184,7 @@ int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const
 bool small_eligible(int32_t D, int32_t K);
 int small_grid(int64_t N, int32_t D, int32_t K);
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
-                 int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
+                 int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode, int32_t* flags,
                  hipStream_t st);
 int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, const float* C_old,
                           float* C_new, int64_t ldcn, int64_t* counts, float* shift, float* sse,

@@ -1,19 +1,28 @@
 // One-sweep Lloyd step for small feature counts (D <= 8) and small K*(D+1): X is read from HBM
 // exactly once per iteration (4D bytes per point) and only the labels are written (4 bytes).
 //
-// Assignment: a lane owns PPT consecutive points in registers; the centroids (scaled by -2, which is
-// exact) and their squared norms sit in LDS and are read as wave-wide broadcasts.  The quadratic
-// expansion of heat/spatial/distance.py:59-64, d2 = |x|^2 + |c|^2 - 2 x.c, is evaluated as a chain of
-// D fused multiply-adds that starts at |c|^2; |x|^2, the same for every centroid, is added to the
-// minimum only.  First index wins ties (torch.min, heat/core/statistics.py:177).  The clamp at 0 is
-// applied lazily: a negative minimum (a point that coincides with a centroid up to rounding)
-// triggers a rescan with the clamp applied to every candidate, so the result equals clamping first.
+// Assignment: a lane owns PPT consecutive points in registers; the centroids and their squared norms are
+// wave-uniform operands -- LDS broadcasts of rows scaled by -2 (exact), or, where a row is one scalar load,
+// scalar registers filled straight from C (scan_centroids_sload).  The quadratic expansion of
+// heat/spatial/distance.py:59-64, d2 = |x|^2 + |c|^2 - 2 x.c, is evaluated as a chain of D fused
+// multiply-adds that starts at |c|^2; |x|^2, the same for every centroid, is added to the minimum only.
+// First index wins ties (torch.min, heat/core/statistics.py:177).  The clamp at 0 is applied lazily: a
+// negative minimum (a point that coincides with a centroid up to rounding) triggers a rescan with the
+// clamp applied to every candidate, so the result equals clamping first.
 //
-// Update (heat/cluster/kmeans.py:76-103) without atomics, three strategies with a fixed summation order:
+// Update (heat/cluster/kmeans.py:76-103), per-cluster sums whose value does not depend on the order in
+// which the hardware happens to run things:
 //   K*(D+1) <= 48: every lane owns a private fp32 column per (cluster, coordinate) in LDS and adds
 //     its own points in program order; the read-add-write round trips of a round are deferred to the
 //     next round and interleaved with its arithmetic.  At the end lanes' columns are added in a fixed
 //     fp64 tree.
+//   otherwise, large N: every coordinate is added as a 64-bit integer, rint(x * 2^(32 - Ec)) with 2^Ec
+//     the bound of the step's largest centroid coordinate, to one of several copies of an integer table
+//     in LDS with ds_add_u64.  Integer addition is exact, so the atomics may land in any order; it costs
+//     two vector instructions per coordinate, a fraction of the assignment.  A workgroup that meets a row
+//     outside the scale's range (|x| >= 2^(Ec + headroom), inf, NaN) or has no usable scale raises a flag,
+//     and a second launch -- the same sweep with one of the two ordered strategies below, which returns at
+//     once when no flag is up -- redoes the step.
 //   otherwise, K <= 32: the sums are a matrix product, (one-hot labels)^T x [X, 1], evaluated on the
 //     fp32 matrix cores with v_mfma_f32_16x16x4_f32 over the wave's points of the round (read back from
 //     the staging buffer); the fp32 accumulators move into the wave's private fp64 row in LDS every
@@ -41,12 +50,27 @@ struct SmallCfg {
     // points per lane so that a lane's chunk is a whole number of 16-byte vectors
     static constexpr int PPT = (D % 4 == 0) ? 2 : (D % 2 == 0) ? 2 : 4;
     static constexpr int SC = (D + 1 + 3) / 4 * 4;  // LDS centroid row: D coords, |c|^2, pad
+    // Centroid rows by scalar loads instead of LDS broadcasts, where a row is ONE scalar load (1, 4 or 8
+    // values): measured on 30-100 M rows with 16-100 clusters, the step is then 4-26 % faster; rows of
+    // 2, 3, 5 or 7 values take several loads per centroid and run 6-10 % slower that way.
+    static constexpr bool SLOAD = D == 1 || D == 4 || D == 8;
 };
 
 bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
 static constexpr int SMALL_T = 256;
+
+// ---- the integer accumulation (acc_mode 4) ----
+// A coordinate is added as the integer rint(x * 2^(QB - Ec)), where 2^Ec bounds the largest centroid
+// coordinate of the step: integer additions are exact, so LDS atomics may deliver them in any order.
+static constexpr int SMALL_QB = 32;
+// copies of the accumulator table per workgroup (a lane uses copy lane % R): fewer lanes of one
+// instruction meet at one address
+__host__ __device__ constexpr int small_replicas(int K) { return K <= 16 ? 16 : K <= 32 ? 8 : 4; }
+// row stride of the table in 64-bit words, odd so that the rows of different clusters spread over the banks
+__host__ __device__ constexpr int small_int_stride(int D) { return (D + 1) | 1; }
+
 // LDS of one workgroup; acc_mode as in the kernel (0 labels only, 1 lane columns, 2 wave rows by the
-// DPP tree, 3 wave rows by the matrix cores)
+// DPP tree, 3 wave rows by the matrix cores, 4 integer tables)
 static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
     const int sc = (D + 1 + 3) / 4 * 4, nv = ppt * D / 4, slots = K * (D + 1);
@@ -54,11 +78,32 @@ static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
            (acc_mode == 2   ? size_t(SMALL_T / 64) * slots * sizeof(double)
             : acc_mode == 3 ? size_t(SMALL_T / 64) * (slots * sizeof(double) + 64 * ppt * sizeof(int))
             : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float)
+            : acc_mode == 4 ? size_t(small_replicas(K)) * K * small_int_stride(D) * 8 + 16
                             : 0);
 }
-// per-lane LDS columns while they fit (slots * 1 KB), the matrix-core product up to 32 clusters, the
-// DPP tree otherwise
-static int small_acc_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : K <= 32 ? 3 : 2; }
+// The ordered strategies: per-lane LDS columns while they fit (slots * 1 KB), the matrix-core product up
+// to 32 clusters, the DPP tree otherwise.
+static int small_ordered_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : K <= 32 ? 3 : 2; }
+
+// HKM_SMALL_SUMS = ordered | integer (looked up per call) overrides the choice by size; tests use it
+static int small_sums_override() {
+    const char* e = getenv("HKM_SMALL_SUMS");
+    if (!e) return 0;
+    return e[0] == 'o' ? 1 : e[0] == 'i' ? 2 : 0;
+}
+
+// Beyond 48 slots the ordered strategies cost more than the assignment itself; the integer tables cost a
+// fraction of it but need a second launch (a re-run in the ordered way that normally returns at once), so
+// they start where a launch no longer shows.
+bool small_integer_sums(int64_t N, int32_t D, int32_t K) {
+    if (K * (D + 1) <= 48) return false;
+    const int o = small_sums_override();
+    if (o) return o == 2;
+    return N >= (K > 32 ? (int64_t(1) << 17) : (int64_t(1) << 20));
+}
+static int small_acc_mode(int64_t N, int32_t D, int32_t K) {
+    return small_integer_sums(N, D, K) ? 4 : small_ordered_mode(D, K);
+}
 
 int small_grid(int64_t N, int32_t D, int32_t K) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
@@ -67,7 +112,7 @@ int small_grid(int64_t N, int32_t D, int32_t K) {
     // accumulating variant's LDS says so: a grid beyond that would run in two uneven batches), then
     // grid-stride
     int64_t want = (groups + SMALL_T - 1) / SMALL_T;
-    int64_t per_cu = int64_t(160 * 1024) / int64_t(small_lds_bytes(D, K, small_acc_mode(D, K)));
+    int64_t per_cu = int64_t(160 * 1024) / int64_t(small_lds_bytes(D, K, small_acc_mode(N, D, K)));
     if (per_cu > 4) per_cu = 4;
     if (per_cu < 1) per_cu = 1;
     int64_t cap = int64_t(num_cus()) * per_cu;
@@ -121,6 +166,48 @@ __device__ __forceinline__ void scan_centroids(const float* sC, int k0, int k1,
     }
 }
 
+// The same scan with the centroid rows fetched straight from the caller's C at wave-uniform addresses:
+// the compiler turns such reads into scalar loads, so a row arrives in scalar registers through the scalar
+// cache and costs neither LDS bandwidth (a broadcast read still returns 64 copies) nor vector registers.
+// The rows in C carry no factor -2, so the chain runs on t = x.c - |c|^2 / 2 and looks for the LARGEST t:
+// every intermediate value is the other chain's divided by -2 (a power of two commutes with rounding), so
+// the comparisons, the ties and -2 t_max = the minimum are the same bits.  |c|^2 still comes from LDS.
+template <int D, int PPT, bool CLAMP>
+__device__ __forceinline__ void scan_centroids_sload(const float* __restrict__ C, int64_t ldc, const float* sC,
+                                                     int k0, int k1, const float (&x)[PPT][D],
+                                                     const float (&xn)[PPT], float (&m)[PPT], int (&mi)[PPT]) {
+    constexpr int SC = SmallCfg<D>::SC;
+    // m is a minimum of distances on entry and on return; in between the plain scan tracks the largest t
+    // (= m / -2, exact both ways), the clamped one the smallest clamped distance
+    float best[PPT];
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) best[p] = CLAMP ? m[p] : -0.5f * m[p];
+#pragma unroll(PPT == 2 ? 4 : 2)
+    for (int k = k0; k < k1; ++k) {
+        const float* ck = C + int64_t(k) * ldc;
+        float c[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) c[d] = ck[d];
+        const float hcn = -0.5f * sC[k * SC + D];
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            float t = fmaf(x[p][0], c[0], hcn);
+#pragma unroll
+            for (int d = 1; d < D; ++d) t = fmaf(x[p][d], c[d], t);
+            if (CLAMP) {
+                const float dist = fmaxf(fmaf(-2.0f, t, xn[p]), 0.0f);
+                mi[p] = dist < best[p] ? k : mi[p];
+                best[p] = fminf(best[p], dist);
+            } else {
+                mi[p] = t > best[p] ? k : mi[p];
+                best[p] = fmaxf(best[p], t);
+            }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) m[p] = CLAMP ? best[p] : -2.0f * best[p];
+}
+
 // The same scan with the centroids in registers that are uniform over the wave (KT rows, those
 // beyond K hold |c|^2 = +inf and never win): no LDS reads and no loop in the round.
 template <int D, int PPT, int KT, bool CLAMP>
@@ -142,13 +229,18 @@ __device__ __forceinline__ void scan_centroids_reg(const float (&cs)[KT][D + 1],
 }
 
 // ACC: 0 = labels only, 1 = per-lane private LDS columns, 2 = DPP wave tree + per-wave fp64 rows,
-//      3 = matrix-core product (one-hot labels x points) + per-wave fp64 rows
-// KT: 0 = centroids read from LDS in a loop over K; otherwise K <= KT and they sit in registers
+//      3 = matrix-core product (one-hot labels x points) + per-wave fp64 rows,
+//      4 = integer tables in LDS, added to with atomics
+// KT: 0 = centroid rows fetched in a loop over K; otherwise K <= KT and they sit in registers
+// flags / aux: ACC == 4 writes flags[workgroup] = 1 if its sums cannot be trusted (a row too large for the
+//   integer scale, or no usable scale), aux = how many bits above the largest centroid coordinate a row
+//   may reach.  The ordered modes, given flags, are the re-run after an ACC == 4 launch of aux workgroups:
+//   they return at once unless one of those raised its flag.
 template <int D, int ACC, bool WANT_MIN, bool WANT_SSE, int KT>
 __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const float* __restrict__ X, int64_t N, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2,
-    double* __restrict__ part, int vec) {
+    double* __restrict__ part, int vec, int32_t* __restrict__ flags, int aux) {
     constexpr int T = SMALL_T;
     constexpr int PPT = SmallCfg<D>::PPT;
     constexpr int SC = SmallCfg<D>::SC;
@@ -166,6 +258,17 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     double* wacc = wacc_all + wave * slots;
+    // ACC == 4: [R][K][LDI] 64-bit integers (column D of a row counts its points), then the bits of the
+    // largest |centroid coordinate| and the workgroup's flag
+    constexpr int LDI = small_int_stride(D);
+    const int nrep = small_replicas(K);
+    unsigned long long* iacc = reinterpret_cast<unsigned long long*>(after);
+    int* imeta = reinterpret_cast<int*>(iacc + nrep * K * LDI);
+    if ((ACC == 2 || ACC == 3) && flags) {
+        int any = 0;
+        for (int g = tid; g < aux; g += T) any |= flags[g];
+        if (!__syncthreads_or(any)) return;
+    }
     int* wlab = reinterpret_cast<int*>(wacc_all + NW * slots) + wave * (64 * PPT);  // ACC==3: [4][16*PPT]
     float* wstage = stage + wave * NV * 256;
 
@@ -199,7 +302,18 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         for (int i = tid; i < NW * slots; i += T) wacc_all[i] = 0.0;
     if (ACC == 1)
         for (int i = tid; i < (slots + D + 1) * T; i += T) cols[i] = 0.f;
+    if (ACC == 4) {
+        for (int i = tid; i < nrep * K * LDI; i += T) iacc[i] = 0ull;
+        if (tid < 2) imeta[tid] = 0;
+    }
     __syncthreads();
+    if (ACC == 4) {
+        // bits of non-negative floats order like integers; NaN and inf end up on top
+        int mx = 0;
+        for (int i = tid; i < K * SC; i += T) mx = max(mx, __float_as_int(sC[i]) & 0x7fffffff);
+        atomicMax(&imeta[0], mx);
+        __syncthreads();  // the scaling below overwrites what the maximum was taken of
+    }
     for (int r = tid; r < K; r += T) {
         float s = 0.f;
 #pragma unroll
@@ -209,6 +323,24 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         for (int d = 0; d < D; ++d) sC[r * SC + d] *= -2.0f;  // exact
     }
     __syncthreads();
+
+    // ACC == 4: 2^Ec > every |centroid coordinate|.  A coordinate x enters as the 64-bit pattern of
+    // fma(x, 2^(QB - Ec), 1.5 * 2^52): for |x| < 2^(Ec + 51 - QB) that is the pattern of the constant plus
+    // the integer rint(x * 2^(QB - Ec)), so the sum of n patterns minus n times the constant's is the exact
+    // sum of the integers (all modulo 2^64; the true sum fits because aux also accounts for the number of
+    // rows a workgroup adds).  A row is inside the range if |x|^2 < 2^(2 (Ec + aux)).
+    double iscale = 0.0, iquantum = 0.0;
+    float xn_limit = 0.f;
+    bool bad = false;
+    if (ACC == 4) {
+        const int ebits = (imeta[0] >> 23) & 0xff;
+        const int Ec = ebits - 127 + 1;
+        bad = ebits == 0 || ebits == 255;  // all centroids zero (or denormal), or a non-finite one: no scale
+        iscale = __hiloint2double((1023 + SMALL_QB - Ec) << 20, 0);
+        iquantum = __hiloint2double((1023 - SMALL_QB + Ec) << 20, 0);
+        const int e2 = 2 * (Ec + aux);
+        xn_limit = e2 > 127 ? HKM_INF : e2 < -126 ? 0.f : __int_as_float((e2 + 127) << 23);
+    }
 
     // 0 < KT <= 8: one copy of the centroid table per wave, in scalar registers
     // KT = 16 / 32 (ACC == 3 only): one / two blocks of 16 clusters in the matrix-core accumulation
@@ -294,12 +426,14 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             rmw_read(1, r);
         }
         if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
+        else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, 0, kh, x, xn, m, mi);
         else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
         if (ACC == 1) {
             rmw_write(PPT == 4 ? 1 : 0, r);
             rmw_read(PPT == 4 ? 2 : 1, r);
         }
         if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
+        else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, kh, K, x, xn, m, mi);
         else scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
         if (ACC == 1 && PPT == 4) {
             rmw_write(2, r);
@@ -319,6 +453,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 mi[p] = 0;
             }
             if constexpr (REGC) scan_centroids_reg<D, PPT, KR, true>(cs, 0, KR, x, xn, m, mi);
+            else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, true>(C, ldc, sC, 0, K, x, xn, m, mi);
             else scan_centroids<D, PPT, true>(sC, 0, K, x, xn, m, mi);
         }
 
@@ -353,6 +488,24 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
                 for (int d = 0; d < D; ++d) px[p][d] = x[p][d];
                 px[p][D] = 1.0f;
+            }
+        }
+        if (ACC == 4) {
+            const double magic = __hiloint2double(0x43380000, 0);  // 1.5 * 2^52
+            const int rep = lane & (nrep - 1);
+#pragma unroll
+            for (int p = 0; p < PPT; ++p) {
+                bad |= !(xn[p] < xn_limit);  // too large for the scale, or not finite
+                if (!GUARD || mi[p] >= 0) {
+                    unsigned long long* row = iacc + (rep * K + mi[p]) * LDI;
+#pragma unroll
+                    for (int d = 0; d < D; ++d) {
+                        const double t = fma(double(x[p][d]), iscale, magic);
+                        __hip_atomic_fetch_add(row + d, (unsigned long long)__double_as_longlong(t), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                    __hip_atomic_fetch_add(row + D, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
             }
         }
         if (ACC == 3) {
@@ -486,9 +639,23 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         }
     }
     if (ACC == 3) flush_macc();
+    if (ACC == 4 && bad) atomicOr(&imeta[1], 1);
     if (ACCUM || WANT_SSE) {
         __syncthreads();
         double* prow = part + int64_t(blockIdx.x) * (slots + 1);
+        if (ACC == 4) {
+            for (int s = tid; s < slots; s += T) {
+                const int k = s / (D + 1), d = s - k * (D + 1);
+                unsigned long long bits = 0ull, cnt = 0ull;
+                for (int r = 0; r < nrep; ++r) {
+                    bits += iacc[(r * K + k) * LDI + d];
+                    cnt += iacc[(r * K + k) * LDI + D];
+                }
+                const long long sum = (long long)(bits - cnt * 0x4338000000000000ull);
+                prow[s] = d == D ? double(cnt) : double(sum) * iquantum;
+            }
+            if (tid == 0) flags[blockIdx.x] = imeta[1];
+        }
         if (ACC == 2 || ACC == 3) {
             for (int s = tid; s < slots; s += T) {
                 double v = 0.0;
@@ -595,13 +762,12 @@ __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
     }
 }
 
+// acc_mode: 0 labels only, else the accumulation strategy; flags / aux as in the kernel
 template <int D>
 static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C, int32_t K,
-                          int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
-                          int grid, hipStream_t st) {
-    const bool accum = mode & 1, want_sse = mode & 2, want_min = min_d2 != nullptr;
-    // per-lane LDS columns while they fit (slots * 1 KB), the DPP tree otherwise
-    const int acc_mode = !accum ? 0 : small_acc_mode(D, K);
+                          int64_t ldc, int32_t* labels, float* min_d2, double* part, bool want_sse,
+                          int acc_mode, int grid, int32_t* flags, int aux, bool timed, hipStream_t st) {
+    const bool want_min = min_d2 != nullptr;
     const size_t lds = small_lds_bytes(D, K, acc_mode);
     // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads
     const int vec = ((ldx == D) && aligned16(X) && aligned16(labels) ? 1 : 0) |
@@ -613,18 +779,18 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     do {                                                                                                 \
         if (A == 3 && K > 16)                                                                            \
             hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A == 3 ? 32 : 0>), dim3(grid), dim3(SMALL_T), lds, \
-                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec);                     \
+                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);         \
         else if (A == 3)                                                                                 \
             hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A == 3 ? 16 : 0>), dim3(grid), dim3(SMALL_T), lds, \
-                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec);                     \
-        else if (reg)                                                                                    \
-            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, KT8>), dim3(grid), dim3(SMALL_T), lds, st, X, \
-                               N, ldx, C, K, ldc, labels, min_d2, part, vec);                            \
+                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);         \
+        else if (reg && A != 4)                                                                          \
+            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A != 4 ? KT8 : 0>), dim3(grid), dim3(SMALL_T), lds, st, X, \
+                               N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);                \
         else                                                                                             \
             hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, 0>), dim3(grid), dim3(SMALL_T), lds, st, X, \
-                               N, ldx, C, K, ldc, labels, min_d2, part, vec);                            \
+                               N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);                \
     } while (0)
-    prof_begin(st);
+    if (timed) prof_begin(st);
     if (acc_mode == 1) {
         if (want_sse) HKM_GO(1, false, true);
         else HKM_GO(1, false, false);
@@ -634,23 +800,53 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     } else if (acc_mode == 3) {
         if (want_sse) HKM_GO(3, false, true);
         else HKM_GO(3, false, false);
+    } else if (acc_mode == 4) {
+        if (want_sse) HKM_GO(4, false, true);
+        else HKM_GO(4, false, false);
     } else {
         if (want_min) HKM_GO(0, true, false);
         else HKM_GO(0, false, false);
     }
-    prof_end(st);
+    if (timed) prof_end(st);
 #undef HKM_GO
     return check_launch("lloyd_small_kernel");
 }
 
-// mode bit 0: accumulate per-cluster sums into `part`; bit 1: also the sum of min d2
+// how many bits above the largest centroid coordinate a row may reach in the integer accumulation:
+// the fused multiply-add needs |x| * 2^(QB - Ec) < 2^51, the 64-bit sum of a workgroup's rows 2^62
+static int small_headroom_bits(int64_t N, int32_t D, int grid) {
+    const int ppt = (D % 2 == 0) ? 2 : 4;
+    const int64_t groups = (N + ppt - 1) / ppt;
+    const int64_t per_wg = int64_t(SMALL_T) * ppt;
+    const int64_t rounds = (groups + int64_t(grid) * SMALL_T - 1) / (int64_t(grid) * SMALL_T);
+    const int64_t rows = rounds * per_wg;
+    int lg = 0;
+    while ((int64_t(1) << lg) < rows) ++lg;
+    return std::min(51 - SMALL_QB, 62 - SMALL_QB - lg);
+}
+
+// mode bit 0: accumulate per-cluster sums into `part`; bit 1: also the sum of min d2.
+// flags: [grid] scratch for the integer accumulation (may be NULL: then the ordered strategies run).
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
-                 int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode,
+                 int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode, int32_t* flags,
                  hipStream_t st) {
     const int grid = small_grid(N, D, K);
-#define HKM_T(d) \
-    case d:      \
-        return launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, mode, grid, st);
+    const bool accum = mode & 1, want_sse = mode & 2;
+    const int headroom = small_headroom_bits(N, D, grid);
+    const bool integer = accum && flags && headroom >= 4 && small_integer_sums(N, D, K);
+    const int ordered = small_ordered_mode(D, K);
+#define HKM_T(d)                                                                                           \
+    case d: {                                                                                              \
+        if (!integer)                                                                                      \
+            return launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, want_sse, accum ? ordered : 0, \
+                                     grid, nullptr, 0, true, st);                                          \
+        int rc = launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, want_sse, 4, grid, flags,   \
+                                   headroom, true, st);                                                    \
+        if (rc) return rc;                                                                                 \
+        /* the same sweep in the ordered way if a workgroup raised its flag; returns at once otherwise */  \
+        return launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, want_sse, ordered, grid, flags, \
+                                 grid, false, st);                                                         \
+    }
     switch (D) {
         HKM_T(1) HKM_T(2) HKM_T(3) HKM_T(4) HKM_T(5) HKM_T(6) HKM_T(7) HKM_T(8)
         default:

@@ -324,6 +324,120 @@ def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
     assert (c_step.cpu() - ref).abs().max() <= 2e-7 * float(xv.abs().max())
 
 
+def _narrow_step(xs, cs, dev, sums, monkeypatch, want_sse=True):
+    """One hkm_lloyd_step_f32 on a narrow shape with the per-cluster sums formed the given way."""
+    monkeypatch.setenv("HKM_SMALL_SUMS", sums)
+    n = xs.shape[0]
+    c_new = torch.empty_like(cs)
+    lab = torch.full((n,), -7, dtype=torch.int32, device=dev)
+    shift = torch.empty((), device=dev)
+    sse = torch.empty((), device=dev) if want_sse else None
+    _native.lloyd_step(xs, cs, c_new, lab, shift, sse, _native.Workspace(dev))
+    torch.cuda.synchronize()
+    return c_new.cpu(), lab.cpu(), shift.cpu(), (sse.cpu() if want_sse else None)
+
+
+# narrow shapes beyond 48 accumulator slots: every D, K up to the limit of 240 slots, ragged N
+NARROW_SHAPES = [(20000, 8, 16), (30011, 8, 26), (50000, 4, 32), (40001, 6, 20), (25000, 7, 30), (60000, 2, 64),
+                 (60002, 3, 40), (50000, 1, 100), (33333, 5, 40), (300, 8, 16), (7, 2, 20)]
+
+
+@pytest.mark.parametrize("n,d,k", NARROW_SHAPES)
+def test_integer_sums_of_the_narrow_step_equal_the_ordered_ones(cuda, n, d, k, monkeypatch):
+    # Large fits form the per-cluster sums of the narrow one-sweep step as exact 64-bit integer sums (LDS
+    # atomics, any order); small ones in a fixed order on the matrix cores or with a wave-wide tree.  Forced
+    # either way on the same input: same labels, same sum of distances, centroids equal to fp32 rounding
+    # and equal to the fp64 means of the labels; the integer way gives the same bits run after run.
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_small" and k * (d + 1) > 48
+    print(f"narrow sums n={n} d={d} k={k}", flush=True)
+    x, _ = _data(n, d, k, seed=3 * n + d)
+    x[::97] = 0.0
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(5))[:k]].contiguous()
+    if n < k:
+        c0 = _data(k, d, k, seed=1)[0]
+    xs, cs = x.to(cuda), c0.to(cuda)
+    c_o, lab_o, shift_o, sse_o = _narrow_step(xs, cs, cuda, "ordered", monkeypatch)
+    c_i, lab_i, shift_i, sse_i = _narrow_step(xs, cs, cuda, "integer", monkeypatch)
+    assert torch.equal(lab_o, lab_i) and torch.equal(sse_o, sse_i)
+    cmax = float(c0.abs().max())
+    assert (c_i - c_o).abs().max() <= 2.4e-7 * cmax
+    ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab_i.long(), x.double())
+    cnt = torch.bincount(lab_i.long(), minlength=k).clamp(min=1).double().unsqueeze(1)
+    ref = (ref / cnt).float()
+    # exact sums of rows rounded to 2^-32 of the largest centroid coordinate, one rounding at the end
+    assert (c_i - ref).abs().max() <= 6e-8 * max(cmax, float(ref.abs().max())) + 2.0 ** -31 * cmax
+    again = _narrow_step(xs, cs, cuda, "integer", monkeypatch)
+    assert torch.equal(again[0], c_i) and torch.equal(again[2], shift_i)
+    # rows with a leading dimension and no alignment: the guarded rounds
+    big = torch.zeros((n, d + 3), device=cuda)
+    big[:, 1:d + 1] = xs
+    c_s, lab_s, shift_s, _ = _narrow_step(big[:, 1:d + 1], cs, cuda, "integer", monkeypatch)
+    assert torch.equal(lab_s, lab_i)
+    assert (c_s - ref).abs().max() <= 6e-8 * max(cmax, float(ref.abs().max())) + 2.0 ** -31 * cmax
+
+
+def test_integer_sums_of_the_narrow_step_fall_back_outside_their_range(cuda, monkeypatch):
+    # The integer scale comes from the largest centroid coordinate.  A row too large for it, a row or a
+    # centroid that is not finite, or centroids that are all zero leave no exact integer sum: the step must
+    # then give exactly what the ordered way gives.  A row 2^10 times larger than the centroids is inside.
+    n, d, k = 30000, 8, 16
+    x, _ = _data(n, d, k, seed=41)
+    g = torch.Generator().manual_seed(6)
+    c_base = x[torch.randperm(n, generator=g)[:k]].contiguous()
+    for variant in ("huge_row", "inf_row", "nan_row", "zero_centroids", "inf_centroid", "large_row_inside"):
+        xv, c0 = x.clone(), c_base.clone()
+        if variant == "huge_row":
+            xv[12345] *= 2.0 ** 40
+        if variant == "inf_row":
+            xv[77, 3] = float("inf")
+        if variant == "nan_row":
+            xv[29999, 0] = float("nan")
+        if variant == "zero_centroids":
+            c0.zero_()
+        if variant == "inf_centroid":
+            c0[3, 2] = float("inf")
+        if variant == "large_row_inside":
+            xv[222] *= 2.0 ** 10
+        xs, cs = xv.to(cuda), c0.to(cuda)
+        c_o, lab_o, shift_o, sse_o = _narrow_step(xs, cs, cuda, "ordered", monkeypatch)
+        c_i, lab_i, shift_i, sse_i = _narrow_step(xs, cs, cuda, "integer", monkeypatch)
+        assert torch.equal(lab_o, lab_i), variant
+        if variant == "large_row_inside":
+            ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab_i.long(), xv.double())
+            cnt = torch.bincount(lab_i.long(), minlength=k).clamp(min=1).double().unsqueeze(1)
+            ref = (ref / cnt).float()
+            assert (c_i - ref).abs().max() <= 6e-8 * float(ref.abs().max()) + 2.0 ** -31 * float(c0.abs().max())
+            continue
+        assert torch.equal(c_o.isnan(), c_i.isnan()), variant
+        assert torch.equal(torch.nan_to_num(c_o), torch.nan_to_num(c_i)), variant
+        assert torch.equal(torch.nan_to_num(shift_o), torch.nan_to_num(shift_i)), variant
+
+
+@pytest.mark.parametrize("d", [1, 4, 8])
+def test_narrow_kernels_take_centroid_rows_at_any_four_byte_address(cuda, d):
+    # For these widths the narrow kernels fetch a centroid row as one scalar load of 1, 4 or 8 values;
+    # the rows of C are only required to be 4-byte aligned.
+    n, k = 20000, 24
+    x, _ = _data(n, d, k, seed=91 + d)
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(8))[:k]].contiguous()
+    xs = x.to(cuda)
+    flat = torch.zeros((k * d + 8,), device=cuda)
+    ref_lab, ref_min = _assign_gpu(x, c0, cuda)
+    for off in (1, 2, 3):
+        flat[off:off + k * d] = c0.to(cuda).reshape(-1)
+        cs = flat[off:off + k * d].view(k, d)
+        assert cs.data_ptr() % 16 == 4 * off
+        lab = torch.full((n,), -7, dtype=torch.int32, device=cuda)
+        md = torch.empty((n,), device=cuda)
+        _native.assign(xs, cs, lab, md, _native.Workspace(cuda))
+        c_new = torch.empty((k, d), device=cuda)
+        lab2 = torch.empty_like(lab)
+        _native.lloyd_step(xs, cs, c_new, lab2, torch.empty((), device=cuda), None, _native.Workspace(cuda))
+        torch.cuda.synchronize()
+        assert torch.equal(lab.cpu(), ref_lab) and torch.equal(md.cpu(), ref_min)
+        assert torch.equal(lab2.cpu(), ref_lab)
+
+
 def test_shift_and_functional_value(cuda):
     g = torch.Generator().manual_seed(9)
     a, b = torch.randn((37, 19), generator=g), torch.randn((37, 19), generator=g)
