@@ -71,16 +71,36 @@ int num_cus() {
     return cached_cus;
 }
 
+// Up to 16 features the vector kernel (one point per lane, K * (D + 3) instructions per point) competes with
+// the matrix cores, whose work comes in blocks of 32 centroids and 8 features with a fixed epilogue per
+// block.  Measured on 10M rows: for the assignment alone the matrix cores win from about 32 centroids on
+// (16 features: equal at 16, 1.4x at 24; 9 features and 16 centroids: the vector kernel is 2x faster), and
+// below 4 features three quarters of their work would be padding (HKM_NARROW_MFMA_MIN_K in the environment
+// moves the threshold).  The one-sweep step is another matter: see fused_eligible.
+static const int NARROW_MFMA_MIN_K = 32;
+static int narrow_mfma_min_k() {
+    const char* e = getenv("HKM_NARROW_MFMA_MIN_K");
+    if (e && e[0]) {
+        const int v = atoi(e);
+        if (v > 0) return v;
+    }
+    return NARROW_MFMA_MIN_K;
+}
+
 AssignKind assign_kind(int32_t D, int32_t K) {
-    if (D <= 16) return ASSIGN_VALU;
-    if (D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024) return ASSIGN_MFMA_RESIDENT;
+    const bool resident = D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024;
+    if (D <= 16 && (D < 4 || K < narrow_mfma_min_k() || !resident)) return ASSIGN_VALU;
+    if (resident) return ASSIGN_MFMA_RESIDENT;
     if (D <= 64) return ASSIGN_MFMA_TILED;
     return ASSIGN_MFMA_STREAM;
 }
 
-// the one-sweep MFMA step needs the centroids, fp64 accumulators and counts of a workgroup in LDS
+// The one-sweep MFMA step needs the centroids, fp64 accumulators and counts of a workgroup in LDS.  From 4
+// features on it is taken whatever K is: what it replaces for narrow rows is the vector assignment PLUS the
+// two-pass update, and reading X once beats that 2-3x even with a single centroid (10M x 16: 0.88 against
+// 1.84 ms at K = 1, 0.30 against 0.79 ms at K = 16).  Below 4 features the two passes stay ahead.
 bool fused_eligible(int32_t D, int32_t K) {
-    return assign_kind(D, K) == ASSIGN_MFMA_RESIDENT && fused_lds_bytes(D, K) <= 160 * 1024;
+    return D >= 4 && D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
 }
 
 static size_t cn_pad(int32_t K) { return (size_t(K) + 127) / 128 * 128; }
@@ -452,7 +472,7 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
 
 int hkm_point_blocks(int32_t D, int32_t* tuned) {
     if (tuned) *tuned = (env_point_blocks() == 0 && tuned_point_blocks() != 0) ? 1 : 0;
-    if (D <= 16 || D > 64) return 0;
+    if (D < 1 || D > 64) return 0;
     return resident_point_blocks(resident_dp(D));
 }
 

@@ -847,7 +847,8 @@ int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx
     if (dp == d && pb == b)                                                                                    \
         return vec ? launch_fused_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st) \
                    : launch_fused_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);
-    HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2) HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
+    HKM_CASE(8, 2) HKM_CASE(8, 1) HKM_CASE(16, 2) HKM_CASE(16, 1) HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2)
+    HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
 #undef HKM_CASE
     return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
 }
@@ -862,7 +863,8 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
     if (dp == d && pb == b)                                                                    \
         return vec ? launch_resident_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, st) \
                    : launch_resident_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
-    HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2) HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
+    HKM_CASE(8, 2) HKM_CASE(8, 1) HKM_CASE(16, 2) HKM_CASE(16, 1) HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2)
+    HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
 #undef HKM_CASE
     return fail(HKM_EUNSUPPORTED, "assign_mfma_resident: D=%d", D);
 }

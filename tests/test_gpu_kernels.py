@@ -209,7 +209,8 @@ def _step_and_two_pass_impl(xs, cs, dev):
 # shapes of the one-sweep MFMA step (16 < D <= 64, centroids + fp64 accumulators fit in LDS):
 # ragged N, K not a multiple of 32, D not a multiple of 4 (scalar loads), every padded width
 @pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (40000, 30, 100),
-                                   (70001, 40, 129), (30000, 64, 128), (768, 17, 5), (100, 48, 7)])
+                                   (70001, 40, 129), (30000, 64, 128), (768, 17, 5), (100, 48, 7),
+                                   (50000, 16, 64), (40000, 8, 40), (30001, 12, 100), (20000, 5, 60), (9000, 4, 256)])
 def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
     assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
     print(f"one-sweep n={n} d={d} k={k}", flush=True)
@@ -228,7 +229,8 @@ def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
     assert torch.equal(again[0], c_step) and torch.equal(again[2], shift)
 
 
-@pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (768, 17, 5)])
+@pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (768, 17, 5), (50000, 16, 64),
+                                   (40000, 8, 40), (30000, 13, 7)])
 def test_one_point_block_per_wave_gives_the_same_labels(cuda, n, d, k, monkeypatch):
     # HKM_POINT_BLOCKS=1 (16 < D <= 32): another launch geometry of the same kernels
     print(f"point blocks n={n} d={d} k={k}", flush=True)
@@ -277,7 +279,7 @@ def test_tuning_call_is_a_step_and_settles_on_a_geometry(cuda, monkeypatch):
     assert torch.equal(lab, want[0]) and torch.equal(cn, want[1]) and float(shift) == want[2]
     # shapes without the choice: wider rows, the narrow kernels
     assert _native.point_blocks(48) == (1, True) or _native.point_blocks(48) == (1, False)
-    assert _native.point_blocks(8)[0] == 0
+    assert _native.point_blocks(100)[0] == 0
     x8 = torch.rand(5000, 8).to(cuda)
     c8 = x8[:16].contiguous()
     assert _native.tune_lloyd_step(x8, c8, torch.empty_like(c8), torch.empty((5000,), dtype=torch.int32, device=cuda),
@@ -286,6 +288,27 @@ def test_tuning_call_is_a_step_and_settles_on_a_geometry(cuda, monkeypatch):
     monkeypatch.setenv("HKM_POINT_BLOCKS", "1")
     assert _native.point_blocks(d) == (1, False)
     assert _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws) == 0
+
+
+@pytest.mark.parametrize("n,d,k", [(30000, 16, 8), (20000, 9, 1), (25000, 12, 20), (10000, 10, 3), (40000, 4, 50), (30000, 7, 31)])
+def test_one_sweep_mfma_step_with_few_centroids_and_narrow_rows(cuda, n, d, k):
+    # From 4 features on the step runs on the matrix cores whatever K is, while the assignment alone stays
+    # on the vector kernel below 32 centroids: the two may break a tie at the resolution of the formula
+    # differently, so the step is checked against the oracle, and its means against its own labels.
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
+    print(f"one-sweep narrow n={n} d={d} k={k}", flush=True)
+    x, _ = _data(n, d, k, seed=7 * n + d)
+    c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(4))[:k]].contiguous()
+    xs, cs = x.to(cuda), c0.to(cuda)
+    c_step, lab_step, shift, _, _, _ = _step_and_two_pass(xs, cs, cuda)
+    lab = lab_step.cpu()
+    ref_lab, _ = orc.assign_to_cluster_literal(x, c0)
+    rep = orc.label_agreement(x, c0, lab, ref_lab)
+    assert rep["n_unexcused"] == 0 and rep["n_strict"] == 0 and rep["agreement"] >= 0.9999, rep
+    ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab.long(), x.double())
+    cnt = torch.bincount(lab.long(), minlength=k).clamp(min=1).double().unsqueeze(1)
+    assert (c_step.cpu() - (ref / cnt).float()).abs().max() <= 2e-7 * float(x.abs().max())
+    assert orc.rel_err_scalar(float(shift), float(orc.centroid_shift(c0, c_step.cpu())), floor=1e-12) <= 1e-5
 
 
 def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
