@@ -88,9 +88,8 @@ static int narrow_mfma_min_k() {
 }
 
 AssignKind assign_kind(int32_t D, int32_t K) {
-    const bool resident = D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024;
-    if (D <= 16 && (D < 4 || K < narrow_mfma_min_k() || !resident)) return ASSIGN_VALU;
-    if (resident) return ASSIGN_MFMA_RESIDENT;
+    if (D <= 16 && (D < 4 || K < narrow_mfma_min_k())) return ASSIGN_VALU;
+    if (D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024) return ASSIGN_MFMA_RESIDENT;
     if (D <= 64) return ASSIGN_MFMA_TILED;
     return ASSIGN_MFMA_STREAM;
 }

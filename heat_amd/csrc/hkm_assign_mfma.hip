@@ -1,4 +1,5 @@
-// Fused distance + argmin on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), for D > 16.
+// Fused distance + argmin on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), for D >= 4 (up to 16 features
+// only from 32 centroids on; the one-sweep step whatever K is).
 //
 // Operand roles: the A operand (M = 32 rows) carries CENTROIDS, the B operand (N = 32 columns)
 // carries POINTS.  In the 32x32 accumulator a lane then owns one point (column lane%32) and 16
@@ -764,7 +765,7 @@ int launch_assign_mfma_tiled(const float* X, int64_t N, int32_t D, int64_t ldx, 
         return vec ? launch_tiled_t<d, true>(X, N, D, ldx, C, K, ldc, cn, labels, min_d2, st)    \
                    : launch_tiled_t<d, false>(X, N, D, ldx, C, K, ldc, cn, labels, min_d2, st);
     switch (dp) {
-        HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
+        HKM_CASE(8) HKM_CASE(16) HKM_CASE(24) HKM_CASE(32) HKM_CASE(48) HKM_CASE(64)
         default:
             return fail(HKM_EUNSUPPORTED, "assign_mfma_tiled: D=%d", D);
     }

@@ -21,6 +21,7 @@ ASSIGN_SHAPES = [
     (1, 3, 8), (1000, 3, 8), (5000, 8, 16), (777, 16, 40), (300, 1, 5), (2000, 5, 700),
     (4096, 32, 256), (1000, 20, 33), (999, 17, 1), (3000, 64, 100), (1300, 50, 37), (257, 24, 64),
     (2048, 64, 1024), (1500, 100, 70), (900, 512, 130), (700, 33, 500), (513, 130, 1030),
+    (3000, 16, 1100), (2500, 8, 1500), (1800, 6, 2000), (4000, 4, 33), (3000, 13, 32),
 ]
 
 
