@@ -19,7 +19,8 @@
  *     synchronises; the library allocates nothing: the caller passes a workspace of at least
  *     hkm_workspace_bytes(N, D, K, flags) bytes (256-byte aligned) that must stay alive until the
  *     enqueued work has finished.  Concurrent calls must use different workspaces;
- *   - all reductions use a fixed order: the same inputs give bit-identical outputs on every run.
+ *   - all reductions use a fixed order, or arithmetic that is exact and therefore independent of the order
+ *     (integer sums, fp64 sums of pre-rounded addends): the same inputs give bit-identical outputs on every run.
  *
  * Environment (looked up on every call, nothing is cached)
  *   HKM_PRODUCTS=bf16x3   hkm_assign_f32 / hkm_lloyd_step_f32, every shape with D > 16 except those with
@@ -29,6 +30,12 @@
  *                         product as fp32, 1.3x to 1.7x the throughput.  Off by default.
  *   HKM_UPDATE_LISTS=1    hkm_update_f32 and the two-pass part of hkm_lloyd_step_f32 use the list-based
  *                         kernels instead of the sort-based ones (a testing aid).
+ *   HKM_SMALL_SUMS=ordered|integer   hkm_lloyd_step_f32 on the narrow shapes (D <= 8, K (D + 1) <= 240) with
+ *                         more than 48 accumulator slots: form the per-cluster sums in a fixed order, or as
+ *                         exact 64-bit integer sums, whatever N is (unset: integer from about a million rows
+ *                         on).  A testing aid; both give the same labels and means equal to fp32 rounding.
+ *   HKM_NARROW_MFMA_MIN_K=n   hkm_assign_f32 with 4 <= D <= 16: use the matrix-core kernels from n centroids
+ *                         on (default 32) and the vector kernel below.  A measuring and testing aid.
  */
 #ifndef HKM_H
 #define HKM_H
@@ -365,7 +372,7 @@ int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, i
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 
 /*
- * The resident matrix-core kernels (16 < D <= 32) come in two launch geometries -- two point blocks per wave,
+ * The resident matrix-core kernels (up to 32 features) come in two launch geometries -- two point blocks per wave,
  * or one with twice the waves -- that produce the same bits and differ in speed by a few percent either way,
  * depending on the clock the individual chip holds under them.  No counterpart in the reference.
  * hkm_tune_lloyd_step_f32: hkm_lloyd_step_f32 with the same arguments and the same results, which -- where the
