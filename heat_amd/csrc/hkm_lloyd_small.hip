@@ -3,7 +3,9 @@
 //
 // Assignment: a lane owns PPT consecutive points in registers; the centroids and their squared norms are
 // wave-uniform operands -- LDS broadcasts of rows scaled by -2 (exact), or, where a row is one scalar load,
-// scalar registers filled straight from C (scan_centroids_sload).  The quadratic expansion of
+// scalar registers filled straight from C (scan_centroids_sload); 14 to 16 centroids of 4 or 8 coordinates
+// are instead one A operand of v_mfma_f32_16x16x4_f32 and the minimum is found in registers after a
+// transpose across the lanes (the matrix-core scan in the kernel body).  The quadratic expansion of
 // heat/spatial/distance.py:59-64, d2 = |x|^2 + |c|^2 - 2 x.c, is evaluated as a chain of D fused
 // multiply-adds that starts at |c|^2; |x|^2, the same for every centroid, is added to the minimum only.
 // First index wins ties (torch.min, heat/core/statistics.py:177).  The clamp at 0 is applied lazily: a
@@ -36,6 +38,18 @@
 #include <type_traits>
 
 #include "hkm_common.h"
+#include "hkm_mfma_util.h"
+
+// Fewest centroids for which the matrix-core scan of the narrow kernel is used (8 / 4 coordinates).  Its cost
+// does not depend on K and equals that of the vector scan over 13 centroids (50M rows, kernel without label
+// stores: 0.36-0.38 ms whatever K is, against 0.35 / 0.37 / 0.39 ms of the vector scan at K = 13 / 14 / 16 with
+// 8 coordinates; 0.222 against 0.228 / 0.245 ms at K = 13 / 16 with 4).
+#ifndef HKM_MSCAN_MIN_K8
+#define HKM_MSCAN_MIN_K8 14
+#endif
+#ifndef HKM_MSCAN_MIN_K4
+#define HKM_MSCAN_MIN_K4 14
+#endif
 
 namespace hkm {
 
@@ -54,6 +68,9 @@ struct SmallCfg {
     // values): measured on 30-100 M rows with 16-100 clusters, the step is then 4-26 % faster; rows of
     // 2, 3, 5 or 7 values take several loads per centroid and run 6-10 % slower that way.
     static constexpr bool SLOAD = D == 1 || D == 4 || D == 8;
+    // Up to 16 centroids of 4 or 8 coordinates are one A operand of v_mfma_f32_16x16x4_f32 (one or two steps
+    // over the coordinates): the cross terms of 16 points then cost one or two matrix instructions.
+    static constexpr bool MSCAN = D == 4 || D == 8;
 };
 
 bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
@@ -74,7 +91,8 @@ __host__ __device__ constexpr int small_int_stride(int D) { return (D + 1) | 1; 
 static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
     const int sc = (D + 1 + 3) / 4 * 4, nv = ppt * D / 4, slots = K * (D + 1);
-    return size_t((K * sc + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) +
+    const size_t xch = (D == 4 || D == 8) ? size_t(SMALL_T / 64) * 256 * sizeof(float) : 0;  // as SmallCfg::MSCAN
+    return size_t((K * sc + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) + xch +
            (acc_mode == 2   ? size_t(SMALL_T / 64) * slots * sizeof(double)
             : acc_mode == 3 ? size_t(SMALL_T / 64) * (slots * sizeof(double) + 64 * ppt * sizeof(int))
             : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float)
@@ -120,6 +138,20 @@ int small_grid(int64_t N, int32_t D, int32_t K) {
     if (want > cap) want = cap;
     if (want < 1) want = 1;
     return int(want);
+}
+
+// Exchanges between the four rows of 16 lanes of a wave (one instruction each): rows 2, 3 of a with rows 0, 1
+// of b; odd rows of a with even rows of b.
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void lane_rows_swap32(float& a, float& b) {
+    const uintx2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void lane_rows_swap16(float& a, float& b) {
+    const uintx2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
 }
 
 // sum over the 64 lanes with a fixed tree; the total is valid in lane 63
@@ -252,7 +284,10 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     constexpr bool ACCUM = ACC != 0;
     const bool stream = (vec & 2) != 0;
     float* stage = lds + ((K * SC + 3) & ~3);                        // [NW][NV*64*4] transpose buffer
-    float* after = stage + NW * NV * 256;
+    // matrix-core scan: [NW][128] (minimum, index) pairs on their way from the lane that found them to the
+    // lane that owns the point
+    float* xch_all = stage + NW * NV * 256;
+    float* after = xch_all + (SmallCfg<D>::MSCAN ? NW * 256 : 0);
     double* wacc_all = reinterpret_cast<double*>(after);             // ACC==2: [NW][slots]
     float* cols = after;                                             // ACC==1: [slots][T]
     const int tid = threadIdx.x;
@@ -358,6 +393,25 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             }
     }
 
+    // The matrix-core scan (K <= 16, D = 4 or 8, PPT = 2): 16 points x 16 centroids per v_mfma_f32_16x16x4_f32,
+    // one instruction per four coordinates.  A = the centroid table (lane: row lane % 16, coordinate 4 s +
+    // lane / 16 of -2c; rows beyond K are zero), held in registers for the whole kernel; C = |c|^2 of the four
+    // rows 4 (lane / 16) + r the lane's results belong to (+inf beyond K: never the minimum); B = 16 points
+    // read back from the staging buffer.
+    constexpr bool MSCAN = SmallCfg<D>::MSCAN && !REGC;
+    const bool mscan = MSCAN && K <= 16 && K >= (D == 8 ? HKM_MSCAN_MIN_K8 : HKM_MSCAN_MIN_K4);
+    float ma[MSCAN ? D / 4 : 1];
+    floatx4 mcn = {HKM_INF, HKM_INF, HKM_INF, HKM_INF};
+    if (mscan) {
+        const int i = lane & 15, kk = lane >> 4;
+#pragma unroll
+        for (int st = 0; st < D / 4; ++st) ma[st] = i < K ? sC[i * SC + 4 * st + kk] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (4 * kk + r < K) mcn[r] = sC[(4 * kk + r) * SC + D];
+    }
+    float* xch = xch_all + wave * 256;
+
     double sse = 0.0;
 
     // ACC == 1: the additions of a round are deferred to the NEXT round and interleaved with its
@@ -425,16 +479,78 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             rmw_write(0, r);
             rmw_read(1, r);
         }
-        if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
-        else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, 0, kh, x, xn, m, mi);
-        else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
+        bool scanned = false;
+        if constexpr (MSCAN) {
+            if (mscan) {
+                scanned = true;
+                // The wave's 128 points of the round sit in the staging buffer as rows; 64 at a time, four
+                // groups of 16 go through the matrix cores.  A lane then holds, of each group, the distances
+                // of point lane % 16 to centroids 4 (lane / 16) + r; two swaps of lane rows per register
+                // (across the halves of the wave, then between neighbouring rows) transpose that, so that
+                // lane 16 g + n ends up with all sixteen distances of point n of group g, in centroid order.
+                const float* brow = wstage + (lane & 15) * D + (lane >> 4);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    floatx4 acc[4];
+                    float bv[4][D / 4];  // all requested before the first matrix instruction waits for one
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int st = 0; st < D / 4; ++st) bv[j][st] = brow[(half * 64 + 16 * j) * D + 4 * st];
+                    wave_lds_sync();
+#pragma unroll
+                    for (int st = 0; st < D / 4; ++st)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ma[st], bv[j][st], st == 0 ? mcn : acc[j], 0, 0, 0);
+                    float dk[4][4];  // [group -> centroid quad after the transpose][r]
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) dk[j][q] = acc[j][q];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        lane_rows_swap32(dk[0][q], dk[2][q]);
+                        lane_rows_swap32(dk[1][q], dk[3][q]);
+                        lane_rows_swap16(dk[0][q], dk[1][q]);
+                        lane_rows_swap16(dk[2][q], dk[3][q]);
+                    }
+                    floatx16 dv;
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) dv[k] = dk[k >> 2][k & 3];
+                    const float best = block_min16(dv);
+                    const int pos = block_pos16(dv, best);  // 8 * (k / 4) + k % 4 for the first k that holds it
+                    const int idx = (pos & 3) | ((pos >> 3) << 2);
+                    // nothing below +inf (all distances inf or NaN): index 0, as the running scan leaves it
+                    const bool any = best < HKM_INF;
+                    float2 out;
+                    out.x = any ? best : HKM_INF;
+                    out.y = __int_as_float(any ? idx : 0);
+                    reinterpret_cast<float2*>(xch)[half * 64 + lane] = out;
+                }
+                wave_lds_sync();
+                const floatx4 mine = reinterpret_cast<const floatx4*>(xch)[lane];  // points 2 lane, 2 lane + 1
+                wave_lds_sync();
+                m[0] = mine[0];
+                mi[0] = __float_as_int(mine[1]);
+                m[PPT - 1] = mine[2];
+                mi[PPT - 1] = __float_as_int(mine[3]);
+            }
+        }
+        if (!scanned) {
+            if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
+            else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, 0, kh, x, xn, m, mi);
+            else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
+        }
         if (ACC == 1) {
             rmw_write(PPT == 4 ? 1 : 0, r);
             rmw_read(PPT == 4 ? 2 : 1, r);
         }
-        if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
-        else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, kh, K, x, xn, m, mi);
-        else scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
+        if (!scanned) {
+            if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
+            else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, kh, K, x, xn, m, mi);
+            else scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
+        }
         if (ACC == 1 && PPT == 4) {
             rmw_write(2, r);
             rmw_read(3, r);
@@ -617,8 +733,8 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
             for (int d = 0; d < D; ++d) x[p][d] = X[r * ldx + d];
         }
-        if (ACC == 3) {
-            // the matrix-core accumulation reads the round's points from the staging buffer
+        if (ACC == 3 || mscan) {
+            // the matrix-core accumulation and the matrix-core scan read the round's points from the staging buffer
             wave_lds_sync();
 #pragma unroll
             for (int p = 0; p < PPT; ++p)

@@ -88,6 +88,45 @@ def test_assign_point_equals_centroid_clamps_at_zero(cuda):
         assert md.max() <= 2e-6 * float((c.double() ** 2).sum(1).max())
 
 
+@pytest.mark.parametrize("d,k", [(8, 16), (8, 14), (4, 16), (4, 15)])
+def test_narrow_matrix_core_scan_keeps_the_reference_rules(cuda, d, k):
+    # 14 to 16 centroids of 4 or 8 coordinates: the narrow kernels take the cross terms from the matrix cores
+    # (16 points x 16 centroids per instruction) and find the minimum in registers after a transpose across
+    # lanes.  Same rules as everywhere: first index on exact ties, clamp at 0, rows of NaN go to cluster 0.
+    g = torch.Generator().manual_seed(40 + d + k)
+    n = 3001
+    base = torch.randn((k // 2, d), generator=g) * 3
+    c = torch.cat([base, base])  # centroid j == j + k/2: exact ties
+    x = base[torch.randint(0, k // 2, (n,), generator=g)] + 0.05 * torch.randn((n, d), generator=g)
+    x[7] = c[3]            # on a centroid: the expansion may come out below zero
+    x[11] = float("nan")
+    lab, md = _assign_gpu(x, c, cuda)
+    ref, _ = orc.assign_to_cluster_literal(torch.nan_to_num(x, nan=0.0), c)
+    ok = torch.ones(n, dtype=torch.bool)
+    ok[11] = False
+    assert int(lab.max()) < k // 2
+    assert bool((lab.long()[ok] == (ref.view(-1) % (k // 2))[ok]).all())
+    assert int(lab[11]) == 0
+    assert float(md[7]) == 0.0 and float(md[ok].min()) >= 0.0
+    # distinct centroids, a leading dimension, an unaligned base, a ragged end: against the oracle, and the
+    # step's labels equal to the assignment's
+    cw = torch.randn((k, d + 3), generator=g) * 3
+    xw = cw[torch.randint(0, k, (n,), generator=g), 2:2 + d] + torch.randn((n, d), generator=g)
+    xbuf = torch.zeros((n, d + 5))
+    xbuf[:, 1:1 + d] = xw
+    xs, cs = xbuf.to(cuda)[:, 1:1 + d], cw.to(cuda)[:, 2:2 + d]
+    lab2 = torch.empty((n,), dtype=torch.int32, device=cuda)
+    _native.assign(xs, cs, lab2, None, _native.Workspace(cuda))
+    ref2, _ = orc.assign_to_cluster_literal(xw.contiguous(), cw[:, 2:2 + d].contiguous())
+    rep = orc.label_agreement(xw, cw[:, 2:2 + d], lab2.cpu(), ref2)
+    assert rep["n_unexcused"] == 0 and rep["n_strict"] == 0, rep
+    c_new = torch.empty((k, d), device=cuda)
+    lab3 = torch.empty_like(lab2)
+    _native.lloyd_step(xs, cs.contiguous(), c_new, lab3, torch.empty((), device=cuda), None, _native.Workspace(cuda))
+    torch.cuda.synchronize()
+    assert torch.equal(lab3, lab2)
+
+
 def test_assign_strided_rows(cuda):
     # X and C as column slices of wider buffers: ld > D, base pointers not 16-byte aligned
     g = torch.Generator().manual_seed(7)
@@ -363,7 +402,7 @@ def _narrow_step(xs, cs, dev, sums, monkeypatch, want_sse=True):
 
 # narrow shapes beyond 48 accumulator slots: every D, K up to the limit of 240 slots, ragged N
 NARROW_SHAPES = [(20000, 8, 16), (30011, 8, 26), (50000, 4, 32), (40001, 6, 20), (25000, 7, 30), (60000, 2, 64),
-                 (60002, 3, 40), (50000, 1, 100), (33333, 5, 40), (300, 8, 16), (7, 2, 20)]
+                 (60002, 3, 40), (50000, 1, 100), (33333, 5, 40), (300, 8, 16), (7, 2, 20), (45001, 4, 15), (30000, 8, 14)]
 
 
 @pytest.mark.parametrize("n,d,k", NARROW_SHAPES)
