@@ -878,6 +878,27 @@ __global__ __launch_bounds__(1024) void lloyd_small_finalize_kernel(
     }
 }
 
+// First level of the finish for many wide partial rows: workgroup b adds rows b * R0 .. of `part` in ascending
+// order (16 loads in flight, additions still in row order) into row b of `out`.  One workgroup walking a
+// thousand rows of 145 values is 30 us of latency; 32 workgroups walking 32 rows each and one walking their
+// 32 results are 10.  The order depends only on (G, R0).
+__global__ __launch_bounds__(256) void lloyd_small_prereduce_kernel(const double* __restrict__ part, int G, int nslot,
+                                                                    int R0, double* __restrict__ out) {
+    const int g0 = blockIdx.x * R0, g1 = min(G, g0 + R0);
+    for (int s = threadIdx.x; s < nslot; s += 256) {
+        double v = 0.0;
+        for (int g = g0; g < g1; g += 16) {
+            double t[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) t[u] = g + u < g1 ? part[int64_t(g + u) * nslot + s] : 0.0;
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (g + u < g1) v += t[u];
+        }
+        out[int64_t(blockIdx.x) * nslot + s] = v;
+    }
+}
+
 // acc_mode: 0 labels only, else the accumulation strategy; flags / aux as in the kernel
 template <int D>
 static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C, int32_t K,
@@ -975,6 +996,16 @@ int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, co
                           float* C_new, int64_t ldcn, int64_t* counts, float* shift, float* sse,
                           hipStream_t st) {
     const int spad = K * (D + 1) + 1;  // <= 241 because K*(D+1) <= 240
+    // many wide rows: two levels (the first writes behind the rows it reads; the workspace holds SMALL_MAX_GRID)
+    if (int64_t(grid) * spad >= 32768 && grid + 32 <= SMALL_MAX_GRID) {
+        const int r0 = (grid + 31) / 32, nb = (grid + r0 - 1) / r0;
+        double* out = const_cast<double*>(part) + int64_t(grid) * spad;
+        hipLaunchKernelGGL(lloyd_small_prereduce_kernel, dim3(nb), dim3(256), 0, st, part, grid, spad, r0, out);
+        int rc = check_launch("lloyd_small_prereduce_kernel");
+        if (rc) return rc;
+        part = out;
+        grid = nb;
+    }
     hipLaunchKernelGGL(lloyd_small_finalize_kernel, dim3(1), dim3(1024), 0, st, part, grid, K, D,
                        C_old, C_new, ldcn, counts, shift, sse, sse ? 1 : 0, spad);
     return check_launch("lloyd_small_finalize_kernel");
