@@ -3,7 +3,7 @@
 //
 // Assignment: a lane owns PPT consecutive points in registers; the centroids and their squared norms are
 // wave-uniform operands -- LDS broadcasts of rows scaled by -2 (exact), or, where a row is one scalar load,
-// scalar registers filled straight from C (scan_centroids_sload); 14 to 16 centroids of 4 or 8 coordinates
+// scalar registers filled straight from C (scan_centroids_sload); 12 to 16 centroids of 4 or 8 coordinates
 // are instead one A operand of v_mfma_f32_16x16x4_f32 and the minimum is found in registers after a
 // transpose across the lanes (the matrix-core scan in the kernel body).  The quadratic expansion of
 // heat/spatial/distance.py:59-64, d2 = |x|^2 + |c|^2 - 2 x.c, is evaluated as a chain of D fused
@@ -41,14 +41,14 @@
 #include "hkm_mfma_util.h"
 
 // Fewest centroids for which the matrix-core scan of the narrow kernel is used (8 / 4 coordinates).  Its cost
-// does not depend on K and equals that of the vector scan over 13 centroids (50M rows, kernel without label
-// stores: 0.36-0.38 ms whatever K is, against 0.35 / 0.37 / 0.39 ms of the vector scan at K = 13 / 14 / 16 with
-// 8 coordinates; 0.222 against 0.228 / 0.245 ms at K = 13 / 16 with 4).
+// does not depend on K and equals that of the vector scan over 11 to 12 centroids (50M rows, kernel without
+// label stores, 8 coordinates: 0.345-0.352 ms whatever K is, against 0.342 / 0.358 / 0.370 ms of the vector
+// scan at K = 11 / 12 / 13; 4 coordinates: 0.222 against 0.219 / 0.231 ms at K = 12 / 13).
 #ifndef HKM_MSCAN_MIN_K8
-#define HKM_MSCAN_MIN_K8 14
+#define HKM_MSCAN_MIN_K8 12
 #endif
 #ifndef HKM_MSCAN_MIN_K4
-#define HKM_MSCAN_MIN_K4 14
+#define HKM_MSCAN_MIN_K4 13
 #endif
 
 namespace hkm {
@@ -80,11 +80,11 @@ static constexpr int SMALL_T = 256;
 // A coordinate is added as the integer rint(x * 2^(QB - Ec)), where 2^Ec bounds the largest centroid
 // coordinate of the step: integer additions are exact, so LDS atomics may deliver them in any order.
 static constexpr int SMALL_QB = 32;
-// copies of the accumulator table per workgroup (a lane uses copy lane % R): fewer lanes of one
-// instruction meet at one address
+// copies of every accumulator per workgroup (a lane uses copy lane % R): fewer lanes of one instruction
+// meet at one address, and with the copies side by side none in a bank more than their share
 __host__ __device__ constexpr int small_replicas(int K) { return K <= 16 ? 16 : K <= 32 ? 8 : 4; }
-// row stride of the table in 64-bit words, odd so that the rows of different clusters spread over the banks
-__host__ __device__ constexpr int small_int_stride(int D) { return (D + 1) | 1; }
+// entries per cluster row of the table
+__host__ __device__ constexpr int small_int_stride(int D) { return D + 1; }
 
 // LDS of one workgroup; acc_mode as in the kernel (0 labels only, 1 lane columns, 2 wave rows by the
 // DPP tree, 3 wave rows by the matrix cores, 4 integer tables)
@@ -293,8 +293,10 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     double* wacc = wacc_all + wave * slots;
-    // ACC == 4: [R][K][LDI] 64-bit integers (column D of a row counts its points), then the bits of the
-    // largest |centroid coordinate| and the workgroup's flag
+    // ACC == 4: [K][LDI][R] 64-bit integers (column D of a row counts its points; the R copies of an entry
+    // lie side by side, so a lane's copy -- lane mod R -- decides its LDS bank and the 64 lanes of an
+    // instruction spread evenly over the banks whatever their labels are), then the bits of the largest
+    // |centroid coordinate| and the workgroup's flag
     constexpr int LDI = small_int_stride(D);
     const int nrep = small_replicas(K);
     unsigned long long* iacc = reinterpret_cast<unsigned long long*>(after);
@@ -613,14 +615,14 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             for (int p = 0; p < PPT; ++p) {
                 bad |= !(xn[p] < xn_limit);  // too large for the scale, or not finite
                 if (!GUARD || mi[p] >= 0) {
-                    unsigned long long* row = iacc + (rep * K + mi[p]) * LDI;
+                    unsigned long long* row = iacc + mi[p] * (LDI * nrep) + rep;
 #pragma unroll
                     for (int d = 0; d < D; ++d) {
                         const double t = fma(double(x[p][d]), iscale, magic);
-                        __hip_atomic_fetch_add(row + d, (unsigned long long)__double_as_longlong(t), __ATOMIC_RELAXED,
+                        __hip_atomic_fetch_add(row + d * nrep, (unsigned long long)__double_as_longlong(t), __ATOMIC_RELAXED,
                                                __HIP_MEMORY_SCOPE_WORKGROUP);
                     }
-                    __hip_atomic_fetch_add(row + D, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(row + D * nrep, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             }
         }
@@ -764,8 +766,8 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 const int k = s / (D + 1), d = s - k * (D + 1);
                 unsigned long long bits = 0ull, cnt = 0ull;
                 for (int r = 0; r < nrep; ++r) {
-                    bits += iacc[(r * K + k) * LDI + d];
-                    cnt += iacc[(r * K + k) * LDI + D];
+                    bits += iacc[(k * LDI + d) * nrep + r];
+                    cnt += iacc[(k * LDI + D) * nrep + r];
                 }
                 const long long sum = (long long)(bits - cnt * 0x4338000000000000ull);
                 prow[s] = d == D ? double(cnt) : double(sum) * iquantum;

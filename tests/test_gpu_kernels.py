@@ -88,9 +88,9 @@ def test_assign_point_equals_centroid_clamps_at_zero(cuda):
         assert md.max() <= 2e-6 * float((c.double() ** 2).sum(1).max())
 
 
-@pytest.mark.parametrize("d,k", [(8, 16), (8, 14), (4, 16), (4, 15)])
+@pytest.mark.parametrize("d,k", [(8, 16), (8, 14), (8, 12), (4, 16), (4, 14)])
 def test_narrow_matrix_core_scan_keeps_the_reference_rules(cuda, d, k):
-    # 14 to 16 centroids of 4 or 8 coordinates: the narrow kernels take the cross terms from the matrix cores
+    # 12 to 16 centroids of 4 or 8 coordinates: the narrow kernels take the cross terms from the matrix cores
     # (16 points x 16 centroids per instruction) and find the minimum in registers after a transpose across
     # lanes.  Same rules as everywhere: first index on exact ties, clamp at 0, rows of NaN go to cluster 0.
     g = torch.Generator().manual_seed(40 + d + k)
@@ -107,7 +107,7 @@ def test_narrow_matrix_core_scan_keeps_the_reference_rules(cuda, d, k):
     assert int(lab.max()) < k // 2
     assert bool((lab.long()[ok] == (ref.view(-1) % (k // 2))[ok]).all())
     assert int(lab[11]) == 0
-    assert float(md[7]) == 0.0 and float(md[ok].min()) >= 0.0
+    assert 0.0 <= float(md[7]) <= 2e-6 * float((c[3].double() ** 2).sum()) and float(md[ok].min()) >= 0.0
     # distinct centroids, a leading dimension, an unaligned base, a ragged end: against the oracle, and the
     # step's labels equal to the assignment's
     cw = torch.randn((k, d + 3), generator=g) * 3
