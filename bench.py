@@ -631,6 +631,8 @@ def main() -> int:
         if tj.get("sources_sha1") == sha and args.scale == 1.0:
             roof["traffic"] = tj.get(w.name)
             roof["traffic_source"] = f"profiles/traffic.json, measured on library sources sha1 {sha} (= this build)"
+        elif args.scale != 1.0:
+            roof["traffic_source"] = "dropped: profiles/traffic.json holds the unscaled workloads only"
         else:
             roof["traffic_source"] = (f"dropped: profiles/traffic.json was measured on library sources sha1 "
                                       f"{tj.get('sources_sha1')}, this build is {sha}")
