@@ -96,8 +96,8 @@ AssignKind assign_kind(int32_t D, int32_t K) {
 
 // The one-sweep MFMA step needs the centroids, fp64 accumulators and counts of a workgroup in LDS.  From 4
 // features on it is taken whatever K is: what it replaces for narrow rows is the vector assignment PLUS the
-// two-pass update, and reading X once beats that 2-3x even with a single centroid (10M x 16: 0.88 against
-// 1.84 ms at K = 1, 0.30 against 0.79 ms at K = 16).  Below 4 features the two passes stay ahead.
+// two-pass update, and reading X once beats that 3x or more even with a single centroid (10M x 16: 0.22 against
+// 1.84 ms at K = 1, 0.24 against 0.79 ms at K = 16).  Below 4 features the two passes stay ahead.
 bool fused_eligible(int32_t D, int32_t K) {
     return D >= 4 && D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
 }

@@ -315,7 +315,7 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles,
     double* __restrict__ fsum, int32_t* __restrict__ fcnt, int32_t* __restrict__ flags,
-    int range_bits) {
+    int range_bits, int nrep) {
     extern __shared__ __align__(16) float lds[];
     constexpr int LDC = DP + 4;
     constexpr int LDA = DP + 1;  // odd row stride (in doubles): rows of different clusters spread over the banks
@@ -323,8 +323,13 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
     const int KP = (K + 31) & ~31;
     float* sC = lds;                                              // [KP][LDC]
     float* sCn = lds + KP * LDC;                                  // [KP] squared norms
-    double* sA = reinterpret_cast<double*>(sCn + KP);             // [K][LDA]
-    int* sN = reinterpret_cast<int*>(sA + size_t(K) * LDA);       // [K] counts, then Emin, Emax
+    // With few clusters many lanes of an atomic instruction meet at one address and are served one after the
+    // other, so the accumulators come in nrep copies (a power of two; a lane uses copy p mod nrep), an odd
+    // number of doubles apart so that the copies of a row start in different banks.
+    const size_t rstride = size_t(K) * LDA + 1;
+    double* sA = reinterpret_cast<double*>(sCn + KP);             // [nrep][K][LDA] (+ 1 pad per copy)
+    int* sN = reinterpret_cast<int*>(sA + nrep * rstride);        // [nrep][K] counts, then Emin, Emax, non-finite
+    int* sMeta = sN + nrep * K;
     const int tid = threadIdx.x, nthr = blockDim.x;
 
     for (int i = tid; i < KP * DP; i += nthr) {
@@ -340,12 +345,12 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
         }
         sCn[r] = s;
     }
-    for (int i = tid; i < K * LDA; i += nthr) sA[i] = 0.0;
-    for (int i = tid; i < K; i += nthr) sN[i] = 0;
+    for (int i = tid; i < int(nrep * rstride); i += nthr) sA[i] = 0.0;
+    for (int i = tid; i < nrep * K; i += nthr) sN[i] = 0;
     if (tid == 0) {
-        sN[K] = 0x7fffffff;
-        sN[K + 1] = -0x7fffffff;
-        sN[K + 2] = 0;
+        sMeta[0] = 0x7fffffff;
+        sMeta[1] = -0x7fffffff;
+        sMeta[2] = 0;
     }
     __syncthreads();
 
@@ -355,6 +360,8 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
     const int64_t tile_rows = int64_t(nw) * PB * 32;
     const bool fast = VEC && D == DP && ldx < (int64_t(1) << 24);
     const unsigned lane_off = unsigned((int64_t(p) * ldx + h * (DP / 2)) * 4);
+    double* sA_lane = sA + (p & (nrep - 1)) * rstride;
+    int* sN_lane = sN + (p & (nrep - 1)) * K;
     int emin = 0x7fffffff, emax = -0x7fffffff;
     int nonfinite = 0;  // a row whose |x|^2 is inf or NaN: its bound 2^E says nothing about its coordinates
 
@@ -391,7 +398,7 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
             if (h == 0 && valid) {
                 labels[rb + p] = mi[pb];
                 if (min_d2) min_d2[rb + p] = m[pb];
-                atomicAdd(&sN[mi[pb]], 1);
+                atomicAdd(&sN_lane[mi[pb]], 1);
             }
             if (valid && xnr[pb] != 0.f) {  // an all-zero row adds nothing
                 // |x_d| < 2^E: |x|^2 < 2^(e2+1) up to rounding, one more bit of slack
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
                 emin = min(emin, E);
                 emax = max(emax, E);
                 const double B = __hiloint2double(((1023 + 52 - FUSED_QBITS + E) << 20) | 0x80000, 0);
-                double* row = sA + size_t(mi[pb]) * LDA + h * (DP / 2);
+                double* row = sA_lane + size_t(mi[pb]) * LDA + h * (DP / 2);
 #pragma unroll
                 for (int j = 0; j < NJ; ++j)
 #pragma unroll
@@ -423,19 +430,25 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
         if (tile + gridDim.x < ntiles) step(tile + gridDim.x, b1, b0);
     }
 
-    atomicMin(&sN[K], emin);
-    atomicMax(&sN[K + 1], emax);
-    if (nonfinite) atomicOr(&sN[K + 2], 1);
+    atomicMin(&sMeta[0], emin);
+    atomicMax(&sMeta[1], emax);
+    if (nonfinite) atomicOr(&sMeta[2], 1);
     __syncthreads();
     double* gs = fsum + size_t(blockIdx.x) * K * D;
     for (int i = tid; i < K * D; i += nthr) {
         const int k = i / D, d = i - k * D;
-        gs[i] = sA[size_t(k) * LDA + d];
+        double v = 0.0;  // exact whatever the order (or the flag is up and the value unused)
+        for (int r = 0; r < nrep; ++r) v += sA[r * rstride + size_t(k) * LDA + d];
+        gs[i] = v;
     }
-    for (int i = tid; i < K; i += nthr) fcnt[size_t(blockIdx.x) * K + i] = sN[i];
+    for (int i = tid; i < K; i += nthr) {
+        int c = 0;
+        for (int r = 0; r < nrep; ++r) c += sN[r * K + i];
+        fcnt[size_t(blockIdx.x) * K + i] = c;
+    }
     if (tid == 0) {
-        const int lo = sN[K], hi = sN[K + 1];
-        flags[blockIdx.x] = ((hi >= lo && hi - lo > range_bits) || sN[K + 2]) ? 1 : 0;
+        const int lo = sMeta[0], hi = sMeta[1];
+        flags[blockIdx.x] = ((hi >= lo && hi - lo > range_bits) || sMeta[2]) ? 1 : 0;
     }
 }
 
@@ -794,11 +807,22 @@ static int launch_resident_t(const float* X, int64_t N, int32_t D, int64_t ldx, 
     return check_launch("assign_mfma_resident_kernel");
 }
 
-size_t fused_lds_bytes(int32_t D, int32_t K) {
+static size_t fused_lds_bytes_with(int32_t D, int32_t K, int nrep) {
     const size_t kp = (size_t(K) + 31) / 32 * 32;
     const int dp = resident_dp(D);
-    return kp * (dp + 5) * sizeof(float) + size_t(K) * (dp + 1) * sizeof(double) + (size_t(K) + 4) * sizeof(int);
+    return kp * (dp + 5) * sizeof(float) + size_t(nrep) * (size_t(K) * (dp + 1) + 1) * sizeof(double) +
+           (size_t(nrep) * K + 4) * sizeof(int);
 }
+
+// Copies of the fp64 accumulators in the one-sweep kernel: up to 64 clusters, as many as bring the lanes
+// that meet at one address down to a few and still fit in 48 KB with everything else.
+int fused_replicas(int32_t D, int32_t K) {
+    int r = K <= 16 ? 16 : K <= 32 ? 8 : K <= 64 ? 4 : 1;
+    while (r > 1 && fused_lds_bytes_with(D, K, r) > 48 * 1024) r >>= 1;
+    return r;
+}
+
+size_t fused_lds_bytes(int32_t D, int32_t K) { return fused_lds_bytes_with(D, K, fused_replicas(D, K)); }
 
 int fused_grid(int64_t N, int32_t D) {
     const int dp = resident_dp(D);
@@ -833,7 +857,7 @@ static int launch_fused_t(const float* X, int64_t N, int32_t D, int64_t ldx, con
     const int range_bits = 53 - FUSED_QBITS - lg;
     prof_begin(st);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(THREADS), lds, st, X, N, D, ldx, C, K, ldc,
-                       labels, min_d2, ntiles, fsum, fcnt, flags, range_bits);
+                       labels, min_d2, ntiles, fsum, fcnt, flags, range_bits, fused_replicas(D, K));
     prof_end(st);
     return check_launch("lloyd_mfma_resident_kernel");
 }
