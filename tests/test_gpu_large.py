@@ -149,12 +149,31 @@ def test_narrow_one_sweep_beyond_4gib(cuda):
     assert torch.equal(lab, lab2)
 
 
-def test_generic_vector_kernel_beyond_4gib(cuda):
-    """D <= 16 outside the one-sweep limits."""
+def test_narrow_rows_on_the_matrix_cores_beyond_4gib(cuda):
+    """4 <= D <= 16 outside the narrow kernel's limits: the matrix-core kernels with the features padded to 16."""
     x, c = _blobs(100_000_000, 12, 64, cuda, 45)
     lab, md = _assign_whole_equals_slices(x, c, cuda)
     _gap_rule(x, c, _probe_rows(*x.shape, cuda), lab, md)
-    lab2 = _step_matches_its_labels(x, c, cuda, _native.lloyd_kernel_name(*x.shape, 64))
+    lab2 = _step_matches_its_labels(x, c, cuda, "lloyd_mfma_resident")
+    assert torch.equal(lab, lab2)
+
+
+def test_narrow_one_sweep_with_integer_sums_beyond_4gib(cuda):
+    """One-sweep vector kernel beyond 48 accumulator slots at a size where it takes the integer sums by itself
+    (and, with 16 centroids of 8 coordinates, the cross terms from the matrix cores)."""
+    x, c = _blobs(150_000_000, 8, 16, cuda, 46)
+    lab, md = _assign_whole_equals_slices(x, c, cuda)
+    _gap_rule(x, c, _probe_rows(*x.shape, cuda), lab, md)
+    lab2 = _step_matches_its_labels(x, c, cuda, "lloyd_small")
+    assert torch.equal(lab, lab2)
+
+
+def test_generic_vector_kernel_beyond_4gib(cuda):
+    """Fewer than 4 features outside the narrow kernel's limits: vector assignment + two-pass update."""
+    x, c = _blobs(600_000_000, 2, 100, cuda, 47)
+    lab, md = _assign_whole_equals_slices(x, c, cuda)
+    _gap_rule(x, c, _probe_rows(*x.shape, cuda), lab, md)
+    lab2 = _step_matches_its_labels(x, c, cuda, "valu+update")
     assert torch.equal(lab, lab2)
 
 
