@@ -16,4 +16,4 @@ from .core import types, devices, communication, factories, base, dndarray  # no
 from . import classification, cluster, graph, spatial, utils  # noqa: F401
 from . import _native  # noqa: F401
 
-__version__ = "0.3.1"  # = hkm_version() of the library this binding was written for (_native.LIB_VERSION)
+__version__ = "0.3.2"  # = hkm_version() of the library this binding was written for (_native.LIB_VERSION)

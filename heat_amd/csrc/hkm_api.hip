@@ -275,7 +275,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 301; }
+int hkm_version(void) { return 302; }
 
 const char* hkm_last_error(void) { return g_err; }
 

@@ -38,7 +38,7 @@ int main() {
     void* const ws = reinterpret_cast<void*>(uintptr_t(1) << 20);
     const size_t big = size_t(1) << 30;
 
-    if (hkm_version() < 301) {
+    if (hkm_version() < 302) {
         std::printf("FAIL version %d\n", hkm_version());
         ++failures;
     }
