@@ -490,28 +490,41 @@ int hkm_tune_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, c
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
         return fail(HKM_EUNSUPPORTED, "hkm_tune_lloyd_step_f32 waits for the device and cannot run under stream capture");
-    hipEvent_t ev[2][2];
+    // Three windows -- two point blocks, one, two again -- each after a warm-up of its own, and the one-block
+    // window is compared with the SECOND two-block window: a device that was idle needs some 30 ms of load to
+    // reach its clock (the first window would lose for that alone), and a chip that lowers its clock under one
+    // geometry has done so 20 ms into it.  Windows are sized in time: a few steps are timed first.
+    hipEvent_t ev[4][2];
     for (auto& pair : ev)
         for (auto& e : pair)
             if (hipEventCreate(&e) != hipSuccess) return fail(HKM_EHIP, "hipEventCreate failed");
-    const int WARM = 10, TIMED = 10;  // a chip that lowers its clock under a kernel does so within milliseconds
-    float ms[3] = {0.f, 0.f, 0.f};
-    for (int pb = 2; pb >= 1 && !rc; --pb) {
+    auto run = [&](int pb, int steps, hipEvent_t e0, hipEvent_t e1) {
         force_point_blocks(pb);
-        for (int i = 0; i < WARM + TIMED && !rc; ++i) {
-            if (i == WARM) (void)hipEventRecord(ev[pb - 1][0], st);
+        if (e0) (void)hipEventRecord(e0, st);
+        for (int i = 0; i < steps && !rc; ++i)
             rc = hkm_lloyd_step_f32(X, N, D, ldx, C, C_new, K, labels, shift, sse, ws, ws_bytes, hip_stream);
-        }
-        (void)hipEventRecord(ev[pb - 1][1], st);
-    }
+        if (e1) (void)hipEventRecord(e1, st);
+    };
+    auto elapsed = [&](hipEvent_t e0, hipEvent_t e1, float& ms) {
+        if (!rc && (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess))
+            rc = fail(HKM_EHIP, "timing the trial steps failed");
+    };
+    float est = 0.f;
+    run(2, 5, ev[0][0], ev[0][1]);
+    elapsed(ev[0][0], ev[0][1], est);
+    const float step_ms = est > 0.f ? est / 5.f : 1.f;
+    const int warm = std::min(2000, std::max(25, int(35.f / step_ms) + 1));
+    const int timed = std::min(2000, std::max(20, int(25.f / step_ms) + 1));
+    float ms[3] = {0.f, 0.f, 0.f};  // [1], [2]: per-step time with one / two point blocks
+    run(2, warm, nullptr, nullptr);
+    run(2, timed, ev[1][0], ev[1][1]);
+    run(1, warm, nullptr, nullptr);
+    run(1, timed, ev[2][0], ev[2][1]);
+    run(2, warm, nullptr, nullptr);
+    run(2, timed, ev[3][0], ev[3][1]);
     force_point_blocks(0);
-    if (!rc) {
-        for (int pb = 1; pb <= 2 && !rc; ++pb) {
-            if (hipEventSynchronize(ev[pb - 1][1]) != hipSuccess ||
-                hipEventElapsedTime(&ms[pb], ev[pb - 1][0], ev[pb - 1][1]) != hipSuccess)
-                rc = fail(HKM_EHIP, "timing the trial steps failed");
-        }
-    }
+    elapsed(ev[2][0], ev[2][1], ms[1]);
+    elapsed(ev[3][0], ev[3][1], ms[2]);
     for (auto& pair : ev)
         for (auto& e : pair) (void)hipEventDestroy(e);
     if (rc) return rc;

@@ -376,9 +376,9 @@ int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_s
  * or one with twice the waves -- that produce the same bits and differ in speed by a few percent either way,
  * depending on the clock the individual chip holds under them.  No counterpart in the reference.
  * hkm_tune_lloyd_step_f32: hkm_lloyd_step_f32 with the same arguments and the same results, which -- where the
- *   shape has the choice and HKM_POINT_BLOCKS is not set -- then runs the same step twenty more times in
- *   either geometry, WAITS for the device, and remembers the faster geometry for the current device until the
- *   process ends.  Returns the point blocks chosen (1 or 2), 0 if the shape has no choice, or a negative
+ *   shape has the choice and HKM_POINT_BLOCKS is not set -- then runs the same step for about 0.2 s more (two
+ *   point blocks, one, two again, each window after a warm-up of its own, sized in time), WAITS for the
+ *   device, and remembers the faster geometry for the current device until the process ends.  Returns the point blocks chosen (1 or 2), 0 if the shape has no choice, or a negative
  *   error; refused under stream capture.  Not calling it leaves the default (two).
  * hkm_point_blocks: the point blocks per wave a call with D features would use now (0: D has no resident
  *   kernel); *tuned (if not NULL) tells whether that came from a measurement on the current device.
