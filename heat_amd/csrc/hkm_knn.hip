@@ -83,7 +83,7 @@ __device__ __forceinline__ void knn_insert_in_place(float (&ld)[KL], unsigned (&
 
 template <int KL>
 __device__ __forceinline__ void knn_offer(float (&ld)[KL], unsigned (&li)[KL], bool ok, float d, unsigned i) {
-    if (__builtin_amdgcn_ballot_w64(ok) != 0) knn_insert_in_place<KL>(ld, li, ok ? d : HKM_INF, i);
+    if (__builtin_amdgcn_ballot_w64(ok) != 0) knn_insert_in_place(ld, li, ok ? d : HKM_INF, i);
 }
 
 template <int KL>
@@ -254,6 +254,21 @@ __device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (
         if (__builtin_amdgcn_ballot_w64(dmin < thr) == 0) return;
     }
     const unsigned gj0 = unsigned(j0) + 4 * h;
+    if (!edge) {
+        // The common tile.  An element is first tested without the clamp (t + |q|^2 < thr: one addition, one
+        // compare); the clamp only raises negative values to 0, so whatever passes the clamped test passes this
+        // one, and the few that pass it are clamped and tested again before they are offered.  A NaN fails both.
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float s = t[i] + qn;
+            if (__builtin_amdgcn_ballot_w64(s < thr) != 0) {
+                const float d = s < 0.0f ? 0.0f : s;
+                knn_insert_in_place(ld, li, d < thr ? d : HKM_INF, gj0 + 8 * (i >> 2) + (i & 3));
+            }
+        }
+        thr = knn_threshold<KL>(ld, kcount);
+        return;
+    }
     float dv[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -262,16 +277,13 @@ __device__ __forceinline__ void knn_block_candidates(float (&ld)[KL], unsigned (
         const float s = t[i] + qn;
         dv[i] = s < 0.0f ? 0.0f : s;
     }
-    if (edge) {
-        // rows past the end and pairs that do not rank after the bound become +inf here, so that one chain
-        // of offers serves every tile
+    // rows past the end and pairs that do not rank after the bound become +inf here
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const unsigned gj = gj0 + 8 * (i >> 2) + (i & 3);
-            bool ok = gj < unsigned(r_end);
-            if (has_bound) ok = ok && (dv[i] > bd || (dv[i] == bd && gj > bi));
-            dv[i] = ok ? dv[i] : HKM_INF;
-        }
+    for (int i = 0; i < 16; ++i) {
+        const unsigned gj = gj0 + 8 * (i >> 2) + (i & 3);
+        bool ok = gj < unsigned(r_end);
+        if (has_bound) ok = ok && (dv[i] > bd || (dv[i] == bd && gj > bi));
+        dv[i] = ok ? dv[i] : HKM_INF;
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) knn_offer<KL>(ld, li, dv[i] < thr, dv[i], gj0 + 8 * (i >> 2) + (i & 3));
@@ -677,7 +689,8 @@ int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N
     if (M == 0) return HKM_OK;
     const KnnPlan p = knn_plan(M, N, knn_target_workgroups(D));
     const bool mfma = knn_uses_mfma(D);
-    const int KL = mfma ? (k <= 8 ? 8 : 16) : (k <= 4 ? 4 : (k <= 8 ? 8 : 16));
+    // list length: the smallest instantiated one that holds k (an insertion costs five instructions per slot)
+    const int KL = mfma ? (k <= 6 ? 6 : k <= 8 ? 8 : 16) : (k <= 4 ? 4 : (k <= 8 ? 8 : 16));
     int rc;
     if (mfma) {
         hipLaunchKernelGGL(knn_norms_kernel, dim3((unsigned)((N + 15) / 16)), dim3(256), 0, st, X, N, ldx, D, xn);
@@ -693,7 +706,12 @@ int launch_knn(const float* Q, int64_t M, int64_t ldq, const float* X, int64_t N
                              dist, ldd, col0, kcount, st)
         if (mfma) {
             const int H = D <= 16 ? 8 : (D <= 32 ? 16 : (D <= 64 ? 32 : 64));
-            if (KL == 8) {
+            if (KL == 6) {
+                if (H == 8) HKM_KNN_MFMA(6, 8);
+                else if (H == 16) HKM_KNN_MFMA(6, 16);
+                else if (H == 32) HKM_KNN_MFMA(6, 32);
+                else HKM_KNN_MFMA(6, 64);
+            } else if (KL == 8) {
                 if (H == 8) HKM_KNN_MFMA(8, 8);
                 else if (H == 16) HKM_KNN_MFMA(8, 16);
                 else if (H == 32) HKM_KNN_MFMA(8, 32);
