@@ -14,7 +14,7 @@ centroids that iteration started from -- the same kernel code, hence the same bi
 returned are exactly those of the sequential loop.
 
 The stop decision.  The two one-sweep kernels form their per-cluster sums on the way (rows pre-rounded
-to 28 bits below their largest coordinate on the matrix cores; fp32 partial sums per lane, or rows rounded
+to 28 bits below their largest coordinate, or below a floor taken from the centroid norms, on the matrix cores; fp32 partial sums per lane, or rows rounded
 to 32 bits below the largest centroid coordinate, in the narrow kernel), so their means can differ from the fp64 divide-then-sum of heat/cluster/kmeans.py:76-103 in the
 last bit.  That is far inside the 1e-4 bar on the centroids but it decides ``shift <= tol`` when the shift
 is (nearly) zero: a fit sitting on a fixed point of the reference's arithmetic would run one iteration

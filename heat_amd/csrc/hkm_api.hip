@@ -94,12 +94,14 @@ AssignKind assign_kind(int32_t D, int32_t K) {
     return ASSIGN_MFMA_STREAM;
 }
 
-// The one-sweep MFMA step needs the centroids, fp64 accumulators and counts of a workgroup in LDS.  From 4
+// The one-sweep MFMA step needs the centroids, fp64 accumulators and counts of a workgroup in LDS.  From 2
 // features on it is taken whatever K is: what it replaces for narrow rows is the vector assignment PLUS the
-// two-pass update, and reading X once beats that 3x or more even with a single centroid (10M x 16: 0.22 against
-// 1.84 ms at K = 1, 0.24 against 0.79 ms at K = 16).  Below 4 features the two passes stay ahead.
+// two-pass update, and reading X once beats that 2-3x even with a single centroid or with three quarters of
+// the matrix work spent on padding (10M x 16: 0.22 against 1.84 ms at K = 1, 0.24 against 0.79 ms at K = 16;
+// 10M x 2, K = 90: 0.28 against 0.55 ms; 10M x 3, K = 256: 0.52 against 0.91 ms).  One feature stays on the
+// two passes (0.57 ms at K = 130; with 130 centroids on a line the two arithmetics part on a thousand ties).
 bool fused_eligible(int32_t D, int32_t K) {
-    return D >= 4 && D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
+    return D >= 2 && D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
 }
 
 static size_t cn_pad(int32_t K) { return (size_t(K) + 127) / 128 * 128; }

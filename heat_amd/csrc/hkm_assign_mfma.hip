@@ -1,5 +1,5 @@
-// Fused distance + argmin on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), for D >= 4 (up to 16 features
-// only from 32 centroids on; the one-sweep step whatever K is).
+// Fused distance + argmin on the fp32 matrix cores (v_mfma_f32_32x32x2_f32): the assignment alone for D >= 4
+// (up to 16 features only from 32 centroids on), the one-sweep step for D >= 2 whatever K is.
 //
 // Operand roles: the A operand (M = 32 rows) carries CENTROIDS, the B operand (N = 32 columns)
 // carries POINTS.  In the 32x32 accumulator a lane then owns one point (column lane%32) and 16
@@ -261,7 +261,8 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 // B_i = 1.5 * 2^52 * q_i.  All addends of a workgroup are then multiples of 2^(Emin - 28) and every
 // partial sum is below n_wg * 2^Emax, so as long as Emax - Emin <= 53 - 28 - ceil(log2 n_wg) every
 // addition is exact in fp64 and the result does not depend on the order.  The rounding keeps 28 bits
-// below the row's largest coordinate (error <= 2^-29 of it per addend).  A workgroup whose rows
+// below the row's largest coordinate (error <= 2^-29 of it per addend) -- or below a floor derived from the
+// centroid norms, for rows far smaller than the centroids (see e_floor in the kernel).  A workgroup whose rows
 // violate the range condition, or hold a row whose |x|^2 is inf or NaN (coordinates above 1.8e19 or
 // non-finite ones: the bound 2^E is then meaningless), raises its flag; the step then falls back to
 // the two-pass update, whose kernels start by looking at the flags.
@@ -328,7 +329,8 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
     // number of doubles apart so that the copies of a row start in different banks.
     const size_t rstride = size_t(K) * LDA + 1;
     double* sA = reinterpret_cast<double*>(sCn + KP);             // [nrep][K][LDA] (+ 1 pad per copy)
-    int* sN = reinterpret_cast<int*>(sA + nrep * rstride);        // [nrep][K] counts, then Emin, Emax, non-finite
+    int* sN = reinterpret_cast<int*>(sA + nrep * rstride);        // [nrep][K] counts, then Emin, Emax, non-finite,
+                                                                  // largest / smallest non-zero centroid norm
     int* sMeta = sN + nrep * K;
     const int tid = threadIdx.x, nthr = blockDim.x;
 
@@ -351,8 +353,33 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
         sMeta[0] = 0x7fffffff;
         sMeta[1] = -0x7fffffff;
         sMeta[2] = 0;
+        sMeta[3] = 0;
+        sMeta[4] = 0x7fffffff;
     }
     __syncthreads();
+    // The squared centroid norms (bits of non-negative floats order like integers) give the rows' expected
+    // magnitude, the same for every workgroup: a row at the largest centroid would get the exponent e_ref
+    // below.  Rows up to 2^head times larger still fit the exact range; rows whose own exponent lies below
+    // e_floor = e_ref + head - range_bits are rounded to the quantum of e_floor instead of their own, so that
+    // a few rows near the origin -- the rule in two or three dimensions -- no longer cost the exact path.
+    // The floor never rises more than 4 above the exponent of the SMALLEST non-zero centroid norm: the sums
+    // of that cluster, too, keep 24 bits below its centroid's magnitude (centroids whose norms span more than
+    // the exact range leave the rows of the large ones outside it, and the step falls back as before).
+    for (int r = tid; r < K; r += nthr) {
+        const int b = __float_as_int(sCn[r]) & 0x7fffffff;
+        atomicMax(&sMeta[3], b);
+        if (b != 0) atomicMin(&sMeta[4], b);
+    }
+    __syncthreads();
+    int e_floor = -0x3fffffff;  // no usable centroid norm (all zero, inf, NaN): every row keeps its own quantum
+    {
+        const int cexp = (sMeta[3] >> 23) & 0xff, cexp_min = (sMeta[4] >> 23) & 0xff;
+        if (cexp != 0 && cexp != 255) {
+            const int e_ref = ((cexp - 127) >> 1) + 2, e_min = ((cexp_min - 127) >> 1) + 2;
+            const int head = range_bits < 4 ? (range_bits < 0 ? 0 : range_bits) : 4;
+            e_floor = min(e_ref + head - range_bits, e_min + 4);
+        }
+    }
 
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), nw = nthr >> 6;
     const int p = lane & 31, h = lane >> 5;
@@ -404,7 +431,7 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
                 // |x_d| < 2^E: |x|^2 < 2^(e2+1) up to rounding, one more bit of slack
                 const int e2 = (__float_as_int(xnr[pb]) >> 23) - 127;
                 nonfinite |= int((e2 & 0xff) == 128);  // exponent field 255 (the sign bit of |x|^2 is clear or NaN)
-                const int E = (e2 >> 1) + 2;
+                const int E = max((e2 >> 1) + 2, e_floor);
                 emin = min(emin, E);
                 emax = max(emax, E);
                 const double B = __hiloint2double(((1023 + 52 - FUSED_QBITS + E) << 20) | 0x80000, 0);
@@ -811,7 +838,7 @@ static size_t fused_lds_bytes_with(int32_t D, int32_t K, int nrep) {
     const size_t kp = (size_t(K) + 31) / 32 * 32;
     const int dp = resident_dp(D);
     return kp * (dp + 5) * sizeof(float) + size_t(nrep) * (size_t(K) * (dp + 1) + 1) * sizeof(double) +
-           (size_t(nrep) * K + 4) * sizeof(int);
+           (size_t(nrep) * K + 8) * sizeof(int);
 }
 
 // Copies of the fp64 accumulators in the one-sweep kernel: up to 64 clusters, as many as bring the lanes

@@ -330,9 +330,10 @@ def test_tuning_call_is_a_step_and_settles_on_a_geometry(cuda, monkeypatch):
     assert _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws) == 0
 
 
-@pytest.mark.parametrize("n,d,k", [(30000, 16, 8), (20000, 9, 1), (25000, 12, 20), (10000, 10, 3), (40000, 4, 50), (30000, 7, 31)])
+@pytest.mark.parametrize("n,d,k", [(30000, 16, 8), (20000, 9, 1), (25000, 12, 20), (10000, 10, 3), (40000, 4, 50), (30000, 7, 31),
+                                   (50000, 2, 90), (40000, 3, 256), (30000, 3, 70)])
 def test_one_sweep_mfma_step_with_few_centroids_and_narrow_rows(cuda, n, d, k):
-    # From 4 features on the step runs on the matrix cores whatever K is, while the assignment alone stays
+    # From 2 features on the step runs on the matrix cores whatever K is, while the assignment alone stays
     # on the vector kernel below 32 centroids: the two may break a tie at the resolution of the formula
     # differently, so the step is checked against the oracle, and its means against its own labels.
     assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
@@ -349,6 +350,27 @@ def test_one_sweep_mfma_step_with_few_centroids_and_narrow_rows(cuda, n, d, k):
     cnt = torch.bincount(lab.long(), minlength=k).clamp(min=1).double().unsqueeze(1)
     assert (c_step.cpu() - (ref / cnt).float()).abs().max() <= 2e-7 * float(x.abs().max())
     assert orc.rel_err_scalar(float(shift), float(orc.centroid_shift(c0, c_step.cpu())), floor=1e-12) <= 1e-5
+
+
+@pytest.mark.parametrize("n,d,k", [(60000, 2, 90), (50000, 4, 60), (40000, 32, 64)])
+def test_one_sweep_mfma_step_keeps_its_exact_sums_with_rows_near_the_origin(cuda, n, d, k):
+    # Rows far smaller than the centroids -- the rule in two or three dimensions, where a blob around the origin
+    # has points at any distance from it -- are rounded to a quantum derived from the largest centroid norm
+    # instead of their own, so they no longer break the range in which the fp64 sums are exact: the step stays
+    # on its own sums (equal to the fp64 means, which the fp32 partials of the two-pass update only approximate).
+    x, _ = _data(n, d, k, seed=13 * n + d)
+    g = torch.Generator().manual_seed(9)
+    tiny = torch.randperm(n, generator=g)[: n // 50]
+    x[tiny] *= torch.pow(2.0, -torch.randint(10, 40, (tiny.numel(), 1), generator=g).float())
+    c0 = _data(n, d, k, seed=13 * n + d)[0][torch.randperm(n, generator=g)[:k]].contiguous()
+    xs, cs = x.to(cuda), c0.to(cuda)
+    c_step, lab_step, shift, c2, lab2, cnt2 = _step_and_two_pass(xs, cs, cuda)
+    lab = lab_step.cpu()
+    ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab.long(), x.double())
+    cnt = torch.bincount(lab.long(), minlength=k).clamp(min=1).double().unsqueeze(1)
+    assert (c_step.cpu() - (ref / cnt).float()).abs().max() <= 1.2e-7 * float(c0.abs().max())
+    again = _step_and_two_pass(xs, cs, cuda)
+    assert torch.equal(again[0], c_step) and torch.equal(again[2], shift)
 
 
 def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):

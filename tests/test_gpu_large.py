@@ -168,13 +168,17 @@ def test_narrow_one_sweep_with_integer_sums_beyond_4gib(cuda):
     assert torch.equal(lab, lab2)
 
 
-def test_generic_vector_kernel_beyond_4gib(cuda):
-    """Fewer than 4 features outside the narrow kernel's limits: vector assignment + two-pass update."""
+def test_two_features_on_the_matrix_cores_beyond_4gib(cuda):
+    """Fewer than 4 features outside the narrow kernel's limits: the assignment alone on the generic vector
+    kernel, the step on the matrix cores (features padded to 8); the two may part on ties, so each is held to
+    the gap rule."""
     x, c = _blobs(600_000_000, 2, 100, cuda, 47)
     lab, md = _assign_whole_equals_slices(x, c, cuda)
-    _gap_rule(x, c, _probe_rows(*x.shape, cuda), lab, md)
-    lab2 = _step_matches_its_labels(x, c, cuda, "valu+update")
-    assert torch.equal(lab, lab2)
+    rows = _probe_rows(*x.shape, cuda)
+    _gap_rule(x, c, rows, lab, md)
+    lab2 = _step_matches_its_labels(x, c, cuda, "lloyd_mfma_resident")
+    _gap_rule(x, c, rows, lab2)
+    assert int((lab != lab2).sum()) <= x.shape[0] // 100_000
 
 
 def test_manhattan_beyond_4gib(cuda):
