@@ -29,6 +29,9 @@ roofline   the dominant kernel -- the fused distance+argmin kernel, or the one-s
            were when it was measured (traffic_source says which)
 cpu_baseline  the CPU restatement of the reference's op sequence (oracle/, torch CPU, all host
            threads) on a bounded row sample of the same workload
+
+--shape N D K times the same loop on K equal blobs of any shape (the lines of profiles/bench_other_shapes.jsonl);
+such a line has no CPU baseline and no traffic figure and is no headline number.
 """
 import argparse
 import json
@@ -471,6 +474,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink N (testing only; invalidates the figure)")
+    ap.add_argument("--shape", type=int, nargs=3, metavar=("N", "D", "K"), default=None,
+                    help="time the Lloyd step on K equal blobs of this shape instead of a named workload "
+                         "(not a headline figure: no CPU baseline, no traffic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--probe", action="store_true",
                     help="run the hardware microbenchmarks (matrix-pipe throughput alone and with interleaved "
@@ -498,7 +504,11 @@ def main() -> int:
     dev = torch.device("cuda:0")
 
     t_gen = time.perf_counter()
-    w = synthetic.CONFIGS[args.config](args.scale)
+    if args.shape:
+        args.config, args.no_cpu_baseline = "shape", True
+        w = synthetic.shape(*args.shape)
+    else:
+        w = synthetic.CONFIGS[args.config](args.scale)
     t_gen = time.perf_counter() - t_gen
     n, d = w.x.shape
     k = w.k
@@ -600,7 +610,9 @@ def main() -> int:
     nbytes = float(n) * (4 * d + 4) if args.config != "c2" else float(n) * (4 * d + 8) + 4.0 * k * d
     tf = flops / (kern_ms * 1e-3) / 1e12
     gbs = nbytes / (kern_ms * 1e-3) / 1e9
-    if args.config in MFMA_BOUND:
+    # a free shape is priced against the matrix pipe where the matrix cores run it, against HBM otherwise
+    mfma_bound = args.config in MFMA_BOUND or (args.config == "shape" and kernel.startswith(("lloyd_mfma", "mfma")))
+    if mfma_bound:
         roof = {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}
     else:
@@ -619,7 +631,7 @@ def main() -> int:
         pb, tuned = _native.point_blocks(d)
         roof["point_blocks_per_wave"] = pb
         roof["point_blocks_measured_here"] = tuned
-    if args.config in MFMA_BOUND:
+    if mfma_bound:
         roof["mfma_alone_tflops_this_chip"] = round(mfma_alone_tflops(), 1)
     roof["traffic"] = None
     roof["traffic_source"] = "none: profiles/traffic.json is missing"

@@ -133,6 +133,17 @@ def config5(scale: float = 1.0) -> Workload:
     return Workload("c5_n200m_d3_k8", x, x[pick].clone(), None, k, 10, seed)
 
 
+def shape(n: int, d: int, k: int, seed: int = 1100) -> Workload:
+    """Any (N, D, K): K equal blobs, centres U[-10,10]^D, sigma 1, shuffled; init = first K rows.  For timing
+    shapes between the five workloads (``bench.py --shape N D K``)."""
+    gen = torch.Generator().manual_seed(seed)
+    centres = torch.rand((k, d), generator=gen) * 20.0 - 10.0
+    sizes = torch.full((k,), n // k, dtype=torch.int64)
+    sizes[: n - int(sizes.sum())] += 1
+    x = _shuffle(_blobs(sizes, centres, torch.ones((k, 1)), gen), gen)
+    return Workload(f"shape_n{n}_d{d}_k{k}", x, x[:k].clone(), None, k, 20, seed)
+
+
 CONFIGS = {"c1": config1, "c2": config2, "c3": config3, "c4": config4, "c5": config5}
 
 
