@@ -7,7 +7,11 @@ host waits for the shift of step i: if the loop goes on (the usual case) the GPU
 stops the extra step is simply not used -- it writes to buffers the results of step i do not live
 in (three centroid buffers, two label buffers, two shift scalars in rotation).  The shift scalars
 live in pinned host memory and are written by the finishing kernel itself, so no copy-engine
-operation sits between two steps on the stream.  For the narrow shapes whose step is one sweep of a
+operation sits between two steps on the stream -- and no event either: before a step is enqueued its
+scalar is set to a value no shift can take (-1: a shift is a sum of squares or NaN), and the host
+waits for the step by reading the scalar until it has changed.  For a step of a few microseconds the
+record and the wait of an event were a third of the host's time per iteration, and the host is what
+bounds such fits.  For the narrow shapes whose step is one sweep of a
 vector kernel (D <= 8), writing N labels is a quarter of the step's memory traffic, so the steps run
 without storing labels and those of the last iteration are computed once, on demand, against the
 centroids that iteration started from -- the same kernel code, hence the same bits.  The values
@@ -28,11 +32,14 @@ shift.  If the loop goes on, the step enqueued ahead is re-issued from the recom
 from __future__ import annotations
 
 import os
+import time
 from typing import Optional
 
 import torch
 
 from .. import _native
+
+_PENDING = -1.0  # what a shift scalar holds while its step has not delivered: no sum of squares is negative
 
 
 class LloydLoop:
@@ -54,7 +61,8 @@ class LloydLoop:
         self.lab = [torch.empty((n,), dtype=torch.int32, device=dev) for _ in range(nbuf)]
         self._lab_of = -1  # iteration whose labels self.lab[0] holds (lazy mode)
         self.shift_host = torch.zeros((2,), dtype=xt.dtype, pin_memory=True)
-        self.ev = [torch.cuda.Event(), torch.cuda.Event()]
+        self._shift_np = self.shift_host.numpy()  # the same two scalars, read without building a tensor
+        self._free_running = False  # steps were enqueued that nobody waited for (tol is None)
         self.enqueued = 0  # steps handed to the stream
         self.done = 0      # steps whose results count
         self._plans = {}   # prepared calls, one per rotation of the buffers (and stream)
@@ -76,28 +84,47 @@ class LloydLoop:
                                               None if self.lazy_labels else self.lab[j % 2],
                                               self.shift_host[j % 2], None, self.ws)
             self._plans[key] = plan
+        self._shift_np[j % 2] = _PENDING
         plan()
-        self.ev[j % 2].record()
         self.enqueued = j + 1
+
+    def _wait(self, i: int) -> float:
+        """The shift of step i, once its finishing kernel has written it."""
+        slot = i % 2
+        spins = 0
+        while self._shift_np[slot] == _PENDING:
+            spins += 1
+            if spins == 1 << 16:
+                t0 = time.monotonic()
+            elif spins > 1 << 16 and (spins & 0xFFF) == 0 and time.monotonic() - t0 > 60.0:
+                torch.cuda.current_stream().synchronize()  # raises what the device has to report
+                if self._shift_np[slot] == _PENDING:
+                    raise RuntimeError(f"Lloyd step {i} finished without delivering its centroid shift")
+        return float(self._shift_np[slot])
 
     def run(self, max_iter: int, tol: Optional[float]) -> int:
         """Up to ``max_iter`` further iterations; stops after the first whose shift is <= tol
         (never if ``tol`` is None, and then without any host read).  Returns the number run."""
         ran = 0
+        if tol is not None and self._free_running:
+            # steps nobody waited for may still be on their way and write the two scalars after a later step
+            # has marked them pending
+            torch.cuda.current_stream().synchronize()
+            self._free_running = False
         for _ in range(max_iter):
             i = self.done
             if self.enqueued == i:
                 self._enqueue()
             if tol is None:
+                self._free_running = True
                 self.done = i + 1
                 ran += 1
                 continue
             if ran + 1 < max_iter and self.enqueued == i + 1:
                 self._enqueue()  # ahead of the host's look at step i
-            self.ev[i % 2].synchronize()
+            shift = self._wait(i)
             self.done = i + 1
             ran += 1
-            shift = float(self.shift_host[i % 2])
             if self._fuzz and shift <= tol + self._margin(tol):
                 shift = self._recompute(i)
             if shift <= tol:
@@ -124,9 +151,8 @@ class LloydLoop:
         _native.update(self.x, lab, self.c[(i + 1) % 3], None, self.ws)
         out = torch.empty((), dtype=self.x.dtype, device=self.x.device)
         _native.shift(self.c[i % 3], self.c[(i + 1) % 3], out)
-        self.shift_host[i % 2] = out.cpu()  # synchronises
-        self.ev[i % 2].record()
-        self.enqueued = i + 1  # a step enqueued ahead started from the centroids just replaced
+        self.shift_host[i % 2] = out.cpu()  # synchronises: a step enqueued ahead has run and written its scalar
+        self.enqueued = i + 1  # that step started from the centroids just replaced
         self.rechecks += 1
         return float(self.shift_host[i % 2])
 
@@ -150,5 +176,5 @@ class LloydLoop:
     def last_shift(self) -> torch.Tensor:
         """0-d device tensor; waits for the step that produced it."""
         i = self.done - 1
-        self.ev[i % 2].synchronize()
+        torch.cuda.current_stream().synchronize()
         return self.shift_host[i % 2].to(self.x.device)
