@@ -301,6 +301,16 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
     b = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
     assert b.run(7, None) == 7
     assert torch.equal(a.centers, b.centers) and torch.equal(a.labels, b.labels)
+    # steps nobody waited for, then steps whose shift the host reads (it recognises a finished step by its
+    # pinned scalar having left the "pending" value, so the earlier ones must not write into it late):
+    # many times over, the shifts read must be those of a loop that waited from the start
+    c = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
+    d = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
+    for _ in range(20):
+        assert c.run(25, None) == 25 and d.run(25, -1.0) == 25
+        assert c.run(1, -1.0) == 1 and d.run(1, -1.0) == 1
+        assert float(c.last_shift) == float(d.last_shift)
+    assert torch.equal(c.centers, d.centers)
     with pytest.raises(ValueError):
         ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(cuda)), max_iter=0).fit(ht.array(x, split=0))
 
