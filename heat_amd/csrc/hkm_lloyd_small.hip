@@ -214,7 +214,8 @@ __device__ __forceinline__ void scan_centroids_sload(const float* __restrict__ C
     float best[PPT];
 #pragma unroll
     for (int p = 0; p < PPT; ++p) best[p] = CLAMP ? m[p] : -0.5f * m[p];
-#pragma unroll(PPT == 2 ? 4 : 2)
+    constexpr int UNROLL_K = PPT == 2 ? 4 : 2;  // centroid rows in flight: bounded by the scalar registers
+#pragma unroll UNROLL_K
     for (int k = k0; k < k1; ++k) {
         const float* ck = C + int64_t(k) * ldc;
         float c[D];
