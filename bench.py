@@ -42,18 +42,21 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# the sources whose code runs in the five clustering workloads (dispatch, the assignment / one-sweep /
-# update kernels and what they include); the other kernels of the library move none of their bytes
-TRAFFIC_SOURCES = ("hkm_api.hip", "hkm_common.h", "hkm_mfma_util.h", "hkm_assign_valu.hip", "hkm_assign_mfma.hip",
-                   "hkm_assign_split.hip", "hkm_lloyd_small.hip", "hkm_update.hip", "hkm_update_sorted.hip")
+# The sources whose code runs in each clustering workload: dispatch and shared headers, then the file of the
+# workload's kernels (the narrow one-sweep kernel for c1 and c5, the matrix-core kernels for c2-c4, with
+# the two-pass update c4 runs and c3 falls back to).  A counter reading is tied to these.
+_SHARED_SOURCES = ("hkm_api.hip", "hkm_common.h", "hkm_mfma_util.h")
+_MFMA_SOURCES = _SHARED_SOURCES + ("hkm_assign_mfma.hip", "hkm_update.hip", "hkm_update_sorted.hip")
+WORKLOAD_SOURCES = {"c1": _SHARED_SOURCES + ("hkm_lloyd_small.hip",), "c5": _SHARED_SOURCES + ("hkm_lloyd_small.hip",),
+                    "c2": _SHARED_SOURCES + ("hkm_assign_mfma.hip",), "c3": _MFMA_SOURCES, "c4": _MFMA_SOURCES}
 
 
-def library_sources_sha1() -> str:
-    """Hash of the HIP sources behind the five workloads' kernels: ties a committed counter reading to the code."""
+def workload_sources_sha1(config: str) -> str:
+    """Hash of the HIP sources behind one workload's kernels: ties a committed counter reading to the code."""
     import hashlib
 
     h = hashlib.sha1()
-    for name in TRAFFIC_SOURCES:
+    for name in WORKLOAD_SOURCES[config]:
         with open(os.path.join(ROOT, "heat_amd", "csrc", name), "rb") as fh:
             h.update(name.encode() + b"\0" + fh.read())
     return h.hexdigest()[:12]
@@ -639,15 +642,19 @@ def main() -> int:
     if os.path.exists(tfile):
         with open(tfile) as f:
             tj = json.load(f)
-        sha = library_sources_sha1()
-        if tj.get("sources_sha1") == sha and args.scale == 1.0:
-            roof["traffic"] = tj.get(w.name)
-            roof["traffic_source"] = f"profiles/traffic.json, measured on library sources sha1 {sha} (= this build)"
+        sha = workload_sources_sha1(args.config) if args.config in WORKLOAD_SOURCES and not args.shape else None
+        measured_on = (tj.get("sources_sha1") or {}).get(w.name)
+        if sha is None:
+            roof["traffic_source"] = "none: profiles/traffic.json holds the five named workloads only"
         elif args.scale != 1.0:
             roof["traffic_source"] = "dropped: profiles/traffic.json holds the unscaled workloads only"
+        elif measured_on == sha:
+            roof["traffic"] = tj.get(w.name)
+            roof["traffic_source"] = (f"profiles/traffic.json, measured on this workload's kernel sources "
+                                      f"sha1 {sha} (= this build)")
         else:
-            roof["traffic_source"] = (f"dropped: profiles/traffic.json was measured on library sources sha1 "
-                                      f"{tj.get('sources_sha1')}, this build is {sha}")
+            roof["traffic_source"] = (f"dropped: profiles/traffic.json was measured on kernel sources sha1 "
+                                      f"{measured_on}, this build is {sha}")
 
     # Not the headline: the same timed loop with the opt-in split-bf16 products (HKM_PRODUCTS=bf16x3;
     # every product still accurate to fp32, evaluated as six bf16 partial products on the bf16 matrix

@@ -5,7 +5,8 @@
 // wave-uniform operands -- LDS broadcasts of rows scaled by -2 (exact), or, where a row is one scalar load,
 // scalar registers filled straight from C (scan_centroids_sload); 12 to 16 centroids of 4 or 8 coordinates
 // are instead one A operand of v_mfma_f32_16x16x4_f32 and the minimum is found in registers after a
-// transpose across the lanes (the matrix-core scan in the kernel body).  The quadratic expansion of
+// transpose across the lanes (the matrix-core scan in the kernel body); a dozen or more centroids of up to
+// 3 coordinates are taken four at a time (scan_centroids_blocked).  The quadratic expansion of
 // heat/spatial/distance.py:59-64, d2 = |x|^2 + |c|^2 - 2 x.c, is evaluated as a chain of D fused
 // multiply-adds that starts at |c|^2; |x|^2, the same for every centroid, is added to the minimum only.
 // First index wins ties (torch.min, heat/core/statistics.py:177).  The clamp at 0 is applied lazily: a
@@ -71,6 +72,11 @@ struct SmallCfg {
     // Up to 16 centroids of 4 or 8 coordinates are one A operand of v_mfma_f32_16x16x4_f32 (one or two steps
     // over the coordinates): the cross terms of 16 points then cost one or two matrix instructions.
     static constexpr bool MSCAN = D == 4 || D == 8;
+    // The scan four centroids at a time, where a centroid row is one 16-byte LDS read: the assignment of
+    // 100M rows takes 1.39 instead of 2.05 ms with 1 coordinate and 100 centroids, 0.66 instead of 1.01 ms
+    // with 2 and 64, 0.53 instead of 0.67 ms with 3 and 40; from a dozen centroids on it is never slower.
+    // Rows of 5 to 7 coordinates (two reads per row, more registers) run 0-18 % slower that way.
+    static constexpr bool BLOCKED = D <= 3;
 };
 
 bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
@@ -92,7 +98,7 @@ static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
     const int sc = (D + 1 + 3) / 4 * 4, nv = ppt * D / 4, slots = K * (D + 1);
     const size_t xch = (D == 4 || D == 8) ? size_t(SMALL_T / 64) * 256 * sizeof(float) : 0;  // as SmallCfg::MSCAN
-    return size_t((K * sc + 3) & ~3) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) + xch +
+    return size_t(((K + 3) & ~3) * sc) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) + xch +
            (acc_mode == 2   ? size_t(SMALL_T / 64) * slots * sizeof(double)
             : acc_mode == 3 ? size_t(SMALL_T / 64) * (slots * sizeof(double) + 64 * ppt * sizeof(int))
             : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float)
@@ -102,6 +108,12 @@ static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
 // The ordered strategies: per-lane LDS columns while they fit (slots * 1 KB), the matrix-core product up
 // to 32 clusters, the DPP tree otherwise.
 static int small_ordered_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : K <= 32 ? 3 : 2; }
+
+// Fewest centroids for which the scan goes four at a time (HKM_SMALL_BLOCKED_MIN_K overrides; looked up per call)
+static int small_blocked_min_k() {
+    const char* e = getenv("HKM_SMALL_BLOCKED_MIN_K");
+    return e ? atoi(e) : 12;
+}
 
 // HKM_SMALL_SUMS = ordered | integer (looked up per call) overrides the choice by size; tests use it
 static int small_sums_override() {
@@ -198,6 +210,75 @@ __device__ __forceinline__ void scan_centroids(const float* sC, int k0, int k1,
     }
 }
 
+// The scan for more than a few centroids, four at a time: the running minimum absorbs a block's four
+// distances with two three-input minima, and of the block only its number is kept where the minimum fell
+// (one compare, one select) -- 4 instead of 12 instructions per four distances besides the products.
+// Which of the four it was is looked up once per point at the end: the lane reads the four rows of ITS
+// block from LDS, evaluates the same chains again (same operands, same order: same bits) and takes the
+// first that equals the minimum.  Strict '<' on blocks and the first equal position inside one give the
+// first centroid that reaches the minimum, as the one-by-one scan does; NaN distances are skipped by the
+// minima, and a point with nothing below +inf keeps index 0.  Rows K .. 4 * ceil(K / 4) - 1 of sC hold
+// zero coordinates and the norm +inf.  m must come in as +inf.
+template <int D, int PPT>
+__device__ __forceinline__ void scan_centroids_blocked(const float* sC, int K, const float (&x)[PPT][D],
+                                                       float (&m)[PPT], int (&mi)[PPT]) {
+    constexpr int SC = SmallCfg<D>::SC;
+    int blk[PPT];
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) blk[p] = 0;
+    const int nb = (K + 3) >> 2;
+    for (int b = 0; b < nb; ++b) {
+        float dist[4][PPT];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float c[SC];
+#pragma unroll
+            for (int q = 0; q < SC / 4; ++q) {
+                const floatx4 v = *reinterpret_cast<const floatx4*>(sC + (4 * b + j) * SC + 4 * q);
+                c[4 * q] = v[0];
+                c[4 * q + 1] = v[1];
+                c[4 * q + 2] = v[2];
+                c[4 * q + 3] = v[3];
+            }
+#pragma unroll
+            for (int p = 0; p < PPT; ++p) {
+                float d2 = fmaf(x[p][0], c[0], c[D]);
+#pragma unroll
+                for (int d = 1; d < D; ++d) d2 = fmaf(x[p][d], c[d], d2);
+                dist[j][p] = d2;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PPT; ++p) {
+            const float nm = fminf(fminf(fminf(fminf(dist[0][p], dist[1][p]), dist[2][p]), dist[3][p]), m[p]);
+            blk[p] = nm < m[p] ? b : blk[p];
+            m[p] = nm;
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) {
+        const float* cb = sC + blk[p] * (4 * SC);
+        int pos = 0;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+            float c[SC];
+#pragma unroll
+            for (int q = 0; q < SC / 4; ++q) {
+                const floatx4 v = *reinterpret_cast<const floatx4*>(cb + j * SC + 4 * q);
+                c[4 * q] = v[0];
+                c[4 * q + 1] = v[1];
+                c[4 * q + 2] = v[2];
+                c[4 * q + 3] = v[3];
+            }
+            float d2 = fmaf(x[p][0], c[0], c[D]);
+#pragma unroll
+            for (int d = 1; d < D; ++d) d2 = fmaf(x[p][d], c[d], d2);
+            pos = d2 == m[p] ? j : pos;
+        }
+        mi[p] = m[p] < HKM_INF ? 4 * blk[p] + pos : 0;
+    }
+}
+
 // The same scan with the centroid rows fetched straight from the caller's C at wave-uniform addresses:
 // the compiler turns such reads into scalar loads, so a row arrives in scalar registers through the scalar
 // cache and costs neither LDS bandwidth (a broadcast read still returns 64 copies) nor vector registers.
@@ -284,7 +365,8 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const int slots = K * (D + 1);
     constexpr bool ACCUM = ACC != 0;
     const bool stream = (vec & 2) != 0;
-    float* stage = lds + ((K * SC + 3) & ~3);                        // [NW][NV*64*4] transpose buffer
+    const int KP = (K + 3) & ~3;                                     // rows of sC: K, then +inf-norm rows up to a multiple of four
+    float* stage = lds + KP * SC;                                    // [NW][NV*64*4] transpose buffer
     // matrix-core scan: [NW][128] (minimum, index) pairs on their way from the lane that found them to the
     // lane that owns the point
     float* xch_all = stage + NW * NV * 256;
@@ -360,6 +442,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
         for (int d = 0; d < D; ++d) sC[r * SC + d] *= -2.0f;  // exact
     }
+    for (int i = K * SC + tid; i < KP * SC; i += T) sC[i] = (i % SC) == D ? HKM_INF : 0.f;
     __syncthreads();
 
     // ACC == 4: 2^Ec > every |centroid coordinate|.  A coordinate x enters as the 64-bit pattern of
@@ -478,6 +561,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             mi[p] = 0;
         }
         const int kh = REGC ? KT / 2 : K >> 1;
+        const bool blocked = !REGC && SmallCfg<D>::BLOCKED && ACC != 1 && (vec & 4) != 0;
         if (ACC == 1 && PPT == 4) {
             rmw_write(0, r);
             rmw_read(1, r);
@@ -541,15 +625,20 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             }
         }
         if (!scanned) {
-            if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
-            else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, 0, kh, x, xn, m, mi);
-            else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
+            if constexpr (!REGC && SmallCfg<D>::BLOCKED) {
+                if (blocked) scan_centroids_blocked<D, PPT>(sC, K, x, m, mi);
+            }
+            if (!blocked) {
+                if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, 0, KR / 2, x, xn, m, mi);
+                else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, 0, kh, x, xn, m, mi);
+                else scan_centroids<D, PPT, false>(sC, 0, kh, x, xn, m, mi);
+            }
         }
         if (ACC == 1) {
             rmw_write(PPT == 4 ? 1 : 0, r);
             rmw_read(PPT == 4 ? 2 : 1, r);
         }
-        if (!scanned) {
+        if (!scanned && !blocked) {
             if constexpr (REGC) scan_centroids_reg<D, PPT, KR, false>(cs, KR / 2, KR, x, xn, m, mi);
             else if constexpr (SmallCfg<D>::SLOAD) scan_centroids_sload<D, PPT, false>(C, ldc, sC, kh, K, x, xn, m, mi);
             else scan_centroids<D, PPT, false>(sC, kh, K, x, xn, m, mi);
@@ -909,9 +998,10 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
                           int acc_mode, int grid, int32_t* flags, int aux, bool timed, hipStream_t st) {
     const bool want_min = min_d2 != nullptr;
     const size_t lds = small_lds_bytes(D, K, acc_mode);
-    // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads
+    // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads;
+    // bit 2: the scan takes the centroids four at a time
     const int vec = ((ldx == D) && aligned16(X) && aligned16(labels) ? 1 : 0) |
-                    (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0);
+                    (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0) | (K >= small_blocked_min_k() ? 4 : 0);
     // the register-resident centroid table: K <= 8 rows of at most 5 values
     constexpr int KT8 = D <= 4 ? 8 : 0;
     const bool reg = KT8 > 0 && K <= KT8;

@@ -36,6 +36,9 @@
  *                         on).  A testing aid; both give the same labels and means equal to fp32 rounding.
  *   HKM_NARROW_MFMA_MIN_K=n   hkm_assign_f32 with 4 <= D <= 16: use the matrix-core kernels from n centroids
  *                         on (default 32) and the vector kernel below.  A measuring and testing aid.
+ *   HKM_SMALL_BLOCKED_MIN_K=n   the narrow kernels with D <= 3 scan the centroids four at a time from n
+ *                         centroids on (default 12), one at a time below.  Same results bit for bit; a
+ *                         measuring and testing aid.
  */
 #ifndef HKM_H
 #define HKM_H

@@ -127,6 +127,48 @@ def test_narrow_matrix_core_scan_keeps_the_reference_rules(cuda, d, k):
     assert torch.equal(lab3, lab2)
 
 
+@pytest.mark.parametrize("d,k", [(2, 64), (2, 13), (3, 40), (3, 57), (2, 80), (3, 14), (1, 100), (1, 30), (1, 13)])
+def test_narrow_scan_four_at_a_time_keeps_the_reference_rules(cuda, d, k, monkeypatch):
+    # Up to 3 coordinates, a dozen centroids or more: the narrow kernels take the centroids four at a time, keep
+    # the block in which the minimum fell and look the position up at the end.  Against the scan one centroid
+    # at a time (forced through the environment) on duplicated centroids -- exact ties, the first index must
+    # win --, a row on a centroid, NaN and inf rows, K not a multiple of four: same labels, same distances,
+    # same step; and against the oracle.
+    print(f"narrow blocked scan d={d} k={k}", flush=True)
+    assert _native.lloyd_kernel_name(3001, d, k) == "lloyd_small"
+    g = torch.Generator().manual_seed(90 + d + k)
+    n = 3001
+    half = (k + 1) // 2
+    base = torch.randn((half, d), generator=g) * 3
+    c = torch.cat([base, base])[:k].contiguous()  # centroid j == j + half: exact ties
+    x = base[torch.randint(0, half, (n,), generator=g)] + 0.05 * torch.randn((n, d), generator=g)
+    x[7] = c[3]
+    x[11] = float("nan")
+    x[13] = float("inf")
+    x[17, 0] = 3e38  # the squared norm and the cross terms overflow
+    res = {}
+    for name, thr in (("one", "100000"), ("four", "2")):
+        monkeypatch.setenv("HKM_SMALL_BLOCKED_MIN_K", thr)
+        lab, md = _assign_gpu(x, c, cuda)
+        c_new = torch.empty((k, d), device=cuda)
+        lab_s = torch.empty((n,), dtype=torch.int32, device=cuda)
+        shift = torch.empty((), device=cuda)
+        _native.lloyd_step(x.to(cuda), c.to(cuda), c_new, lab_s, shift, None, _native.Workspace(cuda))
+        torch.cuda.synchronize()
+        res[name] = (lab, md, lab_s.cpu(), c_new.cpu(), shift.cpu())
+    one, four = res["one"], res["four"]
+    assert torch.equal(one[0], four[0]) and torch.equal(one[2], four[2]) and torch.equal(four[0], four[2])
+    assert torch.equal(torch.nan_to_num(one[1], nan=-1.0), torch.nan_to_num(four[1], nan=-1.0))
+    assert torch.equal(torch.nan_to_num(one[3], nan=-1.0), torch.nan_to_num(four[3], nan=-1.0))
+    lab = four[0]
+    bad = torch.zeros(n, dtype=torch.bool)
+    bad[[11, 13, 17]] = True
+    assert int(lab[~bad].max()) < half and int(lab[11]) == 0
+    ref, _ = orc.assign_to_cluster_literal(x[~bad].contiguous(), c)
+    assert bool((lab.long()[~bad] == ref.view(-1) % half).all())
+    assert 0.0 <= float(four[1][7]) <= 2e-6 * float((c[3].double() ** 2).sum())
+
+
 def test_assign_strided_rows(cuda):
     # X and C as column slices of wider buffers: ld > D, base pointers not 16-byte aligned
     g = torch.Generator().manual_seed(7)
