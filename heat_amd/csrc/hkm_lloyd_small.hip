@@ -561,7 +561,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
             mi[p] = 0;
         }
         const int kh = REGC ? KT / 2 : K >> 1;
-        const bool blocked = !REGC && SmallCfg<D>::BLOCKED && ACC != 1 && (vec & 4) != 0;
+        const bool blocked = !REGC && SmallCfg<D>::BLOCKED && (vec & 4) != 0;
         if (ACC == 1 && PPT == 4) {
             rmw_write(0, r);
             rmw_read(1, r);
