@@ -12,7 +12,7 @@ scalar is set to a value no shift can take (-1: a shift is a sum of squares or N
 waits for the step by reading the scalar until it has changed.  For a step of a few microseconds the
 record and the wait of an event were a third of the host's time per iteration, and the host is what
 bounds such fits.  For the narrow shapes whose step is one sweep of a
-vector kernel (D <= 8), writing N labels is a quarter of the step's memory traffic, so the steps run
+vector kernel (D <= 16, few clusters), writing N labels is a quarter of the step's memory traffic, so the steps run
 without storing labels and those of the last iteration are computed once, on demand, against the
 centroids that iteration started from -- the same kernel code, hence the same bits.  The values
 returned are exactly those of the sequential loop.

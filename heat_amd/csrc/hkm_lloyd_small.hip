@@ -1,4 +1,4 @@
-// One-sweep Lloyd step for small feature counts (D <= 8) and small K*(D+1): X is read from HBM
+// One-sweep Lloyd step for small feature counts (D <= 16) and small K*(D+1): X is read from HBM
 // exactly once per iteration (4D bytes per point) and only the labels are written (4 bytes).
 //
 // Assignment: a lane owns PPT consecutive points in registers; the centroids and their squared norms are
@@ -15,7 +15,7 @@
 //
 // Update (heat/cluster/kmeans.py:76-103), per-cluster sums whose value does not depend on the order in
 // which the hardware happens to run things:
-//   K*(D+1) <= 48: every lane owns a private fp32 column per (cluster, coordinate) in LDS and adds
+//   K*(D+1) <= 48 and D <= 8: every lane owns a private fp32 column per (cluster, coordinate) in LDS and adds
 //     its own points in program order; the read-add-write round trips of a round are deferred to the
 //     next round and interleaved with its arithmetic.  At the end lanes' columns are added in a fixed
 //     fp64 tree.
@@ -26,7 +26,7 @@
 //     outside the scale's range (|x| >= 2^(Ec + headroom), inf, NaN) or has no usable scale raises a flag,
 //     and a second launch -- the same sweep with one of the two ordered strategies below, which returns at
 //     once when no flag is up -- redoes the step.
-//   otherwise, K <= 32: the sums are a matrix product, (one-hot labels)^T x [X, 1], evaluated on the
+//   otherwise, K <= 32 and D <= 8: the sums are a matrix product, (one-hot labels)^T x [X, 1], evaluated on the
 //     fp32 matrix cores with v_mfma_f32_16x16x4_f32 over the wave's points of the round (read back from
 //     the staging buffer); the fp32 accumulators move into the wave's private fp64 row in LDS every
 //     eight rounds.
@@ -79,7 +79,7 @@ struct SmallCfg {
     static constexpr bool BLOCKED = D <= 3;
 };
 
-bool small_eligible(int32_t D, int32_t K) { return D <= 8 && K * (D + 1) <= 240; }
+bool small_eligible(int32_t D, int32_t K) { return D <= 16 && K * (D + 1) <= 240; }
 static constexpr int SMALL_T = 256;
 
 // ---- the integer accumulation (acc_mode 4) ----
@@ -107,7 +107,7 @@ static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
 }
 // The ordered strategies: per-lane LDS columns while they fit (slots * 1 KB), the matrix-core product up
 // to 32 clusters, the DPP tree otherwise.
-static int small_ordered_mode(int32_t D, int32_t K) { return K * (D + 1) <= 48 ? 1 : K <= 32 ? 3 : 2; }
+static int small_ordered_mode(int32_t D, int32_t K) { return D > 8 ? 2 : K * (D + 1) <= 48 ? 1 : K <= 32 ? 3 : 2; }
 
 // Fewest centroids for which the scan goes four at a time (HKM_SMALL_BLOCKED_MIN_K overrides; looked up per call)
 static int small_blocked_min_k() {
@@ -402,7 +402,8 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     // ends up with its own PPT consecutive points.  The first rounds are requested here, before the
     // centroids are staged: for a matrix of a few megabytes the kernel is two memory latencies long,
     // and this way they overlap.
-    constexpr int PF = 3;  // rounds in flight: enough bytes per CU to cover the HBM latency
+    // rounds in flight: enough bytes per CU to cover the HBM latency, within the registers a wide row leaves
+    constexpr int PF = NV <= 4 ? 3 : NV <= 8 ? 2 : 1;
     floatx4 nxt[PF][NV];
     const float* wsrc = X + (base + wave * 64) * (PPT * D) + lane * 4;
     const int64_t rstride = stride * (PPT * D);
@@ -1021,21 +1022,28 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
                                N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);                \
     } while (0)
     if (timed) prof_begin(st);
-    if (acc_mode == 1) {
-        if (want_sse) HKM_GO(1, false, true);
-        else HKM_GO(1, false, false);
-    } else if (acc_mode == 2) {
+    if (acc_mode == 2) {
         if (want_sse) HKM_GO(2, false, true);
         else HKM_GO(2, false, false);
-    } else if (acc_mode == 3) {
-        if (want_sse) HKM_GO(3, false, true);
-        else HKM_GO(3, false, false);
     } else if (acc_mode == 4) {
         if (want_sse) HKM_GO(4, false, true);
         else HKM_GO(4, false, false);
-    } else {
+    } else if (acc_mode == 0) {
         if (want_min) HKM_GO(0, true, false);
         else HKM_GO(0, false, false);
+    } else {
+        // per-lane columns and the matrix-core product exist up to 8 features (small_ordered_mode)
+        if constexpr (D <= 8) {
+            if (acc_mode == 1) {
+                if (want_sse) HKM_GO(1, false, true);
+                else HKM_GO(1, false, false);
+            } else {
+                if (want_sse) HKM_GO(3, false, true);
+                else HKM_GO(3, false, false);
+            }
+        } else {
+            return fail(HKM_EUNSUPPORTED, "lloyd_small: accumulation mode %d with D=%d", acc_mode, D);
+        }
     }
     if (timed) prof_end(st);
 #undef HKM_GO
@@ -1079,8 +1087,9 @@ int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float*
     }
     switch (D) {
         HKM_T(1) HKM_T(2) HKM_T(3) HKM_T(4) HKM_T(5) HKM_T(6) HKM_T(7) HKM_T(8)
+        HKM_T(9) HKM_T(10) HKM_T(11) HKM_T(12) HKM_T(13) HKM_T(14) HKM_T(15) HKM_T(16)
         default:
-            return fail(HKM_EUNSUPPORTED, "lloyd_small: D=%d outside 1..8", D);
+            return fail(HKM_EUNSUPPORTED, "lloyd_small: D=%d outside 1..16", D);
     }
 #undef HKM_T
 }

@@ -30,7 +30,7 @@
  *                         product as fp32, 1.3x to 1.7x the throughput.  Off by default.
  *   HKM_UPDATE_LISTS=1    hkm_update_f32 and the two-pass part of hkm_lloyd_step_f32 use the list-based
  *                         kernels instead of the sort-based ones (a testing aid).
- *   HKM_SMALL_SUMS=ordered|integer   hkm_lloyd_step_f32 on the narrow shapes (D <= 8, K (D + 1) <= 240) with
+ *   HKM_SMALL_SUMS=ordered|integer   hkm_lloyd_step_f32 on the narrow shapes (D <= 16, K (D + 1) <= 240) with
  *                         more than 48 accumulator slots: form the per-cluster sums in a fixed order, or as
  *                         exact 64-bit integer sums, whatever N is (unset: integer from about a million rows
  *                         on).  A testing aid; both give the same labels and means equal to fp32 rounding.

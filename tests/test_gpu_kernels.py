@@ -22,6 +22,8 @@ ASSIGN_SHAPES = [
     (4096, 32, 256), (1000, 20, 33), (999, 17, 1), (3000, 64, 100), (1300, 50, 37), (257, 24, 64),
     (2048, 64, 1024), (1500, 100, 70), (900, 512, 130), (700, 33, 500), (513, 130, 1030),
     (3000, 16, 1100), (2500, 8, 1500), (1800, 6, 2000), (4000, 4, 33), (3000, 13, 32),
+    # 9 to 16 features with few centroids: the narrow kernel
+    (3001, 16, 8), (2000, 9, 24), (4003, 12, 5), (1000, 15, 15), (2500, 10, 1), (3000, 14, 16), (2222, 11, 20), (1999, 13, 3),
 ]
 
 
@@ -230,7 +232,8 @@ def test_update_ignores_out_of_range_labels(cuda):
     assert torch.allclose(c_new.cpu()[1], x[[1, 4, 7, 9]].mean(0))
 
 
-@pytest.mark.parametrize("n,d,k", [(20000, 3, 8), (20000, 8, 16), (30000, 32, 256), (5000, 64, 1024), (4000, 512, 96)])
+@pytest.mark.parametrize("n,d,k", [(20000, 3, 8), (20000, 8, 16), (30000, 32, 256), (5000, 64, 1024), (4000, 512, 96),
+                                   (20000, 16, 8), (15000, 12, 10), (10000, 9, 20), (12000, 15, 4)])
 def test_lloyd_step_matches_oracle_and_is_deterministic(cuda, n, d, k):
     print(f"lloyd n={n} d={d} k={k}", flush=True)
     x, _ = _data(n, d, k, seed=11 * n + k)
@@ -372,7 +375,7 @@ def test_tuning_call_is_a_step_and_settles_on_a_geometry(cuda, monkeypatch):
     assert _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws) == 0
 
 
-@pytest.mark.parametrize("n,d,k", [(30000, 16, 8), (20000, 9, 1), (25000, 12, 20), (10000, 10, 3), (40000, 4, 50), (30000, 7, 31),
+@pytest.mark.parametrize("n,d,k", [(30000, 16, 15), (20000, 9, 25), (25000, 12, 20), (10000, 10, 22), (40000, 4, 50), (30000, 7, 31),
                                    (50000, 2, 90), (40000, 3, 256), (30000, 3, 70)])
 def test_one_sweep_mfma_step_with_few_centroids_and_narrow_rows(cuda, n, d, k):
     # From 2 features on the step runs on the matrix cores whatever K is, while the assignment alone stays
@@ -466,7 +469,10 @@ def _narrow_step(xs, cs, dev, sums, monkeypatch, want_sse=True):
 
 # narrow shapes beyond 48 accumulator slots: every D, K up to the limit of 240 slots, ragged N
 NARROW_SHAPES = [(20000, 8, 16), (30011, 8, 26), (50000, 4, 32), (40001, 6, 20), (25000, 7, 30), (60000, 2, 64),
-                 (60002, 3, 40), (50000, 1, 100), (33333, 5, 40), (300, 8, 16), (7, 2, 20), (45001, 4, 15), (30000, 8, 14)]
+                 (60002, 3, 40), (50000, 1, 100), (33333, 5, 40), (300, 8, 16), (7, 2, 20), (45001, 4, 15), (30000, 8, 14),
+                 # 9 to 16 features, up to 240 accumulator slots
+                 (30000, 16, 8), (25001, 12, 18), (10000, 10, 3), (20000, 9, 24), (40000, 13, 17), (33001, 15, 15),
+                 (20000, 16, 14), (5000, 11, 1), (20002, 14, 16)]
 
 
 @pytest.mark.parametrize("n,d,k", NARROW_SHAPES)
@@ -475,7 +481,7 @@ def test_integer_sums_of_the_narrow_step_equal_the_ordered_ones(cuda, n, d, k, m
     # atomics, any order); small ones in a fixed order on the matrix cores or with a wave-wide tree.  Forced
     # either way on the same input: same labels, same sum of distances, centroids equal to fp32 rounding
     # and equal to the fp64 means of the labels; the integer way gives the same bits run after run.
-    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_small" and k * (d + 1) > 48
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_small" and (k * (d + 1) > 48 or d > 8)
     print(f"narrow sums n={n} d={d} k={k}", flush=True)
     x, _ = _data(n, d, k, seed=3 * n + d)
     x[::97] = 0.0
