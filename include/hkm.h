@@ -33,7 +33,8 @@
  *   HKM_SMALL_SUMS=ordered|integer   hkm_lloyd_step_f32 on the narrow shapes (D <= 16, K (D + 1) <= 240) with
  *                         more than 48 accumulator slots: form the per-cluster sums in a fixed order, or as
  *                         exact 64-bit integer sums, whatever N is (unset: integer from about a million rows
- *                         on).  A testing aid; both give the same labels and means equal to fp32 rounding.
+ *                         on, from 131072 with more than 32 clusters or more than 8 features).  A testing
+ *                         aid; both give the same labels and means equal to fp32 rounding.
  *   HKM_NARROW_MFMA_MIN_K=n   hkm_assign_f32 with 4 <= D <= 16: use the matrix-core kernels from n centroids
  *                         on (default 32) and the vector kernel below.  A measuring and testing aid.
  *   HKM_SMALL_BLOCKED_MIN_K=n   the narrow kernels with D <= 3 scan the centroids four at a time from n
