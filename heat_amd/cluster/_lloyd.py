@@ -27,6 +27,9 @@ in particular before EVERY stop -- the means of that iteration are recomputed fr
 two-pass update (fp64 from the first addition to the division, fixed order: bit-identical to the
 reference's means in all but about one coordinate in a thousand), and the decision is taken on that
 shift.  If the loop goes on, the step enqueued ahead is re-issued from the recomputed centroids.
+One case is decided before that: a one-sweep step whose centroids equal the ones it started from bit for
+bit saw the labels of the step before it, and two iterations with the same labels are where the
+reference stops with a shift of exactly 0 -- the recomputed means are stored, the shift is 0.
 """
 
 from __future__ import annotations
@@ -126,7 +129,16 @@ class LloydLoop:
             self.done = i + 1
             ran += 1
             if self._fuzz and shift <= tol + self._margin(tol):
+                unchanged = shift == 0.0
                 shift = self._recompute(i)
+                if unchanged:
+                    # Bit-identical centroids from a one-sweep step: it saw the labels of the step before it.
+                    # The reference forms the exact means in every iteration and finds no movement between
+                    # two iterations with the same labels (kmeans.py:141-143); the centroids this step
+                    # started from carry the one-sweep rounding, so the exact means just stored would show
+                    # a movement of that size and cost an iteration the reference does not run.
+                    shift = 0.0
+                    self.shift_host[i % 2] = 0.0
             if shift <= tol:
                 break
         return ran

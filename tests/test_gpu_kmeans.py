@@ -191,6 +191,22 @@ def test_scaled_configs_against_oracle(cuda, cfg, scale, parity_report):
     _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
 
 
+@pytest.mark.parametrize("n,d,k", [(60000, 16, 8), (50000, 12, 5), (40000, 9, 20), (200000, 14, 16)])
+def test_few_clusters_of_nine_to_sixteen_features_against_oracle(cuda, n, d, k, parity_report):
+    """Whole fits on the narrow one-sweep kernel's wider rows (9 to 16 features, K (D + 1) <= 240), through the
+    public estimator: step by step and at the end against the oracle, with the labels of the last iteration
+    computed on demand as for every narrow shape.  The largest takes the integer sums by itself."""
+    from heat_amd import _native
+
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_small"
+    w = synthetic.shape(n, d, k, seed=1200 + d)
+    print(f"{w.name}", flush=True)
+    flips, ref = _stepwise_parity(w, cuda, 12, literal=False, report=parity_report)
+    print(f"{w.name}: {flips} excused tie flips over {ref['n_iter']} iterations", flush=True)
+    km, _ = _fit(w.x, w.init, w.k, 12, 0.0, cuda)
+    _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
+
+
 @pytest.mark.parametrize("scale", [1.0 / 16, 1.0])
 def test_config2_cdist_argmin(cuda, scale, parity_report):
     from heat_amd import _native
@@ -282,9 +298,13 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
             n_seq += 1
             _native.lloyd_step(x, c_cur, c_nxt, lab, shift, None, ws)
             if tol is not None and float(shift) <= tol + probe._margin(tol):
-                # the loop's rule: a one-sweep step near the stop decision is settled by the two-pass means
+                # the loop's rule: a one-sweep step near the stop decision is settled by the two-pass means;
+                # a step that reproduced its own centroids bit for bit counts as no movement
+                unchanged = float(shift) == 0.0
                 _native.update(x, lab, c_nxt, None, ws)
                 _native.shift(c_cur, c_nxt, shift)
+                if unchanged:
+                    shift.zero_()
             c_cur, c_nxt = c_nxt, c_cur
             if tol is not None and float(shift) <= tol:
                 break
@@ -318,7 +338,7 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
 # ---- closed forms of the loop (heat/cluster/kmeans.py:131-146) through the public estimator --------
 # shapes: the one-sweep matrix-core step (D = 32), the narrow one-sweep step (D = 3 and D = 8), and a
 # shape that runs assignment + two-pass update (D = 100)
-@pytest.mark.parametrize("n,d", [(64, 32), (200, 32), (8, 3), (16, 8), (30, 5), (50, 100)])
+@pytest.mark.parametrize("n,d", [(64, 32), (200, 32), (8, 3), (16, 8), (30, 5), (50, 100), (14, 16), (20, 11)])
 def test_every_row_its_own_centroid_is_a_fixed_point(cuda, n, d, parity_report):
     """K = N distinct rows as init: every cluster holds exactly its own row, the means are the rows, the
     shift is exactly 0 and the loop stops after ONE iteration (kmeans.py:141-143), as the oracle does."""
@@ -334,7 +354,7 @@ def test_every_row_its_own_centroid_is_a_fixed_point(cuda, n, d, parity_report):
     assert torch.equal(km.labels_.larray.cpu().view(-1), torch.arange(n))
 
 
-@pytest.mark.parametrize("n,d", [(20000, 32), (30000, 3), (20000, 8), (5000, 100)])
+@pytest.mark.parametrize("n,d", [(20000, 32), (30000, 3), (20000, 8), (5000, 100), (20000, 12)])
 def test_init_at_the_means_of_two_far_blobs_stops_like_the_oracle(cuda, n, d, parity_report):
     """Two blobs far apart, init = their means (fp64 means rounded to fp32): the first iteration assigns
     every point to its blob and reproduces the means, so the reference stops at once with shift 0."""
@@ -354,7 +374,7 @@ def test_init_at_the_means_of_two_far_blobs_stops_like_the_oracle(cuda, n, d, pa
     assert orc.rel_err_centers(km.cluster_centers_.larray.cpu(), ref["cluster_centers"]) <= 1e-6
 
 
-@pytest.mark.parametrize("n,d", [(5000, 32), (5000, 3), (3000, 100)])
+@pytest.mark.parametrize("n,d", [(5000, 32), (5000, 3), (3000, 100), (5000, 16)])
 def test_one_cluster_is_the_global_mean(cuda, n, d, parity_report):
     g = torch.Generator().manual_seed(n + d)
     x = torch.randn((n, d), generator=g) * 2.0 + 1.0
