@@ -19,7 +19,7 @@ from . import _f64_paths
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
-LIB_VERSION = 302  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
+LIB_VERSION = 303  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
 WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64 = 1, 2, 3, 4, 8, 16
 
@@ -35,17 +35,10 @@ SIGNATURES = {
     "hkm_static_scratch_bytes": (c_size_t, []),
     "hkm_assign_static_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                              c_void_p, c_void_p, c_void_p]),
-    "hkm_profile_enable": (ctypes.c_int, [c_int32]),
-    "hkm_profile_collect": (ctypes.c_int, [c_void_p, c_int32, c_void_p]),
-    "hkm_probe_mfma_f32": (ctypes.c_int, [c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
-    "hkm_probe_stream": (ctypes.c_int, [c_void_p, c_void_p, c_size_t, c_int32, c_void_p, c_void_p]),
     "hkm_update_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_void_p,
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "hkm_tune_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
-                                          c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "hkm_point_blocks": (ctypes.c_int, [c_int32, c_void_p]),
     "hkm_shift_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "hkm_functional_value_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_cdist_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
@@ -241,19 +234,6 @@ def assign_static(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2
                                        c.stride(0) if k > 1 else d, _ptr(labels), _ptr(min_d2), _stream()))
 
 
-def profile_enable(on: bool) -> None:
-    """Benchmarks: record an event pair around the distance kernel of every assign / lloyd_step call."""
-    check(load().hkm_profile_enable(1 if on else 0))
-
-
-def profile_collect() -> list:
-    """Durations (ms) of the distance kernels launched since the last collect, in call order."""
-    buf = (ctypes.c_float * 512)()
-    cnt = c_int32(0)
-    check(load().hkm_profile_collect(ctypes.cast(buf, c_void_p), 512, ctypes.cast(ctypes.pointer(cnt), c_void_p)))
-    return [float(buf[i]) for i in range(min(cnt.value, 512))]
-
-
 def update(x: torch.Tensor, labels: torch.Tensor, c_new: torch.Tensor, counts: Optional[torch.Tensor],
            ws: Workspace) -> None:
     _require_gpu(x, labels, c_new, counts)
@@ -293,35 +273,6 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Op
     buf = ws.get(need)
     check(load().hkm_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
                                     _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
-
-
-def tune_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: torch.Tensor,
-                    shift: torch.Tensor, ws: Workspace) -> int:
-    """One Lloyd step as ``lloyd_step`` runs it (same results), after which the library times the step in
-    both launch geometries of the resident matrix-core kernels and keeps the faster one for this device
-    (hkm_tune_lloyd_step_f32 in include/hkm.h).  WAITS for the device.  Returns the point blocks per wave
-    chosen, 0 where the shape has no such choice."""
-    _require_gpu(x, c, c_new, labels)
-    _require_rows(x, c, c_new)
-    _require_dense(c, c_new)
-    if x.dtype != torch.float32:
-        return 0
-    n, d = x.shape
-    k = c.shape[0]
-    buf = ws.get(workspace_bytes(n, d, k, WS_LLOYD))
-    rc = load().hkm_tune_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
-                                        _ptr(labels), _ptr(shift), None, _ptr(buf), buf.numel(), _stream())
-    if rc < 0:
-        check(rc)
-    return rc
-
-
-def point_blocks(d: int):
-    """(point blocks per wave a resident matrix-core kernel would use for d features now -- 0 if d has no
-    such kernel --, whether that was measured on the current device)."""
-    tuned = ctypes.c_int32(0)
-    pb = load().hkm_point_blocks(d, ctypes.cast(ctypes.pointer(tuned), c_void_p))
-    return int(pb), bool(tuned.value)
 
 
 def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],

@@ -34,7 +34,6 @@ reference stops with a shift of exactly 0 -- the recomputed means are stored, th
 
 from __future__ import annotations
 
-import os
 import time
 from typing import Optional
 
@@ -55,10 +54,15 @@ class LloydLoop:
         n, d = xt.shape
         kernel = _native.lloyd_kernel_name(n, d, c0.shape[0]) if xt.dtype == torch.float32 else ""
         self.lazy_labels = kernel == "lloyd_small"
-        # relative size (against sum |c|^2) of the squared centroid movement below which a one-sweep step's
-        # shift is within the rounding error of its own sums; 0 for the shapes that run the two-pass update
-        self._fuzz = {"lloyd_small": 1e-11 * d, "lloyd_mfma_resident": 1e-13 * d}.get(kernel, 0.0)
-        self._cscale: Optional[float] = None
+        # Relative size (against sum |c|^2) of the squared rounding error of a one-sweep step's centroids; 0 for the
+        # shapes that run the two-pass update.  From the kernels' quanta: the matrix-core step rounds a row to
+        # 2^-28 of its largest coordinate or, for rows below the floor it derives from the centroid norms, to at
+        # most 2^-23 of the smallest centroid's norm -- squared and summed over K clusters of D coordinates that is
+        # at most D * 2^-46 * sum |c|^2, taken eight times over.  The narrow step sums fp32 partials per lane, or
+        # integers with a quantum of 2^-33 of the largest centroid coordinate: a mean is good to a few dozen ulps,
+        # (2^-18)^2 of its magnitude per coordinate.
+        self._fuzz = {"lloyd_small": d * 2.0 ** -36, "lloyd_mfma_resident": d * 2.0 ** -43}.get(kernel, 0.0)
+        self._cnorm: Optional[float] = None  # upper bound on the Frobenius norm of the current centroids
         self.rechecks = 0  # iterations whose means were recomputed by the two-pass update
         nbuf = 1 if self.lazy_labels else 2
         self.lab = [torch.empty((n,), dtype=torch.int32, device=dev) for _ in range(nbuf)]
@@ -69,13 +73,6 @@ class LloydLoop:
         self.enqueued = 0  # steps handed to the stream
         self.done = 0      # steps whose results count
         self._plans = {}   # prepared calls, one per rotation of the buffers (and stream)
-        # Large fits on the resident matrix-core kernels: let the library measure once per device which of
-        # its two launch geometries this chip runs faster (the results do not depend on it).  The call is a
-        # step from c[0] into c[1] that the loop's own first step then repeats.
-        if kernel == "lloyd_mfma_resident" and n >= (1 << 20):
-            pb, tuned = _native.point_blocks(d)
-            if pb and d <= 32 and not tuned and not os.environ.get("HKM_POINT_BLOCKS"):
-                _native.tune_lloyd_step(self.x, self.c[0], self.c[1], self.lab[0], self.shift_host[0], self.ws)
 
     def _enqueue(self) -> None:
         j = self.enqueued
@@ -120,6 +117,7 @@ class LloydLoop:
                 self._enqueue()
             if tol is None:
                 self._free_running = True
+                self._cnorm = None  # nobody reads these shifts: the bound is taken again when it is needed
                 self.done = i + 1
                 ran += 1
                 continue
@@ -128,27 +126,39 @@ class LloydLoop:
             shift = self._wait(i)
             self.done = i + 1
             ran += 1
-            if self._fuzz and shift <= tol + self._margin(tol):
-                unchanged = shift == 0.0
-                shift = self._recompute(i)
-                if unchanged:
-                    # Bit-identical centroids from a one-sweep step: it saw the labels of the step before it.
-                    # The reference forms the exact means in every iteration and finds no movement between
-                    # two iterations with the same labels (kmeans.py:141-143); the centroids this step
-                    # started from carry the one-sweep rounding, so the exact means just stored would show
-                    # a movement of that size and cost an iteration the reference does not run.
-                    shift = 0.0
-                    self.shift_host[i % 2] = 0.0
+            if self._fuzz:
+                if shift <= tol + self._margin(tol, shift):
+                    # Bit-identical centroids from a one-sweep step (looked at before they are replaced): the step
+                    # saw the labels of the step before it.  The reference forms the exact means in every
+                    # iteration and finds no movement between two iterations with the same labels
+                    # (kmeans.py:141-143); the centroids this step started from carry the one-sweep rounding,
+                    # so the exact means stored below would show a movement of that size and cost an iteration
+                    # the reference does not run.  Not at the first step: nothing came before it, and an init
+                    # that reproduces itself under the one-sweep rounding still moves by the last bit in the
+                    # reference.
+                    unchanged = i > 0 and torch.equal(self.c[i % 3], self.c[(i + 1) % 3])
+                    shift = self._recompute(i)
+                    if unchanged:
+                        shift = 0.0
+                        self.shift_host[i % 2] = 0.0
+                # |c_new| <= |c_old| + sqrt(shift): the bound follows the centroids without a look at them
+                if self._cnorm is not None and shift == shift:
+                    self._cnorm += max(shift, 0.0) ** 0.5
             if shift <= tol:
                 break
         return ran
 
-    def _margin(self, tol: float) -> float:
-        """How far above ``tol`` a one-sweep step's shift may sit while the exact one is <= tol: with
-        e = the rounding error of the step's centroids, |shift - exact| <= 2 sqrt(exact) |e| + |e|^2."""
-        if self._cscale is None:
-            self._cscale = float((self.c[0].double() ** 2).sum())
-        e2 = self._fuzz * self._cscale
+    def _margin(self, tol: float, shift: float) -> float:
+        """How far above ``tol`` the shift of the one-sweep step just waited for may sit while the exact one is
+        <= tol: with e = the rounding error of the step's centroids, |shift - exact| <= 2 sqrt(exact) |e| + |e|^2.
+        e^2 is priced against an upper bound on sum |c|^2 that holds for the centroids the step started from and
+        for those it produced: the norm of the initial centroids (one look at the device, at the first call) plus
+        the square roots of every shift since, so centroids that grow -- an init near the origin, data far from
+        it -- raise the margin with them."""
+        if self._cnorm is None:
+            self._cnorm = float((self.c[(self.done - 1) % 3].double() ** 2).sum()) ** 0.5
+        bound = self._cnorm + (max(shift, 0.0) ** 0.5 if shift == shift else 0.0)
+        e2 = self._fuzz * bound * bound
         return 2.0 * (max(tol, 0.0) * e2) ** 0.5 + e2
 
     def _recompute(self, i: int) -> float:

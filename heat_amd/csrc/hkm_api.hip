@@ -6,6 +6,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include "hkm_bench.h"
 #include "hkm_common.h"
 
 namespace hkm {
@@ -277,7 +278,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 302; }
+int hkm_version(void) { return 303; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -385,7 +386,14 @@ static int static_scratch(void** out) {
     return HKM_OK;
 }
 
-size_t hkm_static_scratch_bytes(void) { return HKM_STATIC_SCRATCH_BYTES; }
+// Also resolves the array's address on the current device, so that a caller who asks for the size first -- the
+// documented warm-up -- never meets the symbol lookup inside hkm_assign_static_f32 (a capturing stream may refuse it).
+size_t hkm_static_scratch_bytes(void) {
+    void* p = nullptr;
+    (void)static_scratch(&p);  // a failure (no device) is reported by the entry point that needs the address
+    g_err[0] = 0;
+    return HKM_STATIC_SCRATCH_BYTES;
+}
 
 int hkm_assign_static_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                           int64_t ldc, int32_t* labels, float* min_d2, void* hip_stream) {
@@ -477,65 +485,7 @@ int hkm_point_blocks(int32_t D, int32_t* tuned) {
     return resident_point_blocks(resident_dp(D));
 }
 
-// The step itself, then -- where there is a choice -- the same step a few more times in either geometry
-// between events; the faster one is remembered for the device.  Every run writes the same bits into the
-// same outputs, so the caller's buffers hold the step's results whatever was measured.
-int hkm_tune_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new,
-                            int32_t K, int32_t* labels, float* shift, float* sse, void* ws, size_t ws_bytes,
-                            void* hip_stream) {
-    int rc = hkm_lloyd_step_f32(X, N, D, ldx, C, C_new, K, labels, shift, sse, ws, ws_bytes, hip_stream);
-    if (rc) return rc;
-    const bool choice = N > 0 && !small_eligible(D, K) && fused_eligible(D, K) && resident_dp(D) <= 32 &&
-                        env_point_blocks() == 0 && !(use_split_products() && split_eligible(D, K, true));
-    if (!choice) return 0;
-    hipStream_t st = static_cast<hipStream_t>(hip_stream);
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
-        return fail(HKM_EUNSUPPORTED, "hkm_tune_lloyd_step_f32 waits for the device and cannot run under stream capture");
-    // Three windows -- two point blocks, one, two again -- each after a warm-up of its own, and the one-block
-    // window is compared with the SECOND two-block window: a device that was idle needs some 30 ms of load to
-    // reach its clock (the first window would lose for that alone), and a chip that lowers its clock under one
-    // geometry has done so 20 ms into it.  Windows are sized in time: a few steps are timed first.
-    hipEvent_t ev[4][2];
-    for (auto& pair : ev)
-        for (auto& e : pair)
-            if (hipEventCreate(&e) != hipSuccess) return fail(HKM_EHIP, "hipEventCreate failed");
-    auto run = [&](int pb, int steps, hipEvent_t e0, hipEvent_t e1) {
-        force_point_blocks(pb);
-        if (e0) (void)hipEventRecord(e0, st);
-        for (int i = 0; i < steps && !rc; ++i)
-            rc = hkm_lloyd_step_f32(X, N, D, ldx, C, C_new, K, labels, shift, sse, ws, ws_bytes, hip_stream);
-        if (e1) (void)hipEventRecord(e1, st);
-    };
-    auto elapsed = [&](hipEvent_t e0, hipEvent_t e1, float& ms) {
-        if (!rc && (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess))
-            rc = fail(HKM_EHIP, "timing the trial steps failed");
-    };
-    float est = 0.f;
-    run(2, 5, ev[0][0], ev[0][1]);
-    elapsed(ev[0][0], ev[0][1], est);
-    const float step_ms = est > 0.f ? est / 5.f : 1.f;
-    const int warm = std::min(2000, std::max(25, int(35.f / step_ms) + 1));
-    const int timed = std::min(2000, std::max(20, int(25.f / step_ms) + 1));
-    float ms[3] = {0.f, 0.f, 0.f};  // [1], [2]: per-step time with one / two point blocks
-    run(2, warm, nullptr, nullptr);
-    run(2, timed, ev[1][0], ev[1][1]);
-    run(1, warm, nullptr, nullptr);
-    run(1, timed, ev[2][0], ev[2][1]);
-    run(2, warm, nullptr, nullptr);
-    run(2, timed, ev[3][0], ev[3][1]);
-    force_point_blocks(0);
-    elapsed(ev[2][0], ev[2][1], ms[1]);
-    elapsed(ev[3][0], ev[3][1], ms[2]);
-    for (auto& pair : ev)
-        for (auto& e : pair) (void)hipEventDestroy(e);
-    if (rc) return rc;
-    // two point blocks unless one is clearly faster here (repeated timings differ by up to half a percent,
-    // and chips on which the two are within one percent of each other exist)
-    const int best = ms[1] < 0.99f * ms[2] ? 1 : 2;
-    set_tuned_point_blocks(best);
-    return best;
-}
+int hkm_point_blocks_trial(float* ms_two, float* ms_one) { return trial_report(ms_two, ms_one); }
 
 int hkm_shift_f32(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,
                   void* hip_stream) {
@@ -868,8 +818,9 @@ int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds,
     return launch_silhouette_finish(S, N, K, lds, labels, counts, out, static_cast<hipStream_t>(hip_stream));
 }
 
-// rows run along grid.x; 2^24 rows would already be a 1 PB matrix
-static const int64_t LAPLACIAN_MAX_N = int64_t(1) << 24;
+// rows run along grid.x, 256-column slices along grid.y (at most 65535 of them); a matrix of that many rows
+// would be a petabyte
+static const int64_t LAPLACIAN_MAX_N = int64_t(65535) * 256;
 
 // 0: nothing to do, 1: arguments fine, launch; negative: error
 static int laplacian_check(size_t elem, const void* S, int64_t N, int64_t lds, int32_t definition, int32_t mode,
@@ -1004,21 +955,6 @@ int hkm_pairwise_f32(const float* X, int64_t M, int64_t ldx, const float* Y, int
                                                                                         : 1;
     const float gauss = gaussian ? 1.0f / (2.0f * sigma * sigma) : 0.f;
     return launch_cdist(X, M, ldx, Y, Nn, ldy, D, out, ldo, form, 1, gauss, static_cast<hipStream_t>(hip_stream));
-}
-
-int hkm_probe_mfma_f32(int32_t op, int32_t nops, int32_t iters, int32_t grid, float* out, void* hip_stream) {
-    g_err[0] = 0;
-    if (iters < 1 || grid < 1 || !out) return fail(HKM_EINVAL, "hkm_probe_mfma_f32: iters and grid must be >= 1 and out not NULL");
-    return launch_probe_mfma(op, nops, iters, grid, out, static_cast<hipStream_t>(hip_stream));
-}
-
-int hkm_probe_stream(const void* src, void* dst, size_t bytes, int32_t mode, float* sink, void* hip_stream) {
-    g_err[0] = 0;
-    if (bytes < 16 || !sink || (mode != 3 && !src) || ((mode == 0 || mode == 3) && !dst))
-        return fail(HKM_EINVAL, "hkm_probe_stream: NULL buffer or fewer than 16 bytes");
-    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u)
-        return fail(HKM_EINVAL, "hkm_probe_stream: buffers must be 16-byte aligned");
-    return launch_probe_stream(src, dst, bytes, mode, sink, static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream) {

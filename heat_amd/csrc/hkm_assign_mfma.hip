@@ -12,7 +12,8 @@
 //
 // Arithmetic mirrors heat/spatial/distance.py:59-64: d2 = (|x|^2 + |c|^2) - 2*(x.c), clamped at 0;
 // first index wins ties (torch.min, heat/core/statistics.py:177).
-#include <atomic>
+#include <pthread.h>
+#include <time.h>
 
 #include "hkm_common.h"
 #include "hkm_mfma_util.h"
@@ -276,20 +277,9 @@ static constexpr int FUSED_QBITS = 28;
 // on those that do not it runs at 2.1-2.2 GHz and two point blocks at 2.3 GHz (1.45 against 1.39 ms).  Both
 // geometries cut the rows into the same tiles of 512 and hand them to the same workgroups, so every output
 // of a step is bit for bit the same whichever runs.  Which one: HKM_POINT_BLOCKS (1 or 2) if set; else what
-// hkm_tune_lloyd_step_f32 measured on this device; else two.  Wider rows leave registers for one point
-// block only (twelve waves).
+// the trial below found on this device; else two.  Wider rows leave registers for one point block only
+// (twelve waves).
 __host__ __device__ constexpr int fused_threads(int pb, int dp) { return pb == 2 ? 512 : (dp <= 32 ? 1024 : 768); }
-
-static const int TUNE_MAX_DEVICES = 64;
-static std::atomic<int> g_tuned_pb[TUNE_MAX_DEVICES];  // per device: 0 not measured, else 1 or 2
-static thread_local int t_forced_pb = 0;                // set by the tuning call around its trial launches
-
-void force_point_blocks(int pb) { t_forced_pb = pb; }
-
-void set_tuned_point_blocks(int pb) {
-    int dev = 0;
-    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < TUNE_MAX_DEVICES) g_tuned_pb[dev].store(pb);
-}
 
 int env_point_blocks() {
     const char* e = getenv("HKM_POINT_BLOCKS");
@@ -297,18 +287,173 @@ int env_point_blocks() {
     return 0;
 }
 
-int tuned_point_blocks() {
+// ---- the trial: which geometry this chip runs faster, found on the caller's own steps ----------------
+// Nothing extra is launched and nothing waits.  While a device has no verdict, the one-sweep steps of large
+// fits (a million rows or more) that follow each other closely on one stream are taken in three windows of
+// consecutive calls -- two point blocks, one, two again -- each long enough (about 30 ms of device time by
+// the step's flop count) for the clock to settle under its geometry: a device coming out of idle needs some
+// 30 ms of load to reach its clock, and a chip that lowers its clock under one geometry has done so 20 ms
+// into it.  The last third of every window lies between two events on the stream.  Later calls look at the
+// last event without waiting; once it has completed, one point block is kept if it beat the SECOND
+// two-block window by at least 1 % (repeated timings differ by half a percent), else two.  A pause between
+// two calls (the device may have gone idle), another shape or another stream starts the windows again, so a
+// process that only ever runs short fits far apart keeps the default, where the choice is worth nothing
+// anyway.  Both geometries write the same bits, so no result depends on any of this.  State: per device,
+// process-wide, behind a mutex.
+static const int TRIAL_MAX_DEVICES = 64;
+static const int64_t TRIAL_MIN_ROWS = int64_t(1) << 20;
+struct GeomTrial {
+    pthread_mutex_t mu = PTHREAD_MUTEX_INITIALIZER;
+    int decided = 0;        // 0: no verdict yet, else 1 or 2
+    int window = 0;         // 0: two point blocks, 1: one, 2: two again; 3: all recorded, verdict pending
+    int calls = 0;          // calls made in the current window
+    int window_calls = 0;   // length of a window for the shape under trial
+    int64_t n = 0;          // the shape and the stream under trial
+    int d = 0, k = 0;
+    hipStream_t stream = nullptr;
+    double last_call = 0.;  // host clock at the previous call, seconds
+    double gap = 0.;        // a longer pause than this between two calls starts over
+    hipEvent_t ev[3][2] = {};
+    bool have_events = false;
+    float window_ms[3] = {0.f, 0.f, 0.f};  // per step, for the query
+};
+static GeomTrial g_trial[TRIAL_MAX_DEVICES];
+
+static double host_seconds() {
+    timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return double(ts.tv_sec) + 1e-9 * double(ts.tv_nsec);
+}
+
+static GeomTrial* trial_of_device() {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TUNE_MAX_DEVICES) return 0;
-    return g_tuned_pb[dev].load();
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TRIAL_MAX_DEVICES) return nullptr;
+    return &g_trial[dev];
+}
+
+int tuned_point_blocks() {
+    GeomTrial* t = trial_of_device();
+    if (!t) return 0;
+    pthread_mutex_lock(&t->mu);
+    const int v = t->decided;
+    pthread_mutex_unlock(&t->mu);
+    return v;
+}
+
+int trial_report(float* ms_two, float* ms_one) {
+    GeomTrial* t = trial_of_device();
+    if (!t) return 0;
+    pthread_mutex_lock(&t->mu);
+    const int v = t->decided;
+    if (ms_two) *ms_two = t->window_ms[2];
+    if (ms_one) *ms_one = t->window_ms[1];
+    pthread_mutex_unlock(&t->mu);
+    return v;
 }
 
 int resident_point_blocks(int dp) {
     if (dp > 32) return 1;
-    if (t_forced_pb) return t_forced_pb;
     if (const int e = env_point_blocks()) return e;
     if (const int t = tuned_point_blocks()) return t;
     return 2;
+}
+
+// What the one-sweep launcher asks before and tells after its launch.  `end` is the event to record behind
+// the launch (the last call of a window), or null.
+struct TrialTicket {
+    int pb = 2;
+    hipEvent_t end = nullptr;
+};
+
+static void trial_restart(GeomTrial& t, int64_t N, int32_t D, int32_t K, hipStream_t st) {
+    t.window = 0;
+    t.calls = 0;
+    t.n = N;
+    t.d = D;
+    t.k = K;
+    t.stream = st;
+    // the step's time from its flop count at about two thirds of the matrix peak: only sizes the windows
+    const double kp = double((K + 31) / 32 * 32);
+    const double est_ms = 2.0 * double(N) * kp * resident_dp(D) / 1.0e11;
+    int c = int(30.0 / (est_ms > 1e-3 ? est_ms : 1e-3)) + 1;
+    t.window_calls = c < 6 ? 6 : c > 600 ? 600 : c;
+    t.gap = 1e-3 * (est_ms * 4.0 > 10.0 ? est_ms * 4.0 : 10.0);
+}
+
+static TrialTicket trial_begin(int64_t N, int32_t D, int32_t K, hipStream_t st) {
+    TrialTicket tk;
+    const int dp = resident_dp(D);
+    if (dp > 32) {
+        tk.pb = 1;
+        return tk;
+    }
+    if (const int e = env_point_blocks()) {
+        tk.pb = e;
+        return tk;
+    }
+    GeomTrial* tp = trial_of_device();
+    if (!tp) return tk;
+    GeomTrial& t = *tp;
+    pthread_mutex_lock(&t.mu);
+    if (t.decided) {
+        tk.pb = t.decided;
+    } else if (N >= TRIAL_MIN_ROWS) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        const bool capturing = hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+        if (t.window == 3) {
+            // every window is recorded: a look at the last event, no wait
+            if (hipEventQuery(t.ev[2][1]) == hipSuccess) {
+                bool ok = true;
+                for (int w = 0; w < 3; ++w) {
+                    float ms = 0.f;
+                    ok = ok && hipEventElapsedTime(&ms, t.ev[w][0], t.ev[w][1]) == hipSuccess;
+                    const int timed = t.window_calls / 3 > 2 ? t.window_calls / 3 : 2;
+                    t.window_ms[w] = ms / float(timed);
+                }
+                if (ok && t.window_ms[1] > 0.f && t.window_ms[2] > 0.f) {
+                    t.decided = t.window_ms[1] < 0.99f * t.window_ms[2] ? 1 : 2;
+                    for (auto& pair : t.ev)
+                        for (auto& e : pair) (void)hipEventDestroy(e);
+                    t.have_events = false;
+                    tk.pb = t.decided;
+                } else {
+                    t.window = 0;  // unusable timings: start over
+                    t.calls = 0;
+                }
+            } else {
+                (void)hipGetLastError();  // hipErrorNotReady is no error of this call
+            }
+        } else if (!capturing) {
+            const double now = host_seconds();
+            const bool other = t.n != N || t.d != D || t.k != K || t.stream != st;
+            if (other || t.window_calls == 0 || (t.calls + t.window > 0 && now - t.last_call > t.gap))
+                trial_restart(t, N, D, K, st);
+            t.last_call = now;
+            if (!t.have_events) {
+                bool ok = true;
+                for (auto& pair : t.ev)
+                    for (auto& e : pair) ok = ok && hipEventCreate(&e) == hipSuccess;
+                t.have_events = ok;
+                if (!ok) (void)hipGetLastError();
+            }
+            if (t.have_events) {
+                tk.pb = t.window == 1 ? 1 : 2;
+                const int timed = t.window_calls / 3 > 2 ? t.window_calls / 3 : 2;
+                if (t.calls == t.window_calls - timed) (void)hipEventRecord(t.ev[t.window][0], st);
+                if (++t.calls == t.window_calls) {
+                    tk.end = t.ev[t.window][1];
+                    t.calls = 0;
+                    ++t.window;
+                }
+            }
+        }
+    }
+    pthread_mutex_unlock(&t.mu);
+    return tk;
+}
+
+static void trial_end(const TrialTicket& tk, hipStream_t st) {
+    if (tk.end) (void)hipEventRecord(tk.end, st);
 }
 
 template <int DP, int PB, bool VEC>
@@ -853,7 +998,7 @@ size_t fused_lds_bytes(int32_t D, int32_t K) { return fused_lds_bytes_with(D, K,
 
 int fused_grid(int64_t N, int32_t D) {
     const int dp = resident_dp(D);
-    const int pb = resident_point_blocks(dp);
+    const int pb = dp > 32 ? 1 : 2;  // up to 32 features both geometries cut the rows into the same tiles
     const int64_t tile_rows = int64_t(fused_threads(pb, dp) / 64) * pb * 32;
     const int64_t ntiles = (N + tile_rows - 1) / tile_rows;
     int64_t grid = num_cus();
@@ -894,15 +1039,22 @@ int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx
                                int32_t* fcnt, int32_t* flags, hipStream_t st) {
     const bool vec = aligned16(X) && (ldx % 4 == 0) && (D % 4 == 0);
     const int dp = resident_dp(D);
-    const int pb = resident_point_blocks(dp);
-#define HKM_CASE(d, b)                                                                                         \
-    if (dp == d && pb == b)                                                                                    \
-        return vec ? launch_fused_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st) \
-                   : launch_fused_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);
+    const TrialTicket tk = trial_begin(N, D, K, st);
+    const int pb = tk.pb;
+    int rc = HKM_EUNSUPPORTED;
+    bool found = false;
+#define HKM_CASE(d, b)                                                                                           \
+    if (!found && dp == d && pb == b) {                                                                          \
+        found = true;                                                                                            \
+        rc = vec ? launch_fused_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st)    \
+                 : launch_fused_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);  \
+    }
     HKM_CASE(8, 2) HKM_CASE(8, 1) HKM_CASE(16, 2) HKM_CASE(16, 1) HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2)
     HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
 #undef HKM_CASE
-    return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
+    trial_end(tk, st);
+    if (!found) return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
+    return rc;
 }
 
 int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,

@@ -170,13 +170,12 @@ bool fused_eligible(int32_t D, int32_t K);
 size_t fused_lds_bytes(int32_t D, int32_t K);
 int fused_grid(int64_t N, int32_t D);
 // point blocks per wave of the resident matrix-core kernels (hkm_assign_mfma.hip): the choice for a padded
-// width, its sources (environment, what the tuning call measured on the current device), and the tuning
-// call's handles
+// width and its sources (environment, what the trial on the caller's own steps found on the current device:
+// 0 while it has no verdict; trial_report also hands out the per-step times of its last two windows)
 int resident_point_blocks(int dp);
 int env_point_blocks();
 int tuned_point_blocks();
-void force_point_blocks(int pb);
-void set_tuned_point_blocks(int pb);
+int trial_report(float* ms_two, float* ms_one);
 int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                                int32_t K, int64_t ldc, int32_t* labels, float* min_d2, double* fsum,
                                int32_t* fcnt, int32_t* flags, hipStream_t st);
@@ -280,9 +279,5 @@ int launch_laplacian(const float* S, int64_t N, int64_t lds, int32_t definition,
                      float eps, float* L, int64_t ldl, float* degree, hipStream_t st);
 int launch_laplacian_f64(const double* S, int64_t N, int64_t lds, int32_t definition, int32_t mode, int32_t weighted,
                          double eps, double* L, int64_t ldl, double* degree, hipStream_t st);
-
-// microbenchmarks (hkm_probe.hip)
-int launch_probe_mfma(int32_t op, int32_t nops, int32_t iters, int32_t grid, float* out, hipStream_t st);
-int launch_probe_stream(const void* src, void* dst, size_t bytes, int32_t mode, float* sink, hipStream_t st);
 
 }  // namespace hkm

@@ -49,7 +49,14 @@ __global__ __launch_bounds__(256) void laplacian_finish_kernel(const T* S, int64
     } else {
         const T di = degree[i] == T(0) ? T(1) : degree[i];
         const T dj = degree[j] == T(0) ? T(1) : degree[j];
-        v = j == i ? T(1) : ((a / sqrt(di)) / sqrt(dj)) * T(-1);
+        if (sizeof(T) == 8 && !weighted && mode != 0) {
+            // an unweighted graph is an int32 adjacency matrix in the reference, divided by the float32 square
+            // roots of its integer degrees (heat/graph/laplacian.py:96-97,129-133): float32 arithmetic whatever
+            // the similarities' type was (adjacency and degrees are small integers, exact in either type)
+            v = j == i ? T(1) : T(((float(a) / sqrtf(float(di))) / sqrtf(float(dj))) * -1.0f);
+        } else {
+            v = j == i ? T(1) : ((a / sqrt(di)) / sqrt(dj)) * T(-1);
+        }
     }
     L[i * ldl + j] = v;
 }

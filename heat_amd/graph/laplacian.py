@@ -42,6 +42,9 @@ class Laplacian:
         S = self.similarity_metric(X)
         if not isinstance(S, DNDarray) or len(S.shape) != 2 or S.shape[0] != S.shape[1]:
             raise ValueError("the similarity function must return a square DNDarray")
+        # the reference zeroes the diagonal of what the similarity call returned, in place (:123): a caller that
+        # keeps that matrix sees the same change here
+        S.larray.fill_diagonal_(0)
         s = S.larray
         if s.dtype not in (torch.float32, torch.float64):
             s = s.to(torch.float32)
@@ -51,7 +54,7 @@ class Laplacian:
         mode = 0 if self.mode == "fully_connected" else (1 if self.epsilon[0] == "upper" else 2)
         degree = torch.empty((n,), dtype=s.dtype, device=s.device)
         # L gets storage of its own: the similarity callable may have returned a matrix it keeps (a cached
-        # or precomputed one), which the reference leaves intact apart from its zeroed diagonal
+        # or precomputed one), which the reference leaves intact apart from the diagonal zeroed above
         out = torch.empty((n, n), dtype=s.dtype, device=s.device)
         _native.laplacian(s, out, 0 if self.definition == "simple" else 1, mode, bool(self.weighted),
                           float(self.epsilon[1]), degree)

@@ -99,6 +99,10 @@ int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const floa
  * (D <= 64: every K up to about four million; D > 64: up to about two million rows, 8 bytes each).
  * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
  * calls on one stream are ordered and each refills what it reads.
+ * The array's device address is looked up once per device (hipGetSymbolAddress), by whichever comes first on
+ * that device: hkm_static_scratch_bytes() or hkm_assign_static_f32.  A stream under capture may refuse that
+ * lookup, so call hkm_static_scratch_bytes() once with the device current BEFORE capturing; after that the
+ * entry point only enqueues kernels and can be captured into a HIP graph and replayed.
  */
 #define HKM_STATIC_SCRATCH_BYTES (16u << 20)
 size_t hkm_static_scratch_bytes(void);
@@ -335,7 +339,7 @@ int hkm_silhouette_finish_f32(const float* S, int64_t N, int32_t K, int64_t lds,
  *   definition HKM_LAPLACIAN_SIMPLE: L = diag(degree) - A;
  *   definition HKM_LAPLACIAN_NORM_SYM: L = -(A / sqrt(d_i)) / sqrt(d_j) with zero degrees taken as 1, and
  *   ones on the diagonal.
- * N <= 2^24.  hkm_laplacian_f64 is the same on float64 matrices (the reference keeps float64 similarities in
+ * N <= 65535 * 256 = 16 776 960.  hkm_laplacian_f64 is the same on float64 matrices (the reference keeps float64 similarities in
  * float64).  The reference's unweighted simple Laplacian is an integer matrix: its entries are small whole
  * numbers here, which the caller may cast.
  */
@@ -374,51 +378,6 @@ int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, i
 
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
-
-/*
- * The resident matrix-core kernels (up to 32 features) come in two launch geometries -- two point blocks per wave,
- * or one with twice the waves -- that produce the same bits and differ in speed by a few percent either way,
- * depending on the clock the individual chip holds under them.  No counterpart in the reference.
- * hkm_tune_lloyd_step_f32: hkm_lloyd_step_f32 with the same arguments and the same results, which -- where the
- *   shape has the choice and HKM_POINT_BLOCKS is not set -- then runs the same step for about 0.2 s more (two
- *   point blocks, one, two again, each window after a warm-up of its own, sized in time), WAITS for the
- *   device, and remembers the faster geometry for the current device until the process ends.  Returns the point blocks chosen (1 or 2), 0 if the shape has no choice, or a negative
- *   error; refused under stream capture.  Not calling it leaves the default (two).
- * hkm_point_blocks: the point blocks per wave a call with D features would use now (0: D has no resident
- *   kernel); *tuned (if not NULL) tells whether that came from a measurement on the current device.
- */
-int hkm_tune_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new,
-                            int32_t K, int32_t* labels, float* shift, float* sse, void* ws, size_t ws_bytes,
-                            void* hip_stream);
-int hkm_point_blocks(int32_t D, int32_t* tuned);
-
-/*
- * Timing of the dominant kernel, for benchmarks (no counterpart in the reference).  After
- * hkm_profile_enable(1) on the calling thread, every hkm_assign_f32 / hkm_assign_static_f32 /
- * hkm_lloyd_step_f32 call of that thread records one pair of events on its stream, right before and right
- * after the launch of its distance kernel (the one hkm_assign_kernel_name / hkm_lloyd_kernel_name names:
- * the fused distance + argmin kernel, or the one-sweep kernel that also forms the per-cluster sums) and of
- * nothing else.  hkm_profile_collect waits for the recorded pairs, writes their durations in milliseconds
- * to ms (HOST pointer, at most cap of them, in call order), the number recorded to *count, and starts
- * over.  At most 512 pairs are kept between two collects.  hkm_profile_enable(0) switches it off.  While
- * off -- the default -- nothing is recorded and no event exists.
- */
-int hkm_profile_enable(int32_t on);
-int hkm_profile_collect(float* ms, int32_t cap, int32_t* count);
-
-/*
- * Microbenchmarks behind the hardware figures the kernels are designed around (no counterpart in the
- * reference; bench.py --probe times them).  Each call enqueues ONE kernel.
- * hkm_probe_mfma_f32: every wave issues iters * 16 fp32 matrix instructions (v_mfma_f32_32x32x2_f32, two
- *   independent accumulators), each followed by `nops` instructions of kind `op`: 0 none (nops = 0),
- *   1 v_fma_f32, 2 v_cndmask_b32, 3 v_min3_f32, 4 s_add_u32 (scalar unit), 5 v_cmp_lt_f32, 6 v_mov_b64;
- *   nops 4 or 8.
- *   grid workgroups of 256 threads; out receives grid * 256 floats.  flops = grid * 4 * iters * 16 * 4096.
- * hkm_probe_stream: mode 0 copies bytes from src to dst, 1 reads src, 2 reads src with non-temporal loads,
- *   3 fills dst; 16-byte vectors, four in flight per thread; sink is one device float.
- */
-int hkm_probe_mfma_f32(int32_t op, int32_t nops, int32_t iters, int32_t grid, float* out, void* hip_stream);
-int hkm_probe_stream(const void* src, void* dst, size_t bytes, int32_t mode, float* sink, void* hip_stream);
 
 /* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "mfma_resident",
  * "mfma_tiled", "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */

@@ -433,14 +433,20 @@ def label_agreement(
     ``n_strict_b_wrong`` those where it is ``labels_b`` (with ``labels_b`` the reference's labels these are
     the rows its own fp32 rounding misorders: an evaluation in exact arithmetic differs from it there too).
 
-    Returns dict(n, n_diff, n_unexcused, agreement, n_strict, n_strict_a_wrong, n_strict_b_wrong,
-    max_strict_gap, max_strict_abs).
+    Which side an unexcused row is due to: ``n_unexcused_a`` counts the differing rows where the centroid
+    ``labels_a`` chose lies outside that limit, ``n_unexcused_b`` the same for ``labels_b``; ``worst_a_ulp`` and
+    ``worst_b_ulp`` are the largest excess of a side's chosen distance over ``(1 + rel_gap) * d2_best``, in units
+    of eps32 * (|x|^2 + |c|^2) (the limit allows max(2, sqrt(D)/4) of them).
+
+    Returns dict(n, n_diff, n_unexcused, n_unexcused_a, n_unexcused_b, worst_a_ulp, worst_b_ulp, agreement,
+    n_strict, n_strict_a_wrong, n_strict_b_wrong, max_strict_gap, max_strict_abs).
     """
     a = labels_a.view(-1).to(torch.int64).cpu()
     b = labels_b.view(-1).to(torch.int64).cpu()
     n = a.numel()
     diff = torch.nonzero(a != b).view(-1)
-    n_unexcused = 0
+    n_unexcused = n_unexcused_a = n_unexcused_b = 0
+    worst_a = worst_b = 0.0
     n_strict = n_strict_a = n_strict_b = 0
     max_strict_gap = 0.0
     max_strict_abs = 0.0
@@ -459,6 +465,11 @@ def label_agreement(
         lim = best * (1.0 + rel_gap) + dfac * mag + 1e-300
         ok = (da <= lim) & (db <= lim)
         n_unexcused += int((~ok).sum())
+        n_unexcused_a += int((da > lim).sum())
+        n_unexcused_b += int((db > lim).sum())
+        res = (eps32 * mag).clamp_min(1e-300)
+        worst_a = max(worst_a, float(((da - best * (1.0 + rel_gap)) / res).max()))
+        worst_b = max(worst_b, float(((db - best * (1.0 + rel_gap)) / res).max()))
         if d2.shape[1] > 1:
             two = torch.topk(d2, 2, dim=1, largest=False).values
             gap_abs = two[:, 1] - two[:, 0]
@@ -474,6 +485,10 @@ def label_agreement(
         "n": n,
         "n_diff": int(diff.numel()),
         "n_unexcused": n_unexcused,
+        "n_unexcused_a": n_unexcused_a,
+        "n_unexcused_b": n_unexcused_b,
+        "worst_a_ulp": worst_a,
+        "worst_b_ulp": worst_b,
         "agreement": 1.0 - diff.numel() / max(n, 1),
         "n_strict": n_strict,
         "n_strict_a_wrong": n_strict_a,

@@ -9,6 +9,7 @@
 #include <cstring>
 
 #include "hkm.h"
+#include "hkm_bench.h"
 
 static int failures = 0;
 
@@ -134,8 +135,11 @@ int main() {
         std::printf("FAIL hkm_point_blocks\n");
         ++failures;
     }
-    EXPECT(hkm_tune_lloyd_step_f32(nullptr, 10, 32, 32, f, f + 4096, 8, i32, f, nullptr, ws, big, nullptr), HKM_EINVAL);
-    EXPECT(hkm_tune_lloyd_step_f32(f, 10, 32, 32, f, f + 4096, 8, i32, f, nullptr, ws, 16, nullptr), HKM_EWORKSPACE);
+    float ms_two = -1.f, ms_one = -1.f;
+    if (hkm_point_blocks_trial(&ms_two, &ms_one) != 0 || hkm_point_blocks_trial(nullptr, nullptr) != 0) {
+        std::printf("FAIL hkm_point_blocks_trial\n");
+        ++failures;
+    }
 
     // ---- the measurement hooks with nothing recorded
     float ms[4];

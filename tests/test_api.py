@@ -156,6 +156,23 @@ def _declared_symbols():
     return sorted(set(re.findall(r"\b(hkm_[a-z0-9_]+)\s*\(", text)))
 
 
+def test_bench_hooks_are_declared_apart_and_exported():
+    """include/hkm_bench.h: the measuring hooks live in libhkm.so, the microbenchmarks in a library of their own
+    that the product never loads; include/hkm.h declares none of them."""
+    from heat_amd.utils import benchhooks
+
+    text = open(os.path.join(ROOT, "include", "hkm_bench.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(hkm_[a-z0-9_]+)\s*\(", text)))
+    assert names == sorted(benchhooks.SIGNATURES)
+    assert not set(names) & set(_declared_symbols())
+    lib, blib = benchhooks.hkm(), benchhooks.bench()
+    for name, (home, _, _) in benchhooks.SIGNATURES.items():
+        assert hasattr(lib if home == "hkm" else blib, name), name
+        if home == "bench":
+            assert not hasattr(lib, name), f"{name} must not be part of the product library"
+
+
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
@@ -453,7 +470,7 @@ def test_argument_validation_of_the_neighbour_silhouette_and_laplacian_entry_poi
     assert lib.hkm_laplacian_f32(good, 10, 10, 0, 3, 1, 1.0, good, 10, other, None) == einval
     assert lib.hkm_laplacian_f32(good, 10, 9, 0, 0, 1, 1.0, good, 10, other, None) == einval
     assert lib.hkm_laplacian_f32(good, 10, 10, 0, 0, 1, 1.0, good, 10, None, None) == einval
-    big = (1 << 24) + 1
+    big = 65535 * 256 + 1
     assert lib.hkm_laplacian_f32(good, big, big, 0, 0, 1, 1.0, good, big, other, None) == eunsup
     assert lib.hkm_laplacian_f64(good, big, big, 0, 0, 1, 1.0, good, big, other, None) == eunsup
     assert lib.hkm_laplacian_f64(good, 10, 10, 0, 0, 1, 1.0, good, 10, None, None) == einval

@@ -343,36 +343,50 @@ def test_one_point_block_per_wave_gives_the_same_labels(cuda, n, d, k, monkeypat
     assert torch.equal(one[3], two[3]) and one[4] == two[4]
 
 
-def test_tuning_call_is_a_step_and_settles_on_a_geometry(cuda, monkeypatch):
+def test_geometry_trial_runs_on_the_callers_own_steps(cuda, monkeypatch):
+    """The choice between the two launch geometries of the resident matrix-core kernels is made on the steps a
+    large fit issues anyway: no extra launch, no wait, the same bits whichever geometry a step ran in, and a
+    verdict for the device once three windows of consecutive steps have been timed."""
+    from heat_amd.cluster._lloyd import LloydLoop
+    from heat_amd.utils import benchhooks
+
     monkeypatch.delenv("HKM_POINT_BLOCKS", raising=False)
-    n, d, k = 300000, 32, 64
+    n, d, k = 1 << 20, 16, 32
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
     x, _ = _data(n, d, k, seed=77)
     c0 = x[torch.randperm(n, generator=torch.Generator().manual_seed(2))[:k]].contiguous()
     xs, cs = x.to(cuda), c0.to(cuda)
-    ws = _native.Workspace(cuda)
-    lab = torch.empty((n,), dtype=torch.int32, device=cuda)
-    cn = torch.empty_like(cs)
-    shift = torch.empty((), device=cuda)
-    _native.lloyd_step(xs, cs, cn, lab, shift, None, ws)
-    torch.cuda.synchronize()
-    want = (lab.clone(), cn.clone(), float(shift))
-    lab.zero_(), cn.zero_()
-    chosen = _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws)
-    torch.cuda.synchronize()
-    assert chosen in (1, 2)
-    assert _native.point_blocks(d) == (chosen, True)
-    assert torch.equal(lab, want[0]) and torch.equal(cn, want[1]) and float(shift) == want[2]
-    # shapes without the choice: wider rows, the narrow kernels
-    assert _native.point_blocks(48) == (1, True) or _native.point_blocks(48) == (1, False)
-    assert _native.point_blocks(100)[0] == 0
-    x8 = torch.rand(5000, 8).to(cuda)
-    c8 = x8[:16].contiguous()
-    assert _native.tune_lloyd_step(x8, c8, torch.empty_like(c8), torch.empty((5000,), dtype=torch.int32, device=cuda),
-                                   shift, ws) == 0
-    # the environment decides where it is set
+    # what a run pinned to one geometry gives
+    monkeypatch.setenv("HKM_POINT_BLOCKS", "2")
+    pinned = LloydLoop(xs, cs, _native.Workspace(cuda))
+    assert pinned.run(12, None) == 12
+    want_c, want_lab = pinned.centers.clone(), pinned.labels.clone()
+    assert benchhooks.point_blocks(d) == (2, False)
     monkeypatch.setenv("HKM_POINT_BLOCKS", "1")
-    assert _native.point_blocks(d) == (1, False)
-    assert _native.tune_lloyd_step(xs, cs, cn, lab, shift, ws) == 0
+    assert benchhooks.point_blocks(d) == (1, False)
+    monkeypatch.delenv("HKM_POINT_BLOCKS")
+    # steps in a row, as a fit issues them: the windows fill, then a later call finds the verdict
+    verdict = benchhooks.point_blocks_trial()[0]
+    loop = LloydLoop(xs, cs, _native.Workspace(cuda))
+    assert loop.run(12, None) == 12
+    assert torch.equal(loop.centers, want_c) and torch.equal(loop.labels, want_lab)
+    for _ in range(40):
+        if verdict:
+            break
+        assert loop.run(100, None) == 100
+        torch.cuda.synchronize()
+        assert loop.run(1, None) == 1  # looks at the last window's event
+        verdict = benchhooks.point_blocks_trial()[0]
+    v, ms_two, ms_one = benchhooks.point_blocks_trial()
+    print(f"geometry trial: verdict {v} point block(s) per wave, {ms_two:.4f} ms per step with two, "
+          f"{ms_one:.4f} ms with one", flush=True)
+    assert v in (1, 2) and benchhooks.point_blocks(d) == (v, True)
+    after = LloydLoop(xs, cs, _native.Workspace(cuda))
+    assert after.run(12, None) == 12
+    assert torch.equal(after.centers, want_c) and torch.equal(after.labels, want_lab)
+    # shapes without the choice: wider rows have one geometry, rows beyond 64 features no resident kernel
+    assert benchhooks.point_blocks(48)[0] == 1
+    assert benchhooks.point_blocks(100)[0] == 0
 
 
 @pytest.mark.parametrize("n,d,k", [(30000, 16, 15), (20000, 9, 25), (25000, 12, 20), (10000, 10, 22), (40000, 4, 50), (30000, 7, 31),

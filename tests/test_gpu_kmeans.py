@@ -14,7 +14,10 @@ distances are more than 1e-5 relative apart.  The reference computes (|x|^2 + |c
 own rounding (an ulp of |x|^2 + |c|^2 is 1e-5 of a typical squared distance on the D = 32 workload and up
 to 1e-4 on the D = 3 one) misorders such rows now and then: an evaluation of its formula in EXACT
 arithmetic differs from it on the same rows (tests/test_oracle_pins.py).  What is asserted:
-  * no difference outside the resolution of the expansion (n_unexcused == 0, see oracle.label_agreement);
+  * on every differing row the centroid the PRODUCT chose lies within one ulp of |x|^2 + |c|^2 -- the resolution
+    of the fp32 expansion -- of (1 + 1e-5) times the best fp64 squared distance (worst_a_ulp <= 1, see
+    oracle.label_agreement; measured at most 0.7).  The centroid the reference chose is held to a sanity bound
+    only (4 ulp, one row per million): on the 10M x 32 workload it strays 2.1 ulp on one row, by its own rounding;
   * on the D >= 8 workloads (c1 - c4) at most 4 strict rows per million comparisons, none with an fp64 gap
     above 5e-5 relative (on such a row either side may be the one that missed the
     fp64 nearest centroid: both evaluate in fp32; the report says which);
@@ -39,8 +42,15 @@ def _label_bar(rep, name, report, narrow=False):
     """The label bar of this file's header on one comparison; ``narrow`` selects the D = 3 form."""
     report(f"{name}: n={rep['n']} differing={rep['n_diff']} strict(>1e-5 fp64 gap)={rep['n_strict']} "
            f"[product misses fp64 nearest: {rep['n_strict_a_wrong']}, reference misses it: {rep['n_strict_b_wrong']}] "
-           f"max_strict_gap={rep['max_strict_gap']:.3e} max_gap_in_ulp_of_expansion={rep['max_strict_abs']:.2f}")
-    assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, (name, rep)
+           f"max_strict_gap={rep['max_strict_gap']:.3e} max_gap_in_ulp_of_expansion={rep['max_strict_abs']:.2f} "
+           f"outside_resolution[product {rep['n_unexcused_a']}, reference {rep['n_unexcused_b']}] "
+           f"worst_excess_ulp[product {rep['worst_a_ulp']:.2f}, reference {rep['worst_b_ulp']:.2f}]")
+    # The product's side of every differing row: its centroid lies within ONE ulp of |x|^2 + |c|^2 (the
+    # resolution of the fp32 expansion) of (1 + 1e-5) times the best fp64 squared distance -- measured at most
+    # 0.7 on the full-size workloads.  The reference's side is a fact about the reference (torch's CPU rounding,
+    # which depends on the host): reported, and only held to a sanity bound that an error in the oracle would break.
+    assert rep["n_unexcused_a"] == 0 and rep["worst_a_ulp"] <= 1.0 and rep["agreement"] >= 0.9999, (name, rep)
+    assert rep["worst_b_ulp"] <= 4.0 and rep["n_unexcused_b"] <= max(1, 1e-6 * rep["n"]), (name, rep)
     if narrow:
         assert rep["max_strict_abs"] <= 2.0 and rep["n_strict"] <= max(2, 2e-6 * rep["n"]), (name, rep)
     else:
@@ -96,7 +106,7 @@ def _stepwise_parity(w, dev, iters, literal, report=print):
     flips = 0
     n_iter = 0
     tot = dict(n=0, n_diff=0, n_strict=0, n_strict_a_wrong=0, n_strict_b_wrong=0, max_strict_gap=0.0,
-               max_strict_abs=0.0, n_unexcused=0)
+               max_strict_abs=0.0, n_unexcused=0, n_unexcused_a=0, n_unexcused_b=0, worst_a_ulp=0.0, worst_b_ulp=0.0)
     for _ in range(iters):
         n_iter += 1
         c_in = c_ref.to(dev)
@@ -111,9 +121,9 @@ def _stepwise_parity(w, dev, iters, literal, report=print):
         rep = orc.label_agreement(w.x, c_ref, lab.cpu(), ref_lab)
         assert rep["n_unexcused"] == 0 and rep["agreement"] >= 0.9999, (n_iter, rep)
         flips += rep["n_diff"]
-        for key in ("n", "n_diff", "n_strict", "n_strict_a_wrong", "n_strict_b_wrong"):
+        for key in ("n", "n_diff", "n_strict", "n_strict_a_wrong", "n_strict_b_wrong", "n_unexcused_a", "n_unexcused_b"):
             tot[key] += rep[key]
-        for key in ("max_strict_gap", "max_strict_abs"):
+        for key in ("max_strict_gap", "max_strict_abs", "worst_a_ulp", "worst_b_ulp"):
             tot[key] = max(tot[key], rep[key])
         own, _ = orc.update_centroids_fast(w.x, lab.cpu().long().view(-1, 1), w.k)
         assert orc.rel_err_centers(c_out.cpu(), own) <= 1e-5, n_iter
@@ -167,14 +177,12 @@ def test_config1_full_size_against_literal_oracle(cuda, parity_report):
     km, xd = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
     _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
     lab, fv = orc.predict(w.x, ref["cluster_centers"])
-    ref_km, _ = _fit(w.x, ref["cluster_centers"], w.k, 1, None, cuda)
-    pred = ref_km.predict(ht.array(w.x.to(cuda), split=0))  # predicts against centroids after 1 more step
     pred0 = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(ref["cluster_centers"].to(cuda)), max_iter=1)
     pred0._cluster_centers = ht.array(ref["cluster_centers"].to(cuda))
     p = pred0.predict(xd)
     assert float((p.larray.cpu() == lab).float().mean()) >= 0.9999
     assert orc.rel_err_scalar(float(pred0.functional_value_), float(fv)) <= 1e-4
-    assert pred.shape == (w.x.shape[0], 1)
+    assert p.shape == (w.x.shape[0], 1)
     km2, _ = _fit(w.x, w.init, w.k, w.max_iter, 0.0, cuda)
     assert torch.equal(km.cluster_centers_.larray, km2.cluster_centers_.larray)
     assert torch.equal(km.labels_.larray, km2.labels_.larray)
@@ -224,9 +232,13 @@ def test_config2_cdist_argmin(cuda, scale, parity_report):
 
 
 def _full_size_properties(w, dev, report, iters):
-    """Properties that hold at any size: counts sum to N, sum_k n_k C_k = sum_i x_i, the shift
-    sequence is what the centroids say, SSE does not increase, predict == re-assignment, and two runs are
-    bit-identical; the labels of the first step are compared with the oracle's on EVERY row."""
+    """The workload at its full size for its own number of iterations (heat/cluster/kmeans.py:131-146).
+    Properties that hold at any size, at every iteration: counts sum to N, sum_k n_k C_k = sum_i x_i, the
+    shift sequence is what the centroids say, SSE does not increase.  Against the oracle, on EVERY row: the
+    labels of the first step and the labels of the LAST iteration (against the centroids that iteration
+    started from).  Through the public estimator: fit == the step loop bit for bit, cluster_centers_ equal the
+    oracle's means of the returned labels, inertia_ equals the fp64 shift between the last two sets of
+    centroids, predict == re-assignment, and a second fit is bit-identical."""
     from heat_amd import _native
 
     n, d = w.x.shape
@@ -256,25 +268,43 @@ def _full_size_properties(w, dev, report, iters):
             _label_bar(rep, f"{w.name} full size, first step", report, narrow=d < 8)
         c_cur, c_nxt = c_nxt, c_cur
     assert all(b <= a * (1 + 1e-5) for a, b in zip(sse_hist, sse_hist[1:])), sse_hist
+    c_start_last = c_nxt.cpu()  # after the swap: the centroids the last iteration started from
     km = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(dev)), max_iter=iters, tol=0.0).fit(xd)
+    assert km.n_iter_ == iters  # none of these workloads reaches a fixed point that early
     assert torch.equal(km.cluster_centers_.larray, c_cur), "fit() and the step loop must agree bit for bit"
     assert torch.equal(km.labels_.larray.view(-1), lab.long())
+    # the last iteration against the oracle: labels on every row, the means of those labels, the shift
+    lab_cpu = km.labels_.larray.cpu()
+    ref_lab, _ = orc.assign_to_cluster_fast(w.x, c_start_last)
+    rep = orc.label_agreement(w.x, c_start_last, lab_cpu.view(-1).to(torch.int32), ref_lab)
+    _label_bar(rep, f"{w.name} full size, iteration {iters} of {iters}", report, narrow=d < 8)
+    want, _ = orc.update_centroids_fast(w.x, lab_cpu, w.k)
+    err = orc.rel_err_centers(km.cluster_centers_.larray.cpu(), want)
+    assert err <= 1e-5, err
+    want_shift = float(((c_start_last.double() - want.double()) ** 2).sum())
+    assert orc.rel_err_scalar(float(km.inertia_), want_shift, floor=1e-12) <= 1e-4, (float(km.inertia_), want_shift)
+    report(f"{w.name} full size, {iters} iterations through KMeans.fit: n_iter_={km.n_iter_} "
+           f"centroids vs oracle means of the same labels {err:.2e}, inertia_ {float(km.inertia_):.6g} "
+           f"(fp64 shift {want_shift:.6g}), SSE {sse_hist[0]:.6g} -> {sse_hist[-1]:.6g}")
     pred = km.predict(xd)
     lab2 = torch.empty_like(lab)
     _native.assign(x, c_cur, lab2, None, ws)
     assert torch.equal(pred.larray.view(-1), lab2.long())
+    km2 = ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(dev)), max_iter=iters, tol=0.0).fit(xd)
+    assert torch.equal(km2.cluster_centers_.larray, km.cluster_centers_.larray)
+    assert torch.equal(km2.labels_.larray, km.labels_.larray) and float(km2.inertia_) == float(km.inertia_)
 
 
 def test_config3_full_size_properties(cuda, parity_report):
-    _full_size_properties(synthetic.config3(), cuda, parity_report, iters=3)
+    _full_size_properties(synthetic.config3(), cuda, parity_report, iters=10)
 
 
 def test_config5_full_size_properties(cuda, parity_report):
-    _full_size_properties(synthetic.config5(), cuda, parity_report, iters=2)
+    _full_size_properties(synthetic.config5(), cuda, parity_report, iters=10)
 
 
 def test_config4_full_size_properties(cuda, parity_report):
-    _full_size_properties(synthetic.config4(), cuda, parity_report, iters=2)
+    _full_size_properties(synthetic.config4(), cuda, parity_report, iters=5)
 
 
 def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
@@ -294,17 +324,23 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
         lab = torch.empty((x.shape[0],), dtype=torch.int32, device=cuda)
         shift = torch.empty((), device=cuda)
         n_seq = 0
-        for _ in range(40):
+        cnorm = float((c_cur.double() ** 2).sum()) ** 0.5
+        for it in range(40):
             n_seq += 1
             _native.lloyd_step(x, c_cur, c_nxt, lab, shift, None, ws)
-            if tol is not None and float(shift) <= tol + probe._margin(tol):
-                # the loop's rule: a one-sweep step near the stop decision is settled by the two-pass means;
-                # a step that reproduced its own centroids bit for bit counts as no movement
-                unchanged = float(shift) == 0.0
-                _native.update(x, lab, c_nxt, None, ws)
-                _native.shift(c_cur, c_nxt, shift)
-                if unchanged:
-                    shift.zero_()
+            sh = float(shift)
+            if tol is not None:
+                # the loop's rule, restated: a one-sweep step whose shift lies within the rounding error of its
+                # own sums of the tolerance is settled by the two-pass means; a step after the first that
+                # reproduced its own centroids bit for bit counts as no movement
+                e2 = probe._fuzz * (cnorm + sh ** 0.5) ** 2
+                if sh <= tol + 2.0 * (max(tol, 0.0) * e2) ** 0.5 + e2:
+                    unchanged = it > 0 and torch.equal(c_cur, c_nxt)
+                    _native.update(x, lab, c_nxt, None, ws)
+                    _native.shift(c_cur, c_nxt, shift)
+                    if unchanged:
+                        shift.zero_()
+                cnorm += max(float(shift), 0.0) ** 0.5
             c_cur, c_nxt = c_nxt, c_cur
             if tol is not None and float(shift) <= tol:
                 break
@@ -372,6 +408,66 @@ def test_init_at_the_means_of_two_far_blobs_stops_like_the_oracle(cuda, n, d, pa
     assert float(km.inertia_) == float(ref["inertia"])
     assert torch.equal(km.labels_.larray.cpu().view(-1), ref["labels"].view(-1))
     assert orc.rel_err_centers(km.cluster_centers_.larray.cpu(), ref["cluster_centers"]) <= 1e-6
+
+
+@pytest.mark.parametrize("n,d,k", [(30000, 32, 6), (30000, 24, 40), (40000, 8, 5), (1 << 17, 12, 9), (30000, 3, 4)])
+def test_init_at_the_one_sweep_means_of_a_fixed_point_stops_like_the_oracle(cuda, n, d, k, parity_report):
+    """Well-separated blobs at their fixed point, with the init taken from the product's own one-sweep step: those
+    centroids equal the exact means of their labels up to the step's rounding (often not bit for bit), and the
+    step reproduces them bit for bit.  The reference moves them onto the exact means in its first iteration (a
+    shift of a last bit, or exactly 0 where the two coincide) and stops in the iteration after; the product must
+    run the same number of iterations and report the same inertia_ -- the first step has no predecessor whose
+    labels it could have repeated, so a zero shift there proves nothing."""
+    from heat_amd import _native
+
+    assert _native.lloyd_kernel_name(n, d, k) in ("lloyd_small", "lloyd_mfma_resident")
+    g = torch.Generator().manual_seed(17 * d + k)
+    centres = (torch.rand((k, d), generator=g) - 0.5) * 400.0
+    x = (torch.randn((n, d), generator=g) + centres[torch.randint(0, k, (n,), generator=g)]).contiguous()
+    xs = x.to(cuda)
+    ws = _native.Workspace(cuda)
+    c0 = centres.to(cuda).contiguous()
+    c1 = torch.empty_like(c0)
+    lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+    shift = torch.empty((), device=cuda)
+    for _ in range(3):  # onto the fixed point, by one-sweep steps
+        _native.lloyd_step(xs, c0, c1, lab, shift, None, ws)
+        c0, c1 = c1, c0
+    assert float(shift) == 0.0, "the one-sweep step must reproduce its own centroids here"
+    exact = torch.empty_like(c0)
+    _native.update(xs, lab, exact, None, ws)
+    init = c0.cpu()
+    ref = orc.kmeans_fit(x, init, 10, 0.0, literal=True)
+    km, _ = _fit(x, init, k, 10, 0.0, cuda)
+    parity_report(f"init at one-sweep means N={n} D={d} K={k}: one-sweep == exact means bit for bit: "
+                  f"{bool(torch.equal(exact, c0))}; n_iter_ {km.n_iter_} (oracle {ref['n_iter']}), inertia_ "
+                  f"{float(km.inertia_):.3g} (oracle {float(ref['inertia']):.3g})")
+    assert km.n_iter_ == ref["n_iter"]
+    assert float(km.inertia_) == float(ref["inertia"])
+    assert torch.equal(km.labels_.larray.cpu().view(-1), ref["labels"].view(-1))
+    assert orc.rel_err_centers(km.cluster_centers_.larray.cpu(), ref["cluster_centers"]) <= 1e-6
+
+
+@pytest.mark.parametrize("n,d,k", [(1 << 17, 32, 8), (1 << 17, 12, 9), (1 << 17, 3, 8), (1 << 17, 8, 40)])
+def test_init_near_the_origin_and_blobs_far_from_it_stop_like_the_oracle(cuda, n, d, k, parity_report):
+    """Centroids that grow a thousandfold after the first step: the margin inside which a one-sweep step's stop
+    decision is settled on the two-pass means must follow them (it is priced against a bound on the centroids'
+    norm that the loop keeps from the shifts it reads)."""
+    g = torch.Generator().manual_seed(5 * d + k)
+    centres = (torch.rand((k, d), generator=g) - 0.5) * 2000.0
+    x = (torch.randn((n, d), generator=g) * 3.0 + centres[torch.randint(0, k, (n,), generator=g)]).contiguous()
+    # a thousandth of the blob centres: the first assignment is still clear-cut in fp32 (the cross terms differ by
+    # hundreds of ulps of |x|^2), the first update multiplies the centroids by a thousand, and the second step
+    # rounds its sums against centroids of another magnitude than the first did
+    init = (centres / 1000.0).contiguous()
+    ref = orc.kmeans_fit(x, init, 30, 0.0, literal=True)
+    km, _ = _fit(x, init, k, 30, 0.0, cuda)
+    parity_report(f"init near the origin N={n} D={d} K={k}: n_iter_ {km.n_iter_} (oracle {ref['n_iter']}), inertia_ "
+                  f"{float(km.inertia_):.3g} (oracle {float(ref['inertia']):.3g})")
+    assert km.n_iter_ == ref["n_iter"]
+    assert float(km.inertia_) == float(ref["inertia"])
+    assert torch.equal(km.labels_.larray.cpu().view(-1), ref["labels"].view(-1))
+    assert orc.rel_err_centers(km.cluster_centers_.larray.cpu(), ref["cluster_centers"]) <= 1e-5
 
 
 @pytest.mark.parametrize("n,d", [(5000, 32), (5000, 3), (3000, 100), (5000, 16)])

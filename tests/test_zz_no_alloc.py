@@ -85,3 +85,36 @@ def test_static_scratch_assign_rejects_what_does_not_fit(cuda):
     _native.assign_static(x[:, :64], c[:, :64], lab, None)
     torch.cuda.synchronize()
     assert int(lab.max()) == 0
+
+
+@pytest.mark.parametrize("n,d,k", [(6000, 64, 1024), (4096, 32, 256), (5000, 130, 300)])
+def test_static_scratch_assign_under_graph_capture(cuda, n, d, k):
+    """After the documented warm-up (hkm_static_scratch_bytes resolves the array's address outside capture)
+    the entry point only enqueues kernels: one call captured into a HIP graph and replayed several times, with
+    eager work and synchronisations between the replays, gives the workspace path's bits every time."""
+    assert _native.load().hkm_static_scratch_bytes() == 16 << 20  # the warm-up, device current
+    print(f"assign_static under capture: n={n} d={d} k={k} kernel={_native.assign_kernel_name(n, d, k)}", flush=True)
+    x, c = _data(n, d, k, seed=3 * n + d)
+    xs, cs = x.to(cuda), c.to(cuda)
+    lab_w = torch.empty((n,), dtype=torch.int32, device=cuda)
+    md_w = torch.empty((n,), dtype=torch.float32, device=cuda)
+    _native.assign(xs, cs, lab_w, md_w, _native.Workspace(cuda))
+    lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+    md = torch.empty((n,), dtype=torch.float32, device=cuda)
+    _native.assign_static(xs, cs, lab, md)  # every kernel of the call has run once before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _native.assign_static(xs, cs, lab, md)
+    for rep in range(4):
+        lab.fill_(-7)
+        md.fill_(-1.0)
+        if rep % 2:
+            # eager work of the same library in between, on the shared scratch array
+            other = torch.empty((1000,), dtype=torch.int32, device=cuda)
+            _native.assign_static(xs[:1000], cs, other, None)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(lab, lab_w), rep
+        assert torch.equal(md.view(torch.int32), md_w.view(torch.int32)), rep
