@@ -19,9 +19,9 @@ from . import _f64_paths
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
-LIB_VERSION = 303  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
+LIB_VERSION = 304  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
-WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64 = 1, 2, 3, 4, 8, 16
+WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64, WS_FIT = 1, 2, 3, 4, 8, 16, 32
 
 # name -> (restype, argtypes); must list every symbol declared in include/hkm.h
 SIGNATURES = {
@@ -39,6 +39,10 @@ SIGNATURES = {
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_lloyd_fit_supported": (ctypes.c_int, [c_int64, c_int32, c_int32]),
+    "hkm_lloyd_fit_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int32, c_int32,
+                                         ctypes.c_double, c_void_p, c_void_p, c_void_p, c_void_p, ctypes.c_uint64,
+                                         c_void_p, c_size_t, c_void_p]),
     "hkm_shift_f32": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "hkm_functional_value_f32": (ctypes.c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_cdist_f32": (ctypes.c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int32,
@@ -273,6 +277,36 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Op
     buf = ws.get(need)
     check(load().hkm_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
                                     _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
+
+
+def lloyd_fit_supported(n: int, d: int, k: int) -> bool:
+    """True where the whole Lloyd loop runs as one launch (hkm_lloyd_fit_f32 in include/hkm.h)."""
+    return bool(load().hkm_lloyd_fit_supported(n, d, k))
+
+
+FIT_WAIT_LIMIT_US = 2_000_000  # how long a workgroup of the one-launch fit waits for the others before it gives up
+
+
+def lloyd_fit(x: torch.Tensor, c0: torch.Tensor, max_iter: int, tol: Optional[float], c_out: torch.Tensor,
+              labels64: torch.Tensor, shift: torch.Tensor, info: torch.Tensor, ws: Workspace,
+              wait_limit_us: Optional[int] = None) -> None:
+    """Enqueue the whole loop (see hkm_lloyd_fit_f32 in include/hkm.h).  ``info`` (two int32, device or pinned
+    host memory) holds the iteration count or a negative status once the stream has finished."""
+    _require_gpu(x, c0, c_out, labels64, shift)
+    _require_rows(x, c0, c_out)
+    _require_dense(c0, c_out)
+    if not (info.is_cuda or info.is_pinned()) or info.dtype != torch.int32 or info.numel() < 2:
+        raise RuntimeError("info must be two int32 on the GPU or in pinned host memory")
+    if labels64.dtype != torch.int64 or not labels64.is_contiguous() or labels64.numel() != x.shape[0]:
+        raise ValueError("labels64 must hold one contiguous int64 per row")
+    n, d = x.shape
+    k = c0.shape[0]
+    buf = ws.get(workspace_bytes(n, d, k, WS_FIT))
+    check(load().hkm_lloyd_fit_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c0), k, int(max_iter),
+                                   0 if tol is None else 1, 0.0 if tol is None else float(tol), _ptr(c_out),
+                                   _ptr(labels64), _ptr(shift), _ptr(info),
+                                   FIT_WAIT_LIMIT_US if wait_limit_us is None else int(wait_limit_us),
+                                   _ptr(buf), buf.numel(), _stream()))
 
 
 def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],

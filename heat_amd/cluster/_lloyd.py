@@ -62,7 +62,10 @@ class LloydLoop:
         # integers with a quantum of 2^-33 of the largest centroid coordinate: a mean is good to a few dozen ulps,
         # (2^-18)^2 of its magnitude per coordinate.
         self._fuzz = {"lloyd_small": d * 2.0 ** -36, "lloyd_mfma_resident": d * 2.0 ** -43}.get(kernel, 0.0)
-        self._cnorm: Optional[float] = None  # upper bound on the Frobenius norm of the current centroids
+        # Upper bound on the Frobenius norm of the current centroids, kept from the shifts the host reads (see
+        # _margin).  It starts at the norm of the init, taken here from a copy on the host, before anything is
+        # in flight: no reduction kernel of the tensor library is loaded or launched for sixteen numbers.
+        self._cnorm: Optional[float] = self._host_norm(c0) if self._fuzz else None
         self.rechecks = 0  # iterations whose means were recomputed by the two-pass update
         nbuf = 1 if self.lazy_labels else 2
         self.lab = [torch.empty((n,), dtype=torch.int32, device=dev) for _ in range(nbuf)]
@@ -155,11 +158,17 @@ class LloydLoop:
         for those it produced: the norm of the initial centroids (one look at the device, at the first call) plus
         the square roots of every shift since, so centroids that grow -- an init near the origin, data far from
         it -- raise the margin with them."""
-        if self._cnorm is None:
-            self._cnorm = float((self.c[(self.done - 1) % 3].double() ** 2).sum()) ** 0.5
+        if self._cnorm is None:  # after steps nobody waited for: one look at the device
+            self._cnorm = self._host_norm(self.c[(self.done - 1) % 3])
         bound = self._cnorm + (max(shift, 0.0) ** 0.5 if shift == shift else 0.0)
         e2 = self._fuzz * bound * bound
         return 2.0 * (max(tol, 0.0) * e2) ** 0.5 + e2
+
+    @staticmethod
+    def _host_norm(c: torch.Tensor) -> float:
+        """Frobenius norm of a (small) device matrix, computed on the host in float64; waits for the stream."""
+        v = c.detach().cpu().double().numpy()
+        return float((v * v).sum()) ** 0.5
 
     def _recompute(self, i: int) -> float:
         """Replace the centroids step i produced by the two-pass means of its labels; returns the shift."""

@@ -6,6 +6,9 @@ shift on the device; the host only reads the 4-byte shift to decide convergence.
 
 from __future__ import annotations
 
+import os
+import threading
+import warnings
 from typing import Optional, Union
 
 import torch
@@ -16,6 +19,21 @@ from ..core import types
 from ..core.dndarray import DNDarray
 from ..spatial import distance
 from ._kcluster import _KCluster
+
+
+# pinned status words of the one-launch fit (iterations run or a negative status, bits of the last shift): one pair
+# per device and host thread, allocated once -- a pinned allocation costs more than the fit it would serve
+_FIT_INFO = {}
+
+
+def _fit_info(device: torch.device):
+    key = (device.index, threading.get_ident())
+    pair = _FIT_INFO.get(key)
+    if pair is None:
+        t = torch.zeros((2,), dtype=torch.int32, pin_memory=True)
+        pair = (t, t.numpy())
+        _FIT_INFO[key] = pair
+    return pair
 
 
 class KMeans(_KCluster):
@@ -77,6 +95,12 @@ class KMeans(_KCluster):
         dev = xt.device
         n, d = xt.shape
         k = self.n_clusters
+        if self.max_iter >= 1 and xt.dtype == torch.float32 and os.environ.get("HKM_FIT") != "steps" \
+                and _native.lloyd_fit_supported(n, d, k):
+            # a few hundred thousand narrow rows: the whole loop is one launch (the rows stay in registers, the
+            # stop decision is taken on the device); on a negative status the loop below runs instead
+            if self._fit_one_launch(x, xt):
+                return self
         # the reference evaluates ``inertia <= tol`` on the host every iteration (kmeans.py:143); the
         # loop keeps the next step enqueued while the host looks at the shift of the current one
         loop = LloydLoop(xt, self._local_f32(self._cluster_centers, like=xt), self._workspace(dev))
@@ -92,3 +116,33 @@ class KMeans(_KCluster):
         self._inertia = DNDarray(shift.clone(), (), ftype, None, x.device, x.comm, True)
         self._labels = DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
         return self
+
+    def _fit_one_launch(self, x: DNDarray, xt: torch.Tensor) -> bool:
+        """The loop of heat/cluster/kmeans.py:131-146 as one launch of hkm_lloyd_fit_f32.  True if it delivered;
+        False if the kernel reported that it could not (a wait between its workgroups ran out, or the data hold a
+        non-finite value), in which case nothing has been set and the caller runs the loop step by step."""
+        dev = xt.device
+        n, d = xt.shape
+        k = self.n_clusters
+        c0 = self._local_f32(self._cluster_centers, like=xt)
+        _native._require_gpu(xt, c0)
+        c_out = torch.empty((k, d), dtype=torch.float32, device=dev)
+        lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
+        shift = torch.empty((), dtype=torch.float32, device=dev)
+        info, info_np = _fit_info(dev)
+        info_np[0] = 0
+        _native.lloyd_fit(xt, c0.contiguous(), self.max_iter, self.tol, c_out, lab64.view(-1), shift, info,
+                          self._workspace(dev))
+        torch.cuda.current_stream().synchronize()
+        n_iter = int(info_np[0])
+        if n_iter < 1:
+            if n_iter == -1:
+                warnings.warn("the one-launch k-means fit gave up waiting for its workgroups (is the GPU shared?); "
+                              "running the loop step by step instead")
+            return False
+        ftype = types.canonical_heat_type(xt.dtype)
+        self._n_iter = n_iter
+        self._cluster_centers = DNDarray(c_out, (k, d), ftype, None, x.device, x.comm, True)
+        self._inertia = DNDarray(shift, (), ftype, None, x.device, x.comm, True)
+        self._labels = DNDarray(lab64, (n, 1), types.int64, x.split, x.device, x.comm, True)
+        return True

@@ -278,7 +278,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 303; }
+int hkm_version(void) { return 304; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -313,6 +313,7 @@ size_t hkm_workspace_bytes(int64_t N, int32_t D, int32_t K, int32_t flags) {
     if (N < 0 || D < 1 || K < 1) return 0;
     if (N > (int64_t(1) << 40) || int64_t(K) * D > (int64_t(1) << 40)) return 0;  // refused by every entry point
     if (flags == HKM_WS_MEDIAN) return carve_median(nullptr, N, D, K).total;
+    if (flags == HKM_WS_FIT) return fit_eligible(N, D, K) ? fit_workspace_bytes(D, K) : 0;
     return carve(nullptr, N, D, K, flags).total;
 }
 
@@ -477,6 +478,34 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     }
     if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
     return rc;
+}
+
+int hkm_lloyd_fit_supported(int64_t N, int32_t D, int32_t K) {
+    if (N < 1 || D < 1 || K < 1) return 0;
+    return fit_eligible(N, D, K) ? 1 : 0;
+}
+
+int hkm_lloyd_fit_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C0, int32_t K, int32_t max_iter,
+                      int32_t use_tol, double tol, float* C_out, int64_t* labels, float* shift, int32_t* info,
+                      uint64_t wait_limit_us, void* ws, size_t ws_bytes, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C0", C0, K, D, D))) return rc;
+    if ((rc = check_matrix("C_out", C_out, K, D, D))) return rc;
+    if (max_iter < 1) return fail(HKM_EINVAL, "max_iter = %d must be >= 1", max_iter);
+    if (!labels || !shift || !info) return fail(HKM_EINVAL, "NULL pointer argument");
+    if (reinterpret_cast<uintptr_t>(labels) & 7u) return fail(HKM_EINVAL, "labels is not 8-byte aligned");
+    if (!fit_eligible(N, D, K))
+        return fail(HKM_EUNSUPPORTED,
+                    "N = %lld, D = %d, K = %d is outside what one launch holds (hkm_lloyd_fit_supported): run "
+                    "hkm_lloyd_step_f32 per iteration", (long long)N, D, K);
+    if ((rc = check_ws(ws, ws_bytes, fit_workspace_bytes(D, K)))) return rc;
+    // the device clock of the waits ticks at 100 MHz
+    const uint64_t ticks = wait_limit_us > (uint64_t(1) << 40) ? (uint64_t(1) << 47) : wait_limit_us * 100u;
+    return launch_lloyd_fit(X, N, D, ldx, C0, K, max_iter, use_tol, tol, C_out, labels, shift, info, ws, ticks,
+                            static_cast<hipStream_t>(hip_stream));
 }
 
 int hkm_point_blocks(int32_t D, int32_t* tuned) {

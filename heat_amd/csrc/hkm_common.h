@@ -182,6 +182,15 @@ int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx
 int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                         int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                         int fgrid, const float* C_old, float* shift, hipStream_t st);
+// the whole Lloyd loop in one launch (hkm_lloyd_fit.hip)
+static const int FIT_MAX_GRID = 64;
+static const int64_t FIT_MAX_ROWS = int64_t(1) << 18;
+bool fit_eligible(int64_t N, int32_t D, int32_t K);
+int fit_grid(int64_t N, int32_t D);
+size_t fit_workspace_bytes(int32_t D, int32_t K);
+int launch_lloyd_fit(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C0, int32_t K, int32_t max_iter,
+                     int32_t use_tol, double tol, float* C_out, int64_t* labels, float* shift_out, int32_t* info,
+                     void* ws, uint64_t wait_limit_ticks, hipStream_t st);
 bool small_eligible(int32_t D, int32_t K);
 int small_grid(int64_t N, int32_t D, int32_t K);
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,

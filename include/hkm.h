@@ -37,6 +37,8 @@
  *                         aid; both give the same labels and means equal to fp32 rounding.
  *   HKM_NARROW_MFMA_MIN_K=n   hkm_assign_f32 with 4 <= D <= 16: use the matrix-core kernels from n centroids
  *                         on (default 32) and the vector kernel below.  A measuring and testing aid.
+ *   HKM_FIT=steps         (read by the Python estimator, not by the library) KMeans.fit runs one hkm_lloyd_step_f32
+ *                         per iteration even where hkm_lloyd_fit_f32 applies.  A testing aid.
  *   HKM_SMALL_BLOCKED_MIN_K=n   the narrow kernels with D <= 3 scan the centroids four at a time from n
  *                         centroids on (default 12), one at a time below.  Same results bit for bit; a
  *                         measuring and testing aid.
@@ -64,6 +66,7 @@ extern "C" {
 #define HKM_WS_SSE 4   /* add when hkm_lloyd_step_f32 is called with sse != NULL (N floats of scratch) */
 #define HKM_WS_MEDIAN 8 /* on its own: scratch of hkm_update_median_f32 / hkm_closest_rows_l1_f32 */
 #define HKM_WS_F64 16   /* add for the *_f64 entry points (partials and scratch are doubles) */
+#define HKM_WS_FIT 32   /* on its own: scratch of hkm_lloyd_fit_f32 (0 where that entry point does not apply) */
 
 /* Library version: major*10000 + minor*100 + patch. */
 int hkm_version(void);
@@ -133,6 +136,33 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
 int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                        float* C_new, int32_t K, int32_t* labels, float* shift, float* sse, void* ws,
                        size_t ws_bytes, void* hip_stream);
+
+/*
+ * The WHOLE Lloyd loop in one launch, for data that stays in the registers of a few dozen workgroups:
+ *   for it in 1..max_iter: labels against C; C = per-cluster means; shift = sum((C_old - C)^2);
+ *                          stop after the first iteration with use_tol != 0 and shift <= tol
+ * with labels (N int64: the (N, 1) matrix the reference returns) those of the LAST assignment, C_out (K x D dense)
+ * the centroids after the last update and *shift (device scalar) the last shift.  X is read once per fit; the
+ * per-cluster sums are exact 64-bit integer sums (a coordinate enters with 44 bits below the largest value of its
+ * column), kept up to date from the rows whose label changed, so two iterations with the same
+ * labels give the same centroids bit for bit, as in the reference; the workgroups exchange their sums once per
+ * iteration and every one of them forms the centroids and takes the stop decision itself.
+ * info (two int32; device memory or pinned, device-accessible host memory) receives, when the launch has
+ * finished: info[0] = the iterations run (>= 1), or -1 if a wait between the workgroups ran out (no output is
+ * valid then: a workgroup that has waited wait_limit_us microseconds gives up and every other one follows, so
+ * the kernel always ends), or -2 if X holds a non-finite coordinate (no output valid either); info[1] = the bits
+ * of the last shift.  On a negative status run the loop with hkm_lloyd_step_f32.
+ * Shapes: hkm_lloyd_fit_supported(N, D, K) != 0, i.e. D <= 16, K (D + 1) <= 240 and N <= 65536 times the rows
+ * a thread holds (4 up to 4 features, 2 up to 8, else 1: 262144 / 131072 / 65536 rows); others return
+ * HKM_EUNSUPPORTED.
+ * ws: hkm_workspace_bytes(N, D, K, HKM_WS_FIT) bytes.  C0 and C_out may be the same matrix.
+ * Replaces heat/cluster/kmeans.py:131-146 (the loop of KMeans.fit) with :76-103 and
+ * heat/cluster/_kcluster.py:352-370 inside it.
+ */
+int hkm_lloyd_fit_supported(int64_t N, int32_t D, int32_t K);
+int hkm_lloyd_fit_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C0, int32_t K, int32_t max_iter,
+                      int32_t use_tol, double tol, float* C_out, int64_t* labels, float* shift, int32_t* info,
+                      uint64_t wait_limit_us, void* ws, size_t ws_bytes, void* hip_stream);
 
 /* *shift = sum((C_old - C_new)^2), fixed order.  Replaces heat/cluster/kmeans.py:141. */
 int hkm_shift_f32(const float* C_old, const float* C_new, int32_t K, int32_t D, float* shift,

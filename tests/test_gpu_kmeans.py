@@ -307,13 +307,14 @@ def test_config4_full_size_properties(cuda, parity_report):
     _full_size_properties(synthetic.config4(), cuda, parity_report, iters=5)
 
 
-def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda):
+def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda, monkeypatch):
     """KMeans.fit keeps the next step enqueued while the host reads the shift of the current one; when
     the tolerance is met the extra step must leave no trace: same iteration count, centroids, labels and
     inertia as a loop that only launches a step after looking at the previous shift."""
     from heat_amd import _native
     from heat_amd.cluster._lloyd import LloydLoop
 
+    monkeypatch.setenv("HKM_FIT", "steps")  # this is about the step loop; data this small would take the one-launch fit
     w = synthetic.config1(0.5)
     x = w.x.to(cuda)
     probe = LloydLoop(x, w.init.to(cuda), _native.Workspace(cuda))
