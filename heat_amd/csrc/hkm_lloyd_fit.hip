@@ -10,24 +10,31 @@
 //     every workgroup adds all published rows itself, forms the new centroids and the shift, and evaluates
 //     `shift <= tol` -- all workgroups run the same instructions on the same numbers, so they agree on when to
 //     stop without another exchange;
-//   * the per-cluster sums are exact 64-bit integer sums: a coordinate enters as rint(x * 2^(44 - E)) with 2^E
+//   * the per-cluster sums are exact 64-bit integer sums: a coordinate enters as rint(x * 2^(43 - E)) with 2^E
 //     above the largest |value| of its COLUMN over the whole data set (found once, before the first iteration;
-//     per column, so that features of very different magnitudes each keep their 44 bits).  Integer
+//     per column, so that features of very different magnitudes each keep their 43 bits).  Integer
 //     additions are exact, so (i) LDS atomics and the addition of the workgroups' rows may happen in any order,
 //     (ii) the sums depend on the labels alone -- two iterations with the same labels give the same centroids
 //     bit for bit, which is where the reference stops with a shift of exactly 0 -- and (iii) they can be
 //     kept UP TO DATE instead of being formed again: a thread touches the table only for rows whose label
 //     changed (subtract from the old cluster, add to the new one), which after the first iterations is a small
 //     part of the rows.  A mean is the integer sum scaled back and divided by the count (rounded through fp32
-//     like the reference, heat/core/rounding.py:156-164).  A value of at least 2^-21 of its column's largest enters
-//     exactly; a smaller one with an error of at most 2^-45 of that largest value, far below the fp32 rounding
+//     like the reference, heat/core/rounding.py:156-164).  A value of at least 2^-20 of its column's largest enters
+//     exactly; a smaller one with an error of at most 2^-44 of that largest value, far below the fp32 rounding
 //     of the mean itself.
 //
 // The hand-over.  The chip's eight L2 caches are not coherent with each other for ordinary accesses, so what
-// workgroups hand to each other (rows, the arrival counter, the abort flag) is written and read with
-// device-scope atomic accesses, which go past the caches; a workgroup waits for its stores to be acknowledged
-// before it counts itself in.  The rows live in two buffers that alternate by iteration: a workgroup can only
-// be one hand-over ahead of the slowest.
+// workgroups hand to each other is written and read with device-scope atomic accesses, which go past the caches.
+// A round trip between workgroups on different dies costs about a microsecond and a half, so an iteration makes
+// exactly one: every 64-bit word a workgroup publishes carries, in its two top bits, a stamp of the iteration it
+// belongs to (the sums need 62 bits: N * 2^43 < 2^61), and a reader simply loads the words it needs until each
+// shows the stamp it expects -- no arrival counter, no flag, no wait for the stores to be acknowledged; a word is
+// written by one 8-byte store, so a word with the right stamp is the right word.  The rows live in two buffers
+// that alternate by iteration, and a buffer's stamps go 1, 3, 1, ... resp. 2, 0, 2, ...: what a buffer held two
+// iterations ago never passes for the current row.  A workgroup cannot publish row it + 2 before every other
+// workgroup has read row it (it needs their rows it + 1 first, which they publish after that read).  Before the
+// first iteration every workgroup clears its own two rows (stamp 0, which iterations 0 and 1 do not expect) and
+// all meet once at an arrival counter, where the column maxima are exchanged too.
 //
 // Every wait is bounded.  A workgroup that has waited longer than the limit the host passed (device clock ticks
 // of 10 ns) raises the abort flag and leaves; every other workgroup sees the flag in its own wait and leaves
@@ -39,7 +46,8 @@
 namespace hkm {
 
 static constexpr int FIT_T = 1024;
-static constexpr int FIT_QB = 44;  // bits kept below 2^E: N * 2^44 stays below 2^62 for N <= FIT_MAX_ROWS
+static constexpr int FIT_QB = 43;  // bits kept below 2^E: N * 2^43 stays below 2^61 for N <= FIT_MAX_ROWS
+static constexpr unsigned long long FIT_VALUE_MASK = (1ull << 62) - 1;  // a published word: 62 bits of sum, 2 of stamp
 static constexpr unsigned long long FIT_MAGIC = 0x4338000000000000ull;  // bits of 1.5 * 2^52
 
 // rows per thread: as few as give a grid of at most FIT_MAX_GRID workgroups
@@ -130,7 +138,7 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
     unsigned long long* itab = reinterpret_cast<unsigned long long*>(sCraw + ((K * D + 3) & ~3));  // [slots][R]
     unsigned long long* tot = itab + slots * R;                                  // [slots]
     unsigned long long* strided = tot + ((slots + 1) & ~1);                      // [T]
-    double* red = reinterpret_cast<double*>(strided + T);                        // [256]
+    double* red = reinterpret_cast<double*>(strided + T);                        // [2][256]
     __shared__ int s_ok;
     __shared__ int s_max[D];
     __shared__ int s_exp[D];  // E of every column: 2^E is above its largest |value|
@@ -171,8 +179,10 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
     }
     __syncthreads();
     if (tid < D) __hip_atomic_fetch_max(&a.bar[2 + tid], unsigned(s_max[tid]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    unsigned arrivals = unsigned(G);
-    if (!grid_handover(a.bar, arrivals, a.wait_limit, &s_ok)) {
+    // whatever an earlier call left in this workgroup's two rows must not pass for a row of this one
+    for (int i = tid; i < 2 * slots; i += T)
+        peer_store(a.rows + (size_t(i / slots) * G + blockIdx.x) * slots + (i % slots), 0ull);
+    if (!grid_handover(a.bar, unsigned(G), a.wait_limit, &s_ok)) {
         if (tid == 0) a.info[0] = -1;
         return;
     }
@@ -192,14 +202,9 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
 
     for (int i = tid; i < K * D; i += T) sCraw[i] = a.C0[i];
     __syncthreads();
-
-    const int SP = slots;            // threads per group of rows in the gather
-    const int J = T / SP;            // groups: thread (j, s) adds rows j, j + J, ... of slot s
-    int n_iter = 0;
-    float shift = 0.f;
-    for (int it = 0; it < a.max_iter; ++it) {
-        // ---- centroid rows for the scan: -2c (exact) and |c|^2, as the one-sweep kernel stages them ----
-        for (int r = tid; r < K; r += T) {
+    // centroid rows for the scan: -2c (exact) and |c|^2, as the one-sweep kernel stages them
+    auto stage_scan_rows = [&]() {
+        for (int r = (tid >= 256 ? tid - 256 : tid); r < K; r += T) {
             float s = 0.f;
 #pragma unroll
             for (int d = 0; d < D; ++d) {
@@ -209,8 +214,30 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
             }
             sC[r * SC + D] = s;
         }
-        __syncthreads();
+    };
+    stage_scan_rows();
+    __syncthreads();
+    __shared__ int s_fail;
+    if (tid == 0) s_fail = 0;
 
+    const int SP = slots;            // threads per group of rows in the gather
+    const int J = T / SP;            // groups: thread (j, s) adds rows j, j + J, ... of slot s
+    int n_iter = 0;
+    float shift = 0.f;
+#ifdef HKM_FIT_TRACE
+    unsigned long long* trace = a.rows + size_t(2) * FIT_MAX_GRID * slots;
+    unsigned long long tprev = clock64();
+#define FIT_TP(i)                                                        \
+    if (tid == 0 && blockIdx.x == 0) {                                   \
+        const unsigned long long tn = clock64();                         \
+        if (it >= 4) trace[i] += tn - tprev;                             \
+        tprev = tn;                                                      \
+    }
+#else
+#define FIT_TP(i)
+#endif
+    for (int it = 0; it < a.max_iter; ++it) {
+        FIT_TP(0)
         // ---- assignment (heat/spatial/distance.py:59-64 + the argmin of heat/cluster/_kcluster.py:352-370) ----
         float m[PPT];
         int mi[PPT];
@@ -263,6 +290,7 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
             }
         }
 
+        FIT_TP(1)
         // ---- the workgroup's sums follow the labels that changed ----
 #pragma unroll
         for (int p = 0; p < PPT; ++p) {
@@ -285,49 +313,78 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
         }
         __syncthreads();
 
-        // ---- publish the workgroup's row, hand over, add everybody's rows ----
+        FIT_TP(2)
+        // ---- publish the workgroup's row; add everybody's rows as they show this iteration's stamp ----
+        const unsigned long long stamp = (unsigned long long)((it + 1) & 3) << 62;
         unsigned long long* mine = a.rows + (size_t(it & 1) * G + blockIdx.x) * slots;
         for (int s = tid; s < slots; s += T) {
             unsigned long long v = 0ull;
 #pragma unroll
             for (int r = 0; r < R; ++r) v += itab[s * R + r];
-            peer_store(mine + s, v);
+            peer_store(mine + s, (v & FIT_VALUE_MASK) | stamp);
         }
-        arrivals += unsigned(G);
-        if (!grid_handover(a.bar, arrivals, a.wait_limit, &s_ok)) {
-            if (tid == 0) a.info[0] = -1;
-            return;
-        }
+        FIT_TP(3)
         {
             const unsigned long long* all = a.rows + size_t(it & 1) * G * slots;
             const int s = tid % SP, j = tid / SP;
             unsigned long long v = 0ull;
+            bool failed = false;
             if (j < J) {
-                for (int g = j; g < G; g += 8 * J) {
-                    unsigned long long t[8];
+                for (int g = j; g < G && !failed; g += 8 * J) {
+                    unsigned pending = 0u;
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) t[u] = g + u * J < G ? peer_load(all + size_t(g + u * J) * slots + s) : 0ull;
+                    for (int u = 0; u < 8; ++u)
+                        if (g + u * J < G) pending |= 1u << u;
+                    unsigned long long t0 = 0ull;
+                    unsigned polls = 0u;
+                    while (pending) {
+                        unsigned long long t[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) v += t[u];
+                        for (int u = 0; u < 8; ++u)
+                            if (pending & (1u << u)) t[u] = peer_load(all + size_t(g + u * J) * slots + s);
+#pragma unroll
+                        for (int u = 0; u < 8; ++u)
+                            if ((pending & (1u << u)) && (t[u] & ~FIT_VALUE_MASK) == stamp) {
+                                v += t[u];
+                                pending &= ~(1u << u);
+                            }
+                        if (pending && (++polls & 15u) == 0u) {
+                            // a word is late: somebody gave up, or the wait has lasted too long
+                            const unsigned long long now = wall_clock64();
+                            if (t0 == 0ull) t0 = now;
+                            if (peer_load32(&a.bar[1]) != 0u || now - t0 > a.wait_limit) {
+                                failed = true;
+                                break;
+                            }
+                        }
+                    }
                 }
             }
             strided[tid] = v;
+            if (failed) s_fail = 1;
         }
         __syncthreads();
-        if (tid < slots) {
-            unsigned long long v = 0ull;
-            for (int q = 0; q < J; ++q) v += strided[q * SP + tid];
-            tot[tid] = v;
+        if (s_fail) {
+            if (tid == 0) {
+                __hip_atomic_store(&a.bar[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                a.info[0] = -1;
+            }
+            return;
         }
-        __syncthreads();
-
+        FIT_TP(4)
         // ---- the new centroids and the shift (heat/cluster/kmeans.py:76-103,141) ----
         double sq = 0.0;
         if (tid < K * D) {
             const int k = tid / D, d = tid - k * D;
-            const long long n = (long long)tot[k * (D + 1) + D];
-            // the table holds the sum of bit patterns: n times the pattern of 1.5 * 2^52 plus the sum of the integers
-            const long long isum = (long long)(tot[k * (D + 1) + d] - (unsigned long long)n * FIT_MAGIC);
+            unsigned long long un = 0ull, us = 0ull;  // the J strided sums of the count and of the coordinate
+            for (int q = 0; q < J; ++q) {
+                un += strided[q * SP + k * (D + 1) + D];
+                us += strided[q * SP + k * (D + 1) + d];
+            }
+            const long long n = (long long)(un & FIT_VALUE_MASK);
+            // the table holds the sum of bit patterns, modulo 2^62: n times the pattern of 1.5 * 2^52 plus the sum
+            // of the integers, which lies within +-2^61 (sign-extended from bit 61)
+            const long long isum = (long long)((us - (unsigned long long)n * FIT_MAGIC) << 2) >> 2;
             const double cnt = double(float(n < 1 ? 1 : n));
             const double quantum = __hiloint2double((1023 - FIT_QB + s_exp[d]) << 20, 0);
             const float c = float(double(isum) * quantum / cnt);
@@ -335,21 +392,23 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
             sq = double(df * df);
             sCraw[tid] = c;  // only this thread reads or writes entry tid between the barriers around
         }
-        // fixed tree over 256 slots of which the first K * D <= 240 are not zero
-        if (tid < 256) red[tid] = sq;
+        // The squared differences of the K * D <= 240 coordinates, added in a fixed order by EVERY wave for itself
+        // (four per lane, then a butterfly over the lanes): all threads of all workgroups get the same bits
+        // without another exchange.  Two buffers by iteration parity: a wave may still be reading one when the
+        // fastest writes the next iteration's.
+        double* rd = red + (it & 1) * 256;
+        if (tid < 256) rd[tid] = sq;
         __syncthreads();
-        if (tid < 128) red[tid] += red[tid + 128];
-        __syncthreads();
-        if (tid < 64) {
-            double r = red[tid] + red[tid + 64];
+        if (tid >= 256) stage_scan_rows();  // the next iteration's scan rows (threads 256 .. 256 + K - 1)
+        {
+            double r = (rd[lane] + rd[lane + 64]) + (rd[lane + 128] + rd[lane + 192]);
 #pragma unroll
-            for (int w = 32; w > 0; w >>= 1) r += __shfl_down(r, w);
-            if (tid == 0) red[0] = r;
+            for (int w = 32; w > 0; w >>= 1) r += __shfl_xor(r, w);
+            shift = float(r);
         }
-        __syncthreads();
-        shift = float(red[0]);
         n_iter = it + 1;
-        __syncthreads();  // red[0] has been read by everybody before the next iteration writes it
+        __syncthreads();  // the scan rows are staged; strided and the table are free again
+        FIT_TP(5)
         if (a.has_tol && double(shift) <= a.tol) break;
     }
 
@@ -371,7 +430,7 @@ __global__ __launch_bounds__(FIT_T) void lloyd_fit_kernel(const FitArgs a) {
 static size_t fit_lds_bytes(int32_t D, int32_t K) {
     const int sc = (D + 1 + 3) / 4 * 4, slots = K * (D + 1);
     return size_t(K) * sc * 4 + size_t((K * D + 3) & ~3) * 4 + size_t(slots) * 8 * 8 + size_t((slots + 1) & ~1) * 8 +
-           size_t(FIT_T) * 8 + 256 * 8;
+           size_t(FIT_T) * 8 + 2 * 256 * 8;
 }
 
 size_t fit_workspace_bytes(int32_t D, int32_t K) {
