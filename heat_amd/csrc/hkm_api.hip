@@ -90,7 +90,7 @@ static int narrow_mfma_min_k() {
 
 AssignKind assign_kind(int32_t D, int32_t K) {
     if (D <= 16 && (D < 4 || K < narrow_mfma_min_k())) return ASSIGN_VALU;
-    if (D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024) return ASSIGN_MFMA_RESIDENT;
+    if (D <= RESIDENT_MAX_D && resident_lds_bytes(D, K) <= 64 * 1024) return ASSIGN_MFMA_RESIDENT;
     if (D <= 64) return ASSIGN_MFMA_TILED;
     return ASSIGN_MFMA_STREAM;
 }
@@ -102,7 +102,7 @@ AssignKind assign_kind(int32_t D, int32_t K) {
 // 10M x 2, K = 90: 0.28 against 0.55 ms; 10M x 3, K = 256: 0.52 against 0.91 ms).  One feature stays on the
 // two passes (0.57 ms at K = 130; with 130 centroids on a line the two arithmetics part on a thousand ties).
 bool fused_eligible(int32_t D, int32_t K) {
-    return D >= 2 && D <= 64 && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
+    return D >= 2 && D <= RESIDENT_MAX_D && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
 }
 
 static size_t cn_pad(int32_t K) { return (size_t(K) + 127) / 128 * 128; }
@@ -510,7 +510,7 @@ int hkm_lloyd_fit_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const f
 
 int hkm_point_blocks(int32_t D, int32_t* tuned) {
     if (tuned) *tuned = (env_point_blocks() == 0 && tuned_point_blocks() != 0) ? 1 : 0;
-    if (D < 1 || D > 64) return 0;
+    if (D < 1 || D > RESIDENT_MAX_D) return 0;
     return resident_point_blocks(resident_dp(D));
 }
 

@@ -58,6 +58,22 @@ __device__ __forceinline__ void resident_block(const float* arow, const floatx16
     }
 }
 
+// The same with the block's A fragments already in registers (the centroids never change during a launch, so
+// a wave with registers to spare keeps its first blocks' fragments for good instead of reading them from LDS
+// for every tile).
+template <int DP, int PB>
+__device__ __forceinline__ void resident_block_regs(const floatx4 (&a)[DP / 8], const floatx16& c0,
+                                                    const floatx4 (&b)[PB][DP / 8], floatx16 (&acc)[PB]) {
+    constexpr int NJ = DP / 8;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int pb = 0; pb < PB; ++pb)
+                acc[pb] = (j == 0 && t == 0) ? MFMA32(a[j][t], b[pb][j][t], c0) : MFMA32(a[j][t], b[pb][j][t], acc[pb]);
+}
+
 // Two centroid blocks at once against one point block: two independent accumulator chains share the
 // point registers, so a wave always has a matrix instruction that does not wait for the one before it,
 // and the first block's minimum tree finds its results complete while the second chain ends.
@@ -82,11 +98,13 @@ __device__ __forceinline__ void resident_block_pair(const float* arow0, const fl
 // whose lazy minimum came out negative).  Two blocks per trip: the squared norms of both are requested
 // at the top of the trip into the registers that then serve, in place, as their accumulators (norms
 // carried over the loop's back edge instead were copied into place, eight moves per block).
-template <int DP, int PB, bool CLAMP>
+// RB > 0 (even; two point blocks only): the A fragments of blocks 0 .. RB - 1 come from `ares` instead of LDS.
+template <int DP, int PB, bool CLAMP, int RB = 0>
 __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn, int ncb, int p, int h,
                                               const floatx4 (&b)[PB][DP / 8],
                                               const float (&xn)[PB], float (&m)[PB],
-                                              int (&mi)[PB]) {
+                                              int (&mi)[PB],
+                                              const floatx4 (*ares)[DP / 8] = nullptr) {
     constexpr int LDC = DP + 4;
     int blk[PB];
     floatx16 keep[PB];
@@ -128,7 +146,27 @@ __device__ __forceinline__ void resident_scan(const float* sC, const float* sCn,
         }
         if (cb < ncb) one_block(cb, load_cn16(sCn + cb * 32 + 4 * h));
     } else {
-        for (int cb = 0; cb < ncb; cb += 2) {
+        int cb = 0;
+        if constexpr (RB > 0) {
+#pragma unroll
+            for (int r = 0; r < RB; r += 2) {
+                if (r < ncb) {
+                    const floatx16 ca = load_cn16(sCn + r * 32 + 4 * h);
+                    const floatx16 cb1 = load_cn16(sCn + (r + 1 < ncb ? r + 1 : r) * 32 + 4 * h);
+                    floatx16 acc[PB];
+                    resident_block_regs<DP, PB>(ares[r], ca, b, acc);
+#pragma unroll
+                    for (int pb = 0; pb < PB; ++pb) block_min_keep(acc[pb], r, m[pb], blk[pb], keep[pb]);
+                    if (r + 1 < ncb) {
+                        resident_block_regs<DP, PB>(ares[r + 1], cb1, b, acc);
+#pragma unroll
+                        for (int pb = 0; pb < PB; ++pb) block_min_keep(acc[pb], r + 1, m[pb], blk[pb], keep[pb]);
+                    }
+                }
+            }
+            cb = RB;
+        }
+        for (; cb < ncb; cb += 2) {
             const floatx16 ca = load_cn16(sCn + cb * 32 + 4 * h);
             const floatx16 cb1 = load_cn16(sCn + (cb + 1 < ncb ? cb + 1 : cb) * 32 + 4 * h);
             one_block(cb, ca);
@@ -269,6 +307,9 @@ __global__ __launch_bounds__(256) void assign_mfma_resident_kernel(
 // the two-pass update, whose kernels start by looking at the flags.
 // ------------------------------------------------------------------------------------------------
 static constexpr int FUSED_QBITS = 28;
+#ifndef HKM_RESIDENT_A_BLOCKS
+#define HKM_RESIDENT_A_BLOCKS 4
+#endif
 // Point blocks per wave of the resident kernels.  Up to 32 padded features there is a choice: TWO point
 // blocks against every centroid row a wave reads from LDS (eight waves per CU in the one-sweep kernel), or ONE
 // with sixteen waves.  Two halve the LDS reads per matrix instruction, and that decides on chips that lower
@@ -279,7 +320,9 @@ static constexpr int FUSED_QBITS = 28;
 // of a step is bit for bit the same whichever runs.  Which one: HKM_POINT_BLOCKS (1 or 2) if set; else what
 // the trial below found on this device; else two.  Wider rows leave registers for one point block only
 // (twelve waves).
-__host__ __device__ constexpr int fused_threads(int pb, int dp) { return pb == 2 ? 512 : (dp <= 32 ? 1024 : 768); }
+__host__ __device__ constexpr int fused_threads(int pb, int dp) {
+    return pb == 2 ? 512 : (dp <= 32 ? 1024 : dp <= 64 ? 768 : 512);  // beyond 64 features a wave needs 256 registers
+}
 
 int env_point_blocks() {
     const char* e = getenv("HKM_POINT_BLOCKS");
@@ -534,6 +577,17 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
     const unsigned lane_off = unsigned((int64_t(p) * ldx + h * (DP / 2)) * 4);
     double* sA_lane = sA + (p & (nrep - 1)) * rstride;
     int* sN_lane = sN + (p & (nrep - 1)) * K;
+    // with two point blocks per wave (eight waves, 256 registers each) the first blocks' A fragments stay in
+    // registers: a quarter of the centroid reads from LDS at K = 256
+    constexpr int RB = PB == 2 ? HKM_RESIDENT_A_BLOCKS : 0;
+    floatx4 ares[RB > 0 ? RB : 1][NJ];
+    if constexpr (RB > 0) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                ares[r][j] = ld4(sC + ((r < ncb ? r : 0) * 32 + p) * LDC + h * (DP / 2) + 4 * j);
+    }
     int emin = 0x7fffffff, emax = -0x7fffffff;
     int nonfinite = 0;  // a row whose |x|^2 is inf or NaN: its bound 2^E says nothing about its coordinates
 
@@ -555,7 +609,7 @@ __global__ __launch_bounds__(fused_threads(PB, DP)) void lloyd_mfma_resident_ker
         if (tile + gridDim.x < ntiles)
             fetch_rows<DP, PB, VEC>(X, N, D, ldx, row0 + int64_t(gridDim.x) * tile_rows, p, h, fast, lane_off, bnext);
 
-        resident_scan<DP, PB, false>(sC, sCn, ncb, p, h, b, xnr, m, mi);
+        resident_scan<DP, PB, false, RB>(sC, sCn, ncb, p, h, b, xnr, m, mi, ares);
         bool neg = false;
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) neg |= m[pb] < 0.f;
@@ -990,7 +1044,9 @@ static size_t fused_lds_bytes_with(int32_t D, int32_t K, int nrep) {
 // that meet at one address down to a few and still fit in 48 KB with everything else.
 int fused_replicas(int32_t D, int32_t K) {
     int r = K <= 16 ? 16 : K <= 32 ? 8 : K <= 64 ? 4 : 1;
-    while (r > 1 && fused_lds_bytes_with(D, K, r) > 48 * 1024) r >>= 1;
+    // (one workgroup per CU runs this kernel: beyond 64 features, where a copy is large, it may take most of the LDS)
+    const size_t cap = resident_dp(D) > 64 ? 128 * 1024 : 48 * 1024;
+    while (r > 1 && fused_lds_bytes_with(D, K, r) > cap) r >>= 1;
     return r;
 }
 
@@ -1050,7 +1106,7 @@ int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx
                  : launch_fused_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st);  \
     }
     HKM_CASE(8, 2) HKM_CASE(8, 1) HKM_CASE(16, 2) HKM_CASE(16, 1) HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2)
-    HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
+    HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1) HKM_CASE(96, 1) HKM_CASE(128, 1)
 #undef HKM_CASE
     trial_end(tk, st);
     if (!found) return fail(HKM_EUNSUPPORTED, "lloyd_mfma_resident: D=%d", D);
@@ -1068,7 +1124,7 @@ int launch_assign_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ld
         return vec ? launch_resident_t<d, b, true>(X, N, D, ldx, C, K, ldc, labels, min_d2, st) \
                    : launch_resident_t<d, b, false>(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
     HKM_CASE(8, 2) HKM_CASE(8, 1) HKM_CASE(16, 2) HKM_CASE(16, 1) HKM_CASE(24, 2) HKM_CASE(24, 1) HKM_CASE(32, 2)
-    HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1)
+    HKM_CASE(32, 1) HKM_CASE(48, 1) HKM_CASE(64, 1) HKM_CASE(96, 1) HKM_CASE(128, 1)
 #undef HKM_CASE
     return fail(HKM_EUNSUPPORTED, "assign_mfma_resident: D=%d", D);
 }

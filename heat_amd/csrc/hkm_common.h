@@ -73,9 +73,10 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 enum AssignKind { ASSIGN_VALU = 0, ASSIGN_MFMA_RESIDENT = 1, ASSIGN_MFMA_STREAM = 2, ASSIGN_MFMA_TILED = 3 };
 AssignKind assign_kind(int32_t D, int32_t K);
 
-// padded feature count used by the resident MFMA kernels (8, 16, 24, 32, 48 or 64)
+// padded feature count used by the resident MFMA kernels (8, 16, 24, 32, 48, 64, 96 or 128)
+static const int RESIDENT_MAX_D = 128;
 static inline int resident_dp(int32_t D) {
-    return D <= 8 ? 8 : D <= 16 ? 16 : D <= 24 ? 24 : D <= 32 ? 32 : D <= 48 ? 48 : 64;
+    return D <= 8 ? 8 : D <= 16 ? 16 : D <= 24 ? 24 : D <= 32 ? 32 : D <= 48 ? 48 : D <= 64 ? 64 : D <= 96 ? 96 : 128;
 }
 static inline size_t resident_lds_bytes(int32_t D, int32_t K) {
     size_t kp = (size_t(K) + 31) / 32 * 32;

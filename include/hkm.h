@@ -24,7 +24,7 @@
  *
  * Environment (looked up on every call, nothing is cached)
  *   HKM_PRODUCTS=bf16x3   hkm_assign_f32 / hkm_lloyd_step_f32, every shape with D > 16 except those with
- *                         32 < D <= 64 whose centroids fit in LDS: the cross term x.c is evaluated on
+ *                         32 < D <= 128 whose centroids fit in LDS: the cross term x.c is evaluated on
  *                         the bf16 matrix cores from operands split three ways (six partial products,
  *                         fp32 accumulation) instead of fp32 matrix instructions.  Same error bound per
  *                         product as fp32, 1.3x to 1.7x the throughput.  Off by default.
@@ -95,11 +95,12 @@ int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const floa
  * hkm_assign_f32 for callers that cannot allocate device memory or carry a workspace: code under HIP
  * graph capture, tight serving loops (predict), harnesses that forbid hipMalloc.  No counterpart in the
  * reference.  Same arguments, results and kernels as hkm_assign_f32, but the scratch (reduction slots,
- * squared centroid norms, the merge keys of the D > 64 kernel) is a device array of
+ * squared centroid norms, the merge keys of the streaming kernel) is a device array of
  * HKM_STATIC_SCRATCH_BYTES built into the library, which every GPU the library runs on holds from the
  * first call on it until the process ends.  The call allocates and frees nothing.  Shapes whose
  * hkm_workspace_bytes(N, D, K, HKM_WS_ASSIGN) exceeds HKM_STATIC_SCRATCH_BYTES return HKM_EUNSUPPORTED
- * (D <= 64: every K up to about four million; D > 64: up to about two million rows, 8 bytes each).
+ * (centroids resident in LDS or D <= 64: every K up to about four million; the streaming kernel -- D > 128, or
+ * D > 64 with more centroids than LDS holds -- up to about two million rows, 8 bytes each).
  * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
  * calls on one stream are ordered and each refills what it reads.
  * The array's device address is looked up once per device (hipGetSymbolAddress), by whichever comes first on

@@ -130,7 +130,7 @@ int main() {
 
     // ---- the launch-geometry choice of the resident kernels: queries and refusals only
     int32_t tuned = -1;
-    if (hkm_point_blocks(0, &tuned) != 0 || hkm_point_blocks(100, nullptr) != 0 || hkm_point_blocks(48, &tuned) != 1 ||
+    if (hkm_point_blocks(0, &tuned) != 0 || hkm_point_blocks(130, nullptr) != 0 || hkm_point_blocks(48, &tuned) != 1 ||
         tuned != 0) {
         std::printf("FAIL hkm_point_blocks\n");
         ++failures;

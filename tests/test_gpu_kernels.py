@@ -21,6 +21,8 @@ ASSIGN_SHAPES = [
     (1, 3, 8), (1000, 3, 8), (5000, 8, 16), (777, 16, 40), (300, 1, 5), (2000, 5, 700),
     (4096, 32, 256), (1000, 20, 33), (999, 17, 1), (3000, 64, 100), (1300, 50, 37), (257, 24, 64),
     (2048, 64, 1024), (1500, 100, 70), (900, 512, 130), (700, 33, 500), (513, 130, 1030),
+    # 65 to 128 features with the centroids resident in LDS (beyond, or with more centroids: the streaming kernel)
+    (3000, 128, 8), (1111, 65, 3), (2000, 96, 32), (1500, 97, 40), (900, 128, 96), (900, 128, 97), (800, 127, 1),
     (3000, 16, 1100), (2500, 8, 1500), (1800, 6, 2000), (4000, 4, 33), (3000, 13, 32),
     # 9 to 16 features with few centroids: the narrow kernel
     (3001, 16, 8), (2000, 9, 24), (4003, 12, 5), (1000, 15, 15), (2500, 10, 1), (3000, 14, 16), (2222, 11, 20), (1999, 13, 3),
@@ -291,11 +293,13 @@ def _step_and_two_pass_impl(xs, cs, dev):
     return c_step, lab_step, shift, c2, lab2, cnt2
 
 
-# shapes of the one-sweep MFMA step (16 < D <= 64, centroids + fp64 accumulators fit in LDS):
+# shapes of the one-sweep MFMA step (up to 128 features, centroids + fp64 accumulators fit in LDS):
 # ragged N, K not a multiple of 32, D not a multiple of 4 (scalar loads), every padded width
 @pytest.mark.parametrize("n,d,k", [(100003, 32, 256), (50000, 20, 37), (1537, 24, 3), (40000, 30, 100),
                                    (70001, 40, 129), (30000, 64, 128), (768, 17, 5), (100, 48, 7),
-                                   (50000, 16, 64), (40000, 8, 40), (30001, 12, 100), (20000, 5, 60), (9000, 4, 256)])
+                                   (50000, 16, 64), (40000, 8, 40), (30001, 12, 100), (20000, 5, 60), (9000, 4, 256),
+                                   (40000, 128, 8), (30001, 100, 16), (20000, 96, 32), (10000, 65, 3), (25000, 128, 90),
+                                   (5000, 77, 1)])
 def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
     assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
     print(f"one-sweep n={n} d={d} k={k}", flush=True)
@@ -384,9 +388,9 @@ def test_geometry_trial_runs_on_the_callers_own_steps(cuda, monkeypatch):
     after = LloydLoop(xs, cs, _native.Workspace(cuda))
     assert after.run(12, None) == 12
     assert torch.equal(after.centers, want_c) and torch.equal(after.labels, want_lab)
-    # shapes without the choice: wider rows have one geometry, rows beyond 64 features no resident kernel
-    assert benchhooks.point_blocks(48)[0] == 1
-    assert benchhooks.point_blocks(100)[0] == 0
+    # shapes without the choice: wider rows have one geometry, rows beyond 128 features no resident kernel
+    assert benchhooks.point_blocks(48)[0] == 1 and benchhooks.point_blocks(100)[0] == 1
+    assert benchhooks.point_blocks(130)[0] == 0
 
 
 @pytest.mark.parametrize("n,d,k", [(30000, 16, 15), (20000, 9, 25), (25000, 12, 20), (10000, 10, 22), (40000, 4, 50), (30000, 7, 31),

@@ -215,6 +215,21 @@ def test_few_clusters_of_nine_to_sixteen_features_against_oracle(cuda, n, d, k, 
     _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
 
 
+@pytest.mark.parametrize("n,d,k", [(60000, 32, 8), (40000, 64, 8), (30000, 128, 8), (30000, 100, 5), (20000, 96, 32)])
+def test_few_clusters_of_wide_rows_against_oracle(cuda, n, d, k, parity_report):
+    """Whole fits with few clusters and 32 to 128 features -- an everyday shape -- on the one-sweep matrix-core
+    step (one read of X per iteration up to 128 features): step by step and at the end against the oracle."""
+    from heat_amd import _native
+
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
+    w = synthetic.shape(n, d, k, seed=1300 + d)
+    print(f"{w.name}", flush=True)
+    flips, ref = _stepwise_parity(w, cuda, 12, literal=False, report=parity_report)
+    print(f"{w.name}: {flips} excused tie flips over {ref['n_iter']} iterations", flush=True)
+    km, _ = _fit(w.x, w.init, w.k, 12, 0.0, cuda)
+    _check_fit(km, w.x, ref["cluster_centers"], ref["labels"], ref["inertia"], ref["n_iter"], tie_flips=flips)
+
+
 @pytest.mark.parametrize("scale", [1.0 / 16, 1.0])
 def test_config2_cdist_argmin(cuda, scale, parity_report):
     from heat_amd import _native

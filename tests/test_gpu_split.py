@@ -54,7 +54,7 @@ def test_split_assign_matches_oracle(cuda, split_products, n, d, k):
 
 # wide rows (D > 64): the 2-D streaming kernel, whose staging threads split the panels; 16 < D <= 64 with
 # more centroids than LDS holds: the tiled kernel, whose staging threads split the centroid tiles
-@pytest.mark.parametrize("n,d,k", [(1500, 100, 70), (900, 512, 130), (513, 130, 1030), (300, 65, 3),
+@pytest.mark.parametrize("n,d,k", [(1500, 100, 170), (900, 512, 130), (513, 130, 1030), (300, 130, 3),
                                    (2048, 64, 1024), (3000, 64, 300), (700, 33, 500), (1300, 50, 437), (5000, 20, 900)])
 def test_split_streaming_and_tiled_assign_match_oracle(cuda, split_products, n, d, k):
     assert _native.assign_kernel_name(n, d, k) in ("mfma_stream", "mfma_tiled")

@@ -4,7 +4,7 @@ allocate -- against hkm_assign_f32 with a caller-owned workspace: labels and min
 must be bit-identical (same kernels, same launch geometry, only the scratch address differs), on two calls
 in a row of which the second has the smaller input, so anything a call leaves behind in the shared array
 would show.  Shapes are chosen to use the scratch: the tiled kernel reads the squared centroid norms from
-it, the D > 64 kernel also merges its partial minima through 8-byte keys kept there.
+it, the streaming kernel (D > 128, or more centroids than LDS holds) also merges its partial minima through 8-byte keys kept there.
 """
 import pytest
 import torch
@@ -71,8 +71,8 @@ def test_static_scratch_assign_without_min_d2_and_strided_rows(cuda):
 
 
 def test_static_scratch_assign_rejects_what_does_not_fit(cuda):
-    # D > 64 keeps 8 bytes per row in the scratch: 3M rows need 24 MB, the array holds 16 MiB
-    n, d, k = 3_000_000, 65, 4
+    # D > 128 keeps 8 bytes per row in the scratch: 3M rows need 24 MB, the array holds 16 MiB
+    n, d, k = 3_000_000, 130, 4
     assert _native.workspace_bytes(n, d, k, _native.WS_ASSIGN) > 16 << 20
     x = torch.zeros((n, d), dtype=torch.float32, device=cuda)
     c = torch.zeros((k, d), dtype=torch.float32, device=cuda)
@@ -81,7 +81,7 @@ def test_static_scratch_assign_rejects_what_does_not_fit(cuda):
         _native.assign_static(x, c, lab, None)
     assert e.value.code == _native.HKM_EUNSUPPORTED
     assert "scratch" in str(e.value)
-    # the same rows with D <= 64 need no per-row scratch and run
+    # the same rows with D <= 128 need no per-row scratch and run
     _native.assign_static(x[:, :64], c[:, :64], lab, None)
     torch.cuda.synchronize()
     assert int(lab.max()) == 0
