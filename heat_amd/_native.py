@@ -19,7 +19,7 @@ from . import _f64_paths
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
-LIB_VERSION = 304  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
+LIB_VERSION = 305  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
 WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64, WS_FIT = 1, 2, 3, 4, 8, 16, 32
 
@@ -32,6 +32,8 @@ SIGNATURES = {
     "hkm_lloyd_kernel_name": (c_char_p, [c_int64, c_int32, c_int32]),
     "hkm_assign_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                       c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_assign_labels64_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
+                                               c_void_p, c_void_p, c_void_p]),
     "hkm_static_scratch_bytes": (c_size_t, []),
     "hkm_assign_static_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int64,
                                              c_void_p, c_void_p, c_void_p]),
@@ -226,6 +228,18 @@ def assign(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optio
     buf = ws.get(need)
     check(load().hkm_assign_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k, c.stride(0) if k > 1 else d,
                                 _ptr(labels), _ptr(min_d2), _ptr(buf), buf.numel(), _stream()))
+
+
+def assign_labels64(x: torch.Tensor, c: torch.Tensor, labels64: torch.Tensor, min_d2: Optional[torch.Tensor]) -> None:
+    """:func:`assign` for the narrow shapes (assign_kernel_name() == "valu_fused") with int64 labels stored at once."""
+    _require_gpu(x, c, labels64, min_d2)
+    _require_rows(x, c)
+    if labels64.dtype != torch.int64 or not labels64.is_contiguous() or labels64.numel() != x.shape[0]:
+        raise ValueError("labels64 must hold one contiguous int64 per row")
+    n, d = x.shape
+    k = c.shape[0]
+    check(load().hkm_assign_labels64_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), k,
+                                         c.stride(0) if k > 1 else d, _ptr(labels64), _ptr(min_d2), _stream()))
 
 
 def assign_static(x: torch.Tensor, c: torch.Tensor, labels: torch.Tensor, min_d2: Optional[torch.Tensor]) -> None:

@@ -203,6 +203,17 @@ class LloydLoop:
             self._lab_of = i
         return self.lab[0]
 
+    def labels64_into(self, out: torch.Tensor) -> None:
+        """The labels of the last iteration that counts as the (N, 1) int64 matrix the reference returns.  Where
+        the steps stored none (the narrow shapes) and none have been computed since, the one assignment pass
+        writes int64 at once instead of int32 labels that a second pass would widen."""
+        i = self.done - 1
+        n, d = self.x.shape
+        if self.lazy_labels and self._lab_of != i and _native.assign_kernel_name(n, d, self.c[0].shape[0]) == "valu_fused":
+            _native.assign_labels64(self.x, self.c[i % 3], out.view(-1), None)
+        else:
+            _native.widen_labels(self.labels, out)
+
     @property
     def last_shift(self) -> torch.Tensor:
         """0-d device tensor; waits for the step that produced it."""

@@ -107,10 +107,9 @@ class KMeans(_KCluster):
         self._n_iter = loop.run(self.max_iter, self.tol)
         if self._n_iter == 0:
             raise ValueError(f"max_iter must be positive, but was {self.max_iter}")
-        c_cur, lab32, shift = loop.centers, loop.labels, loop.last_shift
-
         lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
-        _native.widen_labels(lab32, lab64)
+        loop.labels64_into(lab64)
+        c_cur, shift = loop.centers, loop.last_shift
         ftype = types.canonical_heat_type(xt.dtype)
         self._cluster_centers = DNDarray(c_cur, (k, d), ftype, None, x.device, x.comm, True)
         self._inertia = DNDarray(shift.clone(), (), ftype, None, x.device, x.comm, True)

@@ -278,7 +278,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 304; }
+int hkm_version(void) { return 305; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -354,6 +354,24 @@ int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const floa
     if ((rc = check_ws(ws, ws_bytes, need))) return rc;
     const Workspace w = carve(ws, N, D, K, HKM_WS_ASSIGN);
     return do_assign(X, N, D, ldx, C, K, ldc, labels, min_d2, w, static_cast<hipStream_t>(hip_stream));
+}
+
+int hkm_assign_labels64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                            int64_t ldc, int64_t* labels, float* min_d2, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = check_shape(N, D, K);
+    if (rc) return rc;
+    if ((rc = check_matrix("X", X, N, D, ldx))) return rc;
+    if ((rc = check_matrix("C", C, K, D, ldc))) return rc;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (reinterpret_cast<uintptr_t>(labels) & 7u) return fail(HKM_EINVAL, "labels is not 8-byte aligned");
+    if (!(assign_kind(D, K) == ASSIGN_VALU && small_eligible(D, K)))
+        return fail(HKM_EUNSUPPORTED,
+                    "D = %d, K = %d: only the narrow kernel (hkm_assign_kernel_name() == \"valu_fused\") stores 64-bit "
+                    "labels itself; use hkm_assign_f32 and hkm_widen_labels_i64", D, K);
+    if (N == 0) return HKM_OK;
+    return launch_small(X, N, D, ldx, C, K, ldc, reinterpret_cast<int32_t*>(labels), min_d2, nullptr, 0, nullptr,
+                        static_cast<hipStream_t>(hip_stream), true);
 }
 
 // ---- hkm_assign_static_f32: the assignment without a caller-supplied workspace -----------------

@@ -194,9 +194,10 @@ int launch_lloyd_fit(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
                      void* ws, uint64_t wait_limit_ticks, hipStream_t st);
 bool small_eligible(int32_t D, int32_t K);
 int small_grid(int64_t N, int32_t D, int32_t K);
+// labels64: `labels` points to N 64-bit integers instead of 32-bit ones
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                  int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode, int32_t* flags,
-                 hipStream_t st);
+                 hipStream_t st, bool labels64 = false);
 int launch_small_finalize(const double* part, int grid, int32_t K, int32_t D, const float* C_old,
                           float* C_new, int64_t ldcn, int64_t* counts, float* shift, float* sse,
                           hipStream_t st);

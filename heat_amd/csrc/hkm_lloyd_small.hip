@@ -670,8 +670,14 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 
         // labels == NULL: the caller only wants the sums (a fit needs the labels of its last
         // iteration only and can recompute those)
+        // (vec & 8: `labels` points to 64-bit integers, the type the reference returns its labels in)
+        const bool lab64 = (vec & 8) != 0;
         if constexpr (!GUARD) {
-            if (labels) {
+            if (labels && lab64) {
+                longlong2* out = reinterpret_cast<longlong2*>(reinterpret_cast<long long*>(labels) + i0);
+#pragma unroll
+                for (int q = 0; q < PPT / 2; ++q) out[q] = make_longlong2(mi[2 * q], mi[2 * q + 1]);
+            } else if (labels) {
                 if constexpr (PPT == 4) {
                     *reinterpret_cast<int4*>(labels + i0) = make_int4(mi[0], mi[1], mi[2], mi[3]);
                 } else {
@@ -683,7 +689,10 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         for (int p = 0; p < PPT; ++p) {
             const bool ok = !GUARD || i0 + p < N;
             if (ok) {
-                if (GUARD && labels) labels[i0 + p] = mi[p];
+                if (GUARD && labels) {
+                    if (lab64) reinterpret_cast<long long*>(labels)[i0 + p] = mi[p];
+                    else labels[i0 + p] = mi[p];
+                }
                 if (WANT_MIN) min_d2[i0 + p] = m[p];
                 if (WANT_SSE) sse += double(m[p]);
             } else {
@@ -998,13 +1007,14 @@ __global__ __launch_bounds__(256) void lloyd_small_prereduce_kernel(const double
 template <int D>
 static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C, int32_t K,
                           int64_t ldc, int32_t* labels, float* min_d2, double* part, bool want_sse,
-                          int acc_mode, int grid, int32_t* flags, int aux, bool timed, hipStream_t st) {
+                          int acc_mode, int grid, int32_t* flags, int aux, bool timed, bool labels64, hipStream_t st) {
     const bool want_min = min_d2 != nullptr;
     const size_t lds = small_lds_bytes(D, K, acc_mode);
     // bit 0: 16-byte vector path; bit 1: X exceeds the 256 MB last-level cache -> streaming loads;
-    // bit 2: the scan takes the centroids four at a time
+    // bit 2: the scan takes the centroids four at a time; bit 3: labels are stored as 64-bit integers
     const int vec = ((ldx == D) && aligned16(X) && aligned16(labels) ? 1 : 0) |
-                    (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0) | (K >= small_blocked_min_k() ? 4 : 0);
+                    (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0) | (K >= small_blocked_min_k() ? 4 : 0) |
+                    (labels64 ? 8 : 0);
     // the register-resident centroid table: K <= 8 rows of at most 5 values
     constexpr int KT8 = D <= 4 ? 8 : 0;
     const bool reg = KT8 > 0 && K <= KT8;
@@ -1069,7 +1079,7 @@ static int small_headroom_bits(int64_t N, int32_t D, int grid) {
 // flags: [grid] scratch for the integer accumulation (may be NULL: then the ordered strategies run).
 int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
                  int64_t ldc, int32_t* labels, float* min_d2, double* part, int mode, int32_t* flags,
-                 hipStream_t st) {
+                 hipStream_t st, bool labels64) {
     const int grid = small_grid(N, D, K);
     const bool accum = mode & 1, want_sse = mode & 2;
     const int headroom = small_headroom_bits(N, D, grid);
@@ -1079,13 +1089,13 @@ int launch_small(const float* X, int64_t N, int32_t D, int64_t ldx, const float*
     case d: {                                                                                              \
         if (!integer)                                                                                      \
             return launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, want_sse, accum ? ordered : 0, \
-                                     grid, nullptr, 0, true, st);                                          \
+                                     grid, nullptr, 0, true, labels64, st);                                \
         int rc = launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, want_sse, 4, grid, flags,   \
-                                   headroom, true, st);                                                    \
+                                   headroom, true, labels64, st);                                          \
         if (rc) return rc;                                                                                 \
         /* the same sweep in the ordered way if a workgroup raised its flag; returns at once otherwise */  \
         return launch_small_t<d>(X, N, ldx, C, K, ldc, labels, min_d2, part, want_sse, ordered, grid, flags, \
-                                 grid, false, st);                                                         \
+                                 grid, false, labels64, st);                                               \
     }
     switch (D) {
         HKM_T(1) HKM_T(2) HKM_T(3) HKM_T(4) HKM_T(5) HKM_T(6) HKM_T(7) HKM_T(8)

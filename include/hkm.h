@@ -92,6 +92,17 @@ int hkm_assign_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const floa
                    void* hip_stream);
 
 /*
+ * hkm_assign_f32 with the labels stored as the int64 the reference returns (heat/core/statistics.py:129-200
+ * through heat/core/_operations.py:516-522), for the narrow shapes whose kernel is "valu_fused"
+ * (hkm_assign_kernel_name): their assignment is bound by memory traffic, and storing int64 at once saves the
+ * second pass over the labels that hkm_widen_labels_i64 makes (8 instead of 4 + 4 + 8 bytes per row).  Same
+ * labels and min_d2 as hkm_assign_f32, no workspace.  Other shapes return HKM_EUNSUPPORTED: use hkm_assign_f32
+ * and hkm_widen_labels_i64.
+ */
+int hkm_assign_labels64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K,
+                            int64_t ldc, int64_t* labels, float* min_d2, void* hip_stream);
+
+/*
  * hkm_assign_f32 for callers that cannot allocate device memory or carry a workspace: code under HIP
  * graph capture, tight serving loops (predict), harnesses that forbid hipMalloc.  No counterpart in the
  * reference.  Same arguments, results and kernels as hkm_assign_f32, but the scratch (reduction slots,

@@ -46,6 +46,34 @@ def _assign_gpu(x, c, dev, want_min=True):
     return lab.cpu(), (md.cpu() if want_min else None)
 
 
+@pytest.mark.parametrize("n,d,k", [(1, 3, 8), (1001, 3, 8), (5000, 8, 16), (4003, 12, 5), (300, 1, 5), (2222, 11, 20),
+                                   (70000, 2, 64), (3001, 16, 8), (999, 5, 31)])
+def test_narrow_assign_stores_int64_labels_itself(cuda, n, d, k):
+    """hkm_assign_labels64_f32: the labels of hkm_assign_f32, stored as int64 by the kernel itself (no second pass
+    that widens them), on rows with and without padding; shapes of other kernels are refused."""
+    assert _native.assign_kernel_name(n, d, k) == "valu_fused"
+    x, c = _data(n, d, k, seed=n + d)
+    xs, cs = x.to(cuda), c.to(cuda)
+    pad = torch.zeros((n, d + 3), device=cuda)
+    pad[:, :d] = xs
+    for rows in (xs, pad[:, :d]):
+        lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+        md = torch.empty((n,), device=cuda)
+        _native.assign(rows, cs, lab, md, _native.Workspace(cuda))
+        lab64 = torch.full((n,), -5, dtype=torch.int64, device=cuda)
+        md64 = torch.full((n,), -1.0, device=cuda)
+        _native.assign_labels64(rows, cs, lab64, md64)
+        torch.cuda.synchronize()
+        assert torch.equal(lab64, lab.long()) and torch.equal(md64, md)
+        only = torch.full((n,), -5, dtype=torch.int64, device=cuda)
+        _native.assign_labels64(rows, cs, only, None)
+        assert torch.equal(only, lab.long())
+    with pytest.raises(_native.HkmError) as e:
+        _native.assign_labels64(torch.zeros((10, 32), device=cuda), torch.zeros((4, 32), device=cuda),
+                                torch.zeros((10,), dtype=torch.int64, device=cuda), None)
+    assert e.value.code == _native.HKM_EUNSUPPORTED
+
+
 @pytest.mark.parametrize("n,d,k", ASSIGN_SHAPES)
 def test_assign_matches_oracle(cuda, n, d, k):
     print(f"assign n={n} d={d} k={k} kernel={_native.assign_kernel_name(n, d, k)}", flush=True)
