@@ -81,6 +81,28 @@ int main() {
     EXPECT(hkm_shift_f32(f, f, 0, 3, f, nullptr), HKM_EINVAL);
     EXPECT(hkm_functional_value_f32(f, -1, f, ws, big, nullptr), HKM_EINVAL);
 
+    // ---- the whole loop in one launch, and the assignment that stores 64-bit labels: shapes and arguments
+    int32_t info[2] = {0, 0};
+    if (hkm_lloyd_fit_supported(100000, 8, 16) != 1 || hkm_lloyd_fit_supported(131073, 8, 16) != 0 ||
+        hkm_lloyd_fit_supported(262144, 4, 5) != 1 || hkm_lloyd_fit_supported(1000, 17, 5) != 0 ||
+        hkm_lloyd_fit_supported(1000, 8, 27) != 0 || hkm_lloyd_fit_supported(0, 8, 4) != 0 ||
+        hkm_workspace_bytes(1000, 17, 5, HKM_WS_FIT) != 0 || hkm_workspace_bytes(1000, 8, 16, HKM_WS_FIT) == 0) {
+        std::printf("FAIL hkm_lloyd_fit_supported / HKM_WS_FIT\n");
+        ++failures;
+    }
+    EXPECT(hkm_lloyd_fit_f32(nullptr, 1000, 8, 8, f, 16, 5, 1, 0.0, f + 4096, i64, f, info, 1000, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_lloyd_fit_f32(f, 1000, 8, 8, f, 16, 0, 1, 0.0, f + 4096, i64, f, info, 1000, ws, big, nullptr), HKM_EINVAL);
+    EXPECT_MSG("max_iter");
+    EXPECT(hkm_lloyd_fit_f32(f, 1000, 8, 8, f, 16, 5, 1, 0.0, f + 4096, nullptr, f, info, 1000, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_lloyd_fit_f32(f, 1000, 8, 8, f, 16, 5, 1, 0.0, f + 4096, i64, f, nullptr, 1000, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_lloyd_fit_f32(f, 1000, 8, 8, f, 16, 5, 1, 0.0, f + 4096, i64, f, info, 1000, ws, 16, nullptr), HKM_EWORKSPACE);
+    EXPECT(hkm_lloyd_fit_f32(f, 1000, 32, 32, f, 16, 5, 1, 0.0, f + 4096, i64, f, info, 1000, ws, big, nullptr), HKM_EUNSUPPORTED);
+    EXPECT(hkm_lloyd_fit_f32(f, 300000, 8, 8, f, 16, 5, 1, 0.0, f + 4096, i64, f, info, 1000, ws, big, nullptr), HKM_EUNSUPPORTED);
+    EXPECT(hkm_assign_labels64_f32(f, 10, 3, 3, f, 8, 3, nullptr, nullptr, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_labels64_f32(f, 10, 3, 2, f, 8, 3, i64, nullptr, nullptr), HKM_EINVAL);
+    EXPECT(hkm_assign_labels64_f32(f, 10, 32, 32, f, 8, 32, i64, nullptr, nullptr), HKM_EUNSUPPORTED);
+    EXPECT(hkm_assign_labels64_f32(f, 0, 3, 3, f, 8, 3, i64, nullptr, nullptr), HKM_OK);
+
     // ---- the allocation-free assignment: its built-in scratch has a stated size
     EXPECT(hkm_assign_static_f32(nullptr, 10, 3, 3, f, 8, 3, i32, nullptr, nullptr), HKM_EINVAL);
     EXPECT(hkm_assign_static_f32(f, int64_t(1) << 26, 512, 512, f, 1024, 512, i32, nullptr, nullptr), HKM_EUNSUPPORTED);
