@@ -1041,11 +1041,13 @@ static size_t fused_lds_bytes_with(int32_t D, int32_t K, int nrep) {
 }
 
 // Copies of the fp64 accumulators in the one-sweep kernel: up to 64 clusters, as many as bring the lanes
-// that meet at one address down to a few and still fit in 48 KB with everything else.
+// that meet at one address down to a few.  One workgroup per CU runs this kernel, so the copies may take most of
+// the LDS: with the 48 KB they were held to before, 10M x 64, K = 8 ran on 8 copies in 0.652 ms (16: 0.605 ms),
+// 10M x 32, K = 32 on 4 in 0.360 ms (16: 0.345 ms); more than 16 copies gain nothing (10M x 32, K = 8: 0.3215 /
+// 0.3194 / 0.3166 ms with 16 / 32 / 64).  The sums are exact, so the number of copies does not change a bit.
 int fused_replicas(int32_t D, int32_t K) {
-    int r = K <= 16 ? 16 : K <= 32 ? 8 : K <= 64 ? 4 : 1;
-    // (one workgroup per CU runs this kernel: beyond 64 features, where a copy is large, it may take most of the LDS)
-    const size_t cap = resident_dp(D) > 64 ? 128 * 1024 : 48 * 1024;
+    int r = K <= 32 ? 16 : K <= 64 ? 4 : 1;
+    const size_t cap = 128 * 1024;
     while (r > 1 && fused_lds_bytes_with(D, K, r) > cap) r >>= 1;
     return r;
 }
