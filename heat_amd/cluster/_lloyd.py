@@ -61,7 +61,8 @@ class LloydLoop:
         # at most D * 2^-46 * sum |c|^2, taken eight times over.  The narrow step sums fp32 partials per lane, or
         # integers with a quantum of 2^-33 of the largest centroid coordinate: a mean is good to a few dozen ulps,
         # (2^-18)^2 of its magnitude per coordinate.
-        self._fuzz = {"lloyd_small": d * 2.0 ** -36, "lloyd_mfma_resident": d * 2.0 ** -43}.get(kernel, 0.0)
+        self._fuzz = {"lloyd_small": d * 2.0 ** -36, "lloyd_mfma_resident": d * 2.0 ** -43,
+                      "lloyd_few": d * 2.0 ** -43}.get(kernel, 0.0)  # (lloyd_few rounds its rows as the matrix-core step)
         # Upper bound on the Frobenius norm of the current centroids, kept from the shifts the host reads (see
         # _margin).  It starts at the norm of the init, taken here from a copy on the host, before anything is
         # in flight: no reduction kernel of the tensor library is loaded or launched for sixteen numbers.

@@ -258,6 +258,8 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
         case ASSIGN_MFMA_RESIDENT:
             if (use_split_products() && split_eligible(D, K, false))
                 return launch_split_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, nullptr, nullptr, st);
+            // few clusters of wide rows: the vector ALU needs less time than X takes to arrive
+            if (few_eligible(D, K)) return launch_few(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, nullptr, nullptr, st);
             return launch_assign_mfma_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_TILED: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
@@ -278,7 +280,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 305; }
+int hkm_version(void) { return 306; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -322,7 +324,7 @@ const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K) {
     if (D < 1 || K < 1) return "invalid";
     switch (assign_kind(D, K)) {
         case ASSIGN_VALU: return small_eligible(D, K) ? "valu_fused" : "valu";
-        case ASSIGN_MFMA_RESIDENT: return "mfma_resident";
+        case ASSIGN_MFMA_RESIDENT: return few_eligible(D, K) ? "valu_wide" : "mfma_resident";
         case ASSIGN_MFMA_TILED: return "mfma_tiled";
         default: return "mfma_stream";
     }
@@ -332,7 +334,7 @@ const char* hkm_lloyd_kernel_name(int64_t N, int32_t D, int32_t K) {
     (void)N;
     if (D < 1 || K < 1) return "invalid";
     if (small_eligible(D, K)) return "lloyd_small";
-    if (fused_eligible(D, K)) return "lloyd_mfma_resident";
+    if (fused_eligible(D, K)) return few_eligible(D, K) ? "lloyd_few" : "lloyd_mfma_resident";
     switch (assign_kind(D, K)) {
         case ASSIGN_VALU: return "valu+update";
         case ASSIGN_MFMA_RESIDENT: return "mfma_resident+update";
@@ -480,15 +482,19 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     if (fused_eligible(D, K) && N > 0) {
         // one sweep over X on the matrix cores: labels + fp64 per-cluster sums in LDS
         const bool split = use_split_products() && split_eligible(D, K, true);
+        const bool few = !split && few_eligible(D, K);
         if (split)
             rc = launch_split_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum, w.fcnt,
                                        w.fflags, st);
+        else if (few)
+            rc = launch_few(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum, w.fcnt, w.fflags, st);
         else
             rc = launch_lloyd_mfma_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum,
                                             w.fcnt, w.fflags, st);
         if (rc) return rc;
         if ((rc = launch_update_fused(X, N, D, ldx, labels, K, C_new, D, nullptr, w,
-                                      split ? split_fused_grid(N) : fused_grid(N, D), C, shift, st)))
+                                      split ? split_fused_grid(N) : few ? few_grid(N, D, K) : fused_grid(N, D), C,
+                                      shift, st)))
             return rc;
     } else {
         if ((rc = do_assign(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w, st))) return rc;

@@ -183,6 +183,11 @@ int launch_lloyd_mfma_resident(const float* X, int64_t N, int32_t D, int64_t ldx
 int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const int32_t* labels,
                         int32_t K, float* C_new, int64_t ldcn, int64_t* counts, const Workspace& w,
                         int fgrid, const float* C_old, float* shift, hipStream_t st);
+// few clusters of wide rows on the vector ALU (hkm_lloyd_few.hip); fsum == nullptr: the assignment alone
+bool few_eligible(int32_t D, int32_t K);
+int few_grid(int64_t N, int32_t D, int32_t K);
+int launch_few(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K, int64_t ldc,
+               int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags, hipStream_t st);
 // the whole Lloyd loop in one launch (hkm_lloyd_fit.hip)
 static const int FIT_MAX_GRID = 64;
 static const int64_t FIT_MAX_ROWS = int64_t(1) << 18;

@@ -204,7 +204,7 @@ def test_narrow_scan_four_at_a_time_keeps_the_reference_rules(cuda, d, k, monkey
 def test_assign_strided_rows(cuda):
     # X and C as column slices of wider buffers: ld > D, base pointers not 16-byte aligned
     g = torch.Generator().manual_seed(7)
-    for d, k in ((3, 8), (32, 64), (96, 200)):
+    for d, k in ((3, 8), (32, 64), (96, 200), (32, 8), (44, 5)):
         xw = torch.randn((1200, d + 5), generator=g)
         cw = torch.randn((k, d + 3), generator=g)
         xs, cs = xw.to(cuda)[:, 1 : 1 + d], cw.to(cuda)[:, 2 : 2 + d]
@@ -327,9 +327,17 @@ def _step_and_two_pass_impl(xs, cs, dev):
                                    (70001, 40, 129), (30000, 64, 128), (768, 17, 5), (100, 48, 7),
                                    (50000, 16, 64), (40000, 8, 40), (30001, 12, 100), (20000, 5, 60), (9000, 4, 256),
                                    (40000, 128, 8), (30001, 100, 16), (20000, 96, 32), (10000, 65, 3), (25000, 128, 90),
-                                   (5000, 77, 1)])
+                                   (5000, 77, 1),
+                                   (30000, 64, 16), (20000, 48, 13),
+                                   # few clusters of 17 to 64 features: the vector kernel with the same sums, in each
+                                   # of its launch geometries (workgroups of 256, 512, 1024 lanes; 32 or fewer copies
+                                   # of the accumulators), rows that are no whole 16-byte groups
+                                   (60001, 32, 8), (30000, 64, 12), (20001, 21, 2), (7000, 63, 11), (4000, 36, 16),
+                                   (1000, 64, 1), (300000, 20, 3), (50000, 40, 9), (40000, 48, 12), (25000, 28, 16),
+                                   (33333, 52, 11), (9000, 17, 16)])
 def test_one_sweep_mfma_step_equals_assign_plus_update(cuda, n, d, k):
-    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
+    few = 16 < d <= 64 and k <= (16 if d <= 40 else 12)
+    assert _native.lloyd_kernel_name(n, d, k) == ("lloyd_few" if few else "lloyd_mfma_resident")
     print(f"one-sweep n={n} d={d} k={k}", flush=True)
     x, _ = _data(n, d, k, seed=5 * n + d)
     x[::97] = 0.0  # all-zero rows only count

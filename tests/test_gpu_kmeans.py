@@ -217,11 +217,12 @@ def test_few_clusters_of_nine_to_sixteen_features_against_oracle(cuda, n, d, k, 
 
 @pytest.mark.parametrize("n,d,k", [(60000, 32, 8), (40000, 64, 8), (30000, 128, 8), (30000, 100, 5), (20000, 96, 32)])
 def test_few_clusters_of_wide_rows_against_oracle(cuda, n, d, k, parity_report):
-    """Whole fits with few clusters and 32 to 128 features -- an everyday shape -- on the one-sweep matrix-core
-    step (one read of X per iteration up to 128 features): step by step and at the end against the oracle."""
+    """Whole fits with few clusters and 32 to 128 features -- an everyday shape -- on the one-sweep steps (one
+    read of X per iteration: the vector kernel up to 64 features and 16 clusters, the matrix-core kernel up to
+    128 features): step by step and at the end against the oracle."""
     from heat_amd import _native
 
-    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_mfma_resident"
+    assert _native.lloyd_kernel_name(n, d, k) == ("lloyd_few" if d <= 64 and k <= 12 else "lloyd_mfma_resident")
     w = synthetic.shape(n, d, k, seed=1300 + d)
     print(f"{w.name}", flush=True)
     flips, ref = _stepwise_parity(w, cuda, 12, literal=False, report=parity_report)
@@ -436,7 +437,7 @@ def test_init_at_the_one_sweep_means_of_a_fixed_point_stops_like_the_oracle(cuda
     labels it could have repeated, so a zero shift there proves nothing."""
     from heat_amd import _native
 
-    assert _native.lloyd_kernel_name(n, d, k) in ("lloyd_small", "lloyd_mfma_resident")
+    assert _native.lloyd_kernel_name(n, d, k) in ("lloyd_small", "lloyd_few", "lloyd_mfma_resident")
     g = torch.Generator().manual_seed(17 * d + k)
     centres = (torch.rand((k, d), generator=g) - 0.5) * 400.0
     x = (torch.randn((n, d), generator=g) + centres[torch.randint(0, k, (n,), generator=g)]).contiguous()
