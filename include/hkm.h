@@ -421,12 +421,13 @@ int hkm_pairwise_f64(const double* X, int64_t M, int64_t ldx, const double* Y, i
 /* out[i] = (int64) in[i]: the (N, 1) int64 labels the reference returns (_operations.py:516-522). */
 int hkm_widen_labels_i64(const int32_t* in, int64_t N, int64_t* out, void* hip_stream);
 
-/* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "mfma_resident",
- * "mfma_tiled", "mfma_stream"); host pointer, static storage.  For benchmarks and profiles. */
+/* Name of the kernel family hkm_assign_f32 would launch for this shape ("valu", "valu_fused", "valu_wide" = few
+ * clusters of 17 to 64 features, "mfma_resident", "mfma_tiled", "mfma_stream"); host pointer, static storage.  For
+ * benchmarks and profiles. */
 const char* hkm_assign_kernel_name(int64_t N, int32_t D, int32_t K);
 
-/* Same for hkm_lloyd_step_f32: "lloyd_small" and "lloyd_mfma_resident" read X once per step (labels and
- * per-cluster sums in one kernel); every other shape runs "<assign kernel>+update" (two reads of X). */
+/* Same for hkm_lloyd_step_f32: "lloyd_small", "lloyd_few" and "lloyd_mfma_resident" read X once per step (labels
+ * and per-cluster sums in one kernel); every other shape runs "<assign kernel>+update" (two reads of X). */
 const char* hkm_lloyd_kernel_name(int64_t N, int32_t D, int32_t K);
 
 #ifdef __cplusplus
