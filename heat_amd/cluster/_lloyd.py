@@ -11,9 +11,9 @@ operation sits between two steps on the stream -- and no event either: before a 
 scalar is set to a value no shift can take (-1: a shift is a sum of squares or NaN), and the host
 waits for the step by reading the scalar until it has changed.  For a step of a few microseconds the
 record and the wait of an event were a third of the host's time per iteration, and the host is what
-bounds such fits.  For the narrow shapes whose step is one sweep of a
-vector kernel (D <= 16, few clusters), writing N labels is a quarter of the step's memory traffic, so the steps run
-without storing labels and those of the last iteration are computed once, on demand, against the
+bounds such fits.  For the shapes whose step is one sweep of a vector kernel (few clusters of at most 64
+features), writing N labels is up to a quarter of the step's memory traffic and, next to the stream of
+reads, costs more time than its share, so the steps run without storing labels and those of the last iteration are computed once, on demand, against the
 centroids that iteration started from -- the same kernel code, hence the same bits.  The values
 returned are exactly those of the sequential loop.
 
@@ -53,7 +53,7 @@ class LloydLoop:
         self.c = [c0.clone(), torch.empty_like(c0), torch.empty_like(c0)]
         n, d = xt.shape
         kernel = _native.lloyd_kernel_name(n, d, c0.shape[0]) if xt.dtype == torch.float32 else ""
-        self.lazy_labels = kernel == "lloyd_small"
+        self.lazy_labels = kernel in ("lloyd_small", "lloyd_few")
         # Relative size (against sum |c|^2) of the squared rounding error of a one-sweep step's centroids; 0 for the
         # shapes that run the two-pass update.  From the kernels' quanta: the matrix-core step rounds a row to
         # 2^-28 of its largest coordinate or, for rows below the floor it derives from the centroid norms, to at

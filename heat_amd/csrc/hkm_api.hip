@@ -144,6 +144,7 @@ Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
         w.fsum = reinterpret_cast<double*>(take(size_t(FUSED_MAX_GRID) * K * D * sizeof(double)));
         w.fcnt = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * K * sizeof(int32_t)));
         w.fflags = reinterpret_cast<int32_t*>(take(size_t(FUSED_MAX_GRID) * sizeof(int32_t)));
+        if (few_eligible(D, K)) w.lazy_lab = reinterpret_cast<int32_t*>(take(size_t(N < 1 ? 1 : N) * sizeof(int32_t)));
     }
     if (flags & HKM_WS_SSE)
         w.min_d2 = reinterpret_cast<float*>(
@@ -256,10 +257,10 @@ static int do_assign(const float* X, int64_t N, int32_t D, int64_t ldx, const fl
                 return launch_small(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, 0, nullptr, st);
             return launch_assign_valu(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_RESIDENT:
-            if (use_split_products() && split_eligible(D, K, false))
-                return launch_split_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, nullptr, nullptr, st);
             // few clusters of wide rows: the vector ALU needs less time than X takes to arrive
             if (few_eligible(D, K)) return launch_few(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, nullptr, nullptr, st);
+            if (use_split_products() && split_eligible(D, K, false))
+                return launch_split_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, nullptr, nullptr, nullptr, st);
             return launch_assign_mfma_resident(X, N, D, ldx, C, K, ldc, labels, min_d2, st);
         case ASSIGN_MFMA_TILED: {
             int rc = launch_norms(C, K, D, ldc, w.cn, int32_t(cn_pad(K)), st);
@@ -465,8 +466,8 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     if ((rc = check_matrix("C", C, K, D, D))) return rc;
     if ((rc = check_matrix("C_new", C_new, K, D, D))) return rc;
     if (C == C_new) return fail(HKM_EINVAL, "C and C_new must not alias");
-    if (!labels && N > 0 && !small_eligible(D, K))
-        return fail(HKM_EINVAL, "labels is NULL (only the one-sweep small-D step can run without storing labels)");
+    if (!labels && N > 0 && !small_eligible(D, K) && !few_eligible(D, K))
+        return fail(HKM_EINVAL, "labels is NULL (only the one-sweep vector-ALU steps can run without storing labels)");
     if (!shift) return fail(HKM_EINVAL, "shift is NULL");
     const int32_t flags = HKM_WS_LLOYD | (sse ? HKM_WS_SSE : 0);
     const size_t need = carve(nullptr, N, D, K, flags).total;
@@ -481,8 +482,8 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     }
     if (fused_eligible(D, K) && N > 0) {
         // one sweep over X on the matrix cores: labels + fp64 per-cluster sums in LDS
-        const bool split = use_split_products() && split_eligible(D, K, true);
-        const bool few = !split && few_eligible(D, K);
+        const bool few = few_eligible(D, K);
+        const bool split = !few && use_split_products() && split_eligible(D, K, true);
         if (split)
             rc = launch_split_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum, w.fcnt,
                                        w.fflags, st);
@@ -492,6 +493,14 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
             rc = launch_lloyd_mfma_resident(X, N, D, ldx, C, K, D, labels, sse ? w.min_d2 : nullptr, w.fsum,
                                             w.fcnt, w.fflags, st);
         if (rc) return rc;
+        if (few && !labels) {
+            // the step stored no labels; the two-pass update that redoes the sums of a flagged step needs them:
+            // one more launch, which returns at once unless a flag is up
+            const int grid = few_grid(N, D, K);
+            if ((rc = launch_few(X, N, D, ldx, C, K, D, w.lazy_lab, nullptr, nullptr, nullptr, nullptr, st, w.fflags, grid)))
+                return rc;
+            labels = w.lazy_lab;
+        }
         if ((rc = launch_update_fused(X, N, D, ldx, labels, K, C_new, D, nullptr, w,
                                       split ? split_fused_grid(N) : few ? few_grid(N, D, K) : fused_grid(N, D), C,
                                       shift, st)))

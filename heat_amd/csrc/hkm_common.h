@@ -122,6 +122,7 @@ struct Workspace {
     double* fsum;       // [FUSED_MAX_GRID][K][D] fp64 partial sums of the one-sweep MFMA step
     int32_t* fcnt;      // [FUSED_MAX_GRID][K]
     int32_t* fflags;    // [FUSED_MAX_GRID] 1 = this workgroup's sums may depend on the addition order
+    int32_t* lazy_lab;  // [N] labels of a step that ran without storing any, computed only when a flag is up
     SortedWorkspace srt; // scratch of the sorted update (with the UPDATE flag, K <= 4096)
     size_t total;
 };
@@ -187,7 +188,8 @@ int launch_update_fused(const float* X, int64_t N, int32_t D, int64_t ldx, const
 bool few_eligible(int32_t D, int32_t K);
 int few_grid(int64_t N, int32_t D, int32_t K);
 int launch_few(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K, int64_t ldc,
-               int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags, hipStream_t st);
+               int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags, hipStream_t st,
+               const int32_t* gate = nullptr, int ngate = 0);
 // the whole Lloyd loop in one launch (hkm_lloyd_fit.hip)
 static const int FIT_MAX_GRID = 64;
 static const int64_t FIT_MAX_ROWS = int64_t(1) << 18;

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(T) void lloyd_few_kernel(
     const float* __restrict__ X, int64_t N, int D, int64_t ldx, const float* __restrict__ C, int K, int64_t ldc,
     int32_t* __restrict__ labels, float* __restrict__ min_d2, int64_t ntiles, double* __restrict__ fsum,
     int32_t* __restrict__ fcnt, int32_t* __restrict__ flags, int range_bits, int nrep, int lda, int cstride,
-    int mode) {
+    int mode, const int32_t* __restrict__ gate, int ngate) {
     constexpr int NV = DP / 4;
     extern __shared__ __align__(16) float lds[];
     float* sCn = lds;                                                     // [K]
@@ -110,6 +110,12 @@ __global__ __launch_bounds__(T) void lloyd_few_kernel(
     int* sN = reinterpret_cast<int*>(sA + (FUSED ? nrep * cstride : 0));  // [nrep][K], then the bookkeeping
     int* sMeta = sN + (FUSED ? nrep * K : 0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (gate) {
+        // the labels a step ran without are only wanted if one of its workgroups raised its flag
+        int up = 0;
+        for (int i = tid; i < ngate; i += T) up |= gate[i];
+        if (!__syncthreads_or(up)) return;
+    }
     const bool vec = (mode & 1) != 0;     // rows are whole aligned 16-byte groups
     const bool stream = (mode & 2) != 0;  // X exceeds the last-level cache
     const few_cptr Cc = (few_cptr)C;
@@ -215,8 +221,10 @@ __global__ __launch_bounds__(T) void lloyd_few_kernel(
         m += xn;
         // a row that coincides with a centroid up to rounding: the scan again with the clamp on every value
         if (__any(m < 0.f)) scan(x, xn, true, m, mi);
+        // labels may be absent: a stream of 4 bytes per row next to the reads costs more read bandwidth than its
+        // share, so the fit's steps do without and compute the last iteration's labels once
         if (valid) {
-            labels[row] = mi;
+            if (labels) labels[row] = mi;
             if (WANT_MIN) min_d2[row] = m;
         }
         if (FUSED && valid) {
@@ -274,7 +282,8 @@ __global__ __launch_bounds__(T) void lloyd_few_kernel(
 
 template <int DP, int T>
 static int launch_few_t(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K, int64_t ldc,
-                        int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags, hipStream_t st) {
+                        int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags,
+                        const int32_t* gate, int ngate, hipStream_t st) {
     const bool fused = fsum != nullptr;
     const FewGeometry g = few_geometry(D, K, fused);
     const int64_t ntiles = (N + T - 1) / T;
@@ -302,7 +311,8 @@ static int launch_few_t(const float* X, int64_t N, int32_t D, int64_t ldx, const
         }                                                                                                     \
         prof_begin(st);                                                                                       \
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(T), lds,     st, X, N, D, ldx, C, K, ldc, labels, \
-                           min_d2, ntiles, fsum, fcnt, flags, range_bits, nrep, lda, cstride, mode);          \
+                           min_d2, ntiles, fsum, fcnt, flags, range_bits, nrep, lda, cstride, mode, gate,    \
+                           ngate);                                                                            \
     } while (0)
     if (fused) {
         if (min_d2) HKM_FEW_GO(true, true);
@@ -316,20 +326,22 @@ static int launch_few_t(const float* X, int64_t N, int32_t D, int64_t ldx, const
     return check_launch("lloyd_few_kernel");
 }
 
-// fsum == nullptr: the assignment alone
+// fsum == nullptr: the assignment alone.  labels == nullptr (the step only): none are stored.  gate != nullptr: the
+// launch does nothing unless one of gate[0 .. ngate) is non-zero.
 int launch_few(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, int32_t K, int64_t ldc,
-               int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags, hipStream_t st) {
+               int32_t* labels, float* min_d2, double* fsum, int32_t* fcnt, int32_t* flags, hipStream_t st,
+               const int32_t* gate, int ngate) {
     if (N == 0) return HKM_OK;
     const int threads = few_geometry(D, K, fsum != nullptr).threads;
     switch (few_dp(D)) {
 #define HKM_FEW_CASE(d)                                                                                   \
     case d:                                                                                               \
         switch (threads) {                                                                                \
-            case 256: return launch_few_t<d, 256>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st); \
-            case 512: return launch_few_t<d, 512>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, st); \
+            case 256: return launch_few_t<d, 256>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, gate, ngate, st); \
+            case 512: return launch_few_t<d, 512>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, flags, gate, ngate, st); \
             default:                                                                                      \
                 return launch_few_t<d, (d <= 52 ? 1024 : 512)>(X, N, D, ldx, C, K, ldc, labels, min_d2, fsum, fcnt, \
-                                                               flags, st);                                \
+                                                               flags, gate, ngate, st);                   \
         }
         HKM_FEW_CASE(20) HKM_FEW_CASE(24) HKM_FEW_CASE(28) HKM_FEW_CASE(32) HKM_FEW_CASE(36) HKM_FEW_CASE(40)
         HKM_FEW_CASE(44) HKM_FEW_CASE(48) HKM_FEW_CASE(52) HKM_FEW_CASE(56) HKM_FEW_CASE(60) HKM_FEW_CASE(64)

@@ -508,6 +508,49 @@ def test_one_sweep_mfma_step_falls_back_outside_the_exact_range(cuda):
     assert (c_step.cpu() - ref).abs().max() <= 2e-7 * float(xv.abs().max())
 
 
+@pytest.mark.parametrize("n,d,k", [(60001, 32, 8), (30000, 64, 12), (20001, 21, 2), (25000, 28, 16)])
+def test_few_cluster_step_without_labels_equals_the_step_with_labels(cuda, n, d, k):
+    """The fit's steps on few clusters of 17 to 64 features store no labels.  Same centroids and shift bit for bit
+    as the step that stores them -- on the exact path, and where a workgroup raises its flag (row magnitudes
+    spread over 2^60, non-finite rows): there the labels the two-pass update needs are computed into the
+    workspace by one more launch, which otherwise returns at once."""
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_few"
+    x, _ = _data(n, d, k, seed=3 * n + d)
+    g = torch.Generator().manual_seed(5)
+    for variant in ("plain", "wide", "nonfinite"):
+        xv = x.clone()
+        if variant == "wide":
+            xv = xv * torch.pow(2.0, torch.randint(-30, 31, (n, 1), generator=g).float())
+        if variant == "nonfinite":
+            xv[7, 2] = float("inf")
+            xv[n // 2, 0] = float("nan")
+        c0 = torch.nan_to_num(xv[torch.randperm(n, generator=g)[:k]].contiguous(), nan=0.0, posinf=1.0, neginf=-1.0)
+        xs, cs = xv.to(cuda), c0.to(cuda)
+        ws = _native.Workspace(cuda)
+        out = []
+        for lab in (torch.full((n,), -7, dtype=torch.int32, device=cuda), None, None):
+            c_new = torch.full_like(cs, -3.0)
+            shift = torch.empty((), device=cuda)
+            _native.lloyd_step(xs, cs, c_new, lab, shift, None, ws)
+            torch.cuda.synchronize()
+            out.append((c_new.cpu(), shift.cpu()))
+        for c_new, shift in out[1:]:
+            assert torch.equal(torch.nan_to_num(c_new), torch.nan_to_num(out[0][0])), variant
+            assert torch.equal(c_new.isnan(), out[0][0].isnan()), variant
+            assert torch.equal(torch.nan_to_num(shift), torch.nan_to_num(out[0][1])), variant
+        if variant != "plain":
+            # a flagged step's means are those of the (list-based) two-pass update of its labels; the spread of
+            # magnitudes alone need not raise a flag (rows far below the centroids are rounded to a floor derived
+            # from the centroid norms), and then the means are the fp64 ones
+            _, _, _, c2, lab2, cnt2 = _step_and_two_pass(xs, cs, cuda, lists=True)
+            flagged = torch.equal(torch.nan_to_num(c2.cpu()), torch.nan_to_num(out[1][0]))
+            assert flagged or variant == "wide", variant
+            if not flagged:
+                ref = torch.zeros((k, d), dtype=torch.float64).index_add_(0, lab2.cpu().long(), xv.double())
+                ref = (ref / cnt2.cpu().clamp(min=1).double().unsqueeze(1)).float()
+                assert (out[1][0] - ref).abs().max() <= 2e-7 * float(ref.abs().max())
+
+
 def _narrow_step(xs, cs, dev, sums, monkeypatch, want_sse=True):
     """One hkm_lloyd_step_f32 on a narrow shape with the per-cluster sums formed the given way."""
     monkeypatch.setenv("HKM_SMALL_SUMS", sums)
