@@ -54,6 +54,10 @@ class LloydLoop:
         n, d = xt.shape
         kernel = _native.lloyd_kernel_name(n, d, c0.shape[0]) if xt.dtype == torch.float32 else ""
         self.lazy_labels = kernel in ("lloyd_small", "lloyd_few")
+        # A step known to be the last of a run (the max_iter-th) stores its labels after all: one more stream of
+        # writes in one step instead of one more pass over X afterwards.  Not for the narrow shapes, whose final
+        # pass writes the int64 labels the caller wants at once.
+        self._label_last = kernel == "lloyd_few"
         # Relative size (against sum |c|^2) of the squared rounding error of a one-sweep step's centroids; 0 for the
         # shapes that run the two-pass update.  From the kernels' quanta: the matrix-core step rounds a row to
         # 2^-28 of its largest coordinate or, for rows below the floor it derives from the centroid norms, to at
@@ -78,18 +82,21 @@ class LloydLoop:
         self.done = 0      # steps whose results count
         self._plans = {}   # prepared calls, one per rotation of the buffers (and stream)
 
-    def _enqueue(self) -> None:
+    def _enqueue(self, last: bool = False) -> None:
         j = self.enqueued
-        key = (j % 6, torch.cuda.current_stream().cuda_stream)
+        with_labels = not self.lazy_labels or (last and self._label_last)
+        key = (j % 6, with_labels, torch.cuda.current_stream().cuda_stream)
         plan = self._plans.get(key)
         if plan is None:
             # the argument list of a step only depends on which buffers of the rotation it uses
-            plan = _native.prepare_lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3],
-                                              None if self.lazy_labels else self.lab[j % 2],
+            lab = None if not with_labels else self.lab[0] if self.lazy_labels else self.lab[j % 2]
+            plan = _native.prepare_lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3], lab,
                                               self.shift_host[j % 2], None, self.ws)
             self._plans[key] = plan
         self._shift_np[j % 2] = _PENDING
         plan()
+        if self.lazy_labels and with_labels:
+            self._lab_of = j
         self.enqueued = j + 1
 
     def _wait(self, i: int) -> float:
@@ -118,7 +125,7 @@ class LloydLoop:
         for _ in range(max_iter):
             i = self.done
             if self.enqueued == i:
-                self._enqueue()
+                self._enqueue(last=ran + 1 == max_iter)
             if tol is None:
                 self._free_running = True
                 self._cnorm = None  # nobody reads these shifts: the bound is taken again when it is needed
@@ -126,7 +133,7 @@ class LloydLoop:
                 ran += 1
                 continue
             if ran + 1 < max_iter and self.enqueued == i + 1:
-                self._enqueue()  # ahead of the host's look at step i
+                self._enqueue(last=ran + 2 == max_iter)  # ahead of the host's look at step i
             shift = self._wait(i)
             self.done = i + 1
             ran += 1

@@ -388,6 +388,37 @@ def test_pipelined_loop_stops_exactly_like_the_sequential_one(cuda, monkeypatch)
         ht.cluster.KMeans(n_clusters=w.k, init=ht.array(w.init.to(cuda)), max_iter=0).fit(ht.array(x, split=0))
 
 
+def test_last_step_of_a_run_stores_the_labels_of_few_cluster_fits(cuda):
+    """Few clusters of 17 to 64 features: the steps store no labels, except the one known to be the last of its run
+    (the max_iter-th), so that a fit that ends there needs no pass over X for its labels.  Same labels as the
+    pass would give, whether the run ends at max_iter or earlier, and when a run is continued."""
+    from heat_amd import _native
+    from heat_amd.cluster._lloyd import LloydLoop
+
+    n, d, k = 70001, 32, 8
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_few"
+    g = torch.Generator().manual_seed(11)
+    centres = torch.randn((k, d), generator=g) * 2.0
+    x = (centres[torch.randint(0, k, (n,), generator=g)] + torch.randn((n, d), generator=g)).to(cuda)
+    c0 = x[:k].clone()
+    for steps, tol in ((4, -1.0), (4, None), (40, 1e-3), (1, -1.0)):
+        a = LloydLoop(x, c0, _native.Workspace(cuda))
+        b = LloydLoop(x, c0, _native.Workspace(cuda))
+        b._label_last = False  # every label from the pass afterwards
+        assert a.lazy_labels and a._label_last
+        ra, rb = a.run(steps, tol), b.run(steps, tol)
+        assert ra == rb and torch.equal(a.centers, b.centers)
+        if ra == steps and tol is not None and tol < 0:
+            assert a._lab_of == a.done - 1  # already there
+        assert torch.equal(a.labels, b.labels)
+        lab = torch.empty((n,), dtype=torch.int32, device=cuda)
+        _native.assign(x, a.c[(a.done - 1) % 3], lab, None, _native.Workspace(cuda))
+        assert torch.equal(a.labels, lab)
+        # continued: the labels kept from the first run's last step must not be taken for the second's
+        assert a.run(2, -1.0) == 2 and b.run(2, -1.0) == 2
+        assert torch.equal(a.centers, b.centers) and torch.equal(a.labels, b.labels)
+
+
 # ---- closed forms of the loop (heat/cluster/kmeans.py:131-146) through the public estimator --------
 # shapes: the one-sweep matrix-core step (D = 32), the narrow one-sweep step (D = 3 and D = 8), and a
 # shape that runs assignment + two-pass update (D = 100)
