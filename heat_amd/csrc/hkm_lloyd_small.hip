@@ -54,10 +54,14 @@
 
 namespace hkm {
 
-// stream: the matrix is larger than the last-level cache, so its lines are not worth keeping there
-__device__ __forceinline__ floatx4 ldg4(const float* p, bool stream) {
+// STREAM: the matrix is larger than the last-level cache, so its lines are not worth keeping there.  A template
+// parameter: a run-time choice between a non-temporal and a plain load of one address is compiled into a single
+// plain load.
+template <bool STREAM>
+__device__ __forceinline__ floatx4 ldg4(const float* p) {
     const floatx4* q = reinterpret_cast<const floatx4*>(p);
-    return stream ? __builtin_nontemporal_load(q) : *q;
+    if constexpr (STREAM) return __builtin_nontemporal_load(q);
+    else return *q;
 }
 
 template <int D>
@@ -352,7 +356,7 @@ __device__ __forceinline__ void scan_centroids_reg(const float (&cs)[KT][D + 1],
 //   integer scale, or no usable scale), aux = how many bits above the largest centroid coordinate a row
 //   may reach.  The ordered modes, given flags, are the re-run after an ACC == 4 launch of aux workgroups:
 //   they return at once unless one of those raised its flag.
-template <int D, int ACC, bool WANT_MIN, bool WANT_SSE, int KT>
+template <int D, int ACC, bool WANT_MIN, bool WANT_SSE, int KT, bool STREAM>
 __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const float* __restrict__ X, int64_t N, int64_t ldx, const float* __restrict__ C, int K,
     int64_t ldc, int32_t* __restrict__ labels, float* __restrict__ min_d2,
@@ -366,7 +370,6 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     float* sC = lds;  // [K][SC]
     const int slots = K * (D + 1);
     constexpr bool ACCUM = ACC != 0;
-    const bool stream = (vec & 2) != 0;
     const int KP = (K + 3) & ~3;                                     // rows of sC: K, then +inf-norm rows up to a multiple of four
     float* stage = lds + KP * SC;                                    // [NW][NV*64*4] transpose buffer
     // matrix-core scan: [NW][128] (minimum, index) pairs on their way from the lane that found them to the
@@ -413,7 +416,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     for (int f = 0; f < PF; ++f) {
         if (base + f * stride + T <= full) {
 #pragma unroll
-            for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + f * rstride + v * 256, stream);
+            for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4<STREAM>(wsrc + f * rstride + v * 256);
         }
     }
 
@@ -793,7 +796,9 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     // requested before the current round is processed.
     {
         // The loop is unrolled PF times so that each round's buffer is a fixed set of registers: a
-        // register rotation would make every round wait for ALL outstanding loads.
+        // register rotation would make every round wait for ALL outstanding loads.  (The requests sit under a
+        // condition, so the compiler's wait for a round's rows also covers most of the later rounds' loads; the
+        // loop without conditions, with all PF rounds truly in flight, was measured and is 3-18 % slower.)
         bool more = base + T <= full;
         while (more) {
 #pragma unroll
@@ -810,7 +815,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                     wave_lds_sync();
                     if (base + PF * stride + T <= full) {
 #pragma unroll
-                        for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4(wsrc + PF * rstride + v * 256, stream);
+                        for (int v = 0; v < NV; ++v) nxt[f][v] = ldg4<STREAM>(wsrc + PF * rstride + v * 256);
                     }
                     wsrc += rstride;
 #pragma unroll
@@ -1018,20 +1023,25 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     // the register-resident centroid table: K <= 8 rows of at most 5 values
     constexpr int KT8 = D <= 4 ? 8 : 0;
     const bool reg = KT8 > 0 && K <= KT8;
-#define HKM_GO(A, M, S)                                                                                  \
-    do {                                                                                                 \
-        if (A == 3 && K > 16)                                                                            \
-            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A == 3 ? 32 : 0>), dim3(grid), dim3(SMALL_T), lds, \
-                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);         \
-        else if (A == 3)                                                                                 \
-            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A == 3 ? 16 : 0>), dim3(grid), dim3(SMALL_T), lds, \
-                               st, X, N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);         \
-        else if (reg && A != 4)                                                                          \
-            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, A != 4 ? KT8 : 0>), dim3(grid), dim3(SMALL_T), lds, st, X, \
-                               N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);                \
-        else                                                                                             \
-            hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, 0>), dim3(grid), dim3(SMALL_T), lds, st, X, \
-                               N, ldx, C, K, ldc, labels, min_d2, part, vec, flags, aux);                \
+    // streaming loads only in the modes that large matrices run in (labels only, per-lane columns, integer sums)
+#define HKM_LAUNCH(A, M, S, KTV, STRM)                                                                            \
+    hipLaunchKernelGGL((lloyd_small_kernel<D, A, M, S, KTV, STRM>), dim3(grid), dim3(SMALL_T), lds, st, X, N, ldx, C, \
+                       K, ldc, labels, min_d2, part, vec, flags, aux)
+#define HKM_GO2(A, M, S, KTV)                                          \
+    do {                                                               \
+        if constexpr (A == 0 || A == 1 || A == 4) {                    \
+            if (vec & 2) HKM_LAUNCH(A, M, S, KTV, true);               \
+            else HKM_LAUNCH(A, M, S, KTV, false);                      \
+        } else {                                                       \
+            HKM_LAUNCH(A, M, S, KTV, false);                           \
+        }                                                              \
+    } while (0)
+#define HKM_GO(A, M, S)                                  \
+    do {                                                 \
+        if (A == 3 && K > 16) HKM_GO2(A, M, S, (A == 3 ? 32 : 0));       \
+        else if (A == 3) HKM_GO2(A, M, S, (A == 3 ? 16 : 0));            \
+        else if (reg && A != 4) HKM_GO2(A, M, S, (A != 4 ? KT8 : 0));    \
+        else HKM_GO2(A, M, S, 0);                                        \
     } while (0)
     if (timed) prof_begin(st);
     if (acc_mode == 2) {
@@ -1059,6 +1069,8 @@ static int launch_small_t(const float* X, int64_t N, int64_t ldx, const float* C
     }
     if (timed) prof_end(st);
 #undef HKM_GO
+#undef HKM_GO2
+#undef HKM_LAUNCH
     return check_launch("lloyd_small_kernel");
 }
 
