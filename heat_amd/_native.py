@@ -19,7 +19,7 @@ from . import _f64_paths
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
-LIB_VERSION = 306  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
+LIB_VERSION = 307  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
 WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64, WS_FIT = 1, 2, 3, 4, 8, 16, 32
 
@@ -41,6 +41,8 @@ SIGNATURES = {
                                       c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_step_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "hkm_lloyd_step_labels64_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
+                                                   c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_fit_supported": (ctypes.c_int, [c_int64, c_int32, c_int32]),
     "hkm_lloyd_fit_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int32, c_int32,
                                          ctypes.c_double, c_void_p, c_void_p, c_void_p, c_void_p, ctypes.c_uint64,
@@ -324,11 +326,12 @@ def lloyd_fit(x: torch.Tensor, c0: torch.Tensor, max_iter: int, tol: Optional[fl
 
 
 def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Optional[torch.Tensor],
-                       shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace):
+                       shift: torch.Tensor, sse: Optional[torch.Tensor], ws: Workspace, labels64: bool = False):
     """The same call as :func:`lloyd_step` with every argument converted once: returns a function
     without arguments that enqueues the step on the stream that was current when it was prepared.
     For loops that issue thousands of steps on small problems, where building the argument list costs
-    as much as the step.  The tensors are kept alive by the returned function."""
+    as much as the step.  The tensors are kept alive by the returned function.  ``labels64``: ``labels`` is an
+    int64 vector that the step fills itself (the narrow one-sweep step only)."""
     _require_gpu(x, c, c_new, labels, sse)
     _require_rows(x, c, c_new)
     _require_dense(c, c_new)
@@ -340,6 +343,12 @@ def prepare_lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, la
     flags = WS_LLOYD | (WS_F64 if f64 else 0) | (WS_SSE if sse is not None else 0)
     buf = ws.get(workspace_bytes(n, d, k, flags))
     fn = load().hkm_lloyd_step_f64 if f64 else load().hkm_lloyd_step_f32
+    if labels64:
+        if f64 or labels is None or labels.dtype != torch.int64 or not labels.is_contiguous() or labels.numel() != n:
+            raise ValueError("labels64 needs float32 data and a contiguous int64 vector of N labels")
+        fn = load().hkm_lloyd_step_labels64_f32
+    elif labels is not None and labels.dtype != torch.int32:
+        raise ValueError("labels must be int32")
     args = (_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k, _ptr(labels), _ptr(shift),
             _ptr(sse), _ptr(buf), buf.numel(), _stream())
     keep = (x, c, c_new, labels, shift, sse, buf)

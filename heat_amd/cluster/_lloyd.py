@@ -58,6 +58,11 @@ class LloydLoop:
         # writes in one step instead of one more pass over X afterwards.  Not for the narrow shapes, whose final
         # pass writes the int64 labels the caller wants at once.
         self._label_last = kernel == "lloyd_few"
+        # The narrow shapes' last step can store the int64 labels the caller wants at once, into the caller's own
+        # vector (final_labels64): neither the pass over X nor the widening pass is left.
+        self._narrow = kernel == "lloyd_small"
+        self._lab64_out: Optional[torch.Tensor] = None
+        self._lab64_of = -1  # iteration whose labels self._lab64_out holds
         # Relative size (against sum |c|^2) of the squared rounding error of a one-sweep step's centroids; 0 for the
         # shapes that run the two-pass update.  From the kernels' quanta: the matrix-core step rounds a row to
         # 2^-28 of its largest coordinate or, for rows below the floor it derives from the centroid norms, to at
@@ -82,20 +87,35 @@ class LloydLoop:
         self.done = 0      # steps whose results count
         self._plans = {}   # prepared calls, one per rotation of the buffers (and stream)
 
+    def final_labels64(self, out: Optional[torch.Tensor]) -> None:
+        """A contiguous int64 vector of N entries that the last step of a run may fill with its labels (the narrow
+        shapes only; ignored otherwise).  labels64_into(out) then finds them there."""
+        self._lab64_out = out if self._narrow else None
+        self._lab64_of = -1
+        self._plans = {k: v for k, v in self._plans.items() if k[1] != 2}
+
     def _enqueue(self, last: bool = False) -> None:
         j = self.enqueued
-        with_labels = not self.lazy_labels or (last and self._label_last)
-        key = (j % 6, with_labels, torch.cuda.current_stream().cuda_stream)
+        # 0: no labels; 1: int32 labels; 2: int64 labels into the caller's vector
+        mode = 1 if not self.lazy_labels or (last and self._label_last) else 0
+        if last and self._lab64_out is not None:
+            mode = 2
+        key = (j % 6, mode, torch.cuda.current_stream().cuda_stream)
         plan = self._plans.get(key)
         if plan is None:
             # the argument list of a step only depends on which buffers of the rotation it uses
-            lab = None if not with_labels else self.lab[0] if self.lazy_labels else self.lab[j % 2]
+            if mode == 2:
+                lab = self._lab64_out
+            else:
+                lab = None if mode == 0 else self.lab[0] if self.lazy_labels else self.lab[j % 2]
             plan = _native.prepare_lloyd_step(self.x, self.c[j % 3], self.c[(j + 1) % 3], lab,
-                                              self.shift_host[j % 2], None, self.ws)
+                                              self.shift_host[j % 2], None, self.ws, labels64=mode == 2)
             self._plans[key] = plan
         self._shift_np[j % 2] = _PENDING
         plan()
-        if self.lazy_labels and with_labels:
+        if mode == 2:
+            self._lab64_of = j
+        elif self.lazy_labels and mode == 1:
             self._lab_of = j
         self.enqueued = j + 1
 
@@ -217,6 +237,8 @@ class LloydLoop:
         writes int64 at once instead of int32 labels that a second pass would widen."""
         i = self.done - 1
         n, d = self.x.shape
+        if self._lab64_out is not None and self._lab64_of == i and out.data_ptr() == self._lab64_out.data_ptr():
+            return  # the last step wrote them
         if self.lazy_labels and self._lab_of != i and _native.assign_kernel_name(n, d, self.c[0].shape[0]) == "valu_fused":
             _native.assign_labels64(self.x, self.c[i % 3], out.view(-1), None)
         else:

@@ -104,10 +104,13 @@ class KMeans(_KCluster):
         # the reference evaluates ``inertia <= tol`` on the host every iteration (kmeans.py:143); the
         # loop keeps the next step enqueued while the host looks at the shift of the current one
         loop = LloydLoop(xt, self._local_f32(self._cluster_centers, like=xt), self._workspace(dev))
+        # the (N, 1) int64 labels the reference returns: for the narrow shapes the step known to be the last writes
+        # them itself
+        lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
+        loop.final_labels64(lab64.view(-1))
         self._n_iter = loop.run(self.max_iter, self.tol)
         if self._n_iter == 0:
             raise ValueError(f"max_iter must be positive, but was {self.max_iter}")
-        lab64 = torch.empty((n, 1), dtype=torch.int64, device=dev)
         loop.labels64_into(lab64)
         c_cur, shift = loop.centers, loop.last_shift
         ftype = types.canonical_heat_type(xt.dtype)

@@ -281,7 +281,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 306; }
+int hkm_version(void) { return 307; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -456,9 +456,10 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
                      static_cast<hipStream_t>(hip_stream));
 }
 
-int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
-                       float* C_new, int32_t K, int32_t* labels, float* shift, float* sse, void* ws,
-                       size_t ws_bytes, void* hip_stream) {
+// labels64: `labels` points to 64-bit integers (the narrow one-sweep step only)
+static int lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new, int32_t K,
+                          int32_t* labels, bool labels64, float* shift, float* sse, void* ws, size_t ws_bytes,
+                          void* hip_stream) {
     g_err[0] = 0;
     int rc = check_shape(N, D, K);
     if (rc) return rc;
@@ -476,7 +477,8 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     hipStream_t st = static_cast<hipStream_t>(hip_stream);
     if (small_eligible(D, K) && N > 0) {
         // one sweep over X: labels + private per-lane sums, then a single-workgroup finish
-        if ((rc = launch_small(X, N, D, ldx, C, K, D, labels, nullptr, w.small_part, sse ? 3 : 1, w.small_flags, st)))
+        if ((rc = launch_small(X, N, D, ldx, C, K, D, labels, nullptr, w.small_part, sse ? 3 : 1, w.small_flags, st,
+                               labels64)))
             return rc;
         return launch_small_finalize(w.small_part, small_grid(N, D, K), K, D, C, C_new, D, nullptr, shift, sse, st);
     }
@@ -511,6 +513,26 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
     }
     if (sse) rc = launch_sum_min_d2(w.min_d2, N, sse, w.red, 1, st);
     return rc;
+}
+
+int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
+                       float* C_new, int32_t K, int32_t* labels, float* shift, float* sse, void* ws,
+                       size_t ws_bytes, void* hip_stream) {
+    return lloyd_step_f32(X, N, D, ldx, C, C_new, K, labels, false, shift, sse, ws, ws_bytes, hip_stream);
+}
+
+int hkm_lloyd_step_labels64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new,
+                                int32_t K, int64_t* labels, float* shift, float* sse, void* ws, size_t ws_bytes,
+                                void* hip_stream) {
+    g_err[0] = 0;
+    if (!labels && N > 0) return fail(HKM_EINVAL, "labels is NULL");
+    if (reinterpret_cast<uintptr_t>(labels) & 7u) return fail(HKM_EINVAL, "labels is not 8-byte aligned");
+    if (D >= 1 && K >= 1 && !small_eligible(D, K))
+        return fail(HKM_EUNSUPPORTED,
+                    "D = %d, K = %d: only the narrow one-sweep step (hkm_lloyd_kernel_name() == \"lloyd_small\") stores "
+                    "64-bit labels itself; use hkm_lloyd_step_f32 and hkm_widen_labels_i64", D, K);
+    return lloyd_step_f32(X, N, D, ldx, C, C_new, K, reinterpret_cast<int32_t*>(labels), true, shift, sse, ws, ws_bytes,
+                          hip_stream);
 }
 
 int hkm_lloyd_fit_supported(int64_t N, int32_t D, int32_t K) {

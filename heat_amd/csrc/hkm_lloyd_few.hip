@@ -309,7 +309,7 @@ static int launch_few_t(const float* X, int64_t N, int32_t D, int64_t ldx, const
                                                hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));         \
             if (e != hipSuccess) return fail(HKM_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));      \
         }                                                                                                     \
-        prof_begin(st);                                                                                       \
+        if (!gate) prof_begin(st); /* (a gated launch that returns at once is no sample of the kernel's time) */ \
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(T), lds,     st, X, N, D, ldx, C, K, ldc, labels, \
                            min_d2, ntiles, fsum, fcnt, flags, range_bits, nrep, lda, cstride, mode, gate,    \
                            ngate);                                                                            \
@@ -322,7 +322,7 @@ static int launch_few_t(const float* X, int64_t N, int32_t D, int64_t ldx, const
         else HKM_FEW_GO(false, false);
     }
 #undef HKM_FEW_GO
-    prof_end(st);
+    if (!gate) prof_end(st);
     return check_launch("lloyd_few_kernel");
 }
 

@@ -151,6 +151,18 @@ int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const 
                        size_t ws_bytes, void* hip_stream);
 
 /*
+ * hkm_lloyd_step_f32 with the labels stored as the int64 the reference returns (heat/core/_operations.py:516-522),
+ * for the shapes whose step is "lloyd_small" (hkm_lloyd_kernel_name): a fit whose last iteration is known in
+ * advance (the max_iter-th) runs that one step through this entry point and needs neither a pass over X for its
+ * labels nor a pass over the labels to widen them.  labels must not be NULL here and must be 8-byte aligned; same
+ * centroids, shift and sse as hkm_lloyd_step_f32, bit for bit.  Other shapes return HKM_EUNSUPPORTED.
+ * Replaces the loop body of heat/cluster/kmeans.py:131-143 in the fit's last iteration.
+ */
+int hkm_lloyd_step_labels64_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C, float* C_new,
+                                int32_t K, int64_t* labels, float* shift, float* sse, void* ws, size_t ws_bytes,
+                                void* hip_stream);
+
+/*
  * The WHOLE Lloyd loop in one launch, for data that stays in the registers of a few dozen workgroups:
  *   for it in 1..max_iter: labels against C; C = per-cluster means; shift = sum((C_old - C)^2);
  *                          stop after the first iteration with use_tol != 0 and shift <= tol

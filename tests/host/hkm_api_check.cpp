@@ -102,6 +102,14 @@ int main() {
     EXPECT(hkm_assign_labels64_f32(f, 10, 3, 2, f, 8, 3, i64, nullptr, nullptr), HKM_EINVAL);
     EXPECT(hkm_assign_labels64_f32(f, 10, 32, 32, f, 8, 32, i64, nullptr, nullptr), HKM_EUNSUPPORTED);
     EXPECT(hkm_assign_labels64_f32(f, 0, 3, 3, f, 8, 3, i64, nullptr, nullptr), HKM_OK);
+    // the step that stores 64-bit labels: labels required and aligned, narrow shapes only, the usual checks behind
+    EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 3, 3, f, f + 4096, 8, nullptr, f, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 3, 3, f, f + 4096, 8,
+                                       reinterpret_cast<int64_t*>(reinterpret_cast<char*>(i64) + 4), f, nullptr, ws, big,
+                                       nullptr), HKM_EINVAL);
+    EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 32, 32, f, f + 4096, 8, i64, f, nullptr, ws, big, nullptr), HKM_EUNSUPPORTED);
+    EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 3, 3, f, f, 8, i64, f, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 3, 3, f, f + 4096, 8, i64, f, nullptr, ws, 16, nullptr), HKM_EWORKSPACE);
 
     // ---- the allocation-free assignment: its built-in scratch has a stated size
     EXPECT(hkm_assign_static_f32(nullptr, 10, 3, 3, f, 8, 3, i32, nullptr, nullptr), HKM_EINVAL);

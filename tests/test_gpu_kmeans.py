@@ -419,6 +419,53 @@ def test_last_step_of_a_run_stores_the_labels_of_few_cluster_fits(cuda):
         assert torch.equal(a.centers, b.centers) and torch.equal(a.labels, b.labels)
 
 
+@pytest.mark.parametrize("n,d,k", [(300000, 3, 8), (400001, 8, 16), (1 << 20, 2, 40), (270000, 16, 8), (300000, 5, 12)])
+def test_last_step_of_a_narrow_fit_writes_the_int64_labels_itself(cuda, n, d, k):
+    """Narrow shapes beyond the one-launch fit: the steps store no labels, and the one known to be a run's last
+    (the max_iter-th) writes the (N, 1) int64 labels the reference returns straight into the result
+    (hkm_lloyd_step_labels64_f32) -- same labels as the pass over X afterwards, same centroids and shift as the
+    step without labels, whether the fit ends at max_iter or before."""
+    from heat_amd import _native
+    from heat_amd.cluster._lloyd import LloydLoop
+
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_small" and not _native.lloyd_fit_supported(n, d, k)
+    g = torch.Generator().manual_seed(7 * d + k)
+    centres = torch.randn((k, d), generator=g) * 2.0
+    x = (centres[torch.randint(0, k, (n,), generator=g)] + torch.randn((n, d), generator=g)).to(cuda)
+    c0 = x[:k].clone()
+    for steps, tol in ((3, -1.0), (1, -1.0), (60, 1e-4), (2, None)):
+        out_a = torch.full((n,), -5, dtype=torch.int64, device=cuda)
+        a = LloydLoop(x, c0, _native.Workspace(cuda))
+        a.final_labels64(out_a)
+        b = LloydLoop(x, c0, _native.Workspace(cuda))
+        ra, rb = a.run(steps, tol), b.run(steps, tol)
+        assert ra == rb and torch.equal(a.centers, b.centers)
+        assert float(a.last_shift) == float(b.last_shift)
+        if ra == steps:
+            assert a._lab64_of == a.done - 1  # written by the step
+        a.labels64_into(out_a)
+        out_b = torch.empty((n,), dtype=torch.int64, device=cuda)
+        b.labels64_into(out_b)
+        assert torch.equal(out_a, out_b)
+        assert torch.equal(out_a, a.labels.long())
+    # the entry point refuses other shapes and wrong label vectors
+    ws = _native.Workspace(cuda)
+    wide = torch.zeros((100, 32), device=cuda)
+    with pytest.raises(_native.HkmError):
+        _native.prepare_lloyd_step(wide, wide[:4].clone(), torch.empty((4, 32), device=cuda),
+                                   torch.empty((100,), dtype=torch.int64, device=cuda), torch.empty((), device=cuda),
+                                   None, ws, labels64=True)()
+    with pytest.raises(ValueError):
+        _native.prepare_lloyd_step(x, c0, torch.empty_like(c0), torch.empty((n,), dtype=torch.int32, device=cuda),
+                                   torch.empty((), device=cuda), None, ws, labels64=True)
+    # through the estimator: labels_ of a fit that ends at max_iter equal predict() on the centroids it started from
+    km = ht.cluster.KMeans(n_clusters=k, init=ht.array(c0), max_iter=3, tol=-1.0).fit(ht.array(x, split=0))
+    ref = LloydLoop(x, c0, _native.Workspace(cuda))
+    ref.run(3, -1.0)
+    assert km.n_iter_ == 3 and torch.equal(km.labels_.larray.view(-1), ref.labels.long())
+    assert torch.equal(km.cluster_centers_.larray, ref.centers)
+
+
 # ---- closed forms of the loop (heat/cluster/kmeans.py:131-146) through the public estimator --------
 # shapes: the one-sweep matrix-core step (D = 32), the narrow one-sweep step (D = 3 and D = 8), and a
 # shape that runs assignment + two-pass update (D = 100)
