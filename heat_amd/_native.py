@@ -19,7 +19,7 @@ from . import _f64_paths
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhkm.so")
 _lib: Optional[ctypes.CDLL] = None
 
-LIB_VERSION = 307  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
+LIB_VERSION = 308  # hkm_version() this binding was written for: major * 10000 + minor * 100 + patch
 HKM_OK, HKM_EINVAL, HKM_EWORKSPACE, HKM_EHIP, HKM_EUNSUPPORTED = 0, -1, -2, -3, -4
 WS_ASSIGN, WS_UPDATE, WS_LLOYD, WS_SSE, WS_MEDIAN, WS_F64, WS_FIT = 1, 2, 3, 4, 8, 16, 32
 
@@ -44,6 +44,7 @@ SIGNATURES = {
     "hkm_lloyd_step_labels64_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_void_p, c_int32,
                                                    c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "hkm_lloyd_fit_supported": (ctypes.c_int, [c_int64, c_int32, c_int32]),
+    "hkm_lloyd_step_labels_optional": (ctypes.c_int, [c_int64, c_int32, c_int32]),
     "hkm_lloyd_fit_f32": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int64, c_void_p, c_int32, c_int32, c_int32,
                                          ctypes.c_double, c_void_p, c_void_p, c_void_p, c_void_p, ctypes.c_uint64,
                                          c_void_p, c_size_t, c_void_p]),
@@ -293,6 +294,11 @@ def lloyd_step(x: torch.Tensor, c: torch.Tensor, c_new: torch.Tensor, labels: Op
     buf = ws.get(need)
     check(load().hkm_lloyd_step_f32(_ptr(x), n, d, x.stride(0) if n > 1 else d, _ptr(c), _ptr(c_new), k,
                                     _ptr(labels), _ptr(shift), _ptr(sse), _ptr(buf), buf.numel(), _stream()))
+
+
+def lloyd_step_labels_optional(n: int, d: int, k: int) -> bool:
+    """Whether :func:`lloyd_step` accepts ``labels=None`` for this shape (float32 only)."""
+    return bool(load().hkm_lloyd_step_labels_optional(n, d, k))
 
 
 def lloyd_fit_supported(n: int, d: int, k: int) -> bool:

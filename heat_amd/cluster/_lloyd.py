@@ -53,11 +53,12 @@ class LloydLoop:
         self.c = [c0.clone(), torch.empty_like(c0), torch.empty_like(c0)]
         n, d = xt.shape
         kernel = _native.lloyd_kernel_name(n, d, c0.shape[0]) if xt.dtype == torch.float32 else ""
-        self.lazy_labels = kernel in ("lloyd_small", "lloyd_few")
+        # the one-sweep steps that memory bounds: the two vector kernels'
+        self.lazy_labels = bool(kernel) and _native.lloyd_step_labels_optional(n, d, c0.shape[0])
         # A step known to be the last of a run (the max_iter-th) stores its labels after all: one more stream of
-        # writes in one step instead of one more pass over X afterwards.  Not for the narrow shapes, whose final
-        # pass writes the int64 labels the caller wants at once.
-        self._label_last = kernel == "lloyd_few"
+        # writes in one step instead of one more pass over X afterwards.  (The narrow shapes' last step writes the
+        # int64 labels the caller wants, see below.)
+        self._label_last = self.lazy_labels and kernel != "lloyd_small"
         # The narrow shapes' last step can store the int64 labels the caller wants at once, into the caller's own
         # vector (final_labels64): neither the pass over X nor the widening pass is left.
         self._narrow = kernel == "lloyd_small"

@@ -105,6 +105,11 @@ bool fused_eligible(int32_t D, int32_t K) {
     return D >= 2 && D <= RESIDENT_MAX_D && resident_lds_bytes(D, K) <= 64 * 1024 && fused_lds_bytes(D, K) <= 160 * 1024;
 }
 
+// labels == NULL is accepted by hkm_lloyd_step_f32: the one-sweep steps of the two vector kernels, which memory
+// bounds.  (The matrix-core step with few centroids was tried too: 10M x 128, K = 8: 1.203 -> 1.186 ms, 10M x 96,
+// K = 32: 0.984 -> 0.972 ms -- its fp64 sums bound it, not the labels; it keeps storing them.)
+static bool step_labels_optional(int32_t D, int32_t K) { return small_eligible(D, K) || few_eligible(D, K); }
+
 static size_t cn_pad(int32_t K) { return (size_t(K) + 127) / 128 * 128; }
 
 Workspace carve(void* base, int64_t N, int32_t D, int32_t K, int32_t flags) {
@@ -281,7 +286,7 @@ using namespace hkm;
 
 extern "C" {
 
-int hkm_version(void) { return 307; }
+int hkm_version(void) { return 308; }
 
 const char* hkm_last_error(void) { return g_err; }
 
@@ -467,8 +472,9 @@ static int lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, con
     if ((rc = check_matrix("C", C, K, D, D))) return rc;
     if ((rc = check_matrix("C_new", C_new, K, D, D))) return rc;
     if (C == C_new) return fail(HKM_EINVAL, "C and C_new must not alias");
-    if (!labels && N > 0 && !small_eligible(D, K) && !few_eligible(D, K))
-        return fail(HKM_EINVAL, "labels is NULL (only the one-sweep vector-ALU steps can run without storing labels)");
+    if (!labels && N > 0 && !step_labels_optional(D, K))
+        return fail(HKM_EINVAL, "labels is NULL (hkm_lloyd_step_labels_optional() says which steps can run without "
+                                "storing labels)");
     if (!shift) return fail(HKM_EINVAL, "shift is NULL");
     const int32_t flags = HKM_WS_LLOYD | (sse ? HKM_WS_SSE : 0);
     const size_t need = carve(nullptr, N, D, K, flags).total;
@@ -498,8 +504,8 @@ static int lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, con
         if (few && !labels) {
             // the step stored no labels; the two-pass update that redoes the sums of a flagged step needs them:
             // one more launch, which returns at once unless a flag is up
-            const int grid = few_grid(N, D, K);
-            if ((rc = launch_few(X, N, D, ldx, C, K, D, w.lazy_lab, nullptr, nullptr, nullptr, nullptr, st, w.fflags, grid)))
+            if ((rc = launch_few(X, N, D, ldx, C, K, D, w.lazy_lab, nullptr, nullptr, nullptr, nullptr, st, w.fflags,
+                                 few_grid(N, D, K))))
                 return rc;
             labels = w.lazy_lab;
         }
@@ -533,6 +539,11 @@ int hkm_lloyd_step_labels64_f32(const float* X, int64_t N, int32_t D, int64_t ld
                     "64-bit labels itself; use hkm_lloyd_step_f32 and hkm_widen_labels_i64", D, K);
     return lloyd_step_f32(X, N, D, ldx, C, C_new, K, reinterpret_cast<int32_t*>(labels), true, shift, sse, ws, ws_bytes,
                           hip_stream);
+}
+
+int hkm_lloyd_step_labels_optional(int64_t N, int32_t D, int32_t K) {
+    if (N < 0 || D < 1 || K < 1) return 0;
+    return step_labels_optional(D, K) ? 1 : 0;
 }
 
 int hkm_lloyd_fit_supported(int64_t N, int32_t D, int32_t K) {

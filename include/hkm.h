@@ -137,11 +137,11 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
 /*
  * One Lloyd iteration: labels against C, C_new = per-cluster means, *shift = sum((C - C_new)^2)
  * (fp32 value, device scalar), optional *sse = sum_i min_d2[i] (device scalar; NULL to skip).
- * C and C_new are K x D with leading dimension D.  labels may be NULL for the shapes
- * hkm_lloyd_kernel_name() reports as "lloyd_small" or "lloyd_few": the step then stores no labels (4 of
- * its 4D+4 bytes per point; next to a stream of reads even so small a stream of writes costs a sixth of
- * the read bandwidth) -- a fit needs only those of its last iteration, which hkm_assign_f32 against
- * the previous centroids reproduces bit for bit.  shift (and sse) may also point to pinned,
+ * C and C_new are K x D with leading dimension D.  labels may be NULL where
+ * hkm_lloyd_step_labels_optional() says so -- the one-sweep steps that memory bounds ("lloyd_small" and
+ * "lloyd_few"): the step then stores no labels (4 of its 4D+4 bytes per point; next to a stream of reads even
+ * so small a stream of writes costs up to a sixth of the read bandwidth) -- a fit needs only those of its last
+ * iteration, which hkm_assign_f32 against the previous centroids reproduces bit for bit.  shift (and sse) may also point to pinned,
  * device-accessible host memory: the finishing kernel then delivers the scalar itself and no copy
  * sits between two steps on the stream.
  * Replaces the loop body of heat/cluster/kmeans.py:131-143 (KMeans.fit).
@@ -149,6 +149,9 @@ int hkm_update_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const int3
 int hkm_lloyd_step_f32(const float* X, int64_t N, int32_t D, int64_t ldx, const float* C,
                        float* C_new, int32_t K, int32_t* labels, float* shift, float* sse, void* ws,
                        size_t ws_bytes, void* hip_stream);
+
+/* 1 if hkm_lloyd_step_f32 accepts labels == NULL for this shape, else 0. */
+int hkm_lloyd_step_labels_optional(int64_t N, int32_t D, int32_t K);
 
 /*
  * hkm_lloyd_step_f32 with the labels stored as the int64 the reference returns (heat/core/_operations.py:516-522),

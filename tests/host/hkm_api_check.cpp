@@ -102,6 +102,13 @@ int main() {
     EXPECT(hkm_assign_labels64_f32(f, 10, 3, 2, f, 8, 3, i64, nullptr, nullptr), HKM_EINVAL);
     EXPECT(hkm_assign_labels64_f32(f, 10, 32, 32, f, 8, 32, i64, nullptr, nullptr), HKM_EUNSUPPORTED);
     EXPECT(hkm_assign_labels64_f32(f, 0, 3, 3, f, 8, 3, i64, nullptr, nullptr), HKM_OK);
+    if (hkm_lloyd_step_labels_optional(1000, 32, 8) != 1 || hkm_lloyd_step_labels_optional(1000, 32, 256) != 0 ||
+        hkm_lloyd_step_labels_optional(1000, 0, 8) != 0 || hkm_lloyd_step_labels_optional(-1, 3, 8) != 0) {
+        std::printf("FAIL hkm_lloyd_step_labels_optional\n");
+        ++failures;
+    }
+    EXPECT(hkm_lloyd_step_f32(f, 10, 32, 32, f, f + 4096, 256, nullptr, f, nullptr, ws, big, nullptr), HKM_EINVAL);
+    EXPECT_MSG("labels is NULL");
     // the step that stores 64-bit labels: labels required and aligned, narrow shapes only, the usual checks behind
     EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 3, 3, f, f + 4096, 8, nullptr, f, nullptr, ws, big, nullptr), HKM_EINVAL);
     EXPECT(hkm_lloyd_step_labels64_f32(f, 10, 3, 3, f, f + 4096, 8,

@@ -198,6 +198,10 @@ def test_workspace_and_kernel_selection():
     assert _native.lloyd_kernel_name(200_000_000, 3, 8) == "lloyd_small"
     assert _native.lloyd_kernel_name(10_000_000, 32, 256) == "lloyd_mfma_resident"
     assert _native.lloyd_kernel_name(10_000_000, 64, 512) == "mfma_tiled+update"  # accumulators exceed LDS
+    # steps that may run without storing labels: those of the two vector kernels
+    for d, k, opt in ((3, 8, True), (8, 16, True), (32, 8, True), (64, 12, True), (128, 8, False), (96, 32, False),
+                      (32, 32, False), (32, 256, False), (16, 32, False), (512, 8, False), (8, 64, False)):
+        assert _native.lloyd_step_labels_optional(10_000_000, d, k) == opt, (d, k)
     # few clusters of 17 to 64 features: the vector kernel, for the step and for the assignment alone
     for d, k, few in ((32, 8, True), (17, 1, True), (40, 16, True), (64, 12, True), (64, 13, False), (44, 16, False),
                       (16, 8, False), (65, 8, False), (32, 17, False)):

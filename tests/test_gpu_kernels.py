@@ -514,7 +514,7 @@ def test_few_cluster_step_without_labels_equals_the_step_with_labels(cuda, n, d,
     as the step that stores them -- on the exact path, and where a workgroup raises its flag (row magnitudes
     spread over 2^60, non-finite rows): there the labels the two-pass update needs are computed into the
     workspace by one more launch, which otherwise returns at once."""
-    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_few"
+    assert _native.lloyd_kernel_name(n, d, k) == "lloyd_few" and _native.lloyd_step_labels_optional(n, d, k)
     x, _ = _data(n, d, k, seed=3 * n + d)
     g = torch.Generator().manual_seed(5)
     for variant in ("plain", "wide", "nonfinite"):
