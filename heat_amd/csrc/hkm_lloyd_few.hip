@@ -6,10 +6,10 @@
 // ALU needs K (D + 4) instructions per point -- less than the time X takes to arrive from memory -- so the
 // assignment is bound by HBM: 4 D + 4 bytes per point.
 //
-// A lane owns one row, held in registers (D/4 16-byte loads straight from its row; non-temporal when X exceeds
-// the last-level cache); the next round's rows are requested before the current ones are scanned.  (Fetching a
-// wave's 64 rows as one contiguous piece and handing every lane its row through LDS was measured and is slower:
-// the loads as they are already move what the memory delivers to any kernel, and LDS is busy with the sums.)
+// A lane owns one row, held in registers (D/4 16-byte loads straight from its row -- plain loads: with 16
+// contiguous bytes per lane, loads that pass the caches fetch every line several times and are 2-3 times slower);
+// the next round's rows are requested before the current ones are scanned.  (Fetching a wave's 64 rows in whole
+// cache lines and handing every lane its row through LDS was built and measured: no faster in this kernel.)
 // The centroids
 // are the same for every lane, so they are read through the scalar unit (uniform loads from the constant address
 // space) and enter the multiply-adds as scalar operands: no LDS traffic and no vector registers for them.  The
@@ -117,7 +117,6 @@ __global__ __launch_bounds__(T) void lloyd_few_kernel(
         if (!__syncthreads_or(up)) return;
     }
     const bool vec = (mode & 1) != 0;     // rows are whole aligned 16-byte groups
-    const bool stream = (mode & 2) != 0;  // X exceeds the last-level cache
     const few_cptr Cc = (few_cptr)C;
 
     for (int r = tid; r < K; r += T) {
@@ -166,7 +165,7 @@ __global__ __launch_bounds__(T) void lloyd_few_kernel(
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
                 const floatx4* q = reinterpret_cast<const floatx4*>(xr + 4 * j);
-                dst[j] = stream ? __builtin_nontemporal_load(q) : *q;
+                dst[j] = *q;
             }
         } else {
 #pragma unroll
@@ -295,7 +294,7 @@ static int launch_few_t(const float* X, int64_t N, int32_t D, int64_t ldx, const
     const int nrep = g.rep;
     const size_t lds = few_lds_bytes(D, K, fused ? nrep : 0);
     const int lda = few_lda(D, nrep), cstride = few_copy_stride(D, K, nrep);
-    const int mode = (vec ? 1 : 0) | (N * int64_t(D) * 4 > (int64_t(256) << 20) ? 2 : 0);
+    const int mode = vec ? 1 : 0;
     // rows one workgroup adds up, as a power of two
     const int64_t per_wg = (ntiles + grid - 1) / grid * T;
     int lg = 0;
