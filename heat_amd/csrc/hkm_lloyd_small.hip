@@ -81,6 +81,13 @@ struct SmallCfg {
     // with 2 and 64, 0.53 instead of 0.67 ms with 3 and 40; from a dozen centroids on it is never slower.
     // Rows of 5 to 7 coordinates (two reads per row, more registers) run 0-18 % slower that way.
     static constexpr bool BLOCKED = D <= 3;
+    // The wave's staging buffer holds a round as 64 rows, one per lane, of the lane's PPT points (RL floats); the
+    // rows are RLP floats apart, a multiple of 4 whose quarter is odd: the 16 lanes that read 16 bytes each
+    // together then meet no LDS bank twice (with rows of 16 floats back to back they met four times, with 32 eight
+    // times).  Point q of the round starts at stage_off(q).
+    static constexpr int RL = PPT * D;
+    static constexpr int RLP = (RL / 4) % 2 == 1 ? RL : RL + 4;
+    static constexpr int stage_off(int q) { return (q / PPT) * RLP + (q % PPT) * D; }
 };
 
 bool small_eligible(int32_t D, int32_t K) { return D <= 16 && K * (D + 1) <= 240; }
@@ -100,9 +107,9 @@ __host__ __device__ constexpr int small_int_stride(int D) { return D + 1; }
 // DPP tree, 3 wave rows by the matrix cores, 4 integer tables)
 static size_t small_lds_bytes(int32_t D, int32_t K, int acc_mode) {
     const int ppt = (D % 2 == 0) ? 2 : 4;
-    const int sc = (D + 1 + 3) / 4 * 4, nv = ppt * D / 4, slots = K * (D + 1);
+    const int sc = (D + 1 + 3) / 4 * 4, rl = ppt * D, rlp = (rl / 4) % 2 == 1 ? rl : rl + 4, slots = K * (D + 1);  // as SmallCfg
     const size_t xch = (D == 4 || D == 8) ? size_t(SMALL_T / 64) * 256 * sizeof(float) : 0;  // as SmallCfg::MSCAN
-    return size_t(((K + 3) & ~3) * sc) * sizeof(float) + size_t(SMALL_T / 64) * nv * 256 * sizeof(float) + xch +
+    return size_t(((K + 3) & ~3) * sc) * sizeof(float) + size_t(SMALL_T / 64) * 64 * rlp * sizeof(float) + xch +
            (acc_mode == 2   ? size_t(SMALL_T / 64) * slots * sizeof(double)
             : acc_mode == 3 ? size_t(SMALL_T / 64) * (slots * sizeof(double) + 64 * ppt * sizeof(int))
             : acc_mode == 1 ? size_t(slots + D + 1) * SMALL_T * sizeof(float)
@@ -371,10 +378,11 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
     const int slots = K * (D + 1);
     constexpr bool ACCUM = ACC != 0;
     const int KP = (K + 3) & ~3;                                     // rows of sC: K, then +inf-norm rows up to a multiple of four
-    float* stage = lds + KP * SC;                                    // [NW][NV*64*4] transpose buffer
+    constexpr int RL = SmallCfg<D>::RL, RLP = SmallCfg<D>::RLP;
+    float* stage = lds + KP * SC;                                    // [NW][64][RLP] transpose buffer
     // matrix-core scan: [NW][128] (minimum, index) pairs on their way from the lane that found them to the
     // lane that owns the point
-    float* xch_all = stage + NW * NV * 256;
+    float* xch_all = stage + NW * 64 * RLP;
     float* after = xch_all + (SmallCfg<D>::MSCAN ? NW * 256 : 0);
     double* wacc_all = reinterpret_cast<double*>(after);             // ACC==2: [NW][slots]
     float* cols = after;                                             // ACC==1: [slots][T]
@@ -395,7 +403,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
         if (!__syncthreads_or(any)) return;
     }
     int* wlab = reinterpret_cast<int*>(wacc_all + NW * slots) + wave * (64 * PPT);  // ACC==3: [4][16*PPT]
-    float* wstage = stage + wave * NV * 256;
+    float* wstage = stage + wave * 64 * RLP;
 
     const int64_t groups = (N + PPT - 1) / PPT;
     const int64_t full = (vec & 1) ? N / PPT : 0;  // groups served by the 16-byte vector path
@@ -581,7 +589,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 // of point lane % 16 to centroids 4 (lane / 16) + r; two swaps of lane rows per register
                 // (across the halves of the wave, then between neighbouring rows) transpose that, so that
                 // lane 16 g + n ends up with all sixteen distances of point n of group g, in centroid order.
-                const float* brow = wstage + (lane & 15) * D + (lane >> 4);
+                const float* brow = wstage + SmallCfg<D>::stage_off(lane & 15) + (lane >> 4);  // (16 j, 64 half: whole rows)
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     floatx4 acc[4];
@@ -589,7 +597,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
 #pragma unroll
-                        for (int st = 0; st < D / 4; ++st) bv[j][st] = brow[(half * 64 + 16 * j) * D + 4 * st];
+                        for (int st = 0; st < D / 4; ++st) bv[j][st] = brow[SmallCfg<D>::stage_off(half * 64 + 16 * j) + 4 * st];
                     wave_lds_sync();
 #pragma unroll
                     for (int st = 0; st < D / 4; ++st)
@@ -753,7 +761,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                 const int lbs[4] = {lb.x, lb.y, lb.z, lb.w};
                 float bv[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) bv[u] = wstage[(4 * (g4 + u) + kk) * D + cread];
+                for (int u = 0; u < 4; ++u) bv[u] = wstage[SmallCfg<D>::stage_off(4 * (g4 + u) + kk) + cread];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const float bval = col < D ? bv[u] : bconst;
@@ -811,7 +819,8 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
                     wave_lds_sync();
 #pragma unroll
                     for (int v = 0; v < NV; ++v)
-                        *reinterpret_cast<floatx4*>(wstage + v * 256 + lane * 4) = nxt[f][v];
+                        *reinterpret_cast<floatx4*>(wstage + ((v * 256 + lane * 4) / RL) * RLP + (v * 256 + lane * 4) % RL) =
+                            nxt[f][v];  // (piece v * 64 + lane of the round, in memory order, into its lane's row)
                     wave_lds_sync();
                     if (base + PF * stride + T <= full) {
 #pragma unroll
@@ -821,7 +830,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
                     for (int v = 0; v < NV; ++v) {
                         const floatx4 q =
-                            *reinterpret_cast<const floatx4*>(wstage + lane * (PPT * D) + 4 * v);
+                            *reinterpret_cast<const floatx4*>(wstage + lane * RLP + 4 * v);
 #pragma unroll
                         for (int t = 0; t < 4; ++t) x[(4 * v + t) / D][(4 * v + t) % D] = q[t];
                     }
@@ -848,7 +857,7 @@ __global__ __launch_bounds__(SMALL_T) void lloyd_small_kernel(
 #pragma unroll
             for (int p = 0; p < PPT; ++p)
 #pragma unroll
-                for (int d = 0; d < D; ++d) wstage[(lane * PPT + p) * D + d] = x[p][d];
+                for (int d = 0; d < D; ++d) wstage[lane * RLP + p * D + d] = x[p][d];
             wave_lds_sync();
         }
         process(i0, x, std::true_type{});
